@@ -1,0 +1,201 @@
+/*
+ * lpmm_hip.h -- C ABI of the MI355X (gfx950) kernels for lpmm's 4-bit optimizer-state
+ * hot path.  Plain pointers and sizes only: no torch types, no exceptions, no global
+ * state; every call is asynchronous on the given HIP stream and re-entrant.
+ *
+ * All pointers are DEVICE pointers unless a parameter is documented as host memory.
+ * `stream` is a hipStream_t passed as void* (NULL = the HIP null stream).
+ * Every function returns an lpmm_status; 0 means the work was enqueued.
+ * Argument validation happens before any HIP call, so bad arguments are reported
+ * without touching a GPU.
+ *
+ * Each entry point names the reference interface it replaces (paths relative to the
+ * thu-ml/low-bit-optimizers repository root).
+ */
+#ifndef LPMM_HIP_H
+#define LPMM_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define LPMM_HIP_ABI_VERSION 1
+
+/* One quantisation group of the fused path = 128 elements = one scale
+ * (lpmm/cpp_extension/fused_adamw_kernel.cu:216-219). */
+#define LPMM_GROUP 128
+/* Padding unit of the non-fused packed layout (lpmm/functional.py:362). */
+#define LPMM_PACK_GROUP 2048
+/* Most tensors one multi-tensor launch record can hold. */
+#define LPMM_MULTI_MAX 48
+
+typedef enum lpmm_status {
+    LPMM_OK = 0,
+    LPMM_ERR_NULL = 1,      /* a required pointer is NULL */
+    LPMM_ERR_ALIGN = 2,     /* a pointer does not meet its stated alignment */
+    LPMM_ERR_SIZE = 3,      /* a size/count is negative, zero where it may not be, or too big */
+    LPMM_ERR_LAUNCH = 4,    /* the HIP runtime reported an error at launch */
+    LPMM_ERR_ARG = 5        /* an enum/flag argument has an unknown value */
+} lpmm_status;
+
+const char *lpmm_status_string(int status);
+int lpmm_abi_version(void);
+
+/* ---------------------------------------------------------------------------------------
+ * (a) Fused 4-bit AdamW step on one tensor, in place.
+ * Replaces fused_adamw.adamw4bit_single_tensor
+ *   (lpmm/cpp_extension/fused_adamw.cc:44-78, kernel fused_adamw_kernel.cu:81-174).
+ *   p, g            fp32[n]                       (p updated in place; g read only)
+ *   m_codes,v_codes uint8[(n+1)/2]                two 4-bit codes per byte, low nibble = even index
+ *   m_scale,v_scale fp32[ceil(n/128)]             one scale per 128 elements
+ *   qmap_m, qmap_v  fp32[16]                      ascending quantisation maps
+ *   step            the reference's float step count (>= 1)
+ * p and g need 4-byte alignment; 16-byte alignment of p and g and 4-byte alignment of the
+ * code arrays selects the vectorised path (any torch allocation has it).
+ * ------------------------------------------------------------------------------------- */
+int lpmm_adamw4bit_step(float *p, const float *g, uint8_t *m_codes, uint8_t *v_codes,
+                        float *m_scale, float *v_scale, const float *qmap_m,
+                        const float *qmap_v, int64_t n, float beta1, float beta2, float lr,
+                        float weight_decay, float eps, float step, void *stream);
+
+/* One record of a multi-tensor launch; the array of records is HOST memory. */
+typedef struct lpmm_adamw4bit_tensor {
+    float *p;
+    const float *g;
+    uint8_t *m_codes;
+    uint8_t *v_codes;
+    float *m_scale;
+    float *v_scale;
+    int64_t n;
+    float step;
+    float reserved;
+} lpmm_adamw4bit_tensor;
+
+/* The same step over `count` tensors (host array `tensors`) in as few launches as
+ * possible.  Replaces the per-tensor Python loop of _fused_adamw4bit
+ * (lpmm/optim/adamw.py:463-542), one reference launch per tensor.  Each tensor carries
+ * its own step (adamw.py:498); hyper-parameters are per parameter group, as in the
+ * reference. */
+int lpmm_adamw4bit_step_multi(const lpmm_adamw4bit_tensor *tensors, int64_t count,
+                              const float *qmap_m, const float *qmap_v, float beta1,
+                              float beta2, float lr, float weight_decay, float eps,
+                              void *stream);
+
+/* Fused fp32-state AdamW step (tensors at or under the quantisation threshold).
+ * Replaces fused_adamw.adamw_single_tensor
+ *   (lpmm/cpp_extension/fused_adamw.cc:15-41, kernel fused_adamw_kernel.cu:52-78). */
+int lpmm_adamw_fp32_step(float *p, const float *g, float *m, float *v, int64_t n, float beta1,
+                         float beta2, float lr, float weight_decay, float eps, float step,
+                         void *stream);
+
+typedef struct lpmm_adamw_fp32_tensor {
+    float *p;
+    const float *g;
+    float *m;
+    float *v;
+    int64_t n;
+    float step;
+    float reserved;
+} lpmm_adamw_fp32_tensor;
+
+/* Multi-tensor form of the fp32-state step (the `else` branch of _fused_adamw4bit,
+ * lpmm/optim/adamw.py:543-561). */
+int lpmm_adamw_fp32_step_multi(const lpmm_adamw_fp32_tensor *tensors, int64_t count,
+                               float beta1, float beta2, float lr, float weight_decay,
+                               float eps, void *stream);
+
+/* ---------------------------------------------------------------------------------------
+ * (b) Stand-alone quantise / dequantise in the non-fused packed layout
+ *     (NG*1024 + 1 bytes, NG = ceil(numel_scaled/2048); lpmm/functional.py:359-369,
+ *     quantization_kernel.cu:475-477).  The trailing byte is written as 0.
+ * ------------------------------------------------------------------------------------- */
+
+/* Replaces ext_quantization.pack_nonlinear for bits = 4, stochastic = false
+ *   (lpmm/cpp_extension/quantization.cc:54-63, quantization_kernel.cu:430-513).
+ * x: fp32[n_padded] already normalised, n_padded a multiple of 8; out: n_padded/2 + 1 bytes. */
+int lpmm_pack_nonlinear_4bit(const float *x, const float *qmap, int64_t n_padded, uint8_t *out,
+                             void *stream);
+
+/* Replaces ext_quantization.unpack_nonlinear for bits = 4
+ *   (lpmm/cpp_extension/quantization.cc:65-76, quantization_kernel.cu:604-653).
+ * out[i] = qmap[code_i] for i < n (n = num_groups * group_size in the reference call). */
+int lpmm_unpack_nonlinear_4bit(const uint8_t *codes, const float *qmap, int64_t n, float *out,
+                               void *stream);
+
+/* vectorwise_quant with scale_type 'group' in one pass: per-group max|x| -> max1, x/max1,
+ * code search, pack.  Replaces lpmm/functional.py:184-189 + :359-369 (abs, max, div, cat,
+ * pack_nonlinear as separate passes).  gp_sz must be a multiple of 128 and a divisor of
+ * 2048 or a multiple of it; codes: ceil(G*gp_sz/2048)*1024 + 1 bytes; max1: fp32[G],
+ * G = ceil(n/gp_sz). */
+int lpmm_quant_group(const float *x, int64_t n, int64_t gp_sz, const float *qmap, uint8_t *codes,
+                     float *max1, void *stream);
+
+/* vectorwise_dequant with scale_type 'group': out[i] = qmap[code_i] * max1[i / gp_sz].
+ * Replaces lpmm/functional.py:393-400 + :115-118. */
+int lpmm_dequant_group(const uint8_t *codes, const float *max1, const float *qmap, int64_t n,
+                       int64_t gp_sz, float *out, void *stream);
+
+/* Rank-1 statistics of a row-major R x C tensor: rowmax[r] = max_c |x|, colmax[c] = max_r |x|.
+ * Replaces get_sm3_statistics / _max_reduce_except_dim (lpmm/functional.py:512-531).
+ * colmax is accumulated with atomics on the bit patterns of non-negative floats and is
+ * cleared by the call itself. */
+int lpmm_rank1_stats(const float *x, int64_t rows, int64_t cols, float *rowmax, float *colmax,
+                     void *stream);
+
+/* Rank-1 normalise + search + pack: code(x[r,c] / min(rowmax[r], colmax[c])).
+ * Replaces lpmm/functional.py:199-203 + :503-509 + :359-369.  codes: ceil(R*C/2048)*1024+1. */
+int lpmm_quant_rank1(const float *x, int64_t rows, int64_t cols, const float *rowmax,
+                     const float *colmax, const float *qmap, uint8_t *codes, void *stream);
+
+/* out[r,c] = qmap[code] * min(rowmax[r], colmax[c]).  Replaces lpmm/functional.py:97-106. */
+int lpmm_dequant_rank1(const uint8_t *codes, const float *rowmax, const float *colmax,
+                       const float *qmap, int64_t rows, int64_t cols, float *out, void *stream);
+
+/* ---------------------------------------------------------------------------------------
+ * Non-fused step, elementwise part on fp32 m and v (already dequantised):
+ * decoupled decay, lerp, EMA of g*g, bias-corrected update.
+ * Replaces the PyTorch op sequence of _single_tensor_adamw4bit
+ *   (lpmm/optim/adamw.py:367-369, :412-422).  Scalars are doubles, as in Python.
+ * ------------------------------------------------------------------------------------- */
+int lpmm_nonfused_update(float *p, const float *g, float *m, float *v, int64_t n, double beta1,
+                         double beta2, double lr, double weight_decay, double eps, double step,
+                         void *stream);
+
+/* ---------------------------------------------------------------------------------------
+ * (c) Factored second moment on a row-major R x C tensor.
+ * Replaces _single_quantized_factored_update (lpmm/optim/adamw.py:579-627) and
+ * _approx_sq_grad (:571-576).
+ * ------------------------------------------------------------------------------------- */
+
+/* Pass 1: row/col means of g*g folded into the EMAs
+ *   row = beta2*row + (1-beta2)*mean_c(g^2), col likewise (adamw.py:608-610),
+ * and *row_mean_all = mean(row) after the update (adamw.py:574).
+ * workspace: device scratch of lpmm_factored_workspace_bytes(rows, cols) bytes. */
+int64_t lpmm_factored_workspace_bytes(int64_t rows, int64_t cols);
+int lpmm_factored_stats(const float *g, int64_t rows, int64_t cols, float *row, float *col,
+                        float *row_mean_all, double beta2, void *workspace, void *stream);
+
+/* Pass 2: p *= 1-lr*wd; m = dequant(m_codes); m.lerp_(g, 1-beta1);
+ * v = row/row_mean_all * col; p += -lr/bc1 * m / (sqrt(v)/sqrt(bc2) + eps); m re-quantised
+ * with 'group' scaling, gp_sz 128, into the non-fused packed layout (adamw.py:596-625).
+ * first_step != 0 means m starts at zero and m_codes/m_max1 are only written. */
+int lpmm_factored_update(float *p, const float *g, uint8_t *m_codes, float *m_max1,
+                         const float *qmap_m, const float *row, const float *col,
+                         const float *row_mean_all, int64_t rows, int64_t cols, double beta1,
+                         double beta2, double lr, double weight_decay, double eps, double step,
+                         int first_step, void *stream);
+
+/* The same pass with an fp32 first moment (m read and written as floats): tensors at or
+ * under the quantisation threshold, or first-moment quantisation disabled
+ * (the `else: exp_avg = q_exp_avg` branch, lpmm/optim/adamw.py:603-604). */
+int lpmm_factored_update_fp32m(float *p, const float *g, float *m, const float *row,
+                               const float *col, const float *row_mean_all, int64_t rows,
+                               int64_t cols, double beta1, double beta2, double lr,
+                               double weight_decay, double eps, double step, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LPMM_HIP_H */

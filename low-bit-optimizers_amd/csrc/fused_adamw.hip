@@ -1,0 +1,456 @@
+// Fused AdamW steps for gfx950: the 4-bit-state step (decode -> AdamW -> group absmax ->
+// re-quantise -> pack, one pass over HBM) and the fp32-state step for small tensors.
+//
+// Arithmetic follows lpmm/cpp_extension/fused_adamw_kernel.cu:103-172 of the reference
+// operation by operation, each operation rounded once (the file is compiled with
+// -ffp-contract=off, division and sqrt are the correctly rounded ones).
+//
+// Work layout of the 4-bit step: a lane owns 8 consecutive elements (32 B of p, 32 B of g,
+// one 32-bit word of m codes and one of v codes); 16 lanes = one DPP row own one
+// 128-element group, so the group maxima are 7 in-register max + 4 DPP steps and need
+// neither LDS nor atomics.  A 256-thread workgroup covers a tile of 2048 elements.
+#include "lpmm_common.hpp"
+
+#include <math.h>
+
+namespace lpmm {
+
+constexpr int kThreads = 256;
+constexpr int kEltsPerLane = 8;
+constexpr int kTile = kThreads * kEltsPerLane;  // 2048 elements = 16 groups
+
+struct Tensor4 {
+    float *p;
+    const float *g;
+    uint8_t *mc;
+    uint8_t *vc;
+    float *ms;
+    float *vs;
+    int64_t n;
+    float c1;   // 1 - beta1^step
+    float c2s;  // sqrt(1 - beta2^step)
+};
+
+struct Multi4 {
+    Tensor4 t[LPMM_MULTI_MAX];
+    uint32_t tile_start[LPMM_MULTI_MAX + 1];  // prefix sum of tiles per tensor
+    int count;
+    float beta1, beta2, lr, wd, eps;
+};
+
+struct Hyper {
+    float beta1, beta2, omb1, omb2, lr, wd, eps, c1, c2s;
+};
+
+// AdamW on one element; returns the new parameter, updates m and v in place.
+__device__ __forceinline__ float adamw_elt(float p, float g, float &m, float &v, const Hyper &h)
+{
+    m = h.beta1 * m + h.omb1 * g;
+    v = h.beta2 * v + h.omb2 * g * g;
+    const float denom = (sqrtf(v) / h.c2s + h.eps) * h.c1;
+    const float update = (m / denom) + (h.wd * p);
+    return p - (h.lr * update);
+}
+
+template <bool ALIGNED>
+__global__ __launch_bounds__(kThreads) void adamw4bit_kernel(const Multi4 args,
+                                                             const float *__restrict__ qmap_m,
+                                                             const float *__restrict__ qmap_v)
+{
+    __shared__ float s_qm[16];
+    __shared__ float s_qv[16];
+    if (threadIdx.x < 16)
+        s_qm[threadIdx.x] = qmap_m[threadIdx.x];
+    else if (threadIdx.x < 32)
+        s_qv[threadIdx.x - 16] = qmap_v[threadIdx.x - 16];
+
+    // which tensor does this tile belong to (uniform over the workgroup)
+    int lo = 0, hi = args.count;
+    while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (args.tile_start[mid] <= blockIdx.x)
+            lo = mid;
+        else
+            hi = mid;
+    }
+    const Tensor4 &t = args.t[lo];
+    const int64_t n = t.n;
+    const int64_t base = (int64_t)(blockIdx.x - args.tile_start[lo]) * kTile + (int64_t)threadIdx.x * kEltsPerLane;
+
+    Hyper h;
+    h.beta1 = args.beta1;
+    h.beta2 = args.beta2;
+    h.omb1 = 1 - args.beta1;
+    h.omb2 = 1 - args.beta2;
+    h.lr = args.lr;
+    h.wd = args.wd;
+    h.eps = args.eps;
+    h.c1 = t.c1;
+    h.c2s = t.c2s;
+
+    const Mids mids_m = make_mids(qmap_m);
+    const Mids mids_v = make_mids(qmap_v);
+    __syncthreads();
+
+    const int64_t grp = base / kGroup;
+    const bool any = base < n;
+    const bool full = ALIGNED && (base + kEltsPerLane <= n);
+
+    float pv[kEltsPerLane], gv[kEltsPerLane], m[kEltsPerLane], v[kEltsPerLane];
+    uint32_t wm = 0, wv = 0;
+    float sm = 0.0f, sv = 0.0f;
+
+    if (full) {
+        const float4 *p4 = reinterpret_cast<const float4 *>(t.p + base);
+        const float4 *g4 = reinterpret_cast<const float4 *>(t.g + base);
+        const float4 a0 = p4[0], a1 = p4[1], b0 = g4[0], b1 = g4[1];
+        wm = *reinterpret_cast<const uint32_t *>(t.mc + (base >> 1));
+        wv = *reinterpret_cast<const uint32_t *>(t.vc + (base >> 1));
+        sm = t.ms[grp];
+        sv = t.vs[grp];
+        pv[0] = a0.x; pv[1] = a0.y; pv[2] = a0.z; pv[3] = a0.w;
+        pv[4] = a1.x; pv[5] = a1.y; pv[6] = a1.z; pv[7] = a1.w;
+        gv[0] = b0.x; gv[1] = b0.y; gv[2] = b0.z; gv[3] = b0.w;
+        gv[4] = b1.x; gv[5] = b1.y; gv[6] = b1.z; gv[7] = b1.w;
+    } else if (any) {
+        sm = t.ms[grp];
+        sv = t.vs[grp];
+#pragma unroll
+        for (int k = 0; k < kEltsPerLane; ++k) {
+            const int64_t i = base + k;
+            pv[k] = (i < n) ? t.p[i] : 0.0f;
+            gv[k] = (i < n) ? t.g[i] : 0.0f;
+        }
+#pragma unroll
+        for (int k = 0; k < kEltsPerLane / 2; ++k) {
+            const int64_t i = base + 2 * k;
+            if (i < n) {
+                wm |= (uint32_t)t.mc[i >> 1] << (8 * k);
+                wv |= (uint32_t)t.vc[i >> 1] << (8 * k);
+            }
+        }
+    }
+
+    float amax_m = 0.0f, amax_v = 0.0f;
+    if (any) {
+#pragma unroll
+        for (int k = 0; k < kEltsPerLane; ++k) {
+            m[k] = s_qm[(wm >> (4 * k)) & 0xF] * sm;
+            v[k] = s_qv[(wv >> (4 * k)) & 0xF] * sv;
+            const bool valid = full || (base + k < n);
+            if (valid) {
+                pv[k] = adamw_elt(pv[k], gv[k], m[k], v[k], h);
+                amax_m = fmaxf(amax_m, fabsf(m[k]));
+                amax_v = fmaxf(amax_v, v[k]);
+            } else {
+                m[k] = 0.0f;
+                v[k] = 0.0f;
+            }
+        }
+    }
+    // every lane of the row takes part, also those past the end of the tensor
+    amax_m = row16_max(amax_m);
+    amax_v = row16_max(amax_v);
+    if (!any)
+        return;
+
+    uint32_t om = 0, ov = 0;
+    const bool nan_m = (amax_m == 0.0f);  // x/0 with x == 0: NaN -> code 15 for the whole group
+    const bool nan_v = (amax_v == 0.0f);
+#pragma unroll
+    for (int k = 0; k < kEltsPerLane; ++k) {
+        const bool valid = full || (base + k < n);
+        uint32_t cm = nan_m ? 15u : encode_count(mids_m, m[k] / amax_m);
+        uint32_t cv = nan_v ? 15u : encode_count(mids_v, v[k] / amax_v);
+        if (!valid) {
+            cm = 0;
+            cv = 0;
+        }
+        om |= cm << (4 * k);
+        ov |= cv << (4 * k);
+    }
+
+    if (full) {
+        float4 *p4 = reinterpret_cast<float4 *>(t.p + base);
+        p4[0] = make_float4(pv[0], pv[1], pv[2], pv[3]);
+        p4[1] = make_float4(pv[4], pv[5], pv[6], pv[7]);
+        *reinterpret_cast<uint32_t *>(t.mc + (base >> 1)) = om;
+        *reinterpret_cast<uint32_t *>(t.vc + (base >> 1)) = ov;
+    } else {
+#pragma unroll
+        for (int k = 0; k < kEltsPerLane; ++k)
+            if (base + k < n)
+                t.p[base + k] = pv[k];
+#pragma unroll
+        for (int k = 0; k < kEltsPerLane / 2; ++k) {
+            const int64_t i = base + 2 * k;
+            if (i < n) {
+                t.mc[i >> 1] = (uint8_t)(om >> (8 * k));
+                t.vc[i >> 1] = (uint8_t)(ov >> (8 * k));
+            }
+        }
+    }
+    if ((threadIdx.x & 15) == 0) {
+        t.ms[grp] = amax_m;
+        t.vs[grp] = amax_v;
+    }
+}
+
+// ---------------------------------------------------------------------------------------
+// fp32-state step (lpmm/cpp_extension/fused_adamw_kernel.cu:52-78).
+// ---------------------------------------------------------------------------------------
+struct TensorF {
+    float *p;
+    const float *g;
+    float *m;
+    float *v;
+    int64_t n;
+    float c1;
+    float c2s;
+};
+
+constexpr int kMultiFMax = 64;
+constexpr int kTileF = 1024;  // 256 threads x 4 elements
+
+struct MultiF {
+    TensorF t[kMultiFMax];
+    uint32_t tile_start[kMultiFMax + 1];
+    int count;
+    float beta1, beta2, lr, wd, eps;
+};
+
+__global__ __launch_bounds__(kThreads) void adamw_fp32_kernel(const MultiF args)
+{
+    int lo = 0, hi = args.count;
+    while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (args.tile_start[mid] <= blockIdx.x)
+            lo = mid;
+        else
+            hi = mid;
+    }
+    const TensorF &t = args.t[lo];
+    Hyper h;
+    h.beta1 = args.beta1;
+    h.beta2 = args.beta2;
+    h.omb1 = 1 - args.beta1;
+    h.omb2 = 1 - args.beta2;
+    h.lr = args.lr;
+    h.wd = args.wd;
+    h.eps = args.eps;
+    h.c1 = t.c1;
+    h.c2s = t.c2s;
+    const int64_t tile0 = (int64_t)(blockIdx.x - args.tile_start[lo]) * kTileF;
+#pragma unroll
+    for (int k = 0; k < kTileF / kThreads; ++k) {
+        const int64_t i = tile0 + k * kThreads + threadIdx.x;
+        if (i < t.n) {
+            float m = t.m[i], v = t.v[i];
+            t.p[i] = adamw_elt(t.p[i], t.g[i], m, v, h);
+            t.m[i] = m;
+            t.v[i] = v;
+        }
+    }
+}
+
+// bias corrections exactly as the reference computes them per thread
+// (fused_adamw_kernel.cu:103-104), done once on the host
+inline void bias_corrections(float beta1, float beta2, float step, float *c1, float *c2s)
+{
+    *c1 = 1.0f - powf(beta1, step);
+    *c2s = sqrtf(1.0f - powf(beta2, step));
+}
+
+}  // namespace lpmm
+
+using namespace lpmm;
+
+extern "C" int lpmm_adamw4bit_step_multi(const lpmm_adamw4bit_tensor *tensors, int64_t count,
+                                         const float *qmap_m, const float *qmap_v, float beta1,
+                                         float beta2, float lr, float weight_decay, float eps,
+                                         void *stream)
+{
+    if (count < 0)
+        return LPMM_ERR_SIZE;
+    if (count == 0)
+        return LPMM_OK;
+    LPMM_REQUIRE_PTR(tensors);
+    LPMM_REQUIRE_PTR(qmap_m);
+    LPMM_REQUIRE_PTR(qmap_v);
+    LPMM_REQUIRE_ALIGN(qmap_m, 4);
+    LPMM_REQUIRE_ALIGN(qmap_v, 4);
+    bool aligned = true;
+    for (int64_t i = 0; i < count; ++i) {
+        const lpmm_adamw4bit_tensor &t = tensors[i];
+        if (t.n < 0)
+            return LPMM_ERR_SIZE;
+        if (t.n == 0)
+            continue;
+        LPMM_REQUIRE_PTR(t.p);
+        LPMM_REQUIRE_PTR(t.g);
+        LPMM_REQUIRE_PTR(t.m_codes);
+        LPMM_REQUIRE_PTR(t.v_codes);
+        LPMM_REQUIRE_PTR(t.m_scale);
+        LPMM_REQUIRE_PTR(t.v_scale);
+        LPMM_REQUIRE_ALIGN(t.p, 4);
+        LPMM_REQUIRE_ALIGN(t.g, 4);
+        LPMM_REQUIRE_ALIGN(t.m_scale, 4);
+        LPMM_REQUIRE_ALIGN(t.v_scale, 4);
+        if ((t.n + kTile - 1) / kTile > 0x7fffffffLL)
+            return LPMM_ERR_SIZE;
+        aligned = aligned && aligned_to(t.p, 16) && aligned_to(t.g, 16) && aligned_to(t.m_codes, 4) &&
+                  aligned_to(t.v_codes, 4);
+    }
+
+    Multi4 args;
+    args.beta1 = beta1;
+    args.beta2 = beta2;
+    args.lr = lr;
+    args.wd = weight_decay;
+    args.eps = eps;
+    int64_t i = 0;
+    while (i < count) {
+        int k = 0;
+        uint64_t tiles = 0;
+        args.tile_start[0] = 0;
+        while (i < count && k < LPMM_MULTI_MAX) {
+            const lpmm_adamw4bit_tensor &t = tensors[i];
+            if (t.n == 0) {
+                ++i;
+                continue;
+            }
+            const uint64_t nt = (uint64_t)((t.n + kTile - 1) / kTile);
+            if (tiles + nt > 0x7fffffffULL)
+                break;
+            Tensor4 &d = args.t[k];
+            d.p = t.p;
+            d.g = t.g;
+            d.mc = t.m_codes;
+            d.vc = t.v_codes;
+            d.ms = t.m_scale;
+            d.vs = t.v_scale;
+            d.n = t.n;
+            bias_corrections(beta1, beta2, t.step, &d.c1, &d.c2s);
+            tiles += nt;
+            args.tile_start[++k] = (uint32_t)tiles;
+            ++i;
+        }
+        if (k == 0)
+            continue;
+        args.count = k;
+        for (int j = k + 1; j <= LPMM_MULTI_MAX; ++j)
+            args.tile_start[j] = (uint32_t)tiles;
+        if (aligned)
+            hipLaunchKernelGGL(adamw4bit_kernel<true>, dim3((uint32_t)tiles), dim3(kThreads), 0,
+                               (hipStream_t)stream, args, qmap_m, qmap_v);
+        else
+            hipLaunchKernelGGL(adamw4bit_kernel<false>, dim3((uint32_t)tiles), dim3(kThreads), 0,
+                               (hipStream_t)stream, args, qmap_m, qmap_v);
+        const int st = launch_status();
+        if (st != LPMM_OK)
+            return st;
+    }
+    return LPMM_OK;
+}
+
+extern "C" int lpmm_adamw4bit_step(float *p, const float *g, uint8_t *m_codes, uint8_t *v_codes,
+                                   float *m_scale, float *v_scale, const float *qmap_m,
+                                   const float *qmap_v, int64_t n, float beta1, float beta2, float lr,
+                                   float weight_decay, float eps, float step, void *stream)
+{
+    lpmm_adamw4bit_tensor t;
+    t.p = p;
+    t.g = g;
+    t.m_codes = m_codes;
+    t.v_codes = v_codes;
+    t.m_scale = m_scale;
+    t.v_scale = v_scale;
+    t.n = n;
+    t.step = step;
+    t.reserved = 0.0f;
+    return lpmm_adamw4bit_step_multi(&t, 1, qmap_m, qmap_v, beta1, beta2, lr, weight_decay, eps, stream);
+}
+
+extern "C" int lpmm_adamw_fp32_step_multi(const lpmm_adamw_fp32_tensor *tensors, int64_t count,
+                                          float beta1, float beta2, float lr, float weight_decay,
+                                          float eps, void *stream)
+{
+    if (count < 0)
+        return LPMM_ERR_SIZE;
+    if (count == 0)
+        return LPMM_OK;
+    LPMM_REQUIRE_PTR(tensors);
+    for (int64_t i = 0; i < count; ++i) {
+        const lpmm_adamw_fp32_tensor &t = tensors[i];
+        if (t.n < 0 || (t.n + kTileF - 1) / kTileF > 0x7fffffffLL)
+            return LPMM_ERR_SIZE;
+        if (t.n == 0)
+            continue;
+        LPMM_REQUIRE_PTR(t.p);
+        LPMM_REQUIRE_PTR(t.g);
+        LPMM_REQUIRE_PTR(t.m);
+        LPMM_REQUIRE_PTR(t.v);
+        LPMM_REQUIRE_ALIGN(t.p, 4);
+        LPMM_REQUIRE_ALIGN(t.g, 4);
+        LPMM_REQUIRE_ALIGN(t.m, 4);
+        LPMM_REQUIRE_ALIGN(t.v, 4);
+    }
+    MultiF args;
+    args.beta1 = beta1;
+    args.beta2 = beta2;
+    args.lr = lr;
+    args.wd = weight_decay;
+    args.eps = eps;
+    int64_t i = 0;
+    while (i < count) {
+        int k = 0;
+        uint64_t tiles = 0;
+        args.tile_start[0] = 0;
+        while (i < count && k < kMultiFMax) {
+            const lpmm_adamw_fp32_tensor &t = tensors[i];
+            if (t.n == 0) {
+                ++i;
+                continue;
+            }
+            const uint64_t nt = (uint64_t)((t.n + kTileF - 1) / kTileF);
+            if (tiles + nt > 0x7fffffffULL)
+                break;
+            TensorF &d = args.t[k];
+            d.p = t.p;
+            d.g = t.g;
+            d.m = t.m;
+            d.v = t.v;
+            d.n = t.n;
+            bias_corrections(beta1, beta2, t.step, &d.c1, &d.c2s);
+            tiles += nt;
+            args.tile_start[++k] = (uint32_t)tiles;
+            ++i;
+        }
+        if (k == 0)
+            continue;
+        args.count = k;
+        for (int j = k + 1; j <= kMultiFMax; ++j)
+            args.tile_start[j] = (uint32_t)tiles;
+        hipLaunchKernelGGL(adamw_fp32_kernel, dim3((uint32_t)tiles), dim3(kThreads), 0,
+                           (hipStream_t)stream, args);
+        const int st = launch_status();
+        if (st != LPMM_OK)
+            return st;
+    }
+    return LPMM_OK;
+}
+
+extern "C" int lpmm_adamw_fp32_step(float *p, const float *g, float *m, float *v, int64_t n,
+                                    float beta1, float beta2, float lr, float weight_decay, float eps,
+                                    float step, void *stream)
+{
+    lpmm_adamw_fp32_tensor t;
+    t.p = p;
+    t.g = g;
+    t.m = m;
+    t.v = v;
+    t.n = n;
+    t.step = step;
+    t.reserved = 0.0f;
+    return lpmm_adamw_fp32_step_multi(&t, 1, beta1, beta2, lr, weight_decay, eps, stream);
+}

@@ -1,0 +1,104 @@
+// Shared host/device helpers of the gfx950 kernels.  Wave size is 64; a DPP row is 16 lanes.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "lpmm_hip.h"
+
+namespace lpmm {
+
+constexpr int kWave = 64;
+constexpr int kGroup = LPMM_GROUP;
+
+// ---------------------------------------------------------------------------------------
+// host-side argument checks
+// ---------------------------------------------------------------------------------------
+inline bool aligned_to(const void *p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
+
+#define LPMM_REQUIRE_PTR(p)       \
+    do {                          \
+        if ((p) == nullptr)       \
+            return LPMM_ERR_NULL; \
+    } while (0)
+
+#define LPMM_REQUIRE_ALIGN(p, a)   \
+    do {                           \
+        if (!lpmm::aligned_to(p, a)) \
+            return LPMM_ERR_ALIGN; \
+    } while (0)
+
+inline int launch_status()
+{
+    return hipGetLastError() == hipSuccess ? LPMM_OK : LPMM_ERR_LAUNCH;
+}
+
+// ---------------------------------------------------------------------------------------
+// DPP lane exchange inside a 16-lane row.  The four steps quad xor 1, quad xor 2,
+// half-row mirror and row mirror leave the row-wide result in every lane.
+// ---------------------------------------------------------------------------------------
+template <int CTRL>
+__device__ __forceinline__ float dpp_f32(float v)
+{
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, false));
+}
+
+__device__ __forceinline__ float row16_max(float v)
+{
+    v = fmaxf(v, dpp_f32<0xB1>(v));   // quad_perm [1,0,3,2]
+    v = fmaxf(v, dpp_f32<0x4E>(v));   // quad_perm [2,3,0,1]
+    v = fmaxf(v, dpp_f32<0x141>(v));  // row_half_mirror
+    v = fmaxf(v, dpp_f32<0x140>(v));  // row_mirror
+    return v;
+}
+
+__device__ __forceinline__ float wave_max(float v)
+{
+    v = row16_max(v);
+    v = fmaxf(v, __shfl_xor(v, 16, 64));
+    v = fmaxf(v, __shfl_xor(v, 32, 64));
+    return v;
+}
+
+__device__ __forceinline__ double wave_sum_f64(double v)
+{
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1)
+        v += __shfl_xor(v, o, 64);
+    return v;
+}
+
+// ---------------------------------------------------------------------------------------
+// Code assignment for an ascending 16-entry map given its 15 fp32 midpoints:
+// code = number of midpoints strictly below x.  Identical to the reference's upper-bound
+// search followed by the midpoint test, including "exact tie -> lower code".  NaN compares
+// false everywhere and yields 0 here; callers map NaN to 15 themselves (a NaN arises only
+// from 0/0, i.e. a group whose maximum is 0, which is uniform over the group).
+// ---------------------------------------------------------------------------------------
+struct Mids {
+    float v[15];
+};
+
+__device__ __forceinline__ Mids make_mids(const float *__restrict__ qmap)
+{
+    Mids m;
+    float prev = qmap[0];
+#pragma unroll
+    for (int k = 1; k < 16; ++k) {
+        const float cur = qmap[k];
+        m.v[k - 1] = (prev + cur) * 0.5f;
+        prev = cur;
+    }
+    return m;
+}
+
+__device__ __forceinline__ uint32_t encode_count(const Mids &m, float x)
+{
+    uint32_t c = 0;
+#pragma unroll
+    for (int k = 0; k < 15; ++k)
+        c += (m.v[k] < x) ? 1u : 0u;
+    return c;
+}
+
+}  // namespace lpmm

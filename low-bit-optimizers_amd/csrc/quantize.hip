@@ -1,0 +1,476 @@
+// Stand-alone 4-bit quantise / dequantise kernels for gfx950 in the non-fused packed layout
+// of lpmm: codes of the flattened, zero-padded tensor, two per byte (low nibble = even
+// index), padded to a multiple of 2048 values, plus one trailing byte
+// (lpmm/functional.py:359-369, lpmm/cpp_extension/quantization_kernel.cu:430-477).
+//
+// A lane owns 8 consecutive values = one 32-bit word of codes; a 256-thread workgroup
+// covers one 2048-value pack group.  Group maxima use DPP row reductions (128 values =
+// 16 lanes) and, for larger groups, 16 floats of LDS per workgroup.
+#include "lpmm_common.hpp"
+
+namespace lpmm {
+
+constexpr int kQThreads = 256;
+constexpr int kQElts = 8;
+constexpr int kQTile = kQThreads * kQElts;  // 2048
+
+__device__ __forceinline__ uint32_t encode_nan15(const Mids &mids, float x)
+{
+    return (x != x) ? 15u : encode_count(mids, x);
+}
+
+__device__ __forceinline__ void load8(const float *__restrict__ x, int64_t base, int64_t n, bool vec,
+                                      float (&v)[kQElts])
+{
+    if (vec && base + kQElts <= n) {
+        const float4 a = *reinterpret_cast<const float4 *>(x + base);
+        const float4 b = *reinterpret_cast<const float4 *>(x + base + 4);
+        v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+        v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+    } else {
+#pragma unroll
+        for (int k = 0; k < kQElts; ++k)
+            v[k] = (base + k < n) ? x[base + k] : 0.0f;
+    }
+}
+
+__device__ __forceinline__ void store8(float *__restrict__ out, int64_t base, int64_t n, bool vec,
+                                       const float (&v)[kQElts])
+{
+    if (vec && base + kQElts <= n) {
+        *reinterpret_cast<float4 *>(out + base) = make_float4(v[0], v[1], v[2], v[3]);
+        *reinterpret_cast<float4 *>(out + base + 4) = make_float4(v[4], v[5], v[6], v[7]);
+    } else {
+#pragma unroll
+        for (int k = 0; k < kQElts; ++k)
+            if (base + k < n)
+                out[base + k] = v[k];
+    }
+}
+
+// ---------------------------------------------------------------------------------------
+// pack_nonlinear / unpack_nonlinear (values already normalised)
+// ---------------------------------------------------------------------------------------
+__global__ __launch_bounds__(kQThreads) void pack4_kernel(const float *__restrict__ x,
+                                                          const float *__restrict__ qmap,
+                                                          int64_t n_padded, uint8_t *__restrict__ out,
+                                                          bool vec)
+{
+    const Mids mids = make_mids(qmap);
+    const int64_t base = ((int64_t)blockIdx.x * kQThreads + threadIdx.x) * kQElts;
+    if (base == 0)
+        out[n_padded / 2] = 0;
+    if (base >= n_padded)
+        return;
+    float v[kQElts];
+    load8(x, base, n_padded, vec, v);
+    uint32_t w = 0;
+#pragma unroll
+    for (int k = 0; k < kQElts; ++k)
+        w |= encode_nan15(mids, v[k]) << (4 * k);
+    if (vec) {
+        *reinterpret_cast<uint32_t *>(out + (base >> 1)) = w;
+    } else {
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+            out[(base >> 1) + k] = (uint8_t)(w >> (8 * k));
+    }
+}
+
+// codes hold at least ceil(n/2) bytes; whole words are read only where they lie inside.
+__device__ __forceinline__ uint32_t load_codes8(const uint8_t *__restrict__ codes, int64_t base, int64_t n,
+                                                bool vec)
+{
+    if (vec && base + kQElts <= n)
+        return *reinterpret_cast<const uint32_t *>(codes + (base >> 1));
+    uint32_t w = 0;
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+        if (base + 2 * k < n)
+            w |= (uint32_t)codes[(base >> 1) + k] << (8 * k);
+    return w;
+}
+
+__global__ __launch_bounds__(kQThreads) void unpack4_kernel(const uint8_t *__restrict__ codes,
+                                                            const float *__restrict__ qmap, int64_t n,
+                                                            float *__restrict__ out, bool vec)
+{
+    __shared__ float s_q[16];
+    if (threadIdx.x < 16)
+        s_q[threadIdx.x] = qmap[threadIdx.x];
+    __syncthreads();
+    const int64_t base = ((int64_t)blockIdx.x * kQThreads + threadIdx.x) * kQElts;
+    if (base >= n)
+        return;
+    const uint32_t w = load_codes8(codes, base, n, vec);
+    float v[kQElts];
+#pragma unroll
+    for (int k = 0; k < kQElts; ++k)
+        v[k] = s_q[(w >> (4 * k)) & 0xF];
+    store8(out, base, n, vec, v);
+}
+
+// ---------------------------------------------------------------------------------------
+// 'group' scaling: max|x| per gp_sz values, x / max, search, pack -- one pass.
+// rows_per_group = gp_sz / 128 in {1, 2, 4, 8, 16}.
+// ---------------------------------------------------------------------------------------
+__global__ __launch_bounds__(kQThreads) void quant_group_kernel(const float *__restrict__ x, int64_t n,
+                                                                int rows_per_group,
+                                                                const float *__restrict__ qmap,
+                                                                uint8_t *__restrict__ codes,
+                                                                float *__restrict__ max1, int64_t n_groups,
+                                                                int64_t n_padded, bool vec)
+{
+    __shared__ float s_row[kQThreads / 16];
+    const Mids mids = make_mids(qmap);
+    const int64_t base = ((int64_t)blockIdx.x * kQThreads + threadIdx.x) * kQElts;
+    if (base == 0)
+        codes[n_padded / 2] = 0;
+    float v[kQElts];
+    load8(x, base, n, vec, v);  // zero beyond n: the reference's zero padding
+    float amax = 0.0f;
+#pragma unroll
+    for (int k = 0; k < kQElts; ++k)
+        amax = fmaxf(amax, fabsf(v[k]));
+    amax = row16_max(amax);
+    if (rows_per_group > 1) {
+        const int row = threadIdx.x >> 4;
+        if ((threadIdx.x & 15) == 0)
+            s_row[row] = amax;
+        __syncthreads();
+        const int first = row & ~(rows_per_group - 1);
+        amax = s_row[first];
+        for (int r = 1; r < rows_per_group; ++r)
+            amax = fmaxf(amax, s_row[first + r]);
+    }
+    const int64_t gp_sz = (int64_t)rows_per_group * kGroup;
+    const int64_t grp = base / gp_sz;
+    const bool in_scaled = grp < n_groups;  // else: padding added by the re-grouping to 2048
+    if (in_scaled && (base % gp_sz) == 0)
+        max1[grp] = amax;
+    uint32_t w = 0;
+#pragma unroll
+    for (int k = 0; k < kQElts; ++k) {
+        const float val = in_scaled ? v[k] / amax : 0.0f;
+        w |= encode_nan15(mids, val) << (4 * k);
+    }
+    *reinterpret_cast<uint32_t *>(codes + (base >> 1)) = w;
+}
+
+__global__ __launch_bounds__(kQThreads) void dequant_group_kernel(const uint8_t *__restrict__ codes,
+                                                                  const float *__restrict__ max1,
+                                                                  const float *__restrict__ qmap, int64_t n,
+                                                                  int64_t gp_sz, float *__restrict__ out,
+                                                                  bool vec)
+{
+    __shared__ float s_q[16];
+    if (threadIdx.x < 16)
+        s_q[threadIdx.x] = qmap[threadIdx.x];
+    __syncthreads();
+    const int64_t base = ((int64_t)blockIdx.x * kQThreads + threadIdx.x) * kQElts;
+    if (base >= n)
+        return;
+    const uint32_t w = load_codes8(codes, base, n, vec);
+    const float s = max1[base / gp_sz];  // gp_sz is a multiple of 128, so uniform over the lane's 8
+    float v[kQElts];
+#pragma unroll
+    for (int k = 0; k < kQElts; ++k)
+        v[k] = s_q[(w >> (4 * k)) & 0xF] * s;
+    store8(out, base, n, vec, v);
+}
+
+// ---------------------------------------------------------------------------------------
+// 'rank1' scaling of a row-major R x C tensor.
+// ---------------------------------------------------------------------------------------
+__global__ void fill_zero_kernel(float *__restrict__ a, int64_t na, float *__restrict__ b, int64_t nb)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < na)
+        a[i] = 0.0f;
+    if (i < nb)
+        b[i] = 0.0f;
+}
+
+constexpr int kStatRows = 32;
+constexpr int kStatCols = 1024;  // 256 threads x 4 columns
+
+// max of non-negative floats == max of their bit patterns as unsigned integers
+__device__ __forceinline__ void atomic_max_nonneg(float *addr, float v)
+{
+    atomicMax(reinterpret_cast<unsigned int *>(addr), __float_as_uint(v));
+}
+
+__global__ __launch_bounds__(kQThreads) void rank1_stats_kernel(const float *__restrict__ x, int64_t R,
+                                                                int64_t C, float *__restrict__ rowmax,
+                                                                float *__restrict__ colmax, bool vec)
+{
+    const int64_t c0 = (int64_t)blockIdx.x * kStatCols + (int64_t)threadIdx.x * 4;
+    const int64_t r0 = (int64_t)blockIdx.y * kStatRows;
+    const int64_t r1 = (r0 + kStatRows < R) ? r0 + kStatRows : R;
+    float cm[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (int64_t r = r0; r < r1; ++r) {
+        float a[4];
+        const float *row = x + r * C;
+        if (vec && c0 + 4 <= C) {
+            const float4 t = *reinterpret_cast<const float4 *>(row + c0);
+            a[0] = fabsf(t.x); a[1] = fabsf(t.y); a[2] = fabsf(t.z); a[3] = fabsf(t.w);
+        } else {
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+                a[k] = (c0 + k < C) ? fabsf(row[c0 + k]) : 0.0f;
+        }
+        float rm = fmaxf(fmaxf(a[0], a[1]), fmaxf(a[2], a[3]));
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+            cm[k] = fmaxf(cm[k], a[k]);
+        rm = wave_max(rm);
+        if ((threadIdx.x & 63) == 0)
+            atomic_max_nonneg(rowmax + r, rm);
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+        if (c0 + k < C)
+            atomic_max_nonneg(colmax + c0 + k, cm[k]);
+}
+
+__global__ __launch_bounds__(kQThreads) void quant_rank1_kernel(const float *__restrict__ x, int64_t n,
+                                                                int64_t C, const float *__restrict__ rowmax,
+                                                                const float *__restrict__ colmax,
+                                                                const float *__restrict__ qmap,
+                                                                uint8_t *__restrict__ codes, int64_t n_padded,
+                                                                bool vec)
+{
+    const Mids mids = make_mids(qmap);
+    const int64_t base = ((int64_t)blockIdx.x * kQThreads + threadIdx.x) * kQElts;
+    if (base == 0)
+        codes[n_padded / 2] = 0;
+    float v[kQElts];
+    load8(x, base, n, vec, v);
+    int64_t r = base / C;
+    int64_t c = base - r * C;
+    float rm = (base < n) ? rowmax[r] : 0.0f;
+    uint32_t w = 0;
+#pragma unroll
+    for (int k = 0; k < kQElts; ++k) {
+        float val = 0.0f;  // padding added by the re-grouping to 2048
+        if (base + k < n) {
+            const float cmx = colmax[c];
+            const float st = (cmx < rm) ? cmx : rm;
+            val = v[k] / st;
+            if (++c == C) {
+                c = 0;
+                ++r;
+                rm = (base + k + 1 < n) ? rowmax[r] : 0.0f;
+            }
+        }
+        w |= encode_nan15(mids, val) << (4 * k);
+    }
+    *reinterpret_cast<uint32_t *>(codes + (base >> 1)) = w;
+}
+
+__global__ __launch_bounds__(kQThreads) void dequant_rank1_kernel(const uint8_t *__restrict__ codes,
+                                                                  const float *__restrict__ rowmax,
+                                                                  const float *__restrict__ colmax,
+                                                                  const float *__restrict__ qmap, int64_t n,
+                                                                  int64_t C, float *__restrict__ out, bool vec)
+{
+    __shared__ float s_q[16];
+    if (threadIdx.x < 16)
+        s_q[threadIdx.x] = qmap[threadIdx.x];
+    __syncthreads();
+    const int64_t base = ((int64_t)blockIdx.x * kQThreads + threadIdx.x) * kQElts;
+    if (base >= n)
+        return;
+    const uint32_t w = load_codes8(codes, base, n, vec);
+    int64_t r = base / C;
+    int64_t c = base - r * C;
+    float rm = rowmax[r];
+    float v[kQElts];
+#pragma unroll
+    for (int k = 0; k < kQElts; ++k) {
+        v[k] = 0.0f;
+        if (base + k < n) {
+            const float cmx = colmax[c];
+            const float st = (cmx < rm) ? cmx : rm;
+            v[k] = s_q[(w >> (4 * k)) & 0xF] * st;
+            if (++c == C) {
+                c = 0;
+                ++r;
+                rm = (base + k + 1 < n) ? rowmax[r] : 0.0f;
+            }
+        }
+    }
+    store8(out, base, n, vec, v);
+}
+
+inline bool tiles_ok(int64_t n, int64_t tile, uint32_t *tiles)
+{
+    const int64_t t = (n + tile - 1) / tile;
+    if (t > 0x7fffffffLL)
+        return false;
+    *tiles = (uint32_t)t;
+    return true;
+}
+
+}  // namespace lpmm
+
+using namespace lpmm;
+
+extern "C" int lpmm_pack_nonlinear_4bit(const float *x, const float *qmap, int64_t n_padded,
+                                        uint8_t *out, void *stream)
+{
+    if (n_padded < 0 || (n_padded % 8) != 0)
+        return LPMM_ERR_SIZE;
+    LPMM_REQUIRE_PTR(out);
+    LPMM_REQUIRE_PTR(qmap);
+    LPMM_REQUIRE_ALIGN(qmap, 4);
+    if (n_padded > 0) {
+        LPMM_REQUIRE_PTR(x);
+        LPMM_REQUIRE_ALIGN(x, 4);
+    }
+    uint32_t tiles;
+    if (!tiles_ok(n_padded > 0 ? n_padded : 1, kQTile, &tiles))
+        return LPMM_ERR_SIZE;
+    const bool vec = aligned_to(x, 16) && aligned_to(out, 4);
+    hipLaunchKernelGGL(pack4_kernel, dim3(tiles), dim3(kQThreads), 0, (hipStream_t)stream, x, qmap,
+                       n_padded, out, vec);
+    return launch_status();
+}
+
+extern "C" int lpmm_unpack_nonlinear_4bit(const uint8_t *codes, const float *qmap, int64_t n,
+                                          float *out, void *stream)
+{
+    if (n < 0)
+        return LPMM_ERR_SIZE;
+    if (n == 0)
+        return LPMM_OK;
+    LPMM_REQUIRE_PTR(codes);
+    LPMM_REQUIRE_PTR(qmap);
+    LPMM_REQUIRE_PTR(out);
+    LPMM_REQUIRE_ALIGN(qmap, 4);
+    LPMM_REQUIRE_ALIGN(out, 4);
+    uint32_t tiles;
+    if (!tiles_ok(n, kQTile, &tiles))
+        return LPMM_ERR_SIZE;
+    const bool vec = aligned_to(out, 16) && aligned_to(codes, 4);
+    hipLaunchKernelGGL(unpack4_kernel, dim3(tiles), dim3(kQThreads), 0, (hipStream_t)stream, codes, qmap,
+                       n, out, vec);
+    return launch_status();
+}
+
+extern "C" int lpmm_quant_group(const float *x, int64_t n, int64_t gp_sz, const float *qmap,
+                                uint8_t *codes, float *max1, void *stream)
+{
+    if (n <= 0)
+        return LPMM_ERR_SIZE;
+    if (gp_sz < kGroup || gp_sz > kQTile || (gp_sz & (gp_sz - 1)) != 0)
+        return LPMM_ERR_SIZE;
+    LPMM_REQUIRE_PTR(x);
+    LPMM_REQUIRE_PTR(qmap);
+    LPMM_REQUIRE_PTR(codes);
+    LPMM_REQUIRE_PTR(max1);
+    LPMM_REQUIRE_ALIGN(x, 4);
+    LPMM_REQUIRE_ALIGN(qmap, 4);
+    LPMM_REQUIRE_ALIGN(max1, 4);
+    LPMM_REQUIRE_ALIGN(codes, 4);
+    const int64_t n_groups = (n + gp_sz - 1) / gp_sz;
+    uint32_t tiles;
+    if (!tiles_ok(n_groups * gp_sz, kQTile, &tiles))
+        return LPMM_ERR_SIZE;
+    const int64_t n_padded = (int64_t)tiles * kQTile;
+    hipLaunchKernelGGL(quant_group_kernel, dim3(tiles), dim3(kQThreads), 0, (hipStream_t)stream, x, n,
+                       (int)(gp_sz / kGroup), qmap, codes, max1, n_groups, n_padded, aligned_to(x, 16));
+    return launch_status();
+}
+
+extern "C" int lpmm_dequant_group(const uint8_t *codes, const float *max1, const float *qmap, int64_t n,
+                                  int64_t gp_sz, float *out, void *stream)
+{
+    if (n <= 0 || gp_sz < kGroup || (gp_sz % kGroup) != 0)
+        return LPMM_ERR_SIZE;
+    LPMM_REQUIRE_PTR(codes);
+    LPMM_REQUIRE_PTR(max1);
+    LPMM_REQUIRE_PTR(qmap);
+    LPMM_REQUIRE_PTR(out);
+    LPMM_REQUIRE_ALIGN(max1, 4);
+    LPMM_REQUIRE_ALIGN(qmap, 4);
+    LPMM_REQUIRE_ALIGN(out, 4);
+    uint32_t tiles;
+    if (!tiles_ok(n, kQTile, &tiles))
+        return LPMM_ERR_SIZE;
+    const bool vec = aligned_to(out, 16) && aligned_to(codes, 4);
+    hipLaunchKernelGGL(dequant_group_kernel, dim3(tiles), dim3(kQThreads), 0, (hipStream_t)stream, codes,
+                       max1, qmap, n, gp_sz, out, vec);
+    return launch_status();
+}
+
+extern "C" int lpmm_rank1_stats(const float *x, int64_t rows, int64_t cols, float *rowmax, float *colmax,
+                                void *stream)
+{
+    if (rows <= 0 || cols <= 0)
+        return LPMM_ERR_SIZE;
+    LPMM_REQUIRE_PTR(x);
+    LPMM_REQUIRE_PTR(rowmax);
+    LPMM_REQUIRE_PTR(colmax);
+    LPMM_REQUIRE_ALIGN(x, 4);
+    LPMM_REQUIRE_ALIGN(rowmax, 4);
+    LPMM_REQUIRE_ALIGN(colmax, 4);
+    const int64_t gx = (cols + kStatCols - 1) / kStatCols, gy = (rows + kStatRows - 1) / kStatRows;
+    if (gx > 0x7fffffffLL || gy > 65535)
+        return LPMM_ERR_SIZE;
+    const int64_t mx = rows > cols ? rows : cols;
+    hipLaunchKernelGGL(fill_zero_kernel, dim3((uint32_t)((mx + 255) / 256)), dim3(256), 0,
+                       (hipStream_t)stream, rowmax, rows, colmax, cols);
+    const bool vec = aligned_to(x, 16) && (cols % 4) == 0;
+    hipLaunchKernelGGL(rank1_stats_kernel, dim3((uint32_t)gx, (uint32_t)gy), dim3(kQThreads), 0,
+                       (hipStream_t)stream, x, rows, cols, rowmax, colmax, vec);
+    return launch_status();
+}
+
+extern "C" int lpmm_quant_rank1(const float *x, int64_t rows, int64_t cols, const float *rowmax,
+                                const float *colmax, const float *qmap, uint8_t *codes, void *stream)
+{
+    if (rows <= 0 || cols <= 0)
+        return LPMM_ERR_SIZE;
+    LPMM_REQUIRE_PTR(x);
+    LPMM_REQUIRE_PTR(rowmax);
+    LPMM_REQUIRE_PTR(colmax);
+    LPMM_REQUIRE_PTR(qmap);
+    LPMM_REQUIRE_PTR(codes);
+    LPMM_REQUIRE_ALIGN(x, 4);
+    LPMM_REQUIRE_ALIGN(rowmax, 4);
+    LPMM_REQUIRE_ALIGN(colmax, 4);
+    LPMM_REQUIRE_ALIGN(qmap, 4);
+    LPMM_REQUIRE_ALIGN(codes, 4);
+    const int64_t n = rows * cols;
+    uint32_t tiles;
+    if (!tiles_ok(n, kQTile, &tiles))
+        return LPMM_ERR_SIZE;
+    hipLaunchKernelGGL(quant_rank1_kernel, dim3(tiles), dim3(kQThreads), 0, (hipStream_t)stream, x, n, cols,
+                       rowmax, colmax, qmap, codes, (int64_t)tiles * kQTile, aligned_to(x, 16));
+    return launch_status();
+}
+
+extern "C" int lpmm_dequant_rank1(const uint8_t *codes, const float *rowmax, const float *colmax,
+                                  const float *qmap, int64_t rows, int64_t cols, float *out, void *stream)
+{
+    if (rows <= 0 || cols <= 0)
+        return LPMM_ERR_SIZE;
+    LPMM_REQUIRE_PTR(codes);
+    LPMM_REQUIRE_PTR(rowmax);
+    LPMM_REQUIRE_PTR(colmax);
+    LPMM_REQUIRE_PTR(qmap);
+    LPMM_REQUIRE_PTR(out);
+    LPMM_REQUIRE_ALIGN(rowmax, 4);
+    LPMM_REQUIRE_ALIGN(colmax, 4);
+    LPMM_REQUIRE_ALIGN(qmap, 4);
+    LPMM_REQUIRE_ALIGN(out, 4);
+    const int64_t n = rows * cols;
+    uint32_t tiles;
+    if (!tiles_ok(n, kQTile, &tiles))
+        return LPMM_ERR_SIZE;
+    const bool vec = aligned_to(out, 16) && aligned_to(codes, 4);
+    hipLaunchKernelGGL(dequant_rank1_kernel, dim3(tiles), dim3(kQThreads), 0, (hipStream_t)stream, codes,
+                       rowmax, colmax, qmap, n, cols, out, vec);
+    return launch_status();
+}

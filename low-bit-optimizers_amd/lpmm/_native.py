@@ -1,0 +1,81 @@
+"""ctypes binding of liblpmm_hip.so (the C ABI declared in include/lpmm_hip.h).
+
+There is no fallback: if the library is missing or a call fails, a RuntimeError is raised.
+"""
+import ctypes
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "liblpmm_hip.so")
+ABI_VERSION = 1
+
+_vp = ctypes.c_void_p
+_i64 = ctypes.c_int64
+_f = ctypes.c_float
+_d = ctypes.c_double
+_int = ctypes.c_int
+
+# name -> (restype, argtypes); must list every function of include/lpmm_hip.h
+PROTOTYPES = {
+    "lpmm_status_string": (ctypes.c_char_p, [_int]),
+    "lpmm_abi_version": (_int, []),
+    "lpmm_adamw4bit_step": (_int, [_vp] * 8 + [_i64] + [_f] * 6 + [_vp]),
+    "lpmm_adamw4bit_step_multi": (_int, [_vp, _i64, _vp, _vp] + [_f] * 5 + [_vp]),
+    "lpmm_adamw_fp32_step": (_int, [_vp] * 4 + [_i64] + [_f] * 6 + [_vp]),
+    "lpmm_adamw_fp32_step_multi": (_int, [_vp, _i64] + [_f] * 5 + [_vp]),
+    "lpmm_pack_nonlinear_4bit": (_int, [_vp, _vp, _i64, _vp, _vp]),
+    "lpmm_unpack_nonlinear_4bit": (_int, [_vp, _vp, _i64, _vp, _vp]),
+    "lpmm_quant_group": (_int, [_vp, _i64, _i64, _vp, _vp, _vp, _vp]),
+    "lpmm_dequant_group": (_int, [_vp, _vp, _vp, _i64, _i64, _vp, _vp]),
+    "lpmm_rank1_stats": (_int, [_vp, _i64, _i64, _vp, _vp, _vp]),
+    "lpmm_quant_rank1": (_int, [_vp, _i64, _i64, _vp, _vp, _vp, _vp, _vp]),
+    "lpmm_dequant_rank1": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _vp, _vp]),
+    "lpmm_nonfused_update": (_int, [_vp] * 4 + [_i64] + [_d] * 6 + [_vp]),
+    "lpmm_factored_workspace_bytes": (_i64, [_i64, _i64]),
+    "lpmm_factored_stats": (_int, [_vp, _i64, _i64, _vp, _vp, _vp, _d, _vp, _vp]),
+    "lpmm_factored_update": (_int, [_vp] * 8 + [_i64, _i64] + [_d] * 6 + [_int, _vp]),
+    "lpmm_factored_update_fp32m": (_int, [_vp] * 6 + [_i64, _i64] + [_d] * 6 + [_vp]),
+}
+
+# numpy mirrors of the multi-tensor records (lpmm_adamw4bit_tensor / lpmm_adamw_fp32_tensor)
+ADAMW4BIT_TENSOR = np.dtype([("p", "<u8"), ("g", "<u8"), ("m_codes", "<u8"), ("v_codes", "<u8"),
+                             ("m_scale", "<u8"), ("v_scale", "<u8"), ("n", "<i8"), ("step", "<f4"),
+                             ("reserved", "<f4")])
+ADAMW_FP32_TENSOR = np.dtype([("p", "<u8"), ("g", "<u8"), ("m", "<u8"), ("v", "<u8"), ("n", "<i8"),
+                              ("step", "<f4"), ("reserved", "<f4")])
+
+_lib = None
+
+
+def lib():
+    """The loaded library; raises RuntimeError when it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"lpmm: {LIB_PATH} is missing. Build it with `make -C low-bit-optimizers_amd/csrc` "
+                "(hipcc, gfx950). There is no CPU or PyTorch fallback for the quantised optimizer path.")
+        handle = ctypes.CDLL(LIB_PATH)
+        for name, (restype, argtypes) in PROTOTYPES.items():
+            fn = getattr(handle, name)
+            fn.restype = restype
+            fn.argtypes = argtypes
+        if handle.lpmm_abi_version() != ABI_VERSION:
+            raise RuntimeError("lpmm: liblpmm_hip.so has ABI version "
+                               f"{handle.lpmm_abi_version()}, expected {ABI_VERSION}; rebuild it")
+        _lib = handle
+    return _lib
+
+
+def check(status, what):
+    if status != 0:
+        msg = lib().lpmm_status_string(status).decode()
+        raise RuntimeError(f"lpmm: {what} failed: {msg} (status {status})")
+
+
+def current_stream(device):
+    import torch
+
+    return torch.cuda.current_stream(device).cuda_stream

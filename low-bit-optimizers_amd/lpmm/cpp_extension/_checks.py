@@ -1,0 +1,44 @@
+"""Tensor checks of the operator boundary, same conditions and messages as the reference's
+CHECK_CUDA_TENSOR_* macros (lpmm/cpp_extension/common.h:2-27); failures raise RuntimeError
+like TORCH_CHECK does."""
+import torch
+
+
+def check_cuda_tensor_float(t, name, *, fp32_only=True):
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} must be a CUDA tensor!")
+    if not t.is_contiguous():
+        raise RuntimeError(f"{name} must be contiguous!")
+    if t.dtype not in (torch.float32, torch.float16):
+        raise RuntimeError(f"The type of {name} is not kFloat32 or kFloat16!")
+    if fp32_only and t.dtype != torch.float32:
+        raise RuntimeError(f"The type of {name} is kFloat16: this build implements the fp32 path only")
+
+
+def check_cuda_tensor_dim_float(t, name, n_dim):
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} must be a CUDA tensor!")
+    if not t.is_contiguous():
+        raise RuntimeError(f"{name} must be contiguous!")
+    if t.dim() != n_dim:
+        raise RuntimeError(f"The dimension of {name} is not correct!")
+    check_cuda_tensor_float(t, name)
+
+
+def check_cuda_tensor_dim_type(t, name, n_dim, dtype):
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} must be a CUDA tensor!")
+    if not t.is_contiguous():
+        raise RuntimeError(f"{name} must be contiguous!")
+    if t.dim() != n_dim:
+        raise RuntimeError(f"The dimension of {name} is not correct!")
+    if t.dtype != dtype:
+        raise RuntimeError(f"The type of {name} is not correct!")
+
+
+def same_device(*tensors):
+    dev = tensors[0].device
+    for t in tensors[1:]:
+        if t.device != dev:
+            raise RuntimeError(f"all tensors must be on the same device, got {dev} and {t.device}")
+    return dev

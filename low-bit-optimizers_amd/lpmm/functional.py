@@ -1,0 +1,313 @@
+"""Quantise / dequantise entry points of the 4-bit optimizer-state path.
+
+Same functions and keyword protocol as the slice of lpmm/functional.py the optimizer uses:
+`vectorwise_quant(x, **kw) -> (packed int8, metadata)` (lpmm/functional.py:26-59),
+`vectorwise_dequant(qx, **kw) -> x` (:62-151) and `create_general_qmap` (:244-268), for
+4-bit codes, 'real-nearest' rounding and the scale types 'group' and 'rank1'.  The packed
+layout and the metadata dict are the reference's: int8[NG*1024 + 1] with two codes per byte
+(low nibble = even index), `max1` of shape (G, 1) for 'group', `max_dims` for 'rank1',
+`scaled_shape`, `dtype`, `stride`.
+
+Where the reference chains abs / max / div / cat / pack (and unpack / mul) as separate
+passes, each call here is one HIP kernel (two for rank-1 quantisation: statistics, then
+normalise + search + pack).
+"""
+import math
+
+import torch
+
+from . import _native
+from .cpp_extension import quantization as ext_quantization
+
+PACK_GROUP = 2048
+
+_NONLINEAR_TYPES = ("nonlinear", "power-1", "power-2", "power-3", "float-point", "nonlinear-nozero")
+
+
+# --------------------------------------------------------------------------------------
+# quantisation maps
+# --------------------------------------------------------------------------------------
+def create_dynamic_map(signed=True, max_exponent_bits=7, total_bits=8):
+    """Dynamic-exponent map (lpmm/functional.py:272-315): per decade 10^-(E-1)..10^0 the means
+    of a float32 linspace(0.1, 1) grid whose resolution doubles with the decade, mirrored
+    when signed, plus 0 and 1.  The float32 -> double -> float32 round trip of the
+    reference (tensor * scalar, .tolist(), torch.Tensor) is kept, since it fixes the bits."""
+    non_sign_bits = total_bits - (1 if signed else 0)
+    extra = 2 ** (non_sign_bits - max_exponent_bits) - 1
+    if not signed:
+        extra *= 2
+    values = [0.0, 1.0]
+
+    def add_means(count, decade):
+        edges = torch.linspace(0.1, 1, count)
+        means = decade * ((edges[:-1] + edges[1:]) / 2.0)
+        values.extend(means.tolist())
+        if signed:
+            values.extend((-means).tolist())
+
+    for i in range(max_exponent_bits):
+        decade = 10 ** (i - (max_exponent_bits - 1))
+        shift = i + non_sign_bits - max_exponent_bits
+        add_means(int(2 ** shift + 1) if signed else int(2 ** (shift + 1) + 1), decade)
+        if extra > 0:
+            add_means(extra + 1, decade)
+    return torch.Tensor(sorted(values))
+
+
+def create_pow_map(b, signed, p):
+    """Power map without zero (lpmm/functional.py:644-656): unsigned -> linspace(0,1,2^b+1)[1:]^p."""
+    if signed:
+        qmap = torch.linspace(-1, 1, 2 ** b)
+        if p != 1:
+            qmap = qmap.sign() * (qmap.abs() ** p)
+    else:
+        qmap = torch.linspace(0, 1, 2 ** b + 1)[1:]
+        if p != 1:
+            qmap = qmap ** p
+    return qmap
+
+
+def create_general_qmap(quant_type, bit, signed):
+    """lpmm/functional.py:244-268 for the map families this build quantises with."""
+    if bit == 1:
+        return torch.Tensor([-1.0, 1.0]) if signed else torch.Tensor([0.0, 1.0])
+    if quant_type == "linear":
+        return None
+    if quant_type == "nonlinear":
+        return create_dynamic_map(signed, bit - 1, bit if signed else bit - 1)
+    if quant_type == "nonlinear-nozero":
+        mapping = create_dynamic_map(signed, bit - 1, bit if signed else bit - 1)
+        if not signed:
+            mapping[0] = mapping[1]
+        return mapping
+    if quant_type in ("power-1", "power-2", "power-3"):
+        return create_pow_map(bit, signed, int(quant_type[-1]))
+    raise ValueError(f"Not support {quant_type} quant type.")
+
+
+# --------------------------------------------------------------------------------------
+# grouping helpers (lpmm/functional.py:404-431)
+# --------------------------------------------------------------------------------------
+def group_tensor(input, gp_sz):
+    """Flatten, zero-pad to a multiple of gp_sz, view as (num_groups, gp_sz)."""
+    if not gp_sz > 0:
+        raise ValueError("group size need to be a positive integer, but found {}".format(gp_sz))
+    flat = input.flatten()
+    rem = flat.shape[0] % gp_sz
+    if rem != 0:
+        flat = torch.cat([flat, torch.zeros([gp_sz - rem], dtype=input.dtype, device=input.device)], dim=0)
+    return flat.view(-1, gp_sz)
+
+
+def recon_grouped_tensor(grouped_tensor, shape):
+    """First shape.numel() values of the flattened groups, viewed as shape."""
+    return grouped_tensor.flatten()[: shape.numel()].view(shape)
+
+
+# --------------------------------------------------------------------------------------
+# rank-1 statistics (lpmm/functional.py:503-531)
+# --------------------------------------------------------------------------------------
+def _max_reduce_except_dim(tensor, dim):
+    result = tensor
+    rank = tensor.dim()
+    if rank > 0:
+        assert dim < rank
+        for d in range(rank):
+            if d != dim:
+                result = result.max(dim=d, keepdim=True).values
+    return result
+
+
+def get_sm3_statistics(x, **kwargs):
+    """max|x| over all dimensions but one, for each dimension (keepdim shapes).  2-D float32
+    CUDA tensors take one HIP kernel that reads x once."""
+    if x.dim() == 2 and x.is_cuda and x.dtype == torch.float32:
+        xc = x.contiguous()
+        rows, cols = xc.shape
+        rowmax = torch.empty((rows, 1), dtype=torch.float32, device=x.device)
+        colmax = torch.empty((1, cols), dtype=torch.float32, device=x.device)
+        with torch.cuda.device(x.device):
+            st = _native.lib().lpmm_rank1_stats(xc.data_ptr(), rows, cols, rowmax.data_ptr(), colmax.data_ptr(),
+                                                _native.current_stream(x.device))
+        _native.check(st, "rank1_stats")
+        return [rowmax, colmax]
+    qx = x.abs()
+    return [_max_reduce_except_dim(qx, i) for i in range(x.dim())]
+
+
+def _compute_sm3_scale_tensor(max_dims):
+    scale = max_dims[0].clone()
+    for other in max_dims[1:]:
+        scale = torch.min(scale, other)
+    return scale
+
+
+# --------------------------------------------------------------------------------------
+# code search + packing on already-normalised values (lpmm/functional.py:359-400)
+# --------------------------------------------------------------------------------------
+def nonlinear_quant(qx, qmap, b, round_type="sr"):
+    if round_type != "real-nearest":
+        raise NotImplementedError(f"round_type {round_type!r}: this build implements 'real-nearest' only")
+    return ext_quantization.pack_nonlinear(group_tensor(qx, PACK_GROUP), qmap, b, False)
+
+
+def nonlinear_dequant(qx, qmap, b, shape, round_type="sr"):
+    if not round_type.startswith("real"):
+        raise NotImplementedError(f"round_type {round_type!r}: this build implements 'real-nearest' only")
+    num_groups = (shape.numel() + PACK_GROUP - 1) // PACK_GROUP
+    return recon_grouped_tensor(ext_quantization.unpack_nonlinear(qx, qmap, b, num_groups, PACK_GROUP), shape)
+
+
+# --------------------------------------------------------------------------------------
+# vectorwise_quant / vectorwise_dequant
+# --------------------------------------------------------------------------------------
+def _select_qmap(kwargs):
+    qmap = kwargs["qmap"]
+    if not isinstance(qmap, torch.Tensor):
+        qmap = qmap[(kwargs["b"], kwargs["signed"])][kwargs["quant_type"]]
+    return qmap
+
+
+def _require_supported(kwargs, x):
+    if kwargs["quant_type"] not in _NONLINEAR_TYPES:
+        raise ValueError(f"Not support {kwargs['quant_type']} quant type.")
+    if kwargs["b"] != 4:
+        raise NotImplementedError(f"{kwargs['b']}-bit states: this build implements the 4-bit path only")
+    if not kwargs["round_type"].startswith("real-nearest"):
+        raise NotImplementedError(
+            f"round_type {kwargs['round_type']!r}: this build implements 'real-nearest' only")
+    if not x.is_cuda:
+        raise RuntimeError("x must be a CUDA tensor! (the quantised optimizer path has no CPU implementation)")
+
+
+def packed_nbytes(numel_scaled):
+    """Bytes of the packed tensor for numel_scaled normalised values."""
+    return (numel_scaled + PACK_GROUP - 1) // PACK_GROUP * (PACK_GROUP // 2) + 1
+
+
+def _group_gp_sz_ok(gp_sz):
+    return gp_sz in (128, 256, 512, 1024, 2048)
+
+
+def quant_group_(x, qmap, gp_sz, codes=None, max1=None):
+    """'group' scaling in one kernel.  x: contiguous float32 CUDA tensor.  Optionally writes
+    into caller-owned `codes` / `max1` buffers of the right size."""
+    n = x.numel()
+    groups = (n + gp_sz - 1) // gp_sz
+    if codes is None:
+        codes = torch.empty((packed_nbytes(groups * gp_sz),), dtype=torch.int8, device=x.device)
+    if max1 is None:
+        max1 = torch.empty((groups, 1), dtype=torch.float32, device=x.device)
+    with torch.cuda.device(x.device):
+        st = _native.lib().lpmm_quant_group(x.data_ptr(), n, gp_sz, qmap.data_ptr(), codes.data_ptr(),
+                                            max1.data_ptr(), _native.current_stream(x.device))
+    _native.check(st, "quant_group")
+    return codes, max1
+
+
+def quant_rank1_(x, qmap, codes=None):
+    """'rank1' scaling of a contiguous 2-D float32 CUDA tensor: statistics kernel, then
+    normalise + search + pack kernel."""
+    rows, cols = x.shape
+    max_dims = get_sm3_statistics(x)
+    if codes is None:
+        codes = torch.empty((packed_nbytes(rows * cols),), dtype=torch.int8, device=x.device)
+    with torch.cuda.device(x.device):
+        st = _native.lib().lpmm_quant_rank1(x.data_ptr(), rows, cols, max_dims[0].data_ptr(),
+                                            max_dims[1].data_ptr(), qmap.data_ptr(), codes.data_ptr(),
+                                            _native.current_stream(x.device))
+    _native.check(st, "quant_rank1")
+    return codes, max_dims
+
+
+def vectorwise_quant(x, **kwargs):
+    """Quantise x; returns (packed codes, generated metadata).  lpmm/functional.py:26-59 with
+    quant_scaling's 'group' (:184-189) and 'rank1' (:190-203) branches."""
+    _require_supported(kwargs, x)
+    qmap = _select_qmap(kwargs)
+    md = {"dtype": x.dtype, "stride": x.stride()}
+    src = x.detach()
+    if src.dtype != torch.float32:
+        raise NotImplementedError(f"{src.dtype} states: this build implements the fp32 path only")
+    src = src.contiguous()
+    scale_type = kwargs["scale_type"]
+    as_group = scale_type == "group" or (scale_type == "rank1" and src.dim() == 1)
+    if scale_type == "rank1":
+        md["dim"] = src.dim()
+    if as_group:
+        gp_sz = kwargs["gp_sz"] if scale_type == "group" else 128
+        if _group_gp_sz_ok(gp_sz):
+            codes, max1 = quant_group_(src, qmap, gp_sz)
+        else:  # any other group size: PyTorch reductions, HIP search + pack
+            grouped = group_tensor(src, gp_sz)
+            max1 = _max_reduce_except_dim(grouped.abs(), 0)
+            codes = nonlinear_quant(grouped.div(max1), qmap, 4, round_type="real-nearest")
+        md["max1"] = max1
+        md["scaled_shape"] = torch.Size((max1.shape[0], gp_sz))
+    elif scale_type == "rank1":
+        if src.dim() == 2:
+            codes, max_dims = quant_rank1_(src, qmap)
+        else:
+            max_dims = get_sm3_statistics(src.abs())
+            codes = nonlinear_quant(src.div(_compute_sm3_scale_tensor(max_dims)), qmap, 4,
+                                    round_type="real-nearest")
+        md["max_dims"] = max_dims
+        md["max1"] = None
+        md["scaled_shape"] = src.shape
+    else:
+        raise NotImplementedError(f"scale_type {scale_type!r}: this build implements 'group' and 'rank1'")
+    return codes, md
+
+
+def vectorwise_dequant(qx, denormalized=True, **kwargs):
+    """Dequantise packed codes to a tensor of kwargs['shape'] (the parameter's shape).
+    lpmm/functional.py:62-151."""
+    _require_supported(kwargs, qx)
+    qmap = _select_qmap(kwargs)
+    dtype, stride = kwargs["dtype"], kwargs["stride"]
+    scaled_shape = kwargs["scaled_shape"]
+    scale_type = kwargs["scale_type"]
+    codes = qx.detach()
+    dev = codes.device
+    as_group = scale_type == "group" or (scale_type == "rank1" and kwargs["dim"] == 1)
+    if not denormalized:
+        return nonlinear_dequant(codes, qmap, 4, shape=scaled_shape, round_type=kwargs["round_type"])
+    if as_group:
+        shape = kwargs["shape"]
+        gp_sz = scaled_shape[1]
+        n = shape.numel()
+        if gp_sz % 128 == 0:
+            x = torch.empty(shape, dtype=torch.float32, device=dev)
+            with torch.cuda.device(dev):
+                st = _native.lib().lpmm_dequant_group(codes.data_ptr(), kwargs["max1"].data_ptr(),
+                                                      qmap.data_ptr(), n, gp_sz, x.data_ptr(),
+                                                      _native.current_stream(dev))
+            _native.check(st, "dequant_group")
+        else:
+            x = nonlinear_dequant(codes, qmap, 4, shape=scaled_shape, round_type=kwargs["round_type"])
+            x = recon_grouped_tensor(x.mul(kwargs["max1"]), shape)
+    elif scale_type == "rank1":
+        max_dims = kwargs["max_dims"]
+        if len(scaled_shape) == 2:
+            rows, cols = scaled_shape
+            x = torch.empty(scaled_shape, dtype=torch.float32, device=dev)
+            with torch.cuda.device(dev):
+                st = _native.lib().lpmm_dequant_rank1(codes.data_ptr(), max_dims[0].data_ptr(),
+                                                      max_dims[1].data_ptr(), qmap.data_ptr(), rows, cols,
+                                                      x.data_ptr(), _native.current_stream(dev))
+            _native.check(st, "dequant_rank1")
+        else:
+            x = nonlinear_dequant(codes, qmap, 4, shape=scaled_shape, round_type=kwargs["round_type"])
+            x = x.mul(_compute_sm3_scale_tensor(max_dims))
+    else:
+        raise NotImplementedError(f"scale_type {scale_type!r}: this build implements 'group' and 'rank1'")
+
+    if x.stride() != stride:
+        recon = torch.empty_strided(x.shape, stride, dtype=dtype, layout=torch.strided, device=dev)
+        recon.copy_(x)
+        return recon
+    return x.to(dtype=dtype)
+
+
+def numel(shape):
+    return math.prod(shape)

@@ -1,0 +1,4 @@
+from .adamw import AdamW  # noqa: F401
+from .optimizer import LowBitOptimizer  # noqa: F401
+
+__all__ = ["AdamW", "LowBitOptimizer"]

@@ -1,0 +1,309 @@
+"""AdamW with 4-bit optimizer states on MI355X.
+
+Drop-in for lpmm.optim.AdamW (lpmm/optim/adamw.py:14-230): same constructor, same
+per-parameter state keys (`step`, `exp_avg`, `exp_avg_sq`, `exp_avg_qstate`,
+`exp_avg_sq_qstate`, `exp_avg_sq_row`, `exp_avg_sq_col`), same packed layouts:
+
+* fused=True   -> `exp_avg`/`exp_avg_sq` int8[(numel+1)//2], scales float32[ceil(numel/128)]
+                  in `*_qstate["overhead"]["max1"]` (lpmm/optim/adamw.py:508-523); tensors with
+                  numel <= threshold keep fp32 states (:543-561).
+* fused=False  -> `vectorwise_quant` layout and metadata (lpmm/optim/adamw.py:425-434).
+* factor_second_moment=True on >= 2-D tensors -> fp32 row/col statistics (:124-126, :579-627).
+
+What differs is the execution: all fused tensors of a parameter group go to the GPU in a
+handful of multi-tensor launches instead of one launch per tensor, and each quantise /
+dequantise / update of the non-fused path is one HIP kernel instead of a chain of
+PyTorch passes.
+"""
+from typing import Optional
+
+import numpy as np
+import torch
+
+from .. import _native
+from ..functional import packed_nbytes, vectorwise_dequant, vectorwise_quant
+from .optimizer import LowBitOptimizer
+
+__all__ = ["AdamW"]
+
+
+def _is_placeholder(t):
+    # a state that has not been materialised yet is a 0-dim tensor (adamw.py:121, :128);
+    # the reference tests numel() <= 1 (adamw.py:394, :402, :509, :544)
+    return t.numel() <= 1
+
+
+class AdamW(LowBitOptimizer):
+    def __init__(
+        self,
+        params,
+        lr=1e-3,
+        betas=(0.9, 0.999),
+        eps=1e-8,
+        weight_decay=1e-2,
+        use_first_moment=True,
+        factor_second_moment=False,
+        qconfig=None,
+        *,
+        fused: Optional[bool] = False,
+    ):
+        if not 0.0 <= lr:
+            raise ValueError("Invalid learning rate: {}".format(lr))
+        if not 0.0 <= eps:
+            raise ValueError("Invalid epsilon value: {}".format(eps))
+        if not 0.0 <= betas[0] < 1.0:
+            raise ValueError("Invalid beta parameter at index 0: {}".format(betas[0]))
+        if not 0.0 <= betas[1] < 1.0:
+            raise ValueError("Invalid beta parameter at index 1: {}".format(betas[1]))
+        if not 0.0 <= weight_decay:
+            raise ValueError("Invalid weight_decay value: {}".format(weight_decay))
+        defaults = dict(lr=lr, betas=betas, eps=eps, weight_decay=weight_decay, fused=fused,
+                        use_first_moment=use_first_moment, factor_second_moment=factor_second_moment)
+        super().__init__(params, defaults, qconfig)
+
+    def __setstate__(self, state):
+        super().__setstate__(state)
+        for group in self.param_groups:
+            group.setdefault("fused", None)
+        for s in self.state.values():
+            if "step" in s and not torch.is_tensor(s["step"]):
+                s["step"] = torch.tensor(float(s["step"]))
+
+    def get_subqconfig(self, optimizer_state_name):
+        if optimizer_state_name == "exp_avg":
+            return self.qconfig.QUANT.M
+        if optimizer_state_name == "exp_avg_sq":
+            return self.qconfig.QUANT.SQM
+        raise ValueError(f"unknown optimizer state {optimizer_state_name!r}")
+
+    @staticmethod
+    def _get_options(param_group, param_shape):
+        factored = len(param_shape) >= 2 and param_group["factor_second_moment"]
+        return factored, param_group["use_first_moment"]
+
+    # ---- state ---------------------------------------------------------------------------
+    def _state_of(self, group, p):
+        """Create the parameter's state on first use (lpmm/optim/adamw.py:114-129)."""
+        state = self.state[p]
+        factored, _ = self._get_options(group, p.shape)
+        if len(state) == 0:
+            state["step"] = torch.tensor(0.0)  # on the host: reading it never syncs the GPU
+            state["exp_avg"] = torch.zeros((), dtype=torch.float, device=p.device)
+            self.init_qstate(p, "exp_avg")
+            if factored:
+                state["exp_avg_sq_row"] = torch.zeros(p.shape[:-1], device=p.device)
+                state["exp_avg_sq_col"] = torch.zeros(p.shape[:-2] + p.shape[-1:], device=p.device)
+            else:
+                state["exp_avg_sq"] = torch.zeros((), dtype=torch.float, device=p.device)
+            self.init_qstate(p, "exp_avg_sq")
+        return state, factored
+
+    def _enabled(self, p, state, name):
+        if id(p) in self.override_q_enable:
+            return self.override_q_enable[id(p)]
+        return state[f"{name}_qstate"]["enable"]
+
+    # ---- step ----------------------------------------------------------------------------
+    @torch.no_grad()
+    def step(self, closure=None):
+        """Performs a single optimization step."""
+        loss = None
+        if closure is not None:
+            with torch.enable_grad():
+                loss = closure()
+
+        for group in self.param_groups:
+            work = []
+            for p in group["params"]:
+                if p.grad is None:
+                    continue
+                if p.grad.is_sparse:
+                    raise RuntimeError("AdamW does not support sparse gradients")
+                state, factored = self._state_of(group, p)
+                work.append((p, p.grad, state, factored))
+            if not work:
+                continue
+            if group["fused"]:
+                self._step_fused(group, work)
+            else:
+                self._step_single(group, work)
+        return loss
+
+    # ---- fused path (lpmm/optim/adamw.py:439-561) ---------------------------------------
+    def _step_fused(self, group, work):
+        beta1, beta2 = group["betas"]
+        lr, wd, eps = group["lr"], group["weight_decay"], group["eps"]
+        md_m = self.get_qmetadata_by_state_name("exp_avg")
+        md_v = self.get_qmetadata_by_state_name("exp_avg_sq")
+        quant, plain = {}, {}  # device -> list of records
+        for p, grad, state, factored in work:
+            state["step"] += 1
+            step = state["step"].item()
+            if factored:
+                # the fused kernel does not cover the factored case (adamw.py:472-495)
+                self._factored_step(group, p, grad, state, step)
+                continue
+            en_m, en_v = self._enabled(p, state, "exp_avg"), self._enabled(p, state, "exp_avg_sq")
+            if en_m != en_v:
+                raise ValueError("For same tensor, exp_avg and exp_avg_sq should be both quantized or "
+                                 f"unquantized simultaneously, but get ({en_m} {en_v})")
+            self._check_fp32_cuda(p, grad)
+            if en_m:
+                if md_m["scale_type"] != "group":
+                    print("Warning: fused_adamw4bit only support block-wise scaling, but get exp_avg "
+                          f"scale_type {md_m['scale_type']}.")
+                if md_v["scale_type"] != "group":
+                    print("Warning: fused_adamw4bit only support block-wise scaling, but get exp_avg_sq "
+                          f"scale_type {md_v['scale_type']}.")
+                n = p.numel()
+                if n % 2 != 0:
+                    # the reference's operator demands numel(exp_avg) == numel(p) // 2
+                    # (lpmm/cpp_extension/fused_adamw.cc:68-71) while (numel+1)//2 bytes are allocated
+                    raise RuntimeError("number of elements in exp_avg and p tensors should be equal")
+                nbytes, blocks = (n + 1) // 2, (n + 127) // 128
+                if _is_placeholder(state["exp_avg"]):
+                    state["exp_avg"] = torch.zeros((nbytes,), dtype=torch.int8, device=p.device)
+                if _is_placeholder(state["exp_avg_sq"]):
+                    state["exp_avg_sq"] = torch.zeros((nbytes,), dtype=torch.int8, device=p.device)
+                oh_m, oh_v = state["exp_avg_qstate"]["overhead"], state["exp_avg_sq_qstate"]["overhead"]
+                if "max1" not in oh_m:
+                    oh_m["max1"] = torch.zeros((blocks,), dtype=torch.float32, device=p.device)
+                if "max1" not in oh_v:
+                    oh_v["max1"] = torch.zeros((blocks,), dtype=torch.float32, device=p.device)
+                key = (p.device, state["exp_avg_qstate"]["qmap"].data_ptr(),
+                       state["exp_avg_sq_qstate"]["qmap"].data_ptr())
+                quant.setdefault(key, []).append(
+                    (p.data_ptr(), grad.data_ptr(), state["exp_avg"].data_ptr(), state["exp_avg_sq"].data_ptr(),
+                     oh_m["max1"].data_ptr(), oh_v["max1"].data_ptr(), n, step, 0.0))
+            else:
+                if _is_placeholder(state["exp_avg"]):
+                    state["exp_avg"] = torch.zeros_like(p, memory_format=torch.preserve_format)
+                if _is_placeholder(state["exp_avg_sq"]):
+                    state["exp_avg_sq"] = torch.zeros_like(p, memory_format=torch.preserve_format)
+                plain.setdefault(p.device, []).append(
+                    (p.data_ptr(), grad.data_ptr(), state["exp_avg"].data_ptr(), state["exp_avg_sq"].data_ptr(),
+                     p.numel(), step, 0.0))
+
+        lib = _native.lib()
+        for (dev, qm_ptr, qv_ptr), records in quant.items():
+            table = np.array(records, dtype=_native.ADAMW4BIT_TENSOR)
+            with torch.cuda.device(dev):
+                st = lib.lpmm_adamw4bit_step_multi(table.ctypes.data, len(records), qm_ptr, qv_ptr, beta1, beta2,
+                                                   lr, wd, eps, _native.current_stream(dev))
+            _native.check(st, "fused 4-bit AdamW step")
+        for dev, records in plain.items():
+            table = np.array(records, dtype=_native.ADAMW_FP32_TENSOR)
+            with torch.cuda.device(dev):
+                st = lib.lpmm_adamw_fp32_step_multi(table.ctypes.data, len(records), beta1, beta2, lr, wd, eps,
+                                                    _native.current_stream(dev))
+            _native.check(st, "fused fp32 AdamW step")
+
+    @staticmethod
+    def _check_fp32_cuda(p, grad):
+        for t, name in ((p, "p"), (grad, "g")):
+            if not t.is_cuda:
+                raise RuntimeError(f"{name} must be a CUDA tensor!")
+            if not t.is_contiguous():
+                raise RuntimeError(f"{name} must be contiguous!")
+            if t.dtype != torch.float32:
+                raise RuntimeError(f"The type of {name} is {t.dtype}: this build implements the fp32 path only")
+
+    # ---- non-fused path (lpmm/optim/adamw.py:332-436) -----------------------------------
+    def _step_single(self, group, work):
+        beta1, beta2 = group["betas"]
+        lr, wd, eps = group["lr"], group["weight_decay"], group["eps"]
+        md_m = self.get_qmetadata_by_state_name("exp_avg")
+        md_v = self.get_qmetadata_by_state_name("exp_avg_sq")
+        lib = _native.lib()
+        for p, grad, state, factored in work:
+            state["step"] += 1
+            step = state["step"].item()
+            if factored:
+                self._factored_step(group, p, grad, state, step)
+                continue
+            self._check_fp32_cuda(p, grad)
+            en_m, en_v = self._enabled(p, state, "exp_avg"), self._enabled(p, state, "exp_avg_sq")
+            m = self._materialise(p, state, "exp_avg", en_m, md_m)
+            v = self._materialise(p, state, "exp_avg_sq", en_v, md_v)
+            with torch.cuda.device(p.device):
+                st = lib.lpmm_nonfused_update(p.data_ptr(), grad.data_ptr(), m.data_ptr(), v.data_ptr(), p.numel(),
+                                              beta1, beta2, lr, wd, eps, step, _native.current_stream(p.device))
+            _native.check(st, "non-fused AdamW update")
+            if en_m:
+                self._requantise(p, state, "exp_avg", m, md_m)
+            if en_v:
+                self._requantise(p, state, "exp_avg_sq", v, md_v)
+
+    def _materialise(self, p, state, name, enabled, md):
+        """fp32 view of a state for the update: zeros at the first step, the dequantised
+        tensor when quantised, the state itself otherwise (adamw.py:394-409)."""
+        t = state[name]
+        if _is_placeholder(t):
+            state[name] = t = torch.zeros_like(p, memory_format=torch.contiguous_format)
+            return t
+        if enabled:
+            qstate = state[f"{name}_qstate"]
+            kw = dict(qstate["overhead"])
+            kw.update(md)
+            out = vectorwise_dequant(t, qmap=qstate["qmap"], shape=p.shape, **kw)
+            return out.contiguous()
+        return t
+
+    def _requantise(self, p, state, name, x, md):
+        qstate = state[f"{name}_qstate"]
+        qx, gen = vectorwise_quant(x, qmap=qstate["qmap"], shape=p.shape, **md)
+        state[name] = qx
+        qstate["overhead"].clear()
+        qstate["overhead"].update(gen)
+
+    # ---- factored second moment (lpmm/optim/adamw.py:579-627) ---------------------------
+    def _factored_step(self, group, p, grad, state, step):
+        beta1, beta2 = group["betas"]
+        lr, wd, eps = group["lr"], group["weight_decay"], group["eps"]
+        self._check_fp32_cuda(p, grad)
+        lib = _native.lib()
+        dev = p.device
+        rows, cols = p.shape[-2], p.shape[-1]
+        batch = p.numel() // (rows * cols)  # leading dimensions: independent R x C matrices
+        row, col = state["exp_avg_sq_row"], state["exp_avg_sq_col"]
+        en_m = self._enabled(p, state, "exp_avg")
+        md_m = self.get_qmetadata_by_state_name("exp_avg")
+        qstate = state["exp_avg_qstate"]
+        one_pass = (batch == 1 and en_m and md_m["scale_type"] == "group" and md_m["gp_sz"] == 128
+                    and md_m["b"] == 4 and md_m["round_type"] == "real-nearest")
+        with torch.cuda.device(dev):
+            stream = _native.current_stream(dev)
+            work = torch.empty((lib.lpmm_factored_workspace_bytes(rows, cols),), dtype=torch.uint8, device=dev)
+            mean_all = torch.empty((batch,), dtype=torch.float32, device=dev)
+            for b in range(batch):
+                st = lib.lpmm_factored_stats(grad.data_ptr() + 4 * b * rows * cols, rows, cols,
+                                             row.data_ptr() + 4 * b * rows, col.data_ptr() + 4 * b * cols,
+                                             mean_all.data_ptr() + 4 * b, beta2, work.data_ptr(), stream)
+                _native.check(st, "factored statistics")
+            if one_pass:
+                first = _is_placeholder(state["exp_avg"])
+                groups = (p.numel() + 127) // 128
+                if first:
+                    state["exp_avg"] = torch.empty((packed_nbytes(groups * 128),), dtype=torch.int8, device=dev)
+                    max1 = torch.empty((groups, 1), dtype=torch.float32, device=dev)
+                else:
+                    max1 = qstate["overhead"]["max1"]
+                st = lib.lpmm_factored_update(p.data_ptr(), grad.data_ptr(), state["exp_avg"].data_ptr(),
+                                              max1.data_ptr(), qstate["qmap"].data_ptr(), row.data_ptr(),
+                                              col.data_ptr(), mean_all.data_ptr(), rows, cols, beta1, beta2, lr, wd,
+                                              eps, step, 1 if first else 0, stream)
+                _native.check(st, "factored update")
+                qstate["overhead"].clear()
+                qstate["overhead"].update({"dtype": p.dtype, "stride": p.stride(), "max1": max1,
+                                           "scaled_shape": torch.Size((groups, 128))})
+                return
+            m = self._materialise(p, state, "exp_avg", en_m, md_m)
+            for b in range(batch):
+                off = 4 * b * rows * cols
+                st = lib.lpmm_factored_update_fp32m(p.data_ptr() + off, grad.data_ptr() + off, m.data_ptr() + off,
+                                                    row.data_ptr() + 4 * b * rows, col.data_ptr() + 4 * b * cols,
+                                                    mean_all.data_ptr() + 4 * b, rows, cols, beta1, beta2, lr, wd,
+                                                    eps, step, stream)
+                _native.check(st, "factored update")
+            if en_m:
+                self._requantise(p, state, "exp_avg", m, md_m)

@@ -1,0 +1,345 @@
+"""ctypes/numpy front end of the CPU oracle (oracle/lpmm_oracle.c).
+
+TEST INFRASTRUCTURE ONLY: imported by tests/, by __graft_entry__.smoke() and by the
+cpu_baseline leg of bench.py as the checker.  The shipped package never imports it.
+
+All arrays are C-contiguous numpy arrays; "in place" functions mutate their arguments
+exactly like the reference's kernels mutate the tensors they are given.
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "liblpmm_oracle.so")
+
+GROUP = 128
+PACK_GROUP = 2048
+
+
+def build(force=False):
+    """Compile oracle/lpmm_oracle.c with the committed Makefile."""
+    if force and os.path.exists(_LIB_PATH):
+        os.remove(_LIB_PATH)
+    subprocess.check_call(["make", "-C", _HERE, "liblpmm_oracle.so"], stdout=subprocess.DEVNULL)
+
+
+def _load():
+    if not os.path.exists(_LIB_PATH):
+        build()
+    lib = ctypes.CDLL(_LIB_PATH)
+    return lib
+
+
+_lib = _load()
+
+_f32p = np.ctypeslib.ndpointer(dtype=np.float32, flags="C_CONTIGUOUS")
+_u8p = np.ctypeslib.ndpointer(dtype=np.uint8, flags="C_CONTIGUOUS")
+_i64 = ctypes.c_int64
+_f = ctypes.c_float
+_d = ctypes.c_double
+
+
+def _sig(name, restype, *argtypes):
+    fn = getattr(_lib, name)
+    fn.restype = restype
+    fn.argtypes = list(argtypes)
+    return fn
+
+
+_qmapping = _sig("lpmm_oracle_qmapping", ctypes.c_int, _f32p, ctypes.c_int, _f)
+_qmapping_many = _sig("lpmm_oracle_qmapping_many", None, _f32p, _f32p, _i64, _u8p)
+_pack = _sig("lpmm_oracle_pack_nonlinear_4bit", None, _f32p, _f32p, _i64, _u8p)
+_unpack = _sig("lpmm_oracle_unpack_nonlinear_4bit", None, _u8p, _f32p, _i64, _f32p)
+_adamw_fp32 = _sig("lpmm_oracle_adamw_fp32_step", None, _f32p, _f32p, _f32p, _f32p, _i64,
+                   _f, _f, _f, _f, _f, _f)
+_adamw4bit = _sig("lpmm_oracle_adamw4bit_step", None, _f32p, _f32p, _u8p, _u8p, _f32p, _f32p,
+                  _f32p, _f32p, _i64, _f, _f, _f, _f, _f, _f)
+_quant_group = _sig("lpmm_oracle_quant_group", None, _f32p, _i64, _i64, _f32p, _u8p, _f32p)
+_dequant_group = _sig("lpmm_oracle_dequant_group", None, _u8p, _f32p, _f32p, _i64, _i64, _f32p)
+_rank1_stats = _sig("lpmm_oracle_rank1_stats", None, _f32p, _i64, _i64, _f32p, _f32p)
+_quant_rank1 = _sig("lpmm_oracle_quant_rank1", None, _f32p, _i64, _i64, _f32p, _f32p, _f32p, _u8p)
+_dequant_rank1 = _sig("lpmm_oracle_dequant_rank1", None, _u8p, _f32p, _f32p, _f32p, _i64, _i64,
+                      _f32p)
+_nonfused_update = _sig("lpmm_oracle_nonfused_update", None, _f32p, _f32p, _f32p, _f32p, _i64,
+                        _d, _d, _d, _d, _d, _d)
+_factored_stats = _sig("lpmm_oracle_factored_stats", None, _f32p, _i64, _i64, _f32p, _f32p)
+_factored_ema = _sig("lpmm_oracle_factored_ema", _f, _f32p, _f32p, _f32p, _f32p, _i64, _i64, _d)
+_factored_update = _sig("lpmm_oracle_factored_update", None, _f32p, _f32p, _f32p, _f32p, _f32p,
+                        _f, _i64, _i64, _d, _d, _d, _d, _d, _d)
+_max_threads = _sig("lpmm_oracle_max_threads", ctypes.c_int)
+_set_threads = _sig("lpmm_oracle_set_threads", None, ctypes.c_int)
+
+
+def max_threads():
+    return int(_max_threads())
+
+
+def set_threads(n):
+    _set_threads(int(n))
+
+
+# --------------------------------------------------------------------------------------
+# Quantisation maps.  lpmm/functional.py:244-268 (create_general_qmap), :272-315
+# (create_dynamic_map), :644-656 (create_pow_map).
+# --------------------------------------------------------------------------------------
+def _linspace_f32(start, end, steps):
+    """torch.linspace for float32 on CPU: step = (end-start)/(steps-1) in float32; the first
+    half counts up from start, the second half counts down from end."""
+    f = np.float32
+    start, end = f(start), f(end)
+    if steps == 1:
+        return np.array([start], dtype=f)
+    step = f((end - start) / f(steps - 1))
+    out = np.empty(steps, dtype=f)
+    half = steps // 2
+    for i in range(steps):
+        if i < half:
+            out[i] = f(start + f(step * f(i)))
+        else:
+            out[i] = f(end - f(step * f(steps - i - 1)))
+    return out
+
+
+def create_dynamic_map(signed=True, max_exponent_bits=3, total_bits=4):
+    """lpmm/functional.py:272-315.  The float32 means are scaled by the float32-cast power
+    of ten (tensor * python scalar), widened to double by .tolist(), sorted, and narrowed
+    back to float32 by torch.Tensor(data)."""
+    f = np.float32
+    data = []
+    non_sign_bits = total_bits - (1 if signed else 0)
+    additional_items = 2 ** (non_sign_bits - max_exponent_bits) - 1
+    if not signed:
+        additional_items = 2 * additional_items
+    for i in range(max_exponent_bits):
+        if signed:
+            fraction_items = int(2 ** (i + non_sign_bits - max_exponent_bits) + 1)
+        else:
+            fraction_items = int(2 ** (i + non_sign_bits - max_exponent_bits + 1) + 1)
+        scale = f(10 ** (-(max_exponent_bits - 1) + i))
+        b = _linspace_f32(0.1, 1, fraction_items)
+        means = ((b[:-1] + b[1:]) / f(2.0)).astype(f)
+        data += [float(v) for v in (scale * means).astype(f)]
+        if signed:
+            data += [float(v) for v in (f(-scale) * means).astype(f)]
+        if additional_items > 0:
+            b = _linspace_f32(0.1, 1, additional_items + 1)
+            means = ((b[:-1] + b[1:]) / f(2.0)).astype(f)
+            data += [float(v) for v in (scale * means).astype(f)]
+            if signed:
+                data += [float(v) for v in (f(-scale) * means).astype(f)]
+    data.append(0.0)
+    data.append(1.0)
+    data.sort()
+    return np.array(data, dtype=np.float32)
+
+
+def create_pow_map(b=4, signed=False, p=1):
+    """lpmm/functional.py:644-656 (the 'no zero' versions)."""
+    f = np.float32
+    if signed:
+        q = _linspace_f32(-1, 1, 2 ** b)
+        if p != 1:
+            q = (np.sign(q) * np.abs(q) ** f(p)).astype(f)
+    else:
+        q = _linspace_f32(0, 1, 2 ** b + 1)[1:]
+        if p != 1:
+            q = (q ** f(p)).astype(f)
+    return np.ascontiguousarray(q, dtype=f)
+
+
+def qmap_m():
+    """First-moment map: create_general_qmap('nonlinear', 4, True) (functional.py:250-251)."""
+    return create_dynamic_map(True, 3, 4)
+
+
+def qmap_v():
+    """Second-moment map: create_general_qmap('power-1', 4, False) (functional.py:257-258)."""
+    return create_pow_map(4, False, 1)
+
+
+def midpoints(qmap):
+    q = np.asarray(qmap, dtype=np.float32)
+    return ((q[:-1] + q[1:]) * np.float32(0.5)).astype(np.float32)
+
+
+# --------------------------------------------------------------------------------------
+# thin wrappers
+# --------------------------------------------------------------------------------------
+def _c(a, dtype):
+    a = np.ascontiguousarray(a, dtype=dtype)
+    return a
+
+
+def qmapping_scalar(qmap, x, bits=4):
+    """The reference's int return value (-1 for NaN)."""
+    return int(_qmapping(_c(qmap, np.float32), bits, float(np.float32(x))))
+
+
+def qmapping(qmap, x):
+    x = _c(x, np.float32).reshape(-1)
+    out = np.empty(x.size, dtype=np.uint8)
+    _qmapping_many(_c(qmap, np.float32), x, x.size, out)
+    return out
+
+
+def pack_nonlinear_4bit(x, qmap):
+    x = _c(x, np.float32).reshape(-1)
+    assert x.size % 8 == 0
+    out = np.empty(x.size // 2 + 1, dtype=np.uint8)
+    _pack(x, _c(qmap, np.float32), x.size, out)
+    return out
+
+
+def unpack_nonlinear_4bit(codes, qmap, n):
+    out = np.empty(n, dtype=np.float32)
+    _unpack(_c(codes, np.uint8), _c(qmap, np.float32), n, out)
+    return out
+
+
+def adamw_fp32_step(p, g, m, v, beta1, beta2, lr, wd, eps, step):
+    _adamw_fp32(p, g, m, v, p.size, beta1, beta2, lr, wd, eps, step)
+
+
+def adamw4bit_step(p, g, m_codes, v_codes, m_scale, v_scale, qm, qv, beta1, beta2, lr, wd, eps,
+                   step):
+    n = p.size
+    assert g.size == n and m_codes.size == (n + 1) // 2 and v_codes.size == (n + 1) // 2
+    assert m_scale.size == (n + GROUP - 1) // GROUP and v_scale.size == m_scale.size
+    _adamw4bit(p, g, m_codes, v_codes, m_scale, v_scale, _c(qm, np.float32), _c(qv, np.float32), n,
+               beta1, beta2, lr, wd, eps, step)
+
+
+def packed_nbytes_nonfused(n, gp_sz=GROUP):
+    g = (n + gp_sz - 1) // gp_sz
+    ng = (g * gp_sz + PACK_GROUP - 1) // PACK_GROUP
+    return ng * (PACK_GROUP // 2) + 1
+
+
+def quant_group(x, qmap, gp_sz=GROUP):
+    x = _c(x, np.float32).reshape(-1)
+    n = x.size
+    g = (n + gp_sz - 1) // gp_sz
+    codes = np.empty(packed_nbytes_nonfused(n, gp_sz), dtype=np.uint8)
+    max1 = np.empty(g, dtype=np.float32)
+    _quant_group(x, n, gp_sz, _c(qmap, np.float32), codes, max1)
+    return codes, max1
+
+
+def dequant_group(codes, max1, qmap, n, gp_sz=GROUP):
+    out = np.empty(n, dtype=np.float32)
+    _dequant_group(_c(codes, np.uint8), _c(max1, np.float32).reshape(-1), _c(qmap, np.float32), n,
+                   gp_sz, out)
+    return out
+
+
+def rank1_stats(x):
+    x = _c(x, np.float32)
+    r, c = x.shape
+    rowmax = np.empty(r, dtype=np.float32)
+    colmax = np.empty(c, dtype=np.float32)
+    _rank1_stats(x, r, c, rowmax, colmax)
+    return rowmax, colmax
+
+
+def quant_rank1(x, rowmax, colmax, qmap):
+    x = _c(x, np.float32)
+    r, c = x.shape
+    codes = np.empty(packed_nbytes_nonfused(r * c, 1), dtype=np.uint8)
+    _quant_rank1(x, r, c, rowmax, colmax, _c(qmap, np.float32), codes)
+    return codes
+
+
+def dequant_rank1(codes, rowmax, colmax, qmap, r, c):
+    out = np.empty((r, c), dtype=np.float32)
+    _dequant_rank1(_c(codes, np.uint8), rowmax, colmax, _c(qmap, np.float32), r, c, out)
+    return out
+
+
+def nonfused_update(p, g, m, v, beta1, beta2, lr, wd, eps, step):
+    _nonfused_update(p, g, m, v, p.size, beta1, beta2, lr, wd, eps, step)
+
+
+def factored_stats(g):
+    r, c = g.shape
+    row_mean = np.empty(r, dtype=np.float32)
+    col_mean = np.empty(c, dtype=np.float32)
+    _factored_stats(g, r, c, row_mean, col_mean)
+    return row_mean, col_mean
+
+
+def factored_ema(row, col, row_mean, col_mean, beta2):
+    return float(_factored_ema(row, col, row_mean, col_mean, row.size, col.size, beta2))
+
+
+def factored_update(p, g, m, row, col, row_mean_all, beta1, beta2, lr, wd, eps, step):
+    r, c = p.shape
+    _factored_update(p, g, m, row, col, row_mean_all, r, c, beta1, beta2, lr, wd, eps, step)
+
+
+# --------------------------------------------------------------------------------------
+# Whole non-fused steps on one tensor, composed from the pieces above the way
+# lpmm/optim/adamw.py:332-436 and :579-627 compose them.
+# --------------------------------------------------------------------------------------
+class NonFusedState:
+    """Optimizer state of one tensor in the non-fused layout (adamw.py:119-129,
+    functional.py:32-34, :240): packed codes of NG*1024+1 bytes plus max1 (G,) for 'group'
+    scaling or (rowmax, colmax) for 'rank1' on a 2-D tensor."""
+
+    def __init__(self, shape, v_scale_type="group", factored=False):
+        self.shape = tuple(shape)
+        self.n = int(np.prod(self.shape))
+        self.step = 0
+        self.v_scale_type = v_scale_type
+        self.factored = factored and len(self.shape) >= 2
+        self.m = None  # (codes, max1)
+        self.v = None  # (codes, max1) or (codes, rowmax, colmax)
+        if self.factored:
+            self.row = np.zeros(self.shape[0], dtype=np.float32)
+            self.col = np.zeros(self.shape[1], dtype=np.float32)
+
+
+def _v_is_rank1(state):
+    return state.v_scale_type == "rank1" and len(state.shape) >= 2
+
+
+def nonfused_step(p, g, state, qm, qv, lr, beta1, beta2, eps, wd):
+    """One step of _single_tensor_adamw4bit on one quantised tensor.  p is updated in place."""
+    state.step += 1
+    n = state.n
+    pf, gf = p.reshape(-1), np.ascontiguousarray(g, dtype=np.float32).reshape(-1)
+    if state.factored:
+        return _factored_step(p, g, state, qm, lr, beta1, beta2, eps, wd)
+    m = np.zeros(n, np.float32) if state.m is None else dequant_group(state.m[0], state.m[1], qm, n)
+    if state.v is None:
+        v = np.zeros(n, np.float32)
+    elif _v_is_rank1(state):
+        r, c = state.shape
+        v = dequant_rank1(state.v[0], state.v[1], state.v[2], qv, r, c).reshape(-1)
+    else:
+        v = dequant_group(state.v[0], state.v[1], qv, n)
+    nonfused_update(pf, gf, m, v, beta1, beta2, lr, wd, eps, float(state.step))
+    state.m = quant_group(m, qm)
+    if _v_is_rank1(state):
+        r, c = state.shape
+        v2 = v.reshape(r, c)
+        rowmax, colmax = rank1_stats(v2)
+        state.v = (quant_rank1(v2, rowmax, colmax, qv), rowmax, colmax)
+    else:
+        state.v = quant_group(v, qv)
+    return m, v
+
+
+def _factored_step(p, g, state, qm, lr, beta1, beta2, eps, wd):
+    n = state.n
+    r, c = state.shape
+    g2 = np.ascontiguousarray(g, dtype=np.float32).reshape(r, c)
+    m = np.zeros(n, np.float32) if state.m is None else dequant_group(state.m[0], state.m[1], qm, n)
+    row_mean, col_mean = factored_stats(g2)
+    mean_all = factored_ema(state.row, state.col, row_mean, col_mean, beta2)
+    factored_update(p.reshape(r, c), g2, m, state.row, state.col, mean_all, beta1, beta2, lr, wd,
+                    eps, float(state.step))
+    state.m = quant_group(m, qm)
+    return m, None

@@ -1,0 +1,162 @@
+"""GPU parity of the fused 4-bit AdamW step and the fp32-state step against the CPU oracle,
+called through the C ABI (lpmm._native) on torch device memory."""
+import numpy as np
+import pytest
+import torch
+
+from util import assert_codes, assert_rel, to_dev, to_np
+
+pytestmark = pytest.mark.gpu
+
+HYPER = dict(beta1=0.9, beta2=0.999, lr=1e-3, wd=0.01, eps=1e-8)
+
+
+def _native():
+    from lpmm import _native
+
+    return _native
+
+
+def _run_fused_steps(oracle, qmaps, n, steps, seed, grad_fn=None, p_scale=0.02, offset=0):
+    """Runs `steps` fused steps on GPU and oracle from zero state; compares after every step."""
+    nat = _native()
+    lib = nat.lib()
+    qm, qv = qmaps
+    rng = np.random.default_rng(seed)
+    p_ref = (rng.standard_normal(n) * p_scale).astype(np.float32)
+    nb, ng = (n + 1) // 2, (n + 127) // 128
+    mc_ref, vc_ref = np.zeros(nb, np.uint8), np.zeros(nb, np.uint8)
+    ms_ref, vs_ref = np.zeros(ng, np.float32), np.zeros(ng, np.float32)
+
+    def dev(a):
+        # optional element offset makes the device pointers misaligned for the vector path
+        buf = torch.empty(a.size + offset, dtype=torch.from_numpy(a).dtype, device="cuda")
+        view = buf[offset:]
+        view.copy_(torch.from_numpy(a))
+        return view
+
+    p, mc, vc, ms, vs = dev(p_ref), dev(mc_ref), dev(vc_ref), dev(ms_ref), dev(vs_ref)
+    dqm, dqv = to_dev(qm), to_dev(qv)
+    flips = 0
+    for s in range(1, steps + 1):
+        g_np = grad_fn(rng, n, s) if grad_fn else (rng.standard_normal(n) * 1e-3).astype(np.float32)
+        g = dev(g_np)
+        st = lib.lpmm_adamw4bit_step(p.data_ptr(), g.data_ptr(), mc.data_ptr(), vc.data_ptr(), ms.data_ptr(),
+                                     vs.data_ptr(), dqm.data_ptr(), dqv.data_ptr(), n, HYPER["beta1"],
+                                     HYPER["beta2"], HYPER["lr"], HYPER["wd"], HYPER["eps"], float(s),
+                                     torch.cuda.current_stream().cuda_stream)
+        assert st == 0, lib.lpmm_status_string(st)
+        oracle.adamw4bit_step(p_ref, g_np, mc_ref, vc_ref, ms_ref, vs_ref, qm, qv, HYPER["beta1"], HYPER["beta2"],
+                              HYPER["lr"], HYPER["wd"], HYPER["eps"], float(s))
+        torch.cuda.synchronize()
+        flips += assert_codes(to_np(mc), mc_ref, n, f"m codes step {s}")
+        flips += assert_codes(to_np(vc), vc_ref, n, f"v codes step {s}")
+        assert_rel(to_np(ms), ms_ref, f"m scale step {s}")
+        assert_rel(to_np(vs), vs_ref, f"v scale step {s}")
+        assert_rel(to_np(p), p_ref, f"p step {s}")
+        if flips:
+            # after a tie flip the two runs legitimately diverge: resynchronise the GPU state
+            mc.copy_(torch.from_numpy(mc_ref)); vc.copy_(torch.from_numpy(vc_ref))
+            ms.copy_(torch.from_numpy(ms_ref)); vs.copy_(torch.from_numpy(vs_ref))
+            p.copy_(torch.from_numpy(p_ref))
+    return flips
+
+
+@pytest.mark.parametrize("n", [4098, 128 * 37, 128 * 1000 + 64, 2048 * 33, 1600 * 4800 // 8, 4096 * 1024 + 2])
+def test_fused_step_matches_oracle(oracle, qmaps, n):
+    flips = _run_fused_steps(oracle, qmaps, n, steps=5, seed=n)
+    print(f"n={n}: tie flips {flips}")
+
+
+def test_fused_step_odd_and_tiny(oracle, qmaps):
+    # the C ABI itself accepts any n >= 1, including odd n (last byte holds one code)
+    for n in (1, 2, 7, 127, 129, 4097, 2049 * 3):
+        _run_fused_steps(oracle, qmaps, n, steps=3, seed=100 + n)
+
+
+def test_fused_step_unaligned_pointers(oracle, qmaps):
+    for off in (1, 3):
+        _run_fused_steps(oracle, qmaps, 128 * 50 + 10, steps=3, seed=7, offset=off)
+
+
+def test_fused_step_zero_and_outlier_groups(oracle, qmaps):
+    """All-zero gradient groups (0/0 -> code 15, scale 0) and groups with a huge outlier."""
+
+    def grad_fn(rng, n, s):
+        g = (rng.standard_normal(n) * 1e-3).astype(np.float32)
+        g[: 128 * 3] = 0.0          # three groups that stay exactly zero
+        g[128 * 5 + 17] = 50.0      # one outlier
+        g[128 * 6: 128 * 7] = 1e-30  # g*g underflows to a denormal / zero
+        if s == 2:
+            g[128 * 8: 128 * 9] = 0.0
+        return g
+
+    _run_fused_steps(oracle, qmaps, 128 * 64, steps=4, seed=11, grad_fn=grad_fn)
+
+
+def test_fused_step_heavy_tailed(oracle, qmaps):
+    def grad_fn(rng, n, s):
+        z = rng.standard_normal((4, n))
+        return (z[0] / np.sqrt((z[1] ** 2 + z[2] ** 2 + z[3] ** 2) / 3.0) * 1e-3).astype(np.float32)
+
+    _run_fused_steps(oracle, qmaps, 128 * 4096, steps=6, seed=5, grad_fn=grad_fn)
+
+
+def test_fp32_step_matches_oracle(oracle):
+    nat = _native()
+    lib = nat.lib()
+    rng = np.random.default_rng(3)
+    for n in (1, 1600, 4096, 5000):
+        p_ref = (rng.standard_normal(n) * 0.02).astype(np.float32)
+        m_ref, v_ref = np.zeros(n, np.float32), np.zeros(n, np.float32)
+        p, m, v = to_dev(p_ref), to_dev(m_ref), to_dev(v_ref)
+        for s in range(1, 6):
+            g_np = (rng.standard_normal(n) * 1e-3).astype(np.float32)
+            g = to_dev(g_np)
+            st = lib.lpmm_adamw_fp32_step(p.data_ptr(), g.data_ptr(), m.data_ptr(), v.data_ptr(), n, 0.9, 0.999,
+                                          1e-3, 0.01, 1e-8, float(s), torch.cuda.current_stream().cuda_stream)
+            assert st == 0
+            oracle.adamw_fp32_step(p_ref, g_np, m_ref, v_ref, 0.9, 0.999, 1e-3, 0.01, 1e-8, float(s))
+            torch.cuda.synchronize()
+            np.testing.assert_array_equal(to_np(p), p_ref)
+            np.testing.assert_array_equal(to_np(m), m_ref)
+            np.testing.assert_array_equal(to_np(v), v_ref)
+
+
+def test_multi_tensor_matches_single(oracle, qmaps):
+    """lpmm_adamw4bit_step_multi over many tensors (more than one launch record) gives the
+    same bytes as the oracle run tensor by tensor, each tensor with its own step."""
+    nat = _native()
+    lib = nat.lib()
+    qm, qv = qmaps
+    dqm, dqv = to_dev(qm), to_dev(qv)
+    rng = np.random.default_rng(21)
+    sizes = [4098 + 2 * i for i in range(60)] + [128 * 700, 2048 * 9 + 130]
+    host, devs, recs = [], [], []
+    for i, n in enumerate(sizes):
+        nb, ng = (n + 1) // 2, (n + 127) // 128
+        h = dict(p=(rng.standard_normal(n) * 0.02).astype(np.float32),
+                 g=(rng.standard_normal(n) * 1e-3).astype(np.float32),
+                 mc=rng.integers(0, 256, nb, dtype=np.uint8), vc=rng.integers(0, 256, nb, dtype=np.uint8),
+                 ms=np.abs(rng.standard_normal(ng) * 1e-3).astype(np.float32),
+                 vs=np.abs(rng.standard_normal(ng) * 1e-6).astype(np.float32), step=float(1 + i % 7))
+        if n % 2:
+            h["mc"][-1] &= 0xF
+            h["vc"][-1] &= 0xF
+        d = {k: to_dev(v) for k, v in h.items() if k != "step"}
+        host.append(h); devs.append(d)
+        recs.append((d["p"].data_ptr(), d["g"].data_ptr(), d["mc"].data_ptr(), d["vc"].data_ptr(),
+                     d["ms"].data_ptr(), d["vs"].data_ptr(), n, h["step"], 0.0))
+    table = np.array(recs, dtype=nat.ADAMW4BIT_TENSOR)
+    st = lib.lpmm_adamw4bit_step_multi(table.ctypes.data, len(recs), dqm.data_ptr(), dqv.data_ptr(), 0.9, 0.999,
+                                       1e-3, 0.01, 1e-8, torch.cuda.current_stream().cuda_stream)
+    assert st == 0
+    torch.cuda.synchronize()
+    for h, d, n in zip(host, devs, sizes):
+        oracle.adamw4bit_step(h["p"], h["g"], h["mc"], h["vc"], h["ms"], h["vs"], qm, qv, 0.9, 0.999, 1e-3, 0.01,
+                              1e-8, h["step"])
+        assert_codes(to_np(d["mc"]), h["mc"], n, "m codes")
+        assert_codes(to_np(d["vc"]), h["vc"], n, "v codes")
+        assert_rel(to_np(d["ms"]), h["ms"], "m scale")
+        assert_rel(to_np(d["vs"]), h["vs"], "v scale")
+        assert_rel(to_np(d["p"]), h["p"], "p")

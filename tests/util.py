@@ -1,0 +1,47 @@
+"""Helpers shared by the GPU parity tests: seeded inputs and comparisons at the stated bars.
+
+Bars (from the task's north star): packed 4-bit codes bit-exact except at round-to-nearest
+ties, where they may differ by +-1 code on <= 1e-5 of the elements; scales and updated fp32
+parameters within 1e-6 relative."""
+import numpy as np
+import torch
+
+TIE_BUDGET = 1e-5
+REL_TOL = 1e-6
+
+
+def nibbles(codes, n):
+    c = np.asarray(codes).view(np.uint8).reshape(-1)
+    out = np.empty(c.size * 2, dtype=np.uint8)
+    out[0::2] = c & 0xF
+    out[1::2] = c >> 4
+    return out[:n]
+
+
+def assert_codes(got, want, n, what=""):
+    """Bit-exact, or within the tie budget: a differing code is off by one."""
+    a, b = nibbles(got, n), nibbles(want, n)
+    diff = np.flatnonzero(a != b)
+    if diff.size == 0:
+        return 0
+    assert diff.size <= TIE_BUDGET * n, f"{what}: {diff.size} of {n} codes differ (budget {TIE_BUDGET * n:.1f})"
+    assert np.all(np.abs(a[diff].astype(int) - b[diff].astype(int)) == 1), f"{what}: a code differs by more than 1"
+    return int(diff.size)
+
+
+def assert_rel(got, want, what="", tol=REL_TOL):
+    got = np.asarray(got, dtype=np.float64).reshape(-1)
+    want = np.asarray(want, dtype=np.float64).reshape(-1)
+    assert got.shape == want.shape, f"{what}: shape {got.shape} vs {want.shape}"
+    denom = np.maximum(np.abs(want), np.finfo(np.float32).tiny)
+    rel = np.abs(got - want) / denom
+    bad = np.flatnonzero(~(rel <= tol) & ~(got == want))
+    assert bad.size == 0, f"{what}: {bad.size} values beyond {tol} relative, worst {rel[bad].max():.3e}"
+
+
+def to_dev(a, device="cuda"):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(device)
+
+
+def to_np(t):
+    return t.detach().cpu().numpy()
