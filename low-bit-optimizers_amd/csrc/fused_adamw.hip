@@ -5,11 +5,21 @@
 // operation by operation, each operation rounded once (the file is compiled with
 // -ffp-contract=off, division and sqrt are the correctly rounded ones).
 //
-// Work layout of the 4-bit step: a lane owns 8 consecutive elements (32 B of p, 32 B of g,
-// one 32-bit word of m codes and one of v codes); 16 lanes = one DPP row own one
-// 128-element group, so the group maxima are 7 in-register max + 4 DPP steps and need
-// neither LDS nor atomics.  A 256-thread workgroup covers a tile of 2048 elements.
+// Work layout of the 4-bit step: 16 lanes (one DPP row) own one 128-element group, a lane
+// owns elements [4l, 4l+4) and [64+4l, 64+4l+4) of its group (l = lane within the row), so
+// every 16-byte load of a row covers 256 contiguous bytes and the group maxima are 7
+// in-register max + 4 DPP steps: no LDS traffic and no atomics for the reduction.  A
+// 256-thread workgroup covers a tile of 2048 elements = 16 groups.  LDS holds the two
+// 16-entry maps (decode) and the 2 KB first-moment encode table.
+//
+// When the maps passed in are the standard ones (dynamic-exponent signed map for m,
+// (k+1)/16 for v; checked on the device, no host round trip), the codes are assigned by
+// lpmm_encode.hpp (table for m, closed form for v) and the divisions by the group maximum
+// use the correctly rounded reciprocal plus one fma correction step; both give the same
+// results as the generic search and the plain division, which remain as the fallback for
+// any other map.
 #include "lpmm_common.hpp"
+#include "lpmm_encode.hpp"
 
 #include <math.h>
 
@@ -27,8 +37,8 @@ struct Tensor4 {
     float *ms;
     float *vs;
     int64_t n;
-    float c1;   // 1 - beta1^step
-    float c2s;  // sqrt(1 - beta2^step)
+    float c1;    // 1 - beta1^step
+    float c2s;   // sqrt(1 - beta2^step)
 };
 
 struct Multi4 {
@@ -52,6 +62,34 @@ __device__ __forceinline__ float adamw_elt(float p, float g, float &m, float &v,
     return p - (h.lr * update);
 }
 
+// x / y for |x| <= y given rc = RN(1/y): one multiply and two fmas give the correctly rounded
+// quotient when y lies in [2^-60, 2^60] (no intermediate underflow where it matters).
+__device__ __forceinline__ float div_by_rc(float x, float y, float rc)
+{
+    const float q = x * rc;
+    const float r = __builtin_fmaf(-q, y, x);
+    return __builtin_fmaf(r, rc, q);
+}
+
+__device__ __forceinline__ bool rc_safe(float y)
+{
+    return y >= 0x1p-60f && y <= 0x1p60f;
+}
+
+__device__ __forceinline__ bool maps_are_standard(const float *__restrict__ qmap_m,
+                                                  const float *__restrict__ qmap_v)
+{
+    bool same = true;
+#pragma unroll
+    for (int k = 0; k < 16; ++k)
+        same = same && (__float_as_uint(qmap_m[k]) == kStdQmapMBits[k]) &&
+               (__float_as_uint(qmap_v[k]) == kStdQmapVBits[k]);
+    return same;
+}
+
+// element k (0..7) of a lane sits at this offset inside the lane's group
+__device__ __forceinline__ int elt_offset(int lane16, int k) { return lane16 * 4 + (k & 3) + (k >> 2) * 64; }
+
 template <bool ALIGNED>
 __global__ __launch_bounds__(kThreads) void adamw4bit_kernel(const Multi4 args,
                                                              const float *__restrict__ qmap_m,
@@ -59,10 +97,15 @@ __global__ __launch_bounds__(kThreads) void adamw4bit_kernel(const Multi4 args,
 {
     __shared__ float s_qm[16];
     __shared__ float s_qv[16];
+    __shared__ uint4 s_enc[2 * kEncBuckets];
     if (threadIdx.x < 16)
         s_qm[threadIdx.x] = qmap_m[threadIdx.x];
     else if (threadIdx.x < 32)
         s_qv[threadIdx.x - 16] = qmap_v[threadIdx.x - 16];
+    if (threadIdx.x < 2 * kEncBuckets)
+        s_enc[threadIdx.x] = make_uint4(kEncTableM[threadIdx.x][0], kEncTableM[threadIdx.x][1],
+                                        kEncTableM[threadIdx.x][2], 0u);
+    const bool std_maps = maps_are_standard(qmap_m, qmap_v);
 
     // which tensor does this tile belong to (uniform over the workgroup)
     int lo = 0, hi = args.count;
@@ -75,7 +118,9 @@ __global__ __launch_bounds__(kThreads) void adamw4bit_kernel(const Multi4 args,
     }
     const Tensor4 &t = args.t[lo];
     const int64_t n = t.n;
-    const int64_t base = (int64_t)(blockIdx.x - args.tile_start[lo]) * kTile + (int64_t)threadIdx.x * kEltsPerLane;
+    const int lane16 = threadIdx.x & 15;
+    const int64_t grp = (int64_t)(blockIdx.x - args.tile_start[lo]) * (kTile / kGroup) + (threadIdx.x >> 4);
+    const int64_t gbase = grp * kGroup;
 
     Hyper h;
     h.beta1 = args.beta1;
@@ -87,25 +132,26 @@ __global__ __launch_bounds__(kThreads) void adamw4bit_kernel(const Multi4 args,
     h.eps = args.eps;
     h.c1 = t.c1;
     h.c2s = t.c2s;
-
-    const Mids mids_m = make_mids(qmap_m);
-    const Mids mids_v = make_mids(qmap_v);
     __syncthreads();
 
-    const int64_t grp = base / kGroup;
-    const bool any = base < n;
-    const bool full = ALIGNED && (base + kEltsPerLane <= n);
+    const bool any = gbase + lane16 * 4 < n;           // the lane's first element exists
+    const bool full = ALIGNED && (gbase + kGroup <= n);  // whole group inside: vector path
 
     float pv[kEltsPerLane], gv[kEltsPerLane], m[kEltsPerLane], v[kEltsPerLane];
-    uint32_t wm = 0, wv = 0;
+    uint32_t wm = 0, wv = 0;  // 8 nibbles each: elements 0..3 in the low half-word, 4..7 in the high
     float sm = 0.0f, sv = 0.0f;
 
     if (full) {
-        const float4 *p4 = reinterpret_cast<const float4 *>(t.p + base);
-        const float4 *g4 = reinterpret_cast<const float4 *>(t.g + base);
-        const float4 a0 = p4[0], a1 = p4[1], b0 = g4[0], b1 = g4[1];
-        wm = *reinterpret_cast<const uint32_t *>(t.mc + (base >> 1));
-        wv = *reinterpret_cast<const uint32_t *>(t.vc + (base >> 1));
+        const float *pp = t.p + gbase + lane16 * 4;
+        const float *gp = t.g + gbase + lane16 * 4;
+        const float4 a0 = *reinterpret_cast<const float4 *>(pp);
+        const float4 a1 = *reinterpret_cast<const float4 *>(pp + 64);
+        const float4 b0 = *reinterpret_cast<const float4 *>(gp);
+        const float4 b1 = *reinterpret_cast<const float4 *>(gp + 64);
+        const uint16_t *mcp = reinterpret_cast<const uint16_t *>(t.mc + (gbase >> 1)) + lane16;
+        const uint16_t *vcp = reinterpret_cast<const uint16_t *>(t.vc + (gbase >> 1)) + lane16;
+        wm = (uint32_t)mcp[0] | ((uint32_t)mcp[16] << 16);
+        wv = (uint32_t)vcp[0] | ((uint32_t)vcp[16] << 16);
         sm = t.ms[grp];
         sv = t.vs[grp];
         pv[0] = a0.x; pv[1] = a0.y; pv[2] = a0.z; pv[3] = a0.w;
@@ -117,16 +163,16 @@ __global__ __launch_bounds__(kThreads) void adamw4bit_kernel(const Multi4 args,
         sv = t.vs[grp];
 #pragma unroll
         for (int k = 0; k < kEltsPerLane; ++k) {
-            const int64_t i = base + k;
+            const int64_t i = gbase + elt_offset(lane16, k);
             pv[k] = (i < n) ? t.p[i] : 0.0f;
             gv[k] = (i < n) ? t.g[i] : 0.0f;
         }
 #pragma unroll
-        for (int k = 0; k < kEltsPerLane / 2; ++k) {
-            const int64_t i = base + 2 * k;
+        for (int k = 0; k < kEltsPerLane; k += 2) {
+            const int64_t i = gbase + elt_offset(lane16, k);
             if (i < n) {
-                wm |= (uint32_t)t.mc[i >> 1] << (8 * k);
-                wv |= (uint32_t)t.vc[i >> 1] << (8 * k);
+                wm |= (uint32_t)t.mc[i >> 1] << (4 * k);
+                wv |= (uint32_t)t.vc[i >> 1] << (4 * k);
             }
         }
     }
@@ -137,7 +183,7 @@ __global__ __launch_bounds__(kThreads) void adamw4bit_kernel(const Multi4 args,
         for (int k = 0; k < kEltsPerLane; ++k) {
             m[k] = s_qm[(wm >> (4 * k)) & 0xF] * sm;
             v[k] = s_qv[(wv >> (4 * k)) & 0xF] * sv;
-            const bool valid = full || (base + k < n);
+            const bool valid = full || (gbase + elt_offset(lane16, k) < n);
             if (valid) {
                 pv[k] = adamw_elt(pv[k], gv[k], m[k], v[k], h);
                 amax_m = fmaxf(amax_m, fabsf(m[k]));
@@ -155,42 +201,57 @@ __global__ __launch_bounds__(kThreads) void adamw4bit_kernel(const Multi4 args,
         return;
 
     uint32_t om = 0, ov = 0;
-    const bool nan_m = (amax_m == 0.0f);  // x/0 with x == 0: NaN -> code 15 for the whole group
+    // x/0 with x == 0 is NaN, which the reference turns into code 15 for the whole group
+    const bool nan_m = (amax_m == 0.0f);
     const bool nan_v = (amax_v == 0.0f);
+    if (std_maps && rc_safe(amax_m) && rc_safe(amax_v)) {
+        const float rcm = 1.0f / amax_m, rcv = 1.0f / amax_v;
 #pragma unroll
-    for (int k = 0; k < kEltsPerLane; ++k) {
-        const bool valid = full || (base + k < n);
-        uint32_t cm = nan_m ? 15u : encode_count(mids_m, m[k] / amax_m);
-        uint32_t cv = nan_v ? 15u : encode_count(mids_v, v[k] / amax_v);
-        if (!valid) {
-            cm = 0;
-            cv = 0;
+        for (int k = 0; k < kEltsPerLane; ++k) {
+            const uint32_t xb = __float_as_uint(div_by_rc(m[k], amax_m, rcm));
+            const uint4 e = *reinterpret_cast<const uint4 *>(reinterpret_cast<const char *>(s_enc) + enc_m_offset(xb));
+            om |= enc_m_select(xb, e.x, e.y, e.z) << (4 * k);
+            ov |= enc_v_linear(div_by_rc(v[k], amax_v, rcv)) << (4 * k);
         }
-        om |= cm << (4 * k);
-        ov |= cv << (4 * k);
+    } else {
+        const Mids mids_m = make_mids(qmap_m);
+        const Mids mids_v = make_mids(qmap_v);
+#pragma unroll
+        for (int k = 0; k < kEltsPerLane; ++k) {
+            om |= (nan_m ? 15u : encode_count(mids_m, m[k] / amax_m)) << (4 * k);
+            ov |= (nan_v ? 15u : encode_count(mids_v, v[k] / amax_v)) << (4 * k);
+        }
     }
 
     if (full) {
-        float4 *p4 = reinterpret_cast<float4 *>(t.p + base);
-        p4[0] = make_float4(pv[0], pv[1], pv[2], pv[3]);
-        p4[1] = make_float4(pv[4], pv[5], pv[6], pv[7]);
-        *reinterpret_cast<uint32_t *>(t.mc + (base >> 1)) = om;
-        *reinterpret_cast<uint32_t *>(t.vc + (base >> 1)) = ov;
+        float *pp = t.p + gbase + lane16 * 4;
+        *reinterpret_cast<float4 *>(pp) = make_float4(pv[0], pv[1], pv[2], pv[3]);
+        *reinterpret_cast<float4 *>(pp + 64) = make_float4(pv[4], pv[5], pv[6], pv[7]);
+        uint16_t *mcp = reinterpret_cast<uint16_t *>(t.mc + (gbase >> 1)) + lane16;
+        uint16_t *vcp = reinterpret_cast<uint16_t *>(t.vc + (gbase >> 1)) + lane16;
+        mcp[0] = (uint16_t)om;
+        mcp[16] = (uint16_t)(om >> 16);
+        vcp[0] = (uint16_t)ov;
+        vcp[16] = (uint16_t)(ov >> 16);
     } else {
 #pragma unroll
-        for (int k = 0; k < kEltsPerLane; ++k)
-            if (base + k < n)
-                t.p[base + k] = pv[k];
+        for (int k = 0; k < kEltsPerLane; ++k) {
+            const int64_t i = gbase + elt_offset(lane16, k);
+            if (i < n)
+                t.p[i] = pv[k];
+        }
 #pragma unroll
-        for (int k = 0; k < kEltsPerLane / 2; ++k) {
-            const int64_t i = base + 2 * k;
+        for (int k = 0; k < kEltsPerLane; k += 2) {
+            const int64_t i = gbase + elt_offset(lane16, k);
             if (i < n) {
-                t.mc[i >> 1] = (uint8_t)(om >> (8 * k));
-                t.vc[i >> 1] = (uint8_t)(ov >> (8 * k));
+                // a last odd element leaves the high nibble of its byte 0
+                const uint32_t keep = (i + 1 < n) ? 0xFFu : 0x0Fu;
+                t.mc[i >> 1] = (uint8_t)((om >> (4 * k)) & keep);
+                t.vc[i >> 1] = (uint8_t)((ov >> (4 * k)) & keep);
             }
         }
     }
-    if ((threadIdx.x & 15) == 0) {
+    if (lane16 == 0) {
         t.ms[grp] = amax_m;
         t.vs[grp] = amax_v;
     }
@@ -298,8 +359,8 @@ extern "C" int lpmm_adamw4bit_step_multi(const lpmm_adamw4bit_tensor *tensors, i
         LPMM_REQUIRE_ALIGN(t.v_scale, 4);
         if ((t.n + kTile - 1) / kTile > 0x7fffffffLL)
             return LPMM_ERR_SIZE;
-        aligned = aligned && aligned_to(t.p, 16) && aligned_to(t.g, 16) && aligned_to(t.m_codes, 4) &&
-                  aligned_to(t.v_codes, 4);
+        aligned = aligned && aligned_to(t.p, 16) && aligned_to(t.g, 16) && aligned_to(t.m_codes, 2) &&
+                  aligned_to(t.v_codes, 2);
     }
 
     Multi4 args;
