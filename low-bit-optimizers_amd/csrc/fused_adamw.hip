@@ -39,26 +39,70 @@ struct Tensor4 {
     int64_t n;
     float c1;    // 1 - beta1^step
     float c2s;   // sqrt(1 - beta2^step)
+    float rc2s;  // 1 / c2s, correctly rounded (host division)
+    float pad;
 };
 
 struct Multi4 {
     Tensor4 t[LPMM_MULTI_MAX];
     uint32_t tile_start[LPMM_MULTI_MAX + 1];  // prefix sum of tiles per tensor
     int count;
-    float beta1, beta2, lr, wd, eps;
+    float beta1, beta2, omb1, omb2, lr, wd, eps;  // omb = 1 - beta, subtracted in float on the host
 };
 
+static_assert(sizeof(Multi4) + 2 * sizeof(void *) <= 4096, "kernel arguments exceed 4 KB");
+
 struct Hyper {
-    float beta1, beta2, omb1, omb2, lr, wd, eps, c1, c2s;
+    float beta1, beta2, omb1, omb2, lr, wd, eps, c1, c2s, rc2s;
 };
+
+#ifndef LPMM_P_MODE
+#define LPMM_P_MODE 1
+#endif
+#ifndef LPMM_NT
+#define LPMM_NT 3
+#endif
+
+// sqrt(x) for x >= 0 from the hardware reciprocal square root plus one fma correction of
+// the residual: correctly rounded except for a vanishing fraction of inputs (1 ulp there).
+// Inputs below the smallest normal are treated as that value (their square root is far
+// below any eps it is added to).
+__device__ __forceinline__ float sqrt_fast(float x)
+{
+    const float y = __builtin_amdgcn_rsqf(fmaxf(x, 0x1p-126f));
+    const float s = x * y;
+    const float h = 0.5f * y;
+    const float r = __builtin_fmaf(-s, s, x);
+    return __builtin_fmaf(r, h, s);
+}
+
+// x / d from the hardware reciprocal plus one fma correction of the residual (same remark).
+__device__ __forceinline__ float div_fast(float x, float d)
+{
+    const float rc = __builtin_amdgcn_rcpf(d);
+    const float q = x * rc;
+    const float r = __builtin_fmaf(-q, d, x);
+    return __builtin_fmaf(r, rc, q);
+}
 
 // AdamW on one element; returns the new parameter, updates m and v in place.
 __device__ __forceinline__ float adamw_elt(float p, float g, float &m, float &v, const Hyper &h)
 {
     m = h.beta1 * m + h.omb1 * g;
     v = h.beta2 * v + h.omb2 * g * g;
+#if LPMM_P_MODE == 0
     const float denom = (sqrtf(v) / h.c2s + h.eps) * h.c1;
     const float update = (m / denom) + (h.wd * p);
+#elif LPMM_P_MODE == 1
+    const float s = sqrt_fast(v);
+    const float q = s * h.rc2s;
+    const float sq = __builtin_fmaf(__builtin_fmaf(-q, h.c2s, s), h.rc2s, q);
+    const float denom = (sq + h.eps) * h.c1;
+    const float update = div_fast(m, denom) + (h.wd * p);
+#else
+    const float denom = (__builtin_amdgcn_sqrtf(v) * h.rc2s + h.eps) * h.c1;
+    const float update = m * __builtin_amdgcn_rcpf(denom) + (h.wd * p);
+#endif
     return p - (h.lr * update);
 }
 
@@ -79,79 +123,88 @@ __device__ __forceinline__ bool rc_safe(float y)
 __device__ __forceinline__ bool maps_are_standard(const float *__restrict__ qmap_m,
                                                   const float *__restrict__ qmap_v)
 {
-    bool same = true;
+    // all 32 words are fetched at once (scalar loads) and folded without branches
+    uint32_t diff = 0;
 #pragma unroll
     for (int k = 0; k < 16; ++k)
-        same = same && (__float_as_uint(qmap_m[k]) == kStdQmapMBits[k]) &&
-               (__float_as_uint(qmap_v[k]) == kStdQmapVBits[k]);
-    return same;
+        diff |= (__float_as_uint(qmap_m[k]) ^ kStdQmapMBits[k]) | (__float_as_uint(qmap_v[k]) ^ kStdQmapVBits[k]);
+    return diff == 0;
+}
+
+typedef float v4f __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ float4 load4(const float *p)
+{
+#if LPMM_NT & 1
+    const v4f t = __builtin_nontemporal_load(reinterpret_cast<const v4f *>(p));
+    return make_float4(t.x, t.y, t.z, t.w);
+#else
+    return *reinterpret_cast<const float4 *>(p);
+#endif
+}
+__device__ __forceinline__ void store4(float *p, float4 v)
+{
+#if LPMM_NT & 2
+    const v4f t = {v.x, v.y, v.z, v.w};
+    __builtin_nontemporal_store(t, reinterpret_cast<v4f *>(p));
+#else
+    *reinterpret_cast<float4 *>(p) = v;
+#endif
+}
+__device__ __forceinline__ uint32_t load_u16(const uint16_t *p)
+{
+#if LPMM_NT & 1
+    return __builtin_nontemporal_load(p);
+#else
+    return *p;
+#endif
+}
+__device__ __forceinline__ void store_u16(uint16_t *p, uint32_t v)
+{
+#if LPMM_NT & 2
+    __builtin_nontemporal_store((uint16_t)v, p);
+#else
+    *p = (uint16_t)v;
+#endif
 }
 
 // element k (0..7) of a lane sits at this offset inside the lane's group
 __device__ __forceinline__ int elt_offset(int lane16, int k) { return lane16 * 4 + (k & 3) + (k >> 2) * 64; }
 
-template <bool ALIGNED>
-__global__ __launch_bounds__(kThreads) void adamw4bit_kernel(const Multi4 args,
-                                                             const float *__restrict__ qmap_m,
-                                                             const float *__restrict__ qmap_v)
+// LDS map of the 4-bit kernel (bytes): [0,64) qmap_m, [64,128) qmap_v, then the
+// first-moment encode table at the offsets lpmm_encode.hpp computes.
+constexpr uint32_t kLdsBytes = kEncLdsEnd;
+constexpr uint32_t kLdsQm = 0, kLdsQv = 64;
+static_assert(kLdsQv + 64 <= kEncLdsBegin, "maps overlap the encode table");
+
+template <typename T>
+__device__ __forceinline__ T lds_read(const uint32_t *lds, uint32_t byte_off)
 {
-    __shared__ float s_qm[16];
-    __shared__ float s_qv[16];
-    __shared__ uint4 s_enc[2 * kEncBuckets];
-    if (threadIdx.x < 16)
-        s_qm[threadIdx.x] = qmap_m[threadIdx.x];
-    else if (threadIdx.x < 32)
-        s_qv[threadIdx.x - 16] = qmap_v[threadIdx.x - 16];
-    if (threadIdx.x < 2 * kEncBuckets)
-        s_enc[threadIdx.x] = make_uint4(kEncTableM[threadIdx.x][0], kEncTableM[threadIdx.x][1],
-                                        kEncTableM[threadIdx.x][2], 0u);
-    const bool std_maps = maps_are_standard(qmap_m, qmap_v);
+    return *reinterpret_cast<const T *>(reinterpret_cast<const char *>(lds) + byte_off);
+}
 
-    // which tensor does this tile belong to (uniform over the workgroup)
-    int lo = 0, hi = args.count;
-    while (hi - lo > 1) {
-        const int mid = (lo + hi) >> 1;
-        if (args.tile_start[mid] <= blockIdx.x)
-            lo = mid;
-        else
-            hi = mid;
-    }
-    const Tensor4 &t = args.t[lo];
+// One 128-element group, handled by the 16 lanes of a DPP row.  FULL: the whole group lies
+// inside the tensor and the pointers allow vector access; otherwise every access is
+// guarded per element.  All 16 lanes take the same instantiation.
+template <bool FULL>
+__device__ __forceinline__ void group_step(const Tensor4 &t, const Hyper &h, const uint32_t *lds,
+                                           bool std_maps, int64_t grp, int lane16)
+{
     const int64_t n = t.n;
-    const int lane16 = threadIdx.x & 15;
-    const int64_t grp = (int64_t)(blockIdx.x - args.tile_start[lo]) * (kTile / kGroup) + (threadIdx.x >> 4);
     const int64_t gbase = grp * kGroup;
-
-    Hyper h;
-    h.beta1 = args.beta1;
-    h.beta2 = args.beta2;
-    h.omb1 = 1 - args.beta1;
-    h.omb2 = 1 - args.beta2;
-    h.lr = args.lr;
-    h.wd = args.wd;
-    h.eps = args.eps;
-    h.c1 = t.c1;
-    h.c2s = t.c2s;
-    __syncthreads();
-
-    const bool any = gbase + lane16 * 4 < n;           // the lane's first element exists
-    const bool full = ALIGNED && (gbase + kGroup <= n);  // whole group inside: vector path
-
     float pv[kEltsPerLane], gv[kEltsPerLane], m[kEltsPerLane], v[kEltsPerLane];
     uint32_t wm = 0, wv = 0;  // 8 nibbles each: elements 0..3 in the low half-word, 4..7 in the high
     float sm = 0.0f, sv = 0.0f;
+    const bool any = FULL || (gbase + lane16 * 4 < n);  // the lane's first element exists
 
-    if (full) {
+    if (FULL) {
         const float *pp = t.p + gbase + lane16 * 4;
         const float *gp = t.g + gbase + lane16 * 4;
-        const float4 a0 = *reinterpret_cast<const float4 *>(pp);
-        const float4 a1 = *reinterpret_cast<const float4 *>(pp + 64);
-        const float4 b0 = *reinterpret_cast<const float4 *>(gp);
-        const float4 b1 = *reinterpret_cast<const float4 *>(gp + 64);
+        const float4 a0 = load4(pp), a1 = load4(pp + 64);
+        const float4 b0 = load4(gp), b1 = load4(gp + 64);
         const uint16_t *mcp = reinterpret_cast<const uint16_t *>(t.mc + (gbase >> 1)) + lane16;
         const uint16_t *vcp = reinterpret_cast<const uint16_t *>(t.vc + (gbase >> 1)) + lane16;
-        wm = (uint32_t)mcp[0] | ((uint32_t)mcp[16] << 16);
-        wv = (uint32_t)vcp[0] | ((uint32_t)vcp[16] << 16);
+        wm = load_u16(mcp) | (load_u16(mcp + 16) << 16);
+        wv = load_u16(vcp) | (load_u16(vcp + 16) << 16);
         sm = t.ms[grp];
         sv = t.vs[grp];
         pv[0] = a0.x; pv[1] = a0.y; pv[2] = a0.z; pv[3] = a0.w;
@@ -177,21 +230,25 @@ __global__ __launch_bounds__(kThreads) void adamw4bit_kernel(const Multi4 args,
         }
     }
 
+    // decode: byte j of the *_even / *_odd words holds 4 * nibble (2j) / (2j+1) = LDS offset
+    uint32_t me = (wm << 2) & 0x3C3C3C3Cu, mo = (wm >> 2) & 0x3C3C3C3Cu;
+    uint32_t ve = (wv << 2) & 0x3C3C3C3Cu, vo = (wv >> 2) & 0x3C3C3C3Cu;
+    // keep the four masked words as they are, so that each offset below is one bit-field extract
+    asm volatile("" : "+v"(me), "+v"(mo), "+v"(ve), "+v"(vo));
     float amax_m = 0.0f, amax_v = 0.0f;
-    if (any) {
 #pragma unroll
-        for (int k = 0; k < kEltsPerLane; ++k) {
-            m[k] = s_qm[(wm >> (4 * k)) & 0xF] * sm;
-            v[k] = s_qv[(wv >> (4 * k)) & 0xF] * sv;
-            const bool valid = full || (gbase + elt_offset(lane16, k) < n);
-            if (valid) {
-                pv[k] = adamw_elt(pv[k], gv[k], m[k], v[k], h);
-                amax_m = fmaxf(amax_m, fabsf(m[k]));
-                amax_v = fmaxf(amax_v, v[k]);
-            } else {
-                m[k] = 0.0f;
-                v[k] = 0.0f;
-            }
+    for (int k = 0; k < kEltsPerLane; ++k) {
+        const uint32_t om = __builtin_amdgcn_ubfe((k & 1) ? mo : me, 8 * (k >> 1), 8);
+        const uint32_t ov = __builtin_amdgcn_ubfe((k & 1) ? vo : ve, 8 * (k >> 1), 8);
+        m[k] = lds_read<float>(lds, kLdsQm + om) * sm;
+        v[k] = lds_read<float>(lds, kLdsQv + ov) * sv;
+        if (FULL || (gbase + elt_offset(lane16, k) < n)) {
+            pv[k] = adamw_elt(pv[k], gv[k], m[k], v[k], h);
+            amax_m = fmaxf(amax_m, fabsf(m[k]));
+            amax_v = fmaxf(amax_v, v[k]);
+        } else {
+            m[k] = 0.0f;
+            v[k] = 0.0f;
         }
     }
     // every lane of the row takes part, also those past the end of the tensor
@@ -200,39 +257,46 @@ __global__ __launch_bounds__(kThreads) void adamw4bit_kernel(const Multi4 args,
     if (!any)
         return;
 
-    uint32_t om = 0, ov = 0;
-    // x/0 with x == 0 is NaN, which the reference turns into code 15 for the whole group
-    const bool nan_m = (amax_m == 0.0f);
-    const bool nan_v = (amax_v == 0.0f);
+    uint32_t cm = 0, cv = 0;
     if (std_maps && rc_safe(amax_m) && rc_safe(amax_v)) {
         const float rcm = 1.0f / amax_m, rcv = 1.0f / amax_v;
+        uint32_t vb[2] = {0u, 0u};  // v codes of elements 0..3 / 4..7, one per byte
 #pragma unroll
         for (int k = 0; k < kEltsPerLane; ++k) {
-            const uint32_t xb = __float_as_uint(div_by_rc(m[k], amax_m, rcm));
-            const uint4 e = *reinterpret_cast<const uint4 *>(reinterpret_cast<const char *>(s_enc) + enc_m_offset(xb));
-            om |= enc_m_select(xb, e.x, e.y, e.z) << (4 * k);
-            ov |= enc_v_linear(div_by_rc(v[k], amax_v, rcv)) << (4 * k);
+            const float xm = div_by_rc(m[k], amax_m, rcm);
+            const uint4 e = lds_read<uint4>(lds, enc_m_lds_offset(xm));
+            cm |= enc_m_pick(xm, e.x, e.y, e.z) << (4 * k);
+            // enc_v_linear with the clamp at 0 done by the saturating byte conversion
+            // (0 <= x <= 1 here, so the value never exceeds 15)
+            const float tv = __builtin_ceilf(__builtin_fmaf(div_by_rc(v[k], amax_v, rcv), 16.0f, -1.5f));
+            vb[k >> 2] = __builtin_amdgcn_cvt_pk_u8_f32(tv, k & 3, vb[k >> 2]);
         }
+        // bytes {c0,c1,c2,c3} -> byte 0 = c0|c1<<4, byte 2 = c2|c3<<4; gather bytes 0,2 of both words
+        const uint32_t t0 = vb[0] | (vb[0] >> 4), t1 = vb[1] | (vb[1] >> 4);
+        cv = __builtin_amdgcn_perm(t1, t0, 0x06040200u);
     } else {
-        const Mids mids_m = make_mids(qmap_m);
-        const Mids mids_v = make_mids(qmap_v);
+        // x/0 with x == 0 is NaN, which the reference turns into code 15 for the whole group
+        const bool nan_m = (amax_m == 0.0f), nan_v = (amax_v == 0.0f);
+        // the maps are read back from LDS so that they occupy registers only on this path
+        const Mids mids_m = make_mids(reinterpret_cast<const float *>(lds) + kLdsQm / 4);
+        const Mids mids_v = make_mids(reinterpret_cast<const float *>(lds) + kLdsQv / 4);
 #pragma unroll
         for (int k = 0; k < kEltsPerLane; ++k) {
-            om |= (nan_m ? 15u : encode_count(mids_m, m[k] / amax_m)) << (4 * k);
-            ov |= (nan_v ? 15u : encode_count(mids_v, v[k] / amax_v)) << (4 * k);
+            cm |= (nan_m ? 15u : encode_count(mids_m, m[k] / amax_m)) << (4 * k);
+            cv |= (nan_v ? 15u : encode_count(mids_v, v[k] / amax_v)) << (4 * k);
         }
     }
 
-    if (full) {
+    if (FULL) {
         float *pp = t.p + gbase + lane16 * 4;
-        *reinterpret_cast<float4 *>(pp) = make_float4(pv[0], pv[1], pv[2], pv[3]);
-        *reinterpret_cast<float4 *>(pp + 64) = make_float4(pv[4], pv[5], pv[6], pv[7]);
+        store4(pp, make_float4(pv[0], pv[1], pv[2], pv[3]));
+        store4(pp + 64, make_float4(pv[4], pv[5], pv[6], pv[7]));
         uint16_t *mcp = reinterpret_cast<uint16_t *>(t.mc + (gbase >> 1)) + lane16;
         uint16_t *vcp = reinterpret_cast<uint16_t *>(t.vc + (gbase >> 1)) + lane16;
-        mcp[0] = (uint16_t)om;
-        mcp[16] = (uint16_t)(om >> 16);
-        vcp[0] = (uint16_t)ov;
-        vcp[16] = (uint16_t)(ov >> 16);
+        store_u16(mcp, cm & 0xFFFFu);
+        store_u16(mcp + 16, cm >> 16);
+        store_u16(vcp, cv & 0xFFFFu);
+        store_u16(vcp + 16, cv >> 16);
     } else {
 #pragma unroll
         for (int k = 0; k < kEltsPerLane; ++k) {
@@ -246,8 +310,8 @@ __global__ __launch_bounds__(kThreads) void adamw4bit_kernel(const Multi4 args,
             if (i < n) {
                 // a last odd element leaves the high nibble of its byte 0
                 const uint32_t keep = (i + 1 < n) ? 0xFFu : 0x0Fu;
-                t.mc[i >> 1] = (uint8_t)((om >> (4 * k)) & keep);
-                t.vc[i >> 1] = (uint8_t)((ov >> (4 * k)) & keep);
+                t.mc[i >> 1] = (uint8_t)((cm >> (4 * k)) & keep);
+                t.vc[i >> 1] = (uint8_t)((cv >> (4 * k)) & keep);
             }
         }
     }
@@ -255,6 +319,52 @@ __global__ __launch_bounds__(kThreads) void adamw4bit_kernel(const Multi4 args,
         t.ms[grp] = amax_m;
         t.vs[grp] = amax_v;
     }
+}
+
+template <bool ALIGNED>
+__global__ __launch_bounds__(kThreads) void adamw4bit_kernel(const Multi4 args,
+                                                             const float *__restrict__ qmap_m,
+                                                             const float *__restrict__ qmap_v)
+{
+    __shared__ __align__(16) uint32_t lds[kLdsBytes / 4];
+    if (threadIdx.x < 16)
+        lds[kLdsQm / 4 + threadIdx.x] = __float_as_uint(qmap_m[threadIdx.x]);
+    else if (threadIdx.x < 32)
+        lds[kLdsQv / 4 + threadIdx.x - 16] = __float_as_uint(qmap_v[threadIdx.x - 16]);
+    if (threadIdx.x < 2 * kEncBuckets) {
+        const uint4 e = *reinterpret_cast<const uint4 *>(kEncTableM[threadIdx.x]);
+        *reinterpret_cast<uint4 *>(reinterpret_cast<char *>(lds) + e.w) = e;  // e.w: the entry's LDS offset
+    }
+    const bool std_maps = maps_are_standard(qmap_m, qmap_v);
+
+    // which tensor does this tile belong to (uniform over the workgroup): the number of
+    // later tensors whose first tile is not after this one; unused slots hold the total
+    // (one entry per lane, one ballot per wave)
+    static_assert(LPMM_MULTI_MAX <= kWave, "one tile_start entry per lane");
+    const int lane = threadIdx.x & (kWave - 1);
+    const bool started = lane + 1 < LPMM_MULTI_MAX && args.tile_start[lane + 1] <= blockIdx.x;
+    const int lo = __popcll(__ballot(started));
+    const Tensor4 &t = args.t[lo];
+    const int lane16 = threadIdx.x & 15;
+    const int64_t grp = (int64_t)(blockIdx.x - args.tile_start[lo]) * (kTile / kGroup) + (threadIdx.x >> 4);
+
+    Hyper h;
+    h.beta1 = args.beta1;
+    h.beta2 = args.beta2;
+    h.omb1 = args.omb1;
+    h.omb2 = args.omb2;
+    h.lr = args.lr;
+    h.wd = args.wd;
+    h.eps = args.eps;
+    h.c1 = t.c1;
+    h.c2s = t.c2s;
+    h.rc2s = t.rc2s;
+    __syncthreads();
+
+    if (ALIGNED && (grp + 1) * kGroup <= t.n)
+        group_step<true>(t, h, lds, std_maps, grp, lane16);
+    else
+        group_step<false>(t, h, lds, std_maps, grp, lane16);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -301,6 +411,7 @@ __global__ __launch_bounds__(kThreads) void adamw_fp32_kernel(const MultiF args)
     h.eps = args.eps;
     h.c1 = t.c1;
     h.c2s = t.c2s;
+    h.rc2s = 1.0f / t.c2s;
     const int64_t tile0 = (int64_t)(blockIdx.x - args.tile_start[lo]) * kTileF;
 #pragma unroll
     for (int k = 0; k < kTileF / kThreads; ++k) {
@@ -366,6 +477,8 @@ extern "C" int lpmm_adamw4bit_step_multi(const lpmm_adamw4bit_tensor *tensors, i
     Multi4 args;
     args.beta1 = beta1;
     args.beta2 = beta2;
+    args.omb1 = 1 - beta1;
+    args.omb2 = 1 - beta2;
     args.lr = lr;
     args.wd = weight_decay;
     args.eps = eps;
@@ -392,6 +505,8 @@ extern "C" int lpmm_adamw4bit_step_multi(const lpmm_adamw4bit_tensor *tensors, i
             d.vs = t.v_scale;
             d.n = t.n;
             bias_corrections(beta1, beta2, t.step, &d.c1, &d.c2s);
+            d.rc2s = 1.0f / d.c2s;
+            d.pad = 0.0f;
             tiles += nt;
             args.tile_start[++k] = (uint32_t)tiles;
             ++i;
