@@ -1,0 +1,212 @@
+#!/usr/bin/env python3
+"""Headline benchmark: fused 4-bit AdamW step on a LLaMA-7B-shaped fp32 parameter set.
+
+One "step" = one `lpmm.optim.AdamW(fused=True).step()` over all 291 tensors (6 738 415 616
+parameters) with parameters, gradients and states resident in HBM.  Prints ONE JSON line
+with the step throughput (params/s), the HBM roofline of the dominant kernel measured live
+with events on the launch stream, and a CPU baseline (the reference's non-fused PyTorch op
+sequence on the host cores, bounded sample).
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload llama7b|gpt2xl|tiny]
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, "low-bit-optimizers_amd")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+BYTES_PER_PARAM_4BIT = 14.125  # p r/w 8 + g 4 + m codes 1 + v codes 1 + scales 16/128
+BYTES_PER_PARAM_FP32 = 28.0    # p, m, v r/w + g r
+MULTI_MAX = 48                 # tensors per launch record (LPMM_MULTI_MAX)
+
+
+def llama7b_shapes():
+    shapes = [(32000, 4096)]
+    for _ in range(32):
+        shapes += [(4096, 4096)] * 4 + [(11008, 4096)] * 2 + [(4096, 11008)] + [(4096,)] * 2
+    shapes += [(4096,), (32000, 4096)]
+    return shapes
+
+
+def gpt2xl_shapes():
+    d = 1600
+    shapes = [(50257, d), (1024, d)]
+    for _ in range(48):
+        shapes += [(d,), (d,), (d, 3 * d), (3 * d,), (d, d), (d,), (d,), (d,), (d, 4 * d), (4 * d,), (4 * d, d), (d,)]
+    shapes += [(d,), (d,)]
+    return shapes
+
+
+def tiny_shapes():
+    return [(4096, 1024), (1024, 4096), (4096,), (8192,), (1000, 1000)] * 4
+
+
+WORKLOADS = {
+    "llama7b": ("fused 4-bit AdamW, LLaMA-7B-shaped fp32 set (291 tensors, 6.74e9 params), "
+                "grads Student-t(3) x 1e-3", llama7b_shapes),
+    "gpt2xl": ("fused 4-bit AdamW, GPT-2-XL-shaped fp32 set (580 tensors, 1.56e9 params), grads N(0,1e-3)",
+               gpt2xl_shapes),
+    "tiny": ("fused 4-bit AdamW, small test set", tiny_shapes),
+}
+
+
+def make_params(torch, shapes, dev, heavy_tailed):
+    params = []
+    gen = torch.Generator(device=dev)
+    for i, shape in enumerate(shapes):
+        gen.manual_seed(10000 + i)
+        p = torch.nn.Parameter(torch.randn(shape, device=dev, generator=gen) * 0.02)
+        gen.manual_seed(20000 + i)
+        z = torch.randn(shape, device=dev, generator=gen)
+        if heavy_tailed:  # Student-t, 3 degrees of freedom: z / sqrt((a^2+b^2+c^2)/3)
+            s = torch.zeros(shape, device=dev)
+            for _ in range(3):
+                a = torch.randn(shape, device=dev, generator=gen)
+                s.addcmul_(a, a)
+            z.div_(s.div_(3.0).sqrt_())
+            del s, a
+        p.grad = z.mul_(1e-3)
+        params.append(p)
+    return params
+
+
+def cpu_baseline(torch, steps=3):
+    """The reference's non-fused PyTorch path (op sequence of _single_tensor_adamw4bit) on the
+    host cores: one 4096x4096 fp32 parameter, m group-128 / v rank-1, all threads."""
+    from oracle.nonfused_torch import TorchNonFusedAdamW
+
+    threads = os.cpu_count() or 1
+    torch.set_num_threads(threads)
+    g = torch.Generator().manual_seed(0)
+    p = torch.randn(4096, 4096, generator=g) * 0.02
+    opt = TorchNonFusedAdamW([p], lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01, v_scale_type="rank1")
+    times = []
+    for s in range(steps + 1):
+        gg = torch.Generator().manual_seed(1000 + s)
+        grad = torch.randn(4096, 4096, generator=gg) * 1e-3
+        t0 = time.perf_counter()
+        opt.step([grad])
+        times.append(time.perf_counter() - t0)
+    times = sorted(times[1:])
+    med = times[len(times) // 2]
+    return {
+        "value": p.numel() / med,
+        "unit": "params/s",
+        "cores": threads,
+        "kind": "port",
+        "sample": f"non-fused PyTorch-op path on CPU, one 4096x4096 fp32 tensor, m group-128 / v rank-1, "
+                  f"median of {steps} steps after 1 warm-up",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--workload", default="llama7b", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU; --gpus N with N > 1 is not supported "
+                 "(the step is rank-local; see DESIGN.md for how it would shard).")
+
+    import torch
+
+    import lpmm
+    from lpmm import _native
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    lib = _native.lib()
+
+    desc, shape_fn = WORKLOADS[args.workload]
+    shapes = shape_fn()
+    params = make_params(torch, shapes, dev, heavy_tailed=(args.workload == "llama7b"))
+    opt = lpmm.optim.AdamW(params, lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01, fused=True)
+
+    n_total = sum(p.numel() for p in params)
+    n_quant = sum(p.numel() for p in params if p.numel() > 4096)
+    n_quant_tensors = sum(1 for p in params if p.numel() > 4096)
+    launches_per_step = math.ceil(n_quant_tensors / MULTI_MAX)
+
+    # events around the dominant kernel's launches (same stream as the launches)
+    events = []
+    real_call = lib.lpmm_adamw4bit_step_multi
+    recording = {"on": False}
+
+    def timed_call(*a):
+        if not recording["on"]:
+            return real_call(*a)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        st = real_call(*a)
+        e1.record()
+        events.append((e0, e1))
+        return st
+
+    lib.lpmm_adamw4bit_step_multi = timed_call
+
+    for _ in range(args.warmup):
+        opt.step()
+    torch.cuda.synchronize()
+    recording["on"] = True
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        opt.step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    recording["on"] = False
+
+    ms_per_step = elapsed * 1e3 / args.steps
+    value = n_total / (elapsed / args.steps)
+    kernel_ms_per_step = sum(e0.elapsed_time(e1) for e0, e1 in events) / args.steps
+    launch_ms = kernel_ms_per_step / launches_per_step
+    bytes_per_launch = n_quant * BYTES_PER_PARAM_4BIT / launches_per_step
+    achieved = bytes_per_launch / (launch_ms * 1e-3) / 1e9
+
+    out = {
+        "metric": "fused 4-bit AdamW step: params/sec and % HBM roofline, 1 MI355X",
+        "value": value,
+        "unit": "params/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": desc, "tensors": len(params), "params": n_total, "quantized_params": n_quant,
+                   "launches_per_step": launches_per_step + 1},
+        "effective_gbs": (n_quant * BYTES_PER_PARAM_4BIT + (n_total - n_quant) * BYTES_PER_PARAM_FP32)
+        / (elapsed / args.steps) / 1e9,
+        "roofline": {
+            "bound": "hbm",
+            "kernel": "lpmm::adamw4bit_kernel<true>",
+            "achieved": achieved,
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": achieved / HBM_PEAK_GBS,
+            "traffic": None,
+            "bytes_per_launch": bytes_per_launch,
+            "avg_launch_ms": launch_ms,
+        },
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(torch)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,119 @@
+"""GPU parity of the non-fused elementwise update and of the factored second-moment step
+against the CPU oracle, through the C ABI."""
+import numpy as np
+import pytest
+import torch
+
+from util import assert_rel, to_dev, to_np
+
+pytestmark = pytest.mark.gpu
+
+H = dict(beta1=0.9, beta2=0.999, lr=1e-3, wd=0.01, eps=1e-8)
+
+
+def _lib():
+    from lpmm import _native
+
+    return _native.lib()
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def test_nonfused_update_matches_oracle(oracle):
+    lib = _lib()
+    rng = np.random.default_rng(5)
+    for n in (1, 1000, 4096 * 33 + 5):
+        p = (rng.standard_normal(n) * 0.02).astype(np.float32)
+        m = (rng.standard_normal(n) * 1e-3).astype(np.float32)
+        v = (rng.standard_normal(n) ** 2 * 1e-6).astype(np.float32)
+        dp, dm, dv = to_dev(p), to_dev(m), to_dev(v)
+        for step in (1.0, 2.0, 77.0):
+            g = (rng.standard_normal(n) * 1e-3).astype(np.float32)
+            dg = to_dev(g)
+            st = lib.lpmm_nonfused_update(dp.data_ptr(), dg.data_ptr(), dm.data_ptr(), dv.data_ptr(), n, H["beta1"],
+                                          H["beta2"], H["lr"], H["wd"], H["eps"], step, _stream())
+            assert st == 0
+            oracle.nonfused_update(p, g, m, v, H["beta1"], H["beta2"], H["lr"], H["wd"], H["eps"], step)
+            torch.cuda.synchronize()
+            np.testing.assert_array_equal(to_np(dm), m)
+            np.testing.assert_array_equal(to_np(dv), v)
+            np.testing.assert_array_equal(to_np(dp), p)
+
+
+@pytest.mark.parametrize("shape", [(64, 128), (100, 70), (513, 1025), (1024, 2752), (2752, 1024)])
+def test_factored_step_matches_oracle(oracle, qmaps, shape):
+    lib = _lib()
+    qm = qmaps[0]
+    dqm = to_dev(qm)
+    r, c = shape
+    n = r * c
+    rng = np.random.default_rng(r + c)
+    p = (rng.standard_normal((r, c)) * 0.02).astype(np.float32)
+    row, col = np.zeros(r, np.float32), np.zeros(c, np.float32)
+    dp, drow, dcol = to_dev(p), to_dev(row), to_dev(col)
+    groups = (n + 127) // 128
+    nbytes = (groups * 128 + 2047) // 2048 * 1024 + 1
+    codes = torch.full((nbytes,), 0x55, dtype=torch.uint8, device="cuda")
+    max1 = torch.zeros(groups, dtype=torch.float32, device="cuda")
+    mean_all = torch.zeros(1, dtype=torch.float32, device="cuda")
+    work = torch.empty(lib.lpmm_factored_workspace_bytes(r, c), dtype=torch.uint8, device="cuda")
+    m_state = None
+    for step in range(1, 5):
+        g = (rng.standard_normal((r, c)) * 1e-3 * (1 + rng.random((r, 1)) * 3)).astype(np.float32)
+        dg = to_dev(g)
+        assert lib.lpmm_factored_stats(dg.data_ptr(), r, c, drow.data_ptr(), dcol.data_ptr(), mean_all.data_ptr(),
+                                       H["beta2"], work.data_ptr(), _stream()) == 0
+        assert lib.lpmm_factored_update(dp.data_ptr(), dg.data_ptr(), codes.data_ptr(), max1.data_ptr(),
+                                        dqm.data_ptr(), drow.data_ptr(), dcol.data_ptr(), mean_all.data_ptr(), r, c,
+                                        H["beta1"], H["beta2"], H["lr"], H["wd"], H["eps"], float(step),
+                                        1 if step == 1 else 0, _stream()) == 0
+        # oracle
+        row_mean, col_mean = oracle.factored_stats(g)
+        mean_ref = oracle.factored_ema(row, col, row_mean, col_mean, H["beta2"])
+        m = np.zeros(n, np.float32) if m_state is None else oracle.dequant_group(m_state[0], m_state[1], qm, n)
+        oracle.factored_update(p, g, m, row, col, mean_ref, H["beta1"], H["beta2"], H["lr"], H["wd"], H["eps"],
+                               float(step))
+        m_state = oracle.quant_group(m, qm)
+        torch.cuda.synchronize()
+        # row/col sums are accumulated in double in a different (fixed) order than the oracle's
+        # sequential loop: equal after rounding to float except for rare last-bit differences
+        assert_rel(to_np(drow), row, f"row step {step}", tol=2e-7)
+        assert_rel(to_np(dcol), col, f"col step {step}", tol=2e-7)
+        assert_rel(to_np(mean_all), [mean_ref], f"mean step {step}", tol=2e-7)
+        assert_rel(to_np(dp), p, f"p step {step}")
+        # the first moment does not depend on the second: bit-exact
+        np.testing.assert_array_equal(to_np(max1), m_state[1])
+        np.testing.assert_array_equal(to_np(codes), m_state[0])
+        # continue from the oracle's statistics so that the comparison stays one step deep
+        drow.copy_(torch.from_numpy(row)); dcol.copy_(torch.from_numpy(col)); dp.copy_(torch.from_numpy(p))
+
+
+def test_factored_fp32m_matches_oracle(oracle):
+    lib = _lib()
+    r, c = 48, 64
+    rng = np.random.default_rng(9)
+    p = (rng.standard_normal((r, c)) * 0.02).astype(np.float32)
+    m = np.zeros(r * c, np.float32)
+    row, col = np.zeros(r, np.float32), np.zeros(c, np.float32)
+    dp, dm, drow, dcol = to_dev(p), to_dev(m), to_dev(row), to_dev(col)
+    mean_all = torch.zeros(1, dtype=torch.float32, device="cuda")
+    work = torch.empty(lib.lpmm_factored_workspace_bytes(r, c), dtype=torch.uint8, device="cuda")
+    for step in range(1, 4):
+        g = (rng.standard_normal((r, c)) * 1e-3).astype(np.float32)
+        dg = to_dev(g)
+        assert lib.lpmm_factored_stats(dg.data_ptr(), r, c, drow.data_ptr(), dcol.data_ptr(), mean_all.data_ptr(),
+                                       H["beta2"], work.data_ptr(), _stream()) == 0
+        assert lib.lpmm_factored_update_fp32m(dp.data_ptr(), dg.data_ptr(), dm.data_ptr(), drow.data_ptr(),
+                                              dcol.data_ptr(), mean_all.data_ptr(), r, c, H["beta1"], H["beta2"],
+                                              H["lr"], H["wd"], H["eps"], float(step), _stream()) == 0
+        row_mean, col_mean = oracle.factored_stats(g)
+        mean_ref = oracle.factored_ema(row, col, row_mean, col_mean, H["beta2"])
+        oracle.factored_update(p, g, m, row, col, mean_ref, H["beta1"], H["beta2"], H["lr"], H["wd"], H["eps"],
+                               float(step))
+        torch.cuda.synchronize()
+        assert_rel(to_np(drow), row, "row", tol=2e-7)
+        assert_rel(to_np(dp), p, "p")
+        np.testing.assert_array_equal(to_np(dm), m)
+        drow.copy_(torch.from_numpy(row)); dcol.copy_(torch.from_numpy(col)); dp.copy_(torch.from_numpy(p))
