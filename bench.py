@@ -113,6 +113,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--workload", default="llama7b", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run three plain 1 GiB device copies first (calibration dispatches for "
+                         "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; --gpus N with N > 1 is not supported "
@@ -128,6 +131,14 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     lib = _native.lib()
+
+    if args.copy_probe:
+        src = torch.ones(1 << 28, dtype=torch.float32, device=dev)  # 1 GiB read + 1 GiB written per copy
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     desc, shape_fn = WORKLOADS[args.workload]
     shapes = shape_fn()

@@ -86,8 +86,10 @@ def set_threads(n):
 # (create_dynamic_map), :644-656 (create_pow_map).
 # --------------------------------------------------------------------------------------
 def _linspace_f32(start, end, steps):
-    """torch.linspace for float32 on CPU: step = (end-start)/(steps-1) in float32; the first
-    half counts up from start, the second half counts down from end."""
+    """torch.linspace for float32 on CPU, scalar formula: step = (end-start)/(steps-1) in
+    float32; the first half counts up from start, the second half counts down from end.
+    PyTorch's vectorised path (grids of 8 or more points) rounds differently; the 4-bit maps
+    only use grids of 2, 3 and 5 points, and the 17-point grid of the v map is exact."""
     f = np.float32
     start, end = f(start), f(end)
     if steps == 1:

@@ -1,0 +1,277 @@
+"""End-to-end GPU tests of lpmm.optim.AdamW against the CPU oracle: fused, non-fused
+(group and rank-1 second moment) and factored paths, state layout, checkpointing,
+the 100-step trajectory criterion and the golden fixture."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from util import assert_codes, assert_rel, nibbles, to_dev, to_np
+
+pytestmark = pytest.mark.gpu
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+H = dict(lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01)
+HO = (0.9, 0.999, 1e-3, 0.01, 1e-8)  # oracle order: beta1, beta2, lr, wd, eps
+
+
+def _params(shapes, rng):
+    host = [(rng.standard_normal(s) * 0.02).astype(np.float32) for s in shapes]
+    return host, [torch.nn.Parameter(to_dev(h)) for h in host]
+
+
+def test_fused_optimizer_matches_oracle_and_layout(oracle, qmaps):
+    import lpmm
+
+    qm, qv = qmaps
+    rng = np.random.default_rng(0)
+    shapes = [(64, 130), (1600,), (6400,), (40, 40), (130, 128)]  # 8320 q, 1600 fp32, 6400 q (50 groups), 1600 fp32, 16640 q
+    host, params = _params(shapes, rng)
+    opt = lpmm.optim.AdamW(params, fused=True, **H)
+    ref = []
+    for h in host:
+        n = h.size
+        if n > 4096:
+            ref.append(dict(mc=np.zeros(n // 2, np.uint8), vc=np.zeros(n // 2, np.uint8),
+                            ms=np.zeros((n + 127) // 128, np.float32), vs=np.zeros((n + 127) // 128, np.float32)))
+        else:
+            ref.append(dict(m=np.zeros(n, np.float32), v=np.zeros(n, np.float32)))
+    for step in range(1, 6):
+        grads = [(rng.standard_normal(s) * 1e-3).astype(np.float32) for s in shapes]
+        for p, g in zip(params, grads):
+            p.grad = to_dev(g)
+        opt.step()
+        for h, g, r in zip(host, grads, ref):
+            if "mc" in r:
+                oracle.adamw4bit_step(h.reshape(-1), g.reshape(-1), r["mc"], r["vc"], r["ms"], r["vs"], qm, qv, *HO, float(step))
+            else:
+                oracle.adamw_fp32_step(h.reshape(-1), g.reshape(-1), r["m"], r["v"], *HO, float(step))
+    torch.cuda.synchronize()
+    for p, h, r in zip(params, host, ref):
+        st = opt.state[p]
+        assert float(st["step"]) == 5.0 and st["step"].device.type == "cpu"
+        if "mc" in r:
+            n = h.size
+            assert st["exp_avg"].dtype == torch.int8 and st["exp_avg"].shape == ((n + 1) // 2,)
+            assert st["exp_avg_qstate"]["overhead"]["max1"].shape == ((n + 127) // 128,)
+            assert_codes(to_np(st["exp_avg"]), r["mc"], n, "m codes")
+            assert_codes(to_np(st["exp_avg_sq"]), r["vc"], n, "v codes")
+            assert_rel(to_np(st["exp_avg_qstate"]["overhead"]["max1"]), r["ms"], "m scales")
+            assert_rel(to_np(st["exp_avg_sq_qstate"]["overhead"]["max1"]), r["vs"], "v scales")
+        else:
+            assert st["exp_avg"].dtype == torch.float32 and st["exp_avg"].shape == p.shape
+            np.testing.assert_array_equal(to_np(st["exp_avg"]).reshape(-1), r["m"])
+            np.testing.assert_array_equal(to_np(st["exp_avg_sq"]).reshape(-1), r["v"])
+        assert_rel(to_np(p), h, "p", scale=h)
+
+
+def test_fused_optimizer_error_behaviour(oracle):
+    import lpmm
+
+    # odd numel > 4096: the reference allocates (n+1)//2 bytes and then fails its own size check
+    p = torch.nn.Parameter(torch.zeros(4099, device="cuda"))
+    p.grad = torch.zeros_like(p)
+    with pytest.raises(RuntimeError, match="number of elements in exp_avg and p"):
+        lpmm.optim.AdamW([p], fused=True).step()
+    # m and v must be quantised together on the fused path
+    cfg = os.path.join(os.path.dirname(lpmm.config.__file__), "configs", "2nd_moment_only_group_128.yml")
+    q = torch.nn.Parameter(torch.zeros(128, 64, device="cuda"))
+    q.grad = torch.zeros_like(q)
+    with pytest.raises(ValueError, match="both quantized or unquantized"):
+        lpmm.optim.AdamW([q], fused=True, qconfig=cfg).step()
+    # non-contiguous gradient
+    r = torch.nn.Parameter(torch.zeros(128, 64, device="cuda"))
+    r.grad = torch.zeros(64, 128, device="cuda").t()
+    with pytest.raises(RuntimeError, match="contiguous"):
+        lpmm.optim.AdamW([r], fused=True).step()
+
+
+@pytest.mark.parametrize("v_scale", ["rank1", "group"])
+def test_nonfused_optimizer_matches_oracle(oracle, qmaps, v_scale):
+    import lpmm
+
+    qm, qv = qmaps
+    rng = np.random.default_rng(1)
+    shapes = [(96, 160), (11008,), (2000,)]
+    host, params = _params(shapes, rng)
+    cfg = os.path.join(os.path.dirname(lpmm.config.__file__), "configs",
+                       "default.yml" if v_scale == "rank1" else "2nd_moment_group_128.yml")
+    opt = lpmm.optim.AdamW(params, fused=False, qconfig=cfg, **H)
+    states = [oracle.NonFusedState(s, v_scale_type=v_scale) for s in shapes[:2]]
+    m_small, v_small = np.zeros(2000, np.float32), np.zeros(2000, np.float32)
+    for step in range(1, 5):
+        grads = [(rng.standard_normal(s) * 1e-3).astype(np.float32) for s in shapes]
+        for p, g in zip(params, grads):
+            p.grad = to_dev(g)
+        opt.step()
+        for h, g, st in zip(host[:2], grads[:2], states):
+            oracle.nonfused_step(h, g, st, qm, qv, H["lr"], 0.9, 0.999, H["eps"], H["weight_decay"])
+        oracle.nonfused_update(host[2], grads[2], m_small, v_small, 0.9, 0.999, H["lr"], H["weight_decay"], H["eps"], float(step))
+    torch.cuda.synchronize()
+    # 2-D tensor
+    s0 = opt.state[params[0]]
+    n0 = host[0].size
+    assert s0["exp_avg"].dtype == torch.int8 and s0["exp_avg"].numel() == (n0 + 2047) // 2048 * 1024 + 1
+    np.testing.assert_array_equal(to_np(s0["exp_avg"]).view(np.uint8), states[0].m[0])
+    np.testing.assert_array_equal(to_np(s0["exp_avg_qstate"]["overhead"]["max1"]).reshape(-1), states[0].m[1])
+    oh = s0["exp_avg_sq_qstate"]["overhead"]
+    np.testing.assert_array_equal(to_np(s0["exp_avg_sq"]).view(np.uint8), states[0].v[0])
+    if v_scale == "rank1":
+        assert oh["dim"] == 2 and oh["max1"] is None and oh["scaled_shape"] == torch.Size(shapes[0])
+        np.testing.assert_array_equal(to_np(oh["max_dims"][0]).reshape(-1), states[0].v[1])
+        np.testing.assert_array_equal(to_np(oh["max_dims"][1]).reshape(-1), states[0].v[2])
+    else:
+        assert oh["max1"].shape == ((n0 + 127) // 128, 1) and oh["scaled_shape"] == torch.Size(((n0 + 127) // 128, 128))
+        np.testing.assert_array_equal(to_np(oh["max1"]).reshape(-1), states[0].v[1])
+    np.testing.assert_array_equal(to_np(params[0]), host[0])
+    # 1-D tensor: rank1 falls back to group-128
+    s1 = opt.state[params[1]]
+    np.testing.assert_array_equal(to_np(s1["exp_avg_sq"]).view(np.uint8), states[1].v[0])
+    np.testing.assert_array_equal(to_np(s1["exp_avg_sq_qstate"]["overhead"]["max1"]).reshape(-1), states[1].v[1])
+    np.testing.assert_array_equal(to_np(params[1]), host[1])
+    # small tensor keeps fp32 states
+    s2 = opt.state[params[2]]
+    assert s2["exp_avg"].dtype == torch.float32
+    np.testing.assert_array_equal(to_np(s2["exp_avg"]), m_small)
+    np.testing.assert_array_equal(to_np(s2["exp_avg_sq"]), v_small)
+    np.testing.assert_array_equal(to_np(params[2]), host[2])
+
+
+@pytest.mark.parametrize("fused", [False, True])
+def test_factored_optimizer_matches_oracle(oracle, qmaps, fused):
+    import lpmm
+
+    qm, qv = qmaps
+    rng = np.random.default_rng(2)
+    shapes = [(128, 344), (344, 128), (50, 60), (11008,)]  # quantised m x2, fp32 m (3000 <= 4096), 1-D: 4-bit m and v
+    host, params = _params(shapes, rng)
+    opt = lpmm.optim.AdamW(params, fused=fused, factor_second_moment=True, **H)
+    states = [oracle.NonFusedState(s, factored=True) for s in shapes[:2]]
+    row2, col2, m2 = np.zeros(50, np.float32), np.zeros(60, np.float32), np.zeros(3000, np.float32)
+    st1d = oracle.NonFusedState(shapes[3], v_scale_type="group")
+    fz = dict(mc=np.zeros(5504, np.uint8), vc=np.zeros(5504, np.uint8), ms=np.zeros(86, np.float32), vs=np.zeros(86, np.float32))
+    for step in range(1, 4):
+        grads = [(rng.standard_normal(s) * 1e-3).astype(np.float32) for s in shapes]
+        for p, g in zip(params, grads):
+            p.grad = to_dev(g)
+        opt.step()
+        for h, g, st in zip(host[:2], grads[:2], states):
+            oracle.nonfused_step(h, g, st, qm, qv, H["lr"], 0.9, 0.999, H["eps"], H["weight_decay"])
+        rm, cm = oracle.factored_stats(grads[2])
+        mean_all = oracle.factored_ema(row2, col2, rm, cm, 0.999)
+        oracle.factored_update(host[2], grads[2], m2, row2, col2, mean_all, 0.9, 0.999, H["lr"], H["weight_decay"], H["eps"], float(step))
+        if fused:
+            oracle.adamw4bit_step(host[3], grads[3], fz["mc"], fz["vc"], fz["ms"], fz["vs"], qm, qv, *HO, float(step))
+        else:
+            oracle.nonfused_step(host[3], grads[3], st1d, qm, qv, H["lr"], 0.9, 0.999, H["eps"], H["weight_decay"])
+    torch.cuda.synchronize()
+    for p, h, st in zip(params[:2], host[:2], states):
+        s = opt.state[p]
+        assert "exp_avg_sq" not in s and s["exp_avg_sq_row"].shape == (h.shape[0],) and s["exp_avg_sq_col"].shape == (h.shape[1],)
+        assert_rel(to_np(s["exp_avg_sq_row"]), st.row, "row", tol=1e-6)
+        assert_rel(to_np(s["exp_avg_sq_col"]), st.col, "col", tol=1e-6)
+        np.testing.assert_array_equal(to_np(s["exp_avg"]).view(np.uint8), st.m[0])  # m does not depend on v
+        np.testing.assert_array_equal(to_np(s["exp_avg_qstate"]["overhead"]["max1"]).reshape(-1), st.m[1])
+        assert_rel(to_np(p), h, "p", scale=h)
+    s = opt.state[params[2]]
+    assert s["exp_avg"].dtype == torch.float32
+    np.testing.assert_array_equal(to_np(s["exp_avg"]).reshape(-1), m2)
+    assert_rel(to_np(params[2]), host[2], "p small", scale=host[2])
+    s = opt.state[params[3]]
+    if fused:
+        np.testing.assert_array_equal(to_np(s["exp_avg_sq"]).view(np.uint8), fz["vc"])
+    else:
+        np.testing.assert_array_equal(to_np(s["exp_avg_sq"]).view(np.uint8), st1d.v[0])
+    assert_rel(to_np(params[3]), host[3], "p 1-D", scale=host[3])
+
+
+def test_trajectory_100_steps(oracle, qmaps):
+    """Dequantised m and v over 100 steps stay within 1e-4 relative of the oracle's (measured
+    against the scale of each 128-group, since m has entries near zero)."""
+    import lpmm
+
+    qm, qv = qmaps
+    rng = np.random.default_rng(3)
+    shape = (256, 512)
+    n = shape[0] * shape[1]
+    host, params = _params([shape], rng)
+    h = host[0].reshape(-1)
+    opt = lpmm.optim.AdamW(params, fused=True, **H)
+    mc, vc = np.zeros(n // 2, np.uint8), np.zeros(n // 2, np.uint8)
+    ms, vs = np.zeros(n // 128, np.float32), np.zeros(n // 128, np.float32)
+    total_flips = 0
+    for step in range(1, 101):
+        g = (rng.standard_normal(n) * 1e-3).astype(np.float32)
+        params[0].grad = to_dev(g.reshape(shape))
+        opt.step()
+        oracle.adamw4bit_step(h, g, mc, vc, ms, vs, qm, qv, *HO, float(step))
+        if step % 20 == 0:
+            st = opt.state[params[0]]
+            gm = oracle.dequant_group(to_np(st["exp_avg"]).view(np.uint8), to_np(st["exp_avg_qstate"]["overhead"]["max1"]), qm, n)
+            gv = oracle.dequant_group(to_np(st["exp_avg_sq"]).view(np.uint8), to_np(st["exp_avg_sq_qstate"]["overhead"]["max1"]), qv, n)
+            assert_rel(gm, oracle.dequant_group(mc, ms, qm, n), f"m trajectory step {step}", tol=1e-4, scale=ms.repeat(128))
+            assert_rel(gv, oracle.dequant_group(vc, vs, qv, n), f"v trajectory step {step}", tol=1e-4, scale=vs.repeat(128))
+            assert_rel(to_np(params[0]).reshape(-1), h, f"p trajectory step {step}", tol=1e-6, scale=np.full(n, 0.02))
+            total_flips += int(np.sum(nibbles(to_np(st["exp_avg"]), n) != nibbles(mc, n)))
+    print("code differences after 100 unsynchronised steps:", total_flips)
+
+
+def test_golden_fixture_on_gpu(qmaps):
+    """The committed fixture (tests/golden/fused_step_small.npz), through the reference-named
+    operator lpmm.cpp_extension.fused_adamw.adamw4bit_single_tensor."""
+    from lpmm.cpp_extension import fused_adamw
+
+    gold = np.load(os.path.join(HERE, "golden", "fused_step_small.npz"))
+    n = gold["p0"].size
+    p = to_dev(gold["p0"])
+    mc = torch.zeros(n // 2, dtype=torch.int8, device="cuda")
+    vc = torch.zeros_like(mc)
+    ms, vs = torch.zeros(8, device="cuda"), torch.zeros(8, device="cuda")
+    qm, qv = to_dev(qmaps[0]), to_dev(qmaps[1])
+    for s in range(3):
+        g = to_dev(gold["grads"][s])
+        fused_adamw.adamw4bit_single_tensor(p, g, mc, vc, ms, vs, qm, qv, 0.9, 0.999, 1e-3, 0.01, 1e-8, float(s + 1))
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(to_np(mc).view(np.uint8), gold[f"mc{s + 1}"])
+        np.testing.assert_array_equal(to_np(vc).view(np.uint8), gold[f"vc{s + 1}"])
+        np.testing.assert_array_equal(to_np(ms), gold[f"ms{s + 1}"])
+        np.testing.assert_array_equal(to_np(vs), gold[f"vs{s + 1}"])
+        assert_rel(to_np(p), gold[f"p{s + 1}"], "p", scale=gold["p0"])
+    with pytest.raises(RuntimeError):  # wrong scale length (lpmm/cpp_extension/fused_adamw_kernel.cu:218-219)
+        fused_adamw.adamw4bit_single_tensor(p, g, mc, vc, ms[:7], vs, qm, qv, 0.9, 0.999, 1e-3, 0.01, 1e-8, 4.0)
+    with pytest.raises(RuntimeError):  # numel mismatch
+        fused_adamw.adamw4bit_single_tensor(p, g[:-2], mc, vc, ms, vs, qm, qv, 0.9, 0.999, 1e-3, 0.01, 1e-8, 4.0)
+
+
+def test_checkpoint_resume_on_gpu(oracle):
+    """state_dict -> load_state_dict -> continue gives the same bytes as an uninterrupted run."""
+    import lpmm
+
+    rng = np.random.default_rng(4)
+    shapes = [(64, 130), (1600,)]
+    host, params_a = _params(shapes, rng)
+    params_b = [torch.nn.Parameter(p.detach().clone()) for p in params_a]
+    opt_a = lpmm.optim.AdamW(params_a, fused=True, **H)
+    opt_b = lpmm.optim.AdamW(params_b, fused=True, **H)
+    grads = [[(rng.standard_normal(s) * 1e-3).astype(np.float32) for s in shapes] for _ in range(4)]
+
+    def run(opt, params, steps):
+        for k in steps:
+            for p, g in zip(params, grads[k]):
+                p.grad = to_dev(g)
+            opt.step()
+
+    run(opt_a, params_a, range(4))
+    run(opt_b, params_b, range(2))
+    sd = opt_b.state_dict()
+    params_c = [torch.nn.Parameter(p.detach().clone()) for p in params_b]
+    opt_c = lpmm.optim.AdamW(params_c, fused=True, **H)
+    opt_c.load_state_dict(sd)
+    run(opt_c, params_c, range(2, 4))
+    torch.cuda.synchronize()
+    for pa, pc in zip(params_a, params_c):
+        assert torch.equal(pa, pc)
+        sa, sc = opt_a.state[pa], opt_c.state[pc]
+        assert torch.equal(sa["exp_avg"], sc["exp_avg"]) and torch.equal(sa["exp_avg_sq"], sc["exp_avg_sq"])
+        assert sc["exp_avg"].dtype == sa["exp_avg"].dtype and float(sc["step"]) == 4.0

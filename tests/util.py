@@ -29,11 +29,16 @@ def assert_codes(got, want, n, what=""):
     return int(diff.size)
 
 
-def assert_rel(got, want, what="", tol=REL_TOL):
+def assert_rel(got, want, what="", tol=REL_TOL, scale=None):
+    """|got - want| <= tol * |want| elementwise.  `scale` (e.g. the parameter before the step)
+    widens the yardstick to max(|want|, |scale|): a step that cancels most of a parameter
+    leaves a result whose error is relative to the operands, not to the small difference."""
     got = np.asarray(got, dtype=np.float64).reshape(-1)
     want = np.asarray(want, dtype=np.float64).reshape(-1)
     assert got.shape == want.shape, f"{what}: shape {got.shape} vs {want.shape}"
     denom = np.maximum(np.abs(want), np.finfo(np.float32).tiny)
+    if scale is not None:
+        denom = np.maximum(denom, np.abs(np.asarray(scale, dtype=np.float64).reshape(-1)))
     rel = np.abs(got - want) / denom
     bad = np.flatnonzero(~(rel <= tol) & ~(got == want))
     assert bad.size == 0, f"{what}: {bad.size} values beyond {tol} relative, worst {rel[bad].max():.3e}"
