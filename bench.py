@@ -25,6 +25,10 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 BYTES_PER_PARAM_4BIT = 14.125  # p r/w 8 + g 4 + m codes 1 + v codes 1 + scales 16/128
 BYTES_PER_PARAM_FP32 = 28.0    # p, m, v r/w + g r
 MULTI_MAX = 48                 # tensors per launch record (LPMM_MULTI_MAX)
+# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
+# script (each counter scaled by what it reads for a plain 1 GiB copy, --copy-probe):
+# profiles/fused_adamw4bit_llama7b_pmc.md.  Algorithmic bytes per launch for that workload: 19.035e9.
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"llama7b": 19.12e9}
 
 
 def llama7b_shapes():
@@ -209,7 +213,7 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBS,
-            "traffic": None,
+            "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(args.workload),
             "bytes_per_launch": bytes_per_launch,
             "avg_launch_ms": launch_ms,
         },

@@ -3,9 +3,12 @@
 // Roundings follow the PyTorch CPU kernels that the reference's op sequence runs
 // (lpmm/optim/adamw.py:367-369, :412-422, :579-627): multiply by the float-cast Python
 // scalar, lerp as fma(w, g - m, m) for w < 0.5, addcmul as v + (value*g)*g, true division
-// by the float-cast sqrt(bias_correction2), addcdiv as p + (value*m)/denom.
+// by the float-cast sqrt(bias_correction2), addcdiv as p + (value*m)/denom.  m and v are
+// computed exactly so; the square root and the two divisions of the parameter update use
+// the hardware approximations with one fma correction of the residual (correctly rounded
+// except for a vanishing fraction of inputs; the parameter never feeds back into a state).
 // Row/column means of g*g are summed in double in a fixed order and rounded once.
-#include "lpmm_common.hpp"
+#include "lpmm_codec.hpp"
 
 #include <math.h>
 
@@ -16,7 +19,7 @@ constexpr int kFElts = 8;
 constexpr int kFTile = kFThreads * kFElts;  // 2048
 
 struct NfHyper {
-    float decay, w1, b2, w2, neg_step_size, bc2_sqrt, eps;
+    float decay, w1, b2, w2, neg_step_size, bc2_sqrt, rbc2_sqrt, eps;  // rbc2_sqrt = 1 / bc2_sqrt, correctly rounded
 };
 
 inline NfHyper make_nf_hyper(double beta1, double beta2, double lr, double wd, double eps, double step)
@@ -30,6 +33,7 @@ inline NfHyper make_nf_hyper(double beta1, double beta2, double lr, double wd, d
     const double bc2 = 1.0 - pow(beta2, step);
     h.neg_step_size = (float)(-(lr / bc1));
     h.bc2_sqrt = (float)sqrt(bc2);
+    h.rbc2_sqrt = 1.0f / h.bc2_sqrt;
     h.eps = (float)eps;
     return h;
 }
@@ -39,32 +43,55 @@ __device__ __forceinline__ float lerp_w(float a, float b, float w)
     return (fabsf(w) < 0.5f) ? __builtin_fmaf(w, b - a, a) : __builtin_fmaf(w - 1.0f, b - a, b);
 }
 
+// One lane: 4 consecutive elements per iteration (16-byte accesses), grid-stride.
+__device__ __forceinline__ void nonfused_elt(float &p, float g, float &m, float &v, const NfHyper &h)
+{
+    const float pi = p * h.decay;
+    m = lerp_w(m, g, h.w1);
+    float vi = v * h.b2;
+    vi = vi + (h.w2 * g) * g;
+    v = vi;
+    const float denom = div_by_rc(sqrt_fast(vi), h.bc2_sqrt, h.rbc2_sqrt) + h.eps;
+    p = pi + div_fast(h.neg_step_size * m, denom);
+}
+
 __global__ __launch_bounds__(kFThreads) void nonfused_update_kernel(float *__restrict__ p,
                                                                     const float *__restrict__ g,
                                                                     float *__restrict__ m, float *__restrict__ v,
-                                                                    int64_t n, NfHyper h)
+                                                                    int64_t n, NfHyper h, bool vec)
 {
-    const int64_t stride = (int64_t)gridDim.x * kFThreads;
-    for (int64_t i = (int64_t)blockIdx.x * kFThreads + threadIdx.x; i < n; i += stride) {
-        const float gi = g[i];
-        const float pi = p[i] * h.decay;
-        const float mi = lerp_w(m[i], gi, h.w1);
-        float vi = v[i] * h.b2;
-        vi = vi + (h.w2 * gi) * gi;
-        const float denom = sqrtf(vi) / h.bc2_sqrt + h.eps;
-        p[i] = pi + (h.neg_step_size * mi) / denom;
-        m[i] = mi;
-        v[i] = vi;
+    const int64_t base = ((int64_t)blockIdx.x * kFThreads + threadIdx.x) * 4;
+    if (base >= n)
+        return;
+    if (vec && base + 4 <= n) {
+        float4 pp = load4(p + base), mm = load4(m + base), vv = load4(v + base);
+        const float4 gg = load4(g + base);
+        nonfused_elt(pp.x, gg.x, mm.x, vv.x, h);
+        nonfused_elt(pp.y, gg.y, mm.y, vv.y, h);
+        nonfused_elt(pp.z, gg.z, mm.z, vv.z, h);
+        nonfused_elt(pp.w, gg.w, mm.w, vv.w, h);
+        store4(p + base, pp);
+        store4(m + base, mm);
+        store4(v + base, vv);
+    } else {
+        for (int64_t i = base; i < base + 4 && i < n; ++i) {
+            float pi = p[i], mi = m[i], vi = v[i];
+            nonfused_elt(pi, g[i], mi, vi, h);
+            p[i] = pi;
+            m[i] = mi;
+            v[i] = vi;
+        }
     }
 }
 
 // ---------------------------------------------------------------------------------------
 // Factored statistics, pass A: partial row/column sums of g*g over tiles of
 // kSRows x kSCols, accumulated in double.  Partials go to the workspace:
-//   colpart[ty][c]  (ty = row-tile index)   rowpart[tx*4 + wave][r]  (tx = column-tile index)
+//   colpart[ty][c]  (ty = row-tile index)   rowpart[tx][r]  (tx = column-tile index)
 // ---------------------------------------------------------------------------------------
-constexpr int kSRows = 128;
+constexpr int kSRows = 32;
 constexpr int kSCols = 1024;  // 256 threads x 4 columns
+constexpr int kSUnroll = 8;   // rows in flight per lane
 
 __global__ __launch_bounds__(kFThreads) void factored_partial_kernel(const float *__restrict__ g, int64_t R,
                                                                      int64_t C, double *__restrict__ colpart,
@@ -73,29 +100,41 @@ __global__ __launch_bounds__(kFThreads) void factored_partial_kernel(const float
     const int64_t c0 = (int64_t)blockIdx.x * kSCols + (int64_t)threadIdx.x * 4;
     const int64_t r0 = (int64_t)blockIdx.y * kSRows;
     const int64_t r1 = (r0 + kSRows < R) ? r0 + kSRows : R;
-    // one row partial per wave: rowpart[(column tile * 4 + wave)][r]
-    double *rp = rowpart + ((int64_t)blockIdx.x * (kFThreads / kWave) + (threadIdx.x >> 6)) * R;
+    const bool lane_vec = vec && c0 + 4 <= C;
+    __shared__ double s_part[kFThreads / kWave][kSUnroll];
+    double *rp = rowpart + (int64_t)blockIdx.x * R;  // one row partial per workgroup
     double cs[4] = {0.0, 0.0, 0.0, 0.0};
-    for (int64_t r = r0; r < r1; ++r) {
-        float u[4];
-        const float *row = g + r * C;
-        if (vec && c0 + 4 <= C) {
-            const float4 t = *reinterpret_cast<const float4 *>(row + c0);
-            u[0] = t.x * t.x; u[1] = t.y * t.y; u[2] = t.z * t.z; u[3] = t.w * t.w;
-        } else {
+    for (int64_t rb = r0; rb < r1; rb += kSUnroll) {
+        float u[kSUnroll][4];
 #pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                const float t = (c0 + k < C) ? row[c0 + k] : 0.0f;
-                u[k] = t * t;
+        for (int j = 0; j < kSUnroll; ++j) {
+            const int64_t r = rb + j;
+            if (r < r1 && lane_vec) {
+                const float4 t = load4(g + r * C + c0);
+                u[j][0] = t.x * t.x; u[j][1] = t.y * t.y; u[j][2] = t.z * t.z; u[j][3] = t.w * t.w;
+            } else {
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const float t = (r < r1 && c0 + k < C) ? g[r * C + c0 + k] : 0.0f;
+                    u[j][k] = t * t;
+                }
             }
         }
-        double rs = ((double)u[0] + (double)u[1]) + ((double)u[2] + (double)u[3]);
 #pragma unroll
-        for (int k = 0; k < 4; ++k)
-            cs[k] += (double)u[k];
-        rs = wave_sum_f64(rs);
-        if ((threadIdx.x & 63) == 0)
-            rp[r] = rs;
+        for (int j = 0; j < kSUnroll; ++j) {
+            double rs = ((double)u[j][0] + (double)u[j][1]) + ((double)u[j][2] + (double)u[j][3]);
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+                cs[k] += (double)u[j][k];
+            rs = wave_sum_f64(rs);
+            if ((threadIdx.x & 63) == 0)
+                s_part[threadIdx.x >> 6][j] = rs;
+        }
+        __syncthreads();
+        if (threadIdx.x < kSUnroll && rb + threadIdx.x < r1)
+            rp[rb + threadIdx.x] = (s_part[0][threadIdx.x] + s_part[1][threadIdx.x]) +
+                                   (s_part[2][threadIdx.x] + s_part[3][threadIdx.x]);
+        __syncthreads();
     }
 #pragma unroll
     for (int k = 0; k < 4; ++k)
@@ -103,40 +142,61 @@ __global__ __launch_bounds__(kFThreads) void factored_partial_kernel(const float
             colpart[(int64_t)blockIdx.y * C + c0 + k] = cs[k];
 }
 
-// Pass B: fold the partials in a fixed order, update the EMAs
+// Pass B: fold the partials in a fixed order and update the EMAs
 // (row.mul_(beta2).add_(mean, alpha=1-beta2): fma(mean, 1-beta2, row*beta2)).
-// Workgroups 1.. handle columns; workgroup 0 handles all rows and mean(row).
+// Workgroups [0, row_blocks) take 256 rows each and leave the sum of their new row values in
+// rowblock[b]; the remaining workgroups take 64 columns each.
 __global__ __launch_bounds__(kFThreads) void factored_finalize_kernel(const double *__restrict__ colpart,
                                                                       const double *__restrict__ rowpart,
-                                                                      int64_t R, int64_t C, int tiles_y,
-                                                                      int tiles_x, float *__restrict__ row,
-                                                                      float *__restrict__ col,
-                                                                      float *__restrict__ row_mean_all, float b2,
-                                                                      float w2)
+                                                                      double *__restrict__ rowblock, int64_t R,
+                                                                      int64_t C, int tiles_y, int tiles_x,
+                                                                      int row_blocks, float *__restrict__ row,
+                                                                      float *__restrict__ col, float b2, float w2)
 {
-    if (blockIdx.x > 0) {
-        const int64_t c = (int64_t)(blockIdx.x - 1) * kFThreads + threadIdx.x;
+    if ((int)blockIdx.x >= row_blocks) {
+        // 64 columns per workgroup; the partials of a column are split over 4 threads, each
+        // summing its contiguous quarter 8 loads at a time, and folded in a fixed order
+        __shared__ double s_col[kFThreads];
+        const int64_t c = (int64_t)(blockIdx.x - row_blocks) * 64 + (threadIdx.x & 63);
+        const int quarter = threadIdx.x >> 6;
+        const int per = (tiles_y + 3) / 4;
+        const int t0 = quarter * per, t1 = (t0 + per < tiles_y) ? t0 + per : tiles_y;
+        double s = 0.0;
         if (c < C) {
-            double s = 0.0;
-            for (int t = 0; t < tiles_y; ++t)
+            int t = t0;
+            for (; t + 8 <= t1; t += 8) {
+                double a[8];
+#pragma unroll
+                for (int k = 0; k < 8; ++k)
+                    a[k] = colpart[(int64_t)(t + k) * C + c];
+                s += ((a[0] + a[1]) + (a[2] + a[3])) + ((a[4] + a[5]) + (a[6] + a[7]));
+            }
+            for (; t < t1; ++t)
                 s += colpart[(int64_t)t * C + c];
-            const float mean = (float)(s / (double)R);
+        }
+        s_col[threadIdx.x] = s;
+        __syncthreads();
+        if (quarter == 0 && c < C) {
+            const double tot = (s_col[threadIdx.x] + s_col[threadIdx.x + 64]) +
+                               (s_col[threadIdx.x + 128] + s_col[threadIdx.x + 192]);
+            const float mean = (float)(tot / (double)R);
             col[c] = __builtin_fmaf(mean, w2, col[c] * b2);
         }
         return;
     }
     __shared__ double s_sum[kFThreads];
-    double acc = 0.0;
-    for (int64_t r = threadIdx.x; r < R; r += kFThreads) {
+    const int64_t r = (int64_t)blockIdx.x * kFThreads + threadIdx.x;
+    double mine = 0.0;
+    if (r < R) {
         double s = 0.0;
         for (int t = 0; t < tiles_x; ++t)
             s += rowpart[(int64_t)t * R + r];
         const float mean = (float)(s / (double)C);
         const float nr = __builtin_fmaf(mean, w2, row[r] * b2);
         row[r] = nr;
-        acc += (double)nr;
+        mine = (double)nr;
     }
-    s_sum[threadIdx.x] = acc;
+    s_sum[threadIdx.x] = mine;
     __syncthreads();
     for (int o = kFThreads / 2; o > 0; o >>= 1) {
         if (threadIdx.x < o)
@@ -144,23 +204,38 @@ __global__ __launch_bounds__(kFThreads) void factored_finalize_kernel(const doub
         __syncthreads();
     }
     if (threadIdx.x == 0)
-        *row_mean_all = (float)(s_sum[0] / (double)R);
+        rowblock[blockIdx.x] = s_sum[0];
+}
+
+// Pass C: mean(row) from the per-workgroup sums, in order.
+__global__ void factored_mean_kernel(const double *__restrict__ rowblock, int row_blocks, int64_t R,
+                                     float *__restrict__ row_mean_all)
+{
+    if (threadIdx.x == 0 && blockIdx.x == 0) {
+        double s = 0.0;
+        for (int b = 0; b < row_blocks; ++b)
+            s += rowblock[b];
+        *row_mean_all = (float)(s / (double)R);
+    }
 }
 
 // ---------------------------------------------------------------------------------------
 // Factored update, one pass: decay p, decode m (group-128 codes of the non-fused layout),
 // lerp, v = row/mean(row) * col, update p, re-quantise m and write its pad codes.
+// ROWS: the column count is a multiple of 8, so a lane's 8 elements lie in one row and the
+// row index comes from one division per lane; otherwise every element tracks its own
+// (row, column).
 // ---------------------------------------------------------------------------------------
+template <bool ROWS>
 __global__ __launch_bounds__(kFThreads) void factored_update_kernel(
     float *__restrict__ p, const float *__restrict__ g, uint8_t *__restrict__ m_codes,
     float *__restrict__ m_max1, const float *__restrict__ qmap_m, const float *__restrict__ row,
     const float *__restrict__ col, const float *__restrict__ row_mean_all, int64_t n, int64_t C,
     int64_t n_groups, int64_t n_padded, NfHyper h, bool first_step, bool vec)
 {
-    __shared__ float s_q[16];
-    if (threadIdx.x < 16)
-        s_q[threadIdx.x] = qmap_m[threadIdx.x];
-    const Mids mids = make_mids(qmap_m);
+    __shared__ __align__(16) uint32_t lds[kLdsBytes / 4];
+    lds_fill(lds, qmap_m, nullptr);
+    const int kind = classify_map(qmap_m);
     __syncthreads();
     const int64_t base = ((int64_t)blockIdx.x * kFThreads + threadIdx.x) * kFElts;
     if (base == 0)
@@ -172,10 +247,8 @@ __global__ __launch_bounds__(kFThreads) void factored_update_kernel(
     uint32_t wm = 0;
     float sm = 0.0f;
     if (full) {
-        const float4 a0 = *reinterpret_cast<const float4 *>(p + base);
-        const float4 a1 = *reinterpret_cast<const float4 *>(p + base + 4);
-        const float4 b0 = *reinterpret_cast<const float4 *>(g + base);
-        const float4 b1 = *reinterpret_cast<const float4 *>(g + base + 4);
+        const float4 a0 = load4(p + base), a1 = load4(p + base + 4);
+        const float4 b0 = load4(g + base), b1 = load4(g + base + 4);
         pv[0] = a0.x; pv[1] = a0.y; pv[2] = a0.z; pv[3] = a0.w;
         pv[4] = a1.x; pv[5] = a1.y; pv[6] = a1.z; pv[7] = a1.w;
         gv[0] = b0.x; gv[1] = b0.y; gv[2] = b0.z; gv[3] = b0.w;
@@ -188,27 +261,34 @@ __global__ __launch_bounds__(kFThreads) void factored_update_kernel(
         }
     }
     if (any && !first_step) {
-        wm = *reinterpret_cast<const uint32_t *>(m_codes + (base >> 1));  // padded buffer: always inside
+        wm = load_u32(reinterpret_cast<const uint32_t *>(m_codes + (base >> 1)));  // padded buffer: always inside
         sm = m_max1[grp];
     }
+    const Nibbles nm = split_nibbles(wm);
     const float mean_all = *row_mean_all;
     int64_t r = any ? base / C : 0;
     int64_t c = any ? base - r * C : 0;
     float rf = any ? row[r] / mean_all : 0.0f;
+    float cv[kFElts];
+    if (ROWS && any) {
+        const float4 c0 = *reinterpret_cast<const float4 *>(col + c), c1 = *reinterpret_cast<const float4 *>(col + c + 4);
+        cv[0] = c0.x; cv[1] = c0.y; cv[2] = c0.z; cv[3] = c0.w;
+        cv[4] = c1.x; cv[5] = c1.y; cv[6] = c1.z; cv[7] = c1.w;
+    }
     float amax = 0.0f;
 #pragma unroll
     for (int k = 0; k < kFElts; ++k) {
         m[k] = 0.0f;
         if (base + k < n) {
-            const float m_old = first_step ? 0.0f : s_q[(wm >> (4 * k)) & 0xF] * sm;
+            const float m_old = first_step ? 0.0f : decode_nibble(lds, kLdsQ0, nm, k) * sm;
             const float pi = pv[k] * h.decay;
             const float mi = lerp_w(m_old, gv[k], h.w1);
-            const float vi = rf * col[c];
-            const float denom = sqrtf(vi) / h.bc2_sqrt + h.eps;
-            pv[k] = pi + (h.neg_step_size * mi) / denom;
+            const float vi = rf * (ROWS ? cv[k] : col[c]);
+            const float denom = div_by_rc(sqrt_fast(vi), h.bc2_sqrt, h.rbc2_sqrt) + h.eps;
+            pv[k] = pi + div_fast(h.neg_step_size * mi, denom);
             m[k] = mi;
             amax = fmaxf(amax, fabsf(mi));
-            if (++c == C) {
+            if (!ROWS && ++c == C) {
                 c = 0;
                 ++r;
                 rf = (base + k + 1 < n) ? row[r] / mean_all : 0.0f;
@@ -216,19 +296,21 @@ __global__ __launch_bounds__(kFThreads) void factored_update_kernel(
         }
     }
     amax = row16_max(amax);
-    const bool in_scaled = grp < n_groups;
-    if (in_scaled && (threadIdx.x & 15) == 0)
-        m_max1[grp] = amax;
-    uint32_t om = 0;
-#pragma unroll
-    for (int k = 0; k < kFElts; ++k) {
-        const float val = in_scaled ? m[k] / amax : 0.0f;
-        om |= ((val != val) ? 15u : encode_count(mids, val)) << (4 * k);
+    uint32_t om;
+    if (grp < n_groups) {
+        if ((threadIdx.x & 15) == 0)
+            m_max1[grp] = amax;
+        om = encode8_scaled(lds, kLdsQ0, kind, m, amax);
+    } else {
+        // padding added by the re-grouping to 2048: the code of a plain 0.0
+        const float z[kFElts] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+        om = kind == kMapStdM ? encode8_std_m(lds, z)
+                              : encode8_generic(make_mids(reinterpret_cast<const float *>(lds) + kLdsQ0 / 4), z);
     }
-    *reinterpret_cast<uint32_t *>(m_codes + (base >> 1)) = om;
+    store_u32(reinterpret_cast<uint32_t *>(m_codes + (base >> 1)), om);
     if (full) {
-        *reinterpret_cast<float4 *>(p + base) = make_float4(pv[0], pv[1], pv[2], pv[3]);
-        *reinterpret_cast<float4 *>(p + base + 4) = make_float4(pv[4], pv[5], pv[6], pv[7]);
+        store4(p + base, make_float4(pv[0], pv[1], pv[2], pv[3]));
+        store4(p + base + 4, make_float4(pv[4], pv[5], pv[6], pv[7]));
     } else {
 #pragma unroll
         for (int k = 0; k < kFElts; ++k)
@@ -250,8 +332,8 @@ __global__ __launch_bounds__(kFThreads) void factored_update_fp32m_kernel(
         const float pi = p[i] * h.decay;
         const float mi = lerp_w(m[i], g[i], h.w1);
         const float vi = (row[r] / mean_all) * col[c];
-        const float denom = sqrtf(vi) / h.bc2_sqrt + h.eps;
-        p[i] = pi + (h.neg_step_size * mi) / denom;
+        const float denom = div_by_rc(sqrt_fast(vi), h.bc2_sqrt, h.rbc2_sqrt) + h.eps;
+        p[i] = pi + div_fast(h.neg_step_size * mi, denom);
         m[i] = mi;
     }
 }
@@ -278,12 +360,13 @@ extern "C" int lpmm_nonfused_update(float *p, const float *g, float *m, float *v
     LPMM_REQUIRE_ALIGN(g, 4);
     LPMM_REQUIRE_ALIGN(m, 4);
     LPMM_REQUIRE_ALIGN(v, 4);
-    int64_t blocks = (n + kFThreads - 1) / kFThreads;
-    if (blocks > 256 * 64)
-        blocks = 256 * 64;
+    const int64_t blocks = (n + kFThreads * 4 - 1) / (kFThreads * 4);
+    if (blocks > 0x7fffffffLL)
+        return LPMM_ERR_SIZE;
+    const bool vec = aligned_to(p, 16) && aligned_to(g, 16) && aligned_to(m, 16) && aligned_to(v, 16);
     hipLaunchKernelGGL(nonfused_update_kernel, dim3((uint32_t)blocks), dim3(kFThreads), 0,
                        (hipStream_t)stream, p, g, m, v, n,
-                       make_nf_hyper(beta1, beta2, lr, weight_decay, eps, step));
+                       make_nf_hyper(beta1, beta2, lr, weight_decay, eps, step), vec);
     return launch_status();
 }
 
@@ -292,7 +375,8 @@ extern "C" int64_t lpmm_factored_workspace_bytes(int64_t rows, int64_t cols)
     if (rows <= 0 || cols <= 0)
         return 0;
     const int64_t ty = (rows + kSRows - 1) / kSRows, tx = (cols + kSCols - 1) / kSCols;
-    return (ty * cols + tx * (kFThreads / kWave) * rows) * (int64_t)sizeof(double);
+    const int64_t row_blocks = (rows + kFThreads - 1) / kFThreads;
+    return (ty * cols + tx * rows + row_blocks) * (int64_t)sizeof(double);
 }
 
 extern "C" int lpmm_factored_stats(const float *g, int64_t rows, int64_t cols, float *row, float *col,
@@ -315,16 +399,25 @@ extern "C" int lpmm_factored_stats(const float *g, int64_t rows, int64_t cols, f
         return LPMM_ERR_SIZE;
     double *colpart = static_cast<double *>(workspace);
     double *rowpart = colpart + ty * cols;
+    double *rowblock = rowpart + tx * rows;
+    const int64_t row_blocks = (rows + kFThreads - 1) / kFThreads;
+    const int64_t col_blocks = (cols + 63) / 64;
+    if (row_blocks + col_blocks > 0x7fffffffLL)
+        return LPMM_ERR_SIZE;
     const bool vec = aligned_to(g, 16) && (cols % 4) == 0;
     hipLaunchKernelGGL(factored_partial_kernel, dim3((uint32_t)tx, (uint32_t)ty), dim3(kFThreads), 0,
                        (hipStream_t)stream, g, rows, cols, colpart, rowpart, vec);
     int st = launch_status();
     if (st != LPMM_OK)
         return st;
-    const int64_t col_blocks = (cols + kFThreads - 1) / kFThreads;
-    hipLaunchKernelGGL(factored_finalize_kernel, dim3((uint32_t)(col_blocks + 1)), dim3(kFThreads), 0,
-                       (hipStream_t)stream, colpart, rowpart, rows, cols, (int)ty, (int)tx * (kFThreads / kWave), row, col,
-                       row_mean_all, (float)beta2, (float)(1.0 - beta2));
+    hipLaunchKernelGGL(factored_finalize_kernel, dim3((uint32_t)(row_blocks + col_blocks)), dim3(kFThreads), 0,
+                       (hipStream_t)stream, colpart, rowpart, rowblock, rows, cols, (int)ty, (int)tx,
+                       (int)row_blocks, row, col, (float)beta2, (float)(1.0 - beta2));
+    st = launch_status();
+    if (st != LPMM_OK)
+        return st;
+    hipLaunchKernelGGL(factored_mean_kernel, dim3(1), dim3(kWave), 0, (hipStream_t)stream, rowblock,
+                       (int)row_blocks, rows, row_mean_all);
     return launch_status();
 }
 
@@ -359,10 +452,15 @@ extern "C" int lpmm_factored_update(float *p, const float *g, uint8_t *m_codes, 
     if (tiles > 0x7fffffffLL)
         return LPMM_ERR_SIZE;
     const bool vec = aligned_to(p, 16) && aligned_to(g, 16);
-    hipLaunchKernelGGL(factored_update_kernel, dim3((uint32_t)tiles), dim3(kFThreads), 0,
-                       (hipStream_t)stream, p, g, m_codes, m_max1, qmap_m, row, col, row_mean_all, n, cols,
-                       n_groups, n_padded, make_nf_hyper(beta1, beta2, lr, weight_decay, eps, step),
-                       first_step != 0, vec);
+    const NfHyper h = make_nf_hyper(beta1, beta2, lr, weight_decay, eps, step);
+    if ((cols % 8) == 0 && aligned_to(col, 16))
+        hipLaunchKernelGGL(factored_update_kernel<true>, dim3((uint32_t)tiles), dim3(kFThreads), 0,
+                           (hipStream_t)stream, p, g, m_codes, m_max1, qmap_m, row, col, row_mean_all, n, cols,
+                           n_groups, n_padded, h, first_step != 0, vec);
+    else
+        hipLaunchKernelGGL(factored_update_kernel<false>, dim3((uint32_t)tiles), dim3(kFThreads), 0,
+                           (hipStream_t)stream, p, g, m_codes, m_max1, qmap_m, row, col, row_mean_all, n, cols,
+                           n_groups, n_padded, h, first_step != 0, vec);
     return launch_status();
 }
 

@@ -18,8 +18,7 @@
 // use the correctly rounded reciprocal plus one fma correction step; both give the same
 // results as the generic search and the plain division, which remain as the fallback for
 // any other map.
-#include "lpmm_common.hpp"
-#include "lpmm_encode.hpp"
+#include "lpmm_codec.hpp"
 
 #include <math.h>
 
@@ -57,33 +56,8 @@ struct Hyper {
 };
 
 #ifndef LPMM_P_MODE
-#define LPMM_P_MODE 1
+#define LPMM_P_MODE 1  // 0: IEEE sqrt/div, 1: approximation + residual correction, 2: approximation only
 #endif
-#ifndef LPMM_NT
-#define LPMM_NT 3
-#endif
-
-// sqrt(x) for x >= 0 from the hardware reciprocal square root plus one fma correction of
-// the residual: correctly rounded except for a vanishing fraction of inputs (1 ulp there).
-// Inputs below the smallest normal are treated as that value (their square root is far
-// below any eps it is added to).
-__device__ __forceinline__ float sqrt_fast(float x)
-{
-    const float y = __builtin_amdgcn_rsqf(fmaxf(x, 0x1p-126f));
-    const float s = x * y;
-    const float h = 0.5f * y;
-    const float r = __builtin_fmaf(-s, s, x);
-    return __builtin_fmaf(r, h, s);
-}
-
-// x / d from the hardware reciprocal plus one fma correction of the residual (same remark).
-__device__ __forceinline__ float div_fast(float x, float d)
-{
-    const float rc = __builtin_amdgcn_rcpf(d);
-    const float q = x * rc;
-    const float r = __builtin_fmaf(-q, d, x);
-    return __builtin_fmaf(r, rc, q);
-}
 
 // AdamW on one element; returns the new parameter, updates m and v in place.
 __device__ __forceinline__ float adamw_elt(float p, float g, float &m, float &v, const Hyper &h)
@@ -106,81 +80,8 @@ __device__ __forceinline__ float adamw_elt(float p, float g, float &m, float &v,
     return p - (h.lr * update);
 }
 
-// x / y for |x| <= y given rc = RN(1/y): one multiply and two fmas give the correctly rounded
-// quotient when y lies in [2^-60, 2^60] (no intermediate underflow where it matters).
-__device__ __forceinline__ float div_by_rc(float x, float y, float rc)
-{
-    const float q = x * rc;
-    const float r = __builtin_fmaf(-q, y, x);
-    return __builtin_fmaf(r, rc, q);
-}
-
-__device__ __forceinline__ bool rc_safe(float y)
-{
-    return y >= 0x1p-60f && y <= 0x1p60f;
-}
-
-__device__ __forceinline__ bool maps_are_standard(const float *__restrict__ qmap_m,
-                                                  const float *__restrict__ qmap_v)
-{
-    // all 32 words are fetched at once (scalar loads) and folded without branches
-    uint32_t diff = 0;
-#pragma unroll
-    for (int k = 0; k < 16; ++k)
-        diff |= (__float_as_uint(qmap_m[k]) ^ kStdQmapMBits[k]) | (__float_as_uint(qmap_v[k]) ^ kStdQmapVBits[k]);
-    return diff == 0;
-}
-
-typedef float v4f __attribute__((ext_vector_type(4)));
-__device__ __forceinline__ float4 load4(const float *p)
-{
-#if LPMM_NT & 1
-    const v4f t = __builtin_nontemporal_load(reinterpret_cast<const v4f *>(p));
-    return make_float4(t.x, t.y, t.z, t.w);
-#else
-    return *reinterpret_cast<const float4 *>(p);
-#endif
-}
-__device__ __forceinline__ void store4(float *p, float4 v)
-{
-#if LPMM_NT & 2
-    const v4f t = {v.x, v.y, v.z, v.w};
-    __builtin_nontemporal_store(t, reinterpret_cast<v4f *>(p));
-#else
-    *reinterpret_cast<float4 *>(p) = v;
-#endif
-}
-__device__ __forceinline__ uint32_t load_u16(const uint16_t *p)
-{
-#if LPMM_NT & 1
-    return __builtin_nontemporal_load(p);
-#else
-    return *p;
-#endif
-}
-__device__ __forceinline__ void store_u16(uint16_t *p, uint32_t v)
-{
-#if LPMM_NT & 2
-    __builtin_nontemporal_store((uint16_t)v, p);
-#else
-    *p = (uint16_t)v;
-#endif
-}
-
 // element k (0..7) of a lane sits at this offset inside the lane's group
 __device__ __forceinline__ int elt_offset(int lane16, int k) { return lane16 * 4 + (k & 3) + (k >> 2) * 64; }
-
-// LDS map of the 4-bit kernel (bytes): [0,64) qmap_m, [64,128) qmap_v, then the
-// first-moment encode table at the offsets lpmm_encode.hpp computes.
-constexpr uint32_t kLdsBytes = kEncLdsEnd;
-constexpr uint32_t kLdsQm = 0, kLdsQv = 64;
-static_assert(kLdsQv + 64 <= kEncLdsBegin, "maps overlap the encode table");
-
-template <typename T>
-__device__ __forceinline__ T lds_read(const uint32_t *lds, uint32_t byte_off)
-{
-    return *reinterpret_cast<const T *>(reinterpret_cast<const char *>(lds) + byte_off);
-}
 
 // One 128-element group, handled by the 16 lanes of a DPP row.  FULL: the whole group lies
 // inside the tensor and the pointers allow vector access; otherwise every access is
@@ -230,18 +131,12 @@ __device__ __forceinline__ void group_step(const Tensor4 &t, const Hyper &h, con
         }
     }
 
-    // decode: byte j of the *_even / *_odd words holds 4 * nibble (2j) / (2j+1) = LDS offset
-    uint32_t me = (wm << 2) & 0x3C3C3C3Cu, mo = (wm >> 2) & 0x3C3C3C3Cu;
-    uint32_t ve = (wv << 2) & 0x3C3C3C3Cu, vo = (wv >> 2) & 0x3C3C3C3Cu;
-    // keep the four masked words as they are, so that each offset below is one bit-field extract
-    asm volatile("" : "+v"(me), "+v"(mo), "+v"(ve), "+v"(vo));
+    const Nibbles nm = split_nibbles(wm), nv = split_nibbles(wv);
     float amax_m = 0.0f, amax_v = 0.0f;
 #pragma unroll
     for (int k = 0; k < kEltsPerLane; ++k) {
-        const uint32_t om = __builtin_amdgcn_ubfe((k & 1) ? mo : me, 8 * (k >> 1), 8);
-        const uint32_t ov = __builtin_amdgcn_ubfe((k & 1) ? vo : ve, 8 * (k >> 1), 8);
-        m[k] = lds_read<float>(lds, kLdsQm + om) * sm;
-        v[k] = lds_read<float>(lds, kLdsQv + ov) * sv;
+        m[k] = decode_nibble(lds, kLdsQ0, nm, k) * sm;
+        v[k] = decode_nibble(lds, kLdsQ1, nv, k) * sv;
         if (FULL || (gbase + elt_offset(lane16, k) < n)) {
             pv[k] = adamw_elt(pv[k], gv[k], m[k], v[k], h);
             amax_m = fmaxf(amax_m, fabsf(m[k]));
@@ -257,35 +152,8 @@ __device__ __forceinline__ void group_step(const Tensor4 &t, const Hyper &h, con
     if (!any)
         return;
 
-    uint32_t cm = 0, cv = 0;
-    if (std_maps && rc_safe(amax_m) && rc_safe(amax_v)) {
-        const float rcm = 1.0f / amax_m, rcv = 1.0f / amax_v;
-        uint32_t vb[2] = {0u, 0u};  // v codes of elements 0..3 / 4..7, one per byte
-#pragma unroll
-        for (int k = 0; k < kEltsPerLane; ++k) {
-            const float xm = div_by_rc(m[k], amax_m, rcm);
-            const uint4 e = lds_read<uint4>(lds, enc_m_lds_offset(xm));
-            cm |= enc_m_pick(xm, e.x, e.y, e.z) << (4 * k);
-            // enc_v_linear with the clamp at 0 done by the saturating byte conversion
-            // (0 <= x <= 1 here, so the value never exceeds 15)
-            const float tv = __builtin_ceilf(__builtin_fmaf(div_by_rc(v[k], amax_v, rcv), 16.0f, -1.5f));
-            vb[k >> 2] = __builtin_amdgcn_cvt_pk_u8_f32(tv, k & 3, vb[k >> 2]);
-        }
-        // bytes {c0,c1,c2,c3} -> byte 0 = c0|c1<<4, byte 2 = c2|c3<<4; gather bytes 0,2 of both words
-        const uint32_t t0 = vb[0] | (vb[0] >> 4), t1 = vb[1] | (vb[1] >> 4);
-        cv = __builtin_amdgcn_perm(t1, t0, 0x06040200u);
-    } else {
-        // x/0 with x == 0 is NaN, which the reference turns into code 15 for the whole group
-        const bool nan_m = (amax_m == 0.0f), nan_v = (amax_v == 0.0f);
-        // the maps are read back from LDS so that they occupy registers only on this path
-        const Mids mids_m = make_mids(reinterpret_cast<const float *>(lds) + kLdsQm / 4);
-        const Mids mids_v = make_mids(reinterpret_cast<const float *>(lds) + kLdsQv / 4);
-#pragma unroll
-        for (int k = 0; k < kEltsPerLane; ++k) {
-            cm |= (nan_m ? 15u : encode_count(mids_m, m[k] / amax_m)) << (4 * k);
-            cv |= (nan_v ? 15u : encode_count(mids_v, v[k] / amax_v)) << (4 * k);
-        }
-    }
+    const uint32_t cm = encode8_scaled(lds, kLdsQ0, std_maps ? kMapStdM : kMapGeneric, m, amax_m);
+    const uint32_t cv = encode8_scaled(lds, kLdsQ1, std_maps ? kMapStdV : kMapGeneric, v, amax_v);
 
     if (FULL) {
         float *pp = t.p + gbase + lane16 * 4;
@@ -327,15 +195,8 @@ __global__ __launch_bounds__(kThreads) void adamw4bit_kernel(const Multi4 args,
                                                              const float *__restrict__ qmap_v)
 {
     __shared__ __align__(16) uint32_t lds[kLdsBytes / 4];
-    if (threadIdx.x < 16)
-        lds[kLdsQm / 4 + threadIdx.x] = __float_as_uint(qmap_m[threadIdx.x]);
-    else if (threadIdx.x < 32)
-        lds[kLdsQv / 4 + threadIdx.x - 16] = __float_as_uint(qmap_v[threadIdx.x - 16]);
-    if (threadIdx.x < 2 * kEncBuckets) {
-        const uint4 e = *reinterpret_cast<const uint4 *>(kEncTableM[threadIdx.x]);
-        *reinterpret_cast<uint4 *>(reinterpret_cast<char *>(lds) + e.w) = e;  // e.w: the entry's LDS offset
-    }
-    const bool std_maps = maps_are_standard(qmap_m, qmap_v);
+    lds_fill(lds, qmap_m, qmap_v);
+    const bool std_maps = classify_map(qmap_m) == kMapStdM && classify_map(qmap_v) == kMapStdV;
 
     // which tensor does this tile belong to (uniform over the workgroup): the number of
     // later tensors whose first tile is not after this one; unused slots hold the total

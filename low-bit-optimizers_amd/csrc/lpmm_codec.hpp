@@ -1,0 +1,197 @@
+// Device-side building blocks shared by the gfx950 kernels: streaming (nontemporal) memory
+// access, near-exact sqrt/division from the hardware approximations, the LDS-resident
+// quantisation maps and first-moment encode table, and 4-bit code assignment.
+#pragma once
+
+#include "lpmm_common.hpp"
+#include "lpmm_encode.hpp"
+
+namespace lpmm {
+
+// ---------------------------------------------------------------------------------------
+// Streaming access.  Every large operand of these kernels is touched exactly once per
+// launch, so loads and stores carry the nontemporal hint: on MI355X the same access pattern
+// runs at 5.9 TB/s with it and 4.8 TB/s without.
+// ---------------------------------------------------------------------------------------
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ float4 load4(const float *p)
+{
+    const v4f t = __builtin_nontemporal_load(reinterpret_cast<const v4f *>(p));
+    return make_float4(t.x, t.y, t.z, t.w);
+}
+__device__ __forceinline__ void store4(float *p, float4 v)
+{
+    const v4f t = {v.x, v.y, v.z, v.w};
+    __builtin_nontemporal_store(t, reinterpret_cast<v4f *>(p));
+}
+__device__ __forceinline__ uint32_t load_u16(const uint16_t *p) { return __builtin_nontemporal_load(p); }
+__device__ __forceinline__ void store_u16(uint16_t *p, uint32_t v) { __builtin_nontemporal_store((uint16_t)v, p); }
+__device__ __forceinline__ uint32_t load_u32(const uint32_t *p) { return __builtin_nontemporal_load(p); }
+__device__ __forceinline__ void store_u32(uint32_t *p, uint32_t v) { __builtin_nontemporal_store(v, p); }
+
+// ---------------------------------------------------------------------------------------
+// Near-exact arithmetic: hardware approximation + one fma correction of the exact residual.
+// ---------------------------------------------------------------------------------------
+
+// sqrt(x) for x >= 0: correctly rounded except for a vanishing fraction of inputs (1 ulp
+// there).  Inputs below the smallest normal are treated as that value (their square root is
+// far below any eps it is added to).
+__device__ __forceinline__ float sqrt_fast(float x)
+{
+    const float y = __builtin_amdgcn_rsqf(fmaxf(x, 0x1p-126f));
+    const float s = x * y;
+    const float h = 0.5f * y;
+    const float r = __builtin_fmaf(-s, s, x);
+    return __builtin_fmaf(r, h, s);
+}
+
+// x / d (same remark).
+__device__ __forceinline__ float div_fast(float x, float d)
+{
+    const float rc = __builtin_amdgcn_rcpf(d);
+    const float q = x * rc;
+    const float r = __builtin_fmaf(-q, d, x);
+    return __builtin_fmaf(r, rc, q);
+}
+
+// x / y given rc = RN(1/y): one multiply and two fmas give the correctly rounded quotient
+// when y lies in [2^-60, 2^60] and |x| <= y (no intermediate underflow where a code depends
+// on it).
+__device__ __forceinline__ float div_by_rc(float x, float y, float rc)
+{
+    const float q = x * rc;
+    const float r = __builtin_fmaf(-q, y, x);
+    return __builtin_fmaf(r, rc, q);
+}
+
+__device__ __forceinline__ bool rc_safe(float y) { return y >= 0x1p-60f && y <= 0x1p60f; }
+
+// ---------------------------------------------------------------------------------------
+// Which map is this?  Decided on the device from the 16 values themselves (scalar loads,
+// xor/or, no branches, no host round trip).
+// ---------------------------------------------------------------------------------------
+enum MapKind : int { kMapGeneric = 0, kMapStdM = 1, kMapStdV = 2 };
+
+__device__ __forceinline__ int classify_map(const float *__restrict__ qmap)
+{
+    uint32_t dm = 0, dv = 0;
+#pragma unroll
+    for (int k = 0; k < 16; ++k) {
+        const uint32_t b = __float_as_uint(qmap[k]);
+        dm |= b ^ kStdQmapMBits[k];
+        dv |= b ^ kStdQmapVBits[k];
+    }
+    return dm == 0 ? kMapStdM : (dv == 0 ? kMapStdV : kMapGeneric);
+}
+
+// ---------------------------------------------------------------------------------------
+// LDS map (bytes): [0,64) first map, [64,128) second map, then the first-moment encode
+// table at the offsets lpmm_encode.hpp computes (the bytes in between stay unused).
+// ---------------------------------------------------------------------------------------
+constexpr uint32_t kLdsBytes = kEncLdsEnd;
+constexpr uint32_t kLdsQ0 = 0, kLdsQ1 = 64;
+static_assert(kLdsQ1 + 64 <= kEncLdsBegin, "maps overlap the encode table");
+
+template <typename T>
+__device__ __forceinline__ T lds_read(const uint32_t *lds, uint32_t byte_off)
+{
+    return *reinterpret_cast<const T *>(reinterpret_cast<const char *>(lds) + byte_off);
+}
+
+// Threads [0,16) copy map 0, [16,32) map 1 (if given), [0, 2*kEncBuckets) the encode table.
+// The caller synchronises the workgroup afterwards.
+__device__ __forceinline__ void lds_fill(uint32_t *lds, const float *__restrict__ q0, const float *__restrict__ q1)
+{
+    if (threadIdx.x < 16)
+        lds[kLdsQ0 / 4 + threadIdx.x] = __float_as_uint(q0[threadIdx.x]);
+    else if (threadIdx.x < 32 && q1 != nullptr)
+        lds[kLdsQ1 / 4 + threadIdx.x - 16] = __float_as_uint(q1[threadIdx.x - 16]);
+    if (threadIdx.x < 2 * kEncBuckets) {
+        const uint4 e = *reinterpret_cast<const uint4 *>(kEncTableM[threadIdx.x]);
+        *reinterpret_cast<uint4 *>(reinterpret_cast<char *>(lds) + e.w) = e;  // e.w: the entry's LDS offset
+    }
+}
+
+// Codes of 8 already divided values with the standard first-moment map: nibble k = code of x[k].
+__device__ __forceinline__ uint32_t encode8_std_m(const uint32_t *lds, const float (&x)[8])
+{
+    uint32_t w = 0;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        const uint4 e = lds_read<uint4>(lds, enc_m_lds_offset(x[k]));
+        w |= enc_m_pick(x[k], e.x, e.y, e.z) << (4 * k);
+    }
+    return w;
+}
+
+// The same for the standard second-moment map; requires 0 <= x[k] <= 1 (so the code never
+// exceeds 15) -- the clamp at 0 is done by the saturating byte conversion.
+__device__ __forceinline__ uint32_t encode8_std_v(const float (&x)[8])
+{
+    uint32_t b[2] = {0u, 0u};  // codes of elements 0..3 / 4..7, one per byte
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        const float t = __builtin_ceilf(__builtin_fmaf(x[k], 16.0f, -1.5f));
+        b[k >> 2] = __builtin_amdgcn_cvt_pk_u8_f32(t, k & 3, b[k >> 2]);
+    }
+    // bytes {c0,c1,c2,c3} -> byte 0 = c0|c1<<4, byte 2 = c2|c3<<4; gather bytes 0, 2 of both words
+    const uint32_t t0 = b[0] | (b[0] >> 4), t1 = b[1] | (b[1] >> 4);
+    return __builtin_amdgcn_perm(t1, t0, 0x06040200u);
+}
+
+// Any ascending map: count of midpoints below x; NaN -> 15.
+__device__ __forceinline__ uint32_t encode8_generic(const Mids &mids, const float (&x)[8])
+{
+    uint32_t w = 0;
+#pragma unroll
+    for (int k = 0; k < 8; ++k)
+        w |= ((x[k] != x[k]) ? 15u : encode_count(mids, x[k])) << (4 * k);
+    return w;
+}
+
+// Codes of v[k] / amax for the 8 values of a lane (amax uniform over the lanes that share a
+// scale).  `kind` says which map sits at LDS offset `lds_map`; an all-zero group (0/0 -> NaN)
+// gives code 15 throughout, as in the reference.  For kMapStdV the values must be >= 0.
+__device__ __forceinline__ uint32_t encode8_scaled(const uint32_t *lds, uint32_t lds_map, int kind,
+                                                   const float (&v)[8], float amax)
+{
+    float x[8];
+    if (kind != kMapGeneric && rc_safe(amax)) {
+        const float rc = 1.0f / amax;
+#pragma unroll
+        for (int k = 0; k < 8; ++k)
+            x[k] = div_by_rc(v[k], amax, rc);
+        return kind == kMapStdM ? encode8_std_m(lds, x) : encode8_std_v(x);
+    }
+#pragma unroll
+    for (int k = 0; k < 8; ++k)
+        x[k] = v[k] / amax;
+    // the map is read back from LDS so that it occupies registers only on this path
+    const Mids mids = make_mids(reinterpret_cast<const float *>(lds) + lds_map / 4);
+    return encode8_generic(mids, x);
+}
+
+// Decode offsets: byte j of `even` / `odd` holds 4 * nibble (2j) / (2j+1) of the code word.
+struct Nibbles {
+    uint32_t even, odd;
+};
+
+__device__ __forceinline__ Nibbles split_nibbles(uint32_t w)
+{
+    Nibbles n;
+    n.even = (w << 2) & 0x3C3C3C3Cu;
+    n.odd = (w >> 2) & 0x3C3C3C3Cu;
+    // keep the masked words as they are, so that each offset below is one bit-field extract
+    asm volatile("" : "+v"(n.even), "+v"(n.odd));
+    return n;
+}
+
+// qmap[nibble k] from the map at LDS offset lds_map
+__device__ __forceinline__ float decode_nibble(const uint32_t *lds, uint32_t lds_map, const Nibbles &n, int k)
+{
+    const uint32_t off = __builtin_amdgcn_ubfe((k & 1) ? n.odd : n.even, 8 * (k >> 1), 8);
+    return lds_read<float>(lds, lds_map + off);
+}
+
+}  // namespace lpmm

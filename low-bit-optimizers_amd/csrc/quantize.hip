@@ -5,8 +5,10 @@
 //
 // A lane owns 8 consecutive values = one 32-bit word of codes; a 256-thread workgroup
 // covers one 2048-value pack group.  Group maxima use DPP row reductions (128 values =
-// 16 lanes) and, for larger groups, 16 floats of LDS per workgroup.
-#include "lpmm_common.hpp"
+// 16 lanes) and, for larger groups, 16 floats of LDS per workgroup.  Code assignment uses
+// the table / closed-form encoders of lpmm_codec.hpp when the map is one of the two
+// standard ones and the count-of-midpoints search otherwise.
+#include "lpmm_codec.hpp"
 
 namespace lpmm {
 
@@ -14,17 +16,11 @@ constexpr int kQThreads = 256;
 constexpr int kQElts = 8;
 constexpr int kQTile = kQThreads * kQElts;  // 2048
 
-__device__ __forceinline__ uint32_t encode_nan15(const Mids &mids, float x)
-{
-    return (x != x) ? 15u : encode_count(mids, x);
-}
-
 __device__ __forceinline__ void load8(const float *__restrict__ x, int64_t base, int64_t n, bool vec,
                                       float (&v)[kQElts])
 {
     if (vec && base + kQElts <= n) {
-        const float4 a = *reinterpret_cast<const float4 *>(x + base);
-        const float4 b = *reinterpret_cast<const float4 *>(x + base + 4);
+        const float4 a = load4(x + base), b = load4(x + base + 4);
         v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
         v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
     } else {
@@ -38,14 +34,51 @@ __device__ __forceinline__ void store8(float *__restrict__ out, int64_t base, in
                                        const float (&v)[kQElts])
 {
     if (vec && base + kQElts <= n) {
-        *reinterpret_cast<float4 *>(out + base) = make_float4(v[0], v[1], v[2], v[3]);
-        *reinterpret_cast<float4 *>(out + base + 4) = make_float4(v[4], v[5], v[6], v[7]);
+        store4(out + base, make_float4(v[0], v[1], v[2], v[3]));
+        store4(out + base + 4, make_float4(v[4], v[5], v[6], v[7]));
     } else {
 #pragma unroll
         for (int k = 0; k < kQElts; ++k)
             if (base + k < n)
                 out[base + k] = v[k];
     }
+}
+
+// codes hold at least ceil(n/2) bytes; whole words are read only where they lie inside.
+__device__ __forceinline__ uint32_t load_codes8(const uint8_t *__restrict__ codes, int64_t base, int64_t n,
+                                                bool vec)
+{
+    if (vec && base + kQElts <= n)
+        return load_u32(reinterpret_cast<const uint32_t *>(codes + (base >> 1)));
+    uint32_t w = 0;
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+        if (base + 2 * k < n)
+            w |= (uint32_t)codes[(base >> 1) + k] << (8 * k);
+    return w;
+}
+
+// Codes of 8 values that are already normalised (no division): NaN -> 15 like the reference.
+__device__ __forceinline__ uint32_t encode8_plain(const uint32_t *lds, int kind, const float (&x)[kQElts])
+{
+    if (kind == kMapGeneric)
+        return encode8_generic(make_mids(reinterpret_cast<const float *>(lds) + kLdsQ0 / 4), x);
+    uint32_t w;
+    if (kind == kMapStdM) {
+        w = encode8_std_m(lds, x);
+    } else {
+        // the closed form needs x <= 1 for the upper clamp; larger inputs are legal here
+        float y[kQElts];
+#pragma unroll
+        for (int k = 0; k < kQElts; ++k)
+            y[k] = fminf(x[k], 1.0f);
+        w = encode8_std_v(y);
+    }
+#pragma unroll
+    for (int k = 0; k < kQElts; ++k)
+        if (x[k] != x[k])
+            w |= 15u << (4 * k);
+    return w;
 }
 
 // ---------------------------------------------------------------------------------------
@@ -56,7 +89,10 @@ __global__ __launch_bounds__(kQThreads) void pack4_kernel(const float *__restric
                                                           int64_t n_padded, uint8_t *__restrict__ out,
                                                           bool vec)
 {
-    const Mids mids = make_mids(qmap);
+    __shared__ __align__(16) uint32_t lds[kLdsBytes / 4];
+    lds_fill(lds, qmap, nullptr);
+    const int kind = classify_map(qmap);
+    __syncthreads();
     const int64_t base = ((int64_t)blockIdx.x * kQThreads + threadIdx.x) * kQElts;
     if (base == 0)
         out[n_padded / 2] = 0;
@@ -64,12 +100,9 @@ __global__ __launch_bounds__(kQThreads) void pack4_kernel(const float *__restric
         return;
     float v[kQElts];
     load8(x, base, n_padded, vec, v);
-    uint32_t w = 0;
-#pragma unroll
-    for (int k = 0; k < kQElts; ++k)
-        w |= encode_nan15(mids, v[k]) << (4 * k);
+    const uint32_t w = encode8_plain(lds, kind, v);
     if (vec) {
-        *reinterpret_cast<uint32_t *>(out + (base >> 1)) = w;
+        store_u32(reinterpret_cast<uint32_t *>(out + (base >> 1)), w);
     } else {
 #pragma unroll
         for (int k = 0; k < 4; ++k)
@@ -77,36 +110,22 @@ __global__ __launch_bounds__(kQThreads) void pack4_kernel(const float *__restric
     }
 }
 
-// codes hold at least ceil(n/2) bytes; whole words are read only where they lie inside.
-__device__ __forceinline__ uint32_t load_codes8(const uint8_t *__restrict__ codes, int64_t base, int64_t n,
-                                                bool vec)
-{
-    if (vec && base + kQElts <= n)
-        return *reinterpret_cast<const uint32_t *>(codes + (base >> 1));
-    uint32_t w = 0;
-#pragma unroll
-    for (int k = 0; k < 4; ++k)
-        if (base + 2 * k < n)
-            w |= (uint32_t)codes[(base >> 1) + k] << (8 * k);
-    return w;
-}
-
 __global__ __launch_bounds__(kQThreads) void unpack4_kernel(const uint8_t *__restrict__ codes,
                                                             const float *__restrict__ qmap, int64_t n,
                                                             float *__restrict__ out, bool vec)
 {
-    __shared__ float s_q[16];
+    __shared__ __align__(16) uint32_t lds[32];
     if (threadIdx.x < 16)
-        s_q[threadIdx.x] = qmap[threadIdx.x];
+        lds[threadIdx.x] = __float_as_uint(qmap[threadIdx.x]);
     __syncthreads();
     const int64_t base = ((int64_t)blockIdx.x * kQThreads + threadIdx.x) * kQElts;
     if (base >= n)
         return;
-    const uint32_t w = load_codes8(codes, base, n, vec);
+    const Nibbles nb = split_nibbles(load_codes8(codes, base, n, vec));
     float v[kQElts];
 #pragma unroll
     for (int k = 0; k < kQElts; ++k)
-        v[k] = s_q[(w >> (4 * k)) & 0xF];
+        v[k] = decode_nibble(lds, kLdsQ0, nb, k);
     store8(out, base, n, vec, v);
 }
 
@@ -121,8 +140,10 @@ __global__ __launch_bounds__(kQThreads) void quant_group_kernel(const float *__r
                                                                 float *__restrict__ max1, int64_t n_groups,
                                                                 int64_t n_padded, bool vec)
 {
+    __shared__ __align__(16) uint32_t lds[kLdsBytes / 4];
     __shared__ float s_row[kQThreads / 16];
-    const Mids mids = make_mids(qmap);
+    lds_fill(lds, qmap, nullptr);
+    const int kind = classify_map(qmap);
     const int64_t base = ((int64_t)blockIdx.x * kQThreads + threadIdx.x) * kQElts;
     if (base == 0)
         codes[n_padded / 2] = 0;
@@ -133,28 +154,28 @@ __global__ __launch_bounds__(kQThreads) void quant_group_kernel(const float *__r
     for (int k = 0; k < kQElts; ++k)
         amax = fmaxf(amax, fabsf(v[k]));
     amax = row16_max(amax);
+    if ((threadIdx.x & 15) == 0)
+        s_row[threadIdx.x >> 4] = amax;
+    __syncthreads();
     if (rows_per_group > 1) {
-        const int row = threadIdx.x >> 4;
-        if ((threadIdx.x & 15) == 0)
-            s_row[row] = amax;
-        __syncthreads();
-        const int first = row & ~(rows_per_group - 1);
+        const int first = (threadIdx.x >> 4) & ~(rows_per_group - 1);
         amax = s_row[first];
         for (int r = 1; r < rows_per_group; ++r)
             amax = fmaxf(amax, s_row[first + r]);
     }
     const int64_t gp_sz = (int64_t)rows_per_group * kGroup;
     const int64_t grp = base / gp_sz;
-    const bool in_scaled = grp < n_groups;  // else: padding added by the re-grouping to 2048
-    if (in_scaled && (base % gp_sz) == 0)
-        max1[grp] = amax;
-    uint32_t w = 0;
-#pragma unroll
-    for (int k = 0; k < kQElts; ++k) {
-        const float val = in_scaled ? v[k] / amax : 0.0f;
-        w |= encode_nan15(mids, val) << (4 * k);
+    uint32_t w;
+    if (grp < n_groups) {
+        if ((base % gp_sz) == 0)
+            max1[grp] = amax;
+        w = encode8_scaled(lds, kLdsQ0, kind, v, amax);
+    } else {
+        // padding added by the re-grouping to 2048: plain zeros, not divided by anything
+        const float z[kQElts] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+        w = encode8_plain(lds, kind, z);
     }
-    *reinterpret_cast<uint32_t *>(codes + (base >> 1)) = w;
+    store_u32(reinterpret_cast<uint32_t *>(codes + (base >> 1)), w);
 }
 
 __global__ __launch_bounds__(kQThreads) void dequant_group_kernel(const uint8_t *__restrict__ codes,
@@ -163,19 +184,19 @@ __global__ __launch_bounds__(kQThreads) void dequant_group_kernel(const uint8_t 
                                                                   int64_t gp_sz, float *__restrict__ out,
                                                                   bool vec)
 {
-    __shared__ float s_q[16];
+    __shared__ __align__(16) uint32_t lds[32];
     if (threadIdx.x < 16)
-        s_q[threadIdx.x] = qmap[threadIdx.x];
+        lds[threadIdx.x] = __float_as_uint(qmap[threadIdx.x]);
     __syncthreads();
     const int64_t base = ((int64_t)blockIdx.x * kQThreads + threadIdx.x) * kQElts;
     if (base >= n)
         return;
-    const uint32_t w = load_codes8(codes, base, n, vec);
+    const Nibbles nb = split_nibbles(load_codes8(codes, base, n, vec));
     const float s = max1[base / gp_sz];  // gp_sz is a multiple of 128, so uniform over the lane's 8
     float v[kQElts];
 #pragma unroll
     for (int k = 0; k < kQElts; ++k)
-        v[k] = s_q[(w >> (4 * k)) & 0xF] * s;
+        v[k] = decode_nibble(lds, kLdsQ0, nb, k) * s;
     store8(out, base, n, vec, v);
 }
 
@@ -193,6 +214,7 @@ __global__ void fill_zero_kernel(float *__restrict__ a, int64_t na, float *__res
 
 constexpr int kStatRows = 32;
 constexpr int kStatCols = 1024;  // 256 threads x 4 columns
+constexpr int kStatUnroll = 8;   // rows in flight per lane
 
 // max of non-negative floats == max of their bit patterns as unsigned integers
 __device__ __forceinline__ void atomic_max_nonneg(float *addr, float v)
@@ -200,6 +222,8 @@ __device__ __forceinline__ void atomic_max_nonneg(float *addr, float v)
     atomicMax(reinterpret_cast<unsigned int *>(addr), __float_as_uint(v));
 }
 
+// Tile of kStatRows x kStatCols; a lane keeps 4 column maxima in registers, row maxima are
+// reduced over the wave and merged with atomics (max is exact and order-independent).
 __global__ __launch_bounds__(kQThreads) void rank1_stats_kernel(const float *__restrict__ x, int64_t R,
                                                                 int64_t C, float *__restrict__ rowmax,
                                                                 float *__restrict__ colmax, bool vec)
@@ -207,25 +231,32 @@ __global__ __launch_bounds__(kQThreads) void rank1_stats_kernel(const float *__r
     const int64_t c0 = (int64_t)blockIdx.x * kStatCols + (int64_t)threadIdx.x * 4;
     const int64_t r0 = (int64_t)blockIdx.y * kStatRows;
     const int64_t r1 = (r0 + kStatRows < R) ? r0 + kStatRows : R;
+    const bool lane_vec = vec && c0 + 4 <= C;
     float cm[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-    for (int64_t r = r0; r < r1; ++r) {
-        float a[4];
-        const float *row = x + r * C;
-        if (vec && c0 + 4 <= C) {
-            const float4 t = *reinterpret_cast<const float4 *>(row + c0);
-            a[0] = fabsf(t.x); a[1] = fabsf(t.y); a[2] = fabsf(t.z); a[3] = fabsf(t.w);
-        } else {
+    for (int64_t rb = r0; rb < r1; rb += kStatUnroll) {
+        float a[kStatUnroll][4];
+#pragma unroll
+        for (int u = 0; u < kStatUnroll; ++u) {
+            const int64_t r = rb + u;
+            if (r < r1 && lane_vec) {
+                const float4 t = load4(x + r * C + c0);
+                a[u][0] = fabsf(t.x); a[u][1] = fabsf(t.y); a[u][2] = fabsf(t.z); a[u][3] = fabsf(t.w);
+            } else {
+#pragma unroll
+                for (int k = 0; k < 4; ++k)
+                    a[u][k] = (r < r1 && c0 + k < C) ? fabsf(x[r * C + c0 + k]) : 0.0f;
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kStatUnroll; ++u) {
+            float rm = fmaxf(fmaxf(a[u][0], a[u][1]), fmaxf(a[u][2], a[u][3]));
 #pragma unroll
             for (int k = 0; k < 4; ++k)
-                a[k] = (c0 + k < C) ? fabsf(row[c0 + k]) : 0.0f;
+                cm[k] = fmaxf(cm[k], a[u][k]);
+            rm = wave_max(rm);
+            if ((threadIdx.x & 63) == 0 && rb + u < r1)
+                atomic_max_nonneg(rowmax + rb + u, rm);
         }
-        float rm = fmaxf(fmaxf(a[0], a[1]), fmaxf(a[2], a[3]));
-#pragma unroll
-        for (int k = 0; k < 4; ++k)
-            cm[k] = fmaxf(cm[k], a[k]);
-        rm = wave_max(rm);
-        if ((threadIdx.x & 63) == 0)
-            atomic_max_nonneg(rowmax + r, rm);
     }
 #pragma unroll
     for (int k = 0; k < 4; ++k)
@@ -233,6 +264,8 @@ __global__ __launch_bounds__(kQThreads) void rank1_stats_kernel(const float *__r
             atomic_max_nonneg(colmax + c0 + k, cm[k]);
 }
 
+// Normalise by min(rowmax[r], colmax[c]), search, pack.  Flattened indexing: a lane's 8
+// values may straddle rows (any C).
 __global__ __launch_bounds__(kQThreads) void quant_rank1_kernel(const float *__restrict__ x, int64_t n,
                                                                 int64_t C, const float *__restrict__ rowmax,
                                                                 const float *__restrict__ colmax,
@@ -240,32 +273,75 @@ __global__ __launch_bounds__(kQThreads) void quant_rank1_kernel(const float *__r
                                                                 uint8_t *__restrict__ codes, int64_t n_padded,
                                                                 bool vec)
 {
-    const Mids mids = make_mids(qmap);
+    __shared__ __align__(16) uint32_t lds[kLdsBytes / 4];
+    lds_fill(lds, qmap, nullptr);
+    const int kind = classify_map(qmap);
+    __syncthreads();
     const int64_t base = ((int64_t)blockIdx.x * kQThreads + threadIdx.x) * kQElts;
     if (base == 0)
         codes[n_padded / 2] = 0;
-    float v[kQElts];
+    float v[kQElts], xs[kQElts];
     load8(x, base, n, vec, v);
     int64_t r = base / C;
     int64_t c = base - r * C;
     float rm = (base < n) ? rowmax[r] : 0.0f;
-    uint32_t w = 0;
 #pragma unroll
     for (int k = 0; k < kQElts; ++k) {
-        float val = 0.0f;  // padding added by the re-grouping to 2048
+        xs[k] = 0.0f;  // padding added by the re-grouping to 2048
         if (base + k < n) {
             const float cmx = colmax[c];
             const float st = (cmx < rm) ? cmx : rm;
-            val = v[k] / st;
+            xs[k] = v[k] / st;
             if (++c == C) {
                 c = 0;
                 ++r;
                 rm = (base + k + 1 < n) ? rowmax[r] : 0.0f;
             }
         }
-        w |= encode_nan15(mids, val) << (4 * k);
     }
-    *reinterpret_cast<uint32_t *>(codes + (base >> 1)) = w;
+    store_u32(reinterpret_cast<uint32_t *>(codes + (base >> 1)), encode8_plain(lds, kind, xs));
+}
+
+// The same when C is a multiple of 8: a lane's 8 values lie in one row, the grid is
+// (column chunks, rows) and no index division is needed.  Workgroup (0,0) also writes the
+// pad codes past the tensor.
+constexpr int kR1Cols = kQThreads * kQElts;  // columns per workgroup
+
+__global__ __launch_bounds__(kQThreads) void quant_rank1_rows_kernel(const float *__restrict__ x, int64_t R,
+                                                                     int64_t C, const float *__restrict__ rowmax,
+                                                                     const float *__restrict__ colmax,
+                                                                     const float *__restrict__ qmap,
+                                                                     uint8_t *__restrict__ codes, int64_t n_padded)
+{
+    __shared__ __align__(16) uint32_t lds[kLdsBytes / 4];
+    lds_fill(lds, qmap, nullptr);
+    const int kind = classify_map(qmap);
+    __syncthreads();
+    const int64_t n = R * C;
+    if (blockIdx.x == 0 && blockIdx.y == 0) {
+        const float z[kQElts] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+        const uint32_t wz = encode8_plain(lds, kind, z);
+        for (int64_t i = n + (int64_t)threadIdx.x * kQElts; i < n_padded; i += kR1Cols)
+            *reinterpret_cast<uint32_t *>(codes + (i >> 1)) = wz;
+        if (threadIdx.x == 0)
+            codes[n_padded / 2] = 0;
+    }
+    const int64_t r = blockIdx.y;
+    const int64_t c = (int64_t)blockIdx.x * kR1Cols + (int64_t)threadIdx.x * kQElts;
+    if (c >= C)
+        return;
+    const float rm = rowmax[r];
+    const float4 a = load4(x + r * C + c), b = load4(x + r * C + c + 4);
+    const float4 ca = *reinterpret_cast<const float4 *>(colmax + c), cb = *reinterpret_cast<const float4 *>(colmax + c + 4);
+    const float v[kQElts] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+    const float cmx[kQElts] = {ca.x, ca.y, ca.z, ca.w, cb.x, cb.y, cb.z, cb.w};
+    float xs[kQElts];
+#pragma unroll
+    for (int k = 0; k < kQElts; ++k) {
+        const float st = (cmx[k] < rm) ? cmx[k] : rm;
+        xs[k] = v[k] / st;
+    }
+    store_u32(reinterpret_cast<uint32_t *>(codes + ((r * C + c) >> 1)), encode8_plain(lds, kind, xs));
 }
 
 __global__ __launch_bounds__(kQThreads) void dequant_rank1_kernel(const uint8_t *__restrict__ codes,
@@ -274,14 +350,14 @@ __global__ __launch_bounds__(kQThreads) void dequant_rank1_kernel(const uint8_t 
                                                                   const float *__restrict__ qmap, int64_t n,
                                                                   int64_t C, float *__restrict__ out, bool vec)
 {
-    __shared__ float s_q[16];
+    __shared__ __align__(16) uint32_t lds[32];
     if (threadIdx.x < 16)
-        s_q[threadIdx.x] = qmap[threadIdx.x];
+        lds[threadIdx.x] = __float_as_uint(qmap[threadIdx.x]);
     __syncthreads();
     const int64_t base = ((int64_t)blockIdx.x * kQThreads + threadIdx.x) * kQElts;
     if (base >= n)
         return;
-    const uint32_t w = load_codes8(codes, base, n, vec);
+    const Nibbles nb = split_nibbles(load_codes8(codes, base, n, vec));
     int64_t r = base / C;
     int64_t c = base - r * C;
     float rm = rowmax[r];
@@ -292,7 +368,7 @@ __global__ __launch_bounds__(kQThreads) void dequant_rank1_kernel(const uint8_t 
         if (base + k < n) {
             const float cmx = colmax[c];
             const float st = (cmx < rm) ? cmx : rm;
-            v[k] = s_q[(w >> (4 * k)) & 0xF] * st;
+            v[k] = decode_nibble(lds, kLdsQ0, nb, k) * st;
             if (++c == C) {
                 c = 0;
                 ++r;
@@ -301,6 +377,33 @@ __global__ __launch_bounds__(kQThreads) void dequant_rank1_kernel(const uint8_t 
         }
     }
     store8(out, base, n, vec, v);
+}
+
+__global__ __launch_bounds__(kQThreads) void dequant_rank1_rows_kernel(const uint8_t *__restrict__ codes,
+                                                                       const float *__restrict__ rowmax,
+                                                                       const float *__restrict__ colmax,
+                                                                       const float *__restrict__ qmap, int64_t C,
+                                                                       float *__restrict__ out)
+{
+    __shared__ __align__(16) uint32_t lds[32];
+    if (threadIdx.x < 16)
+        lds[threadIdx.x] = __float_as_uint(qmap[threadIdx.x]);
+    __syncthreads();
+    const int64_t r = blockIdx.y;
+    const int64_t c = (int64_t)blockIdx.x * kR1Cols + (int64_t)threadIdx.x * kQElts;
+    if (c >= C)
+        return;
+    const float rm = rowmax[r];
+    const Nibbles nb = split_nibbles(load_u32(reinterpret_cast<const uint32_t *>(codes + ((r * C + c) >> 1))));
+    const float4 ca = *reinterpret_cast<const float4 *>(colmax + c), cb = *reinterpret_cast<const float4 *>(colmax + c + 4);
+    const float cmx[kQElts] = {ca.x, ca.y, ca.z, ca.w, cb.x, cb.y, cb.z, cb.w};
+    float v[kQElts];
+#pragma unroll
+    for (int k = 0; k < kQElts; ++k)
+        v[k] = decode_nibble(lds, kLdsQ0, nb, k) * ((cmx[k] < rm) ? cmx[k] : rm);
+    float *o = out + r * C + c;
+    store4(o, make_float4(v[0], v[1], v[2], v[3]));
+    store4(o + 4, make_float4(v[4], v[5], v[6], v[7]));
 }
 
 inline bool tiles_ok(int64_t n, int64_t tile, uint32_t *tiles)
@@ -427,6 +530,12 @@ extern "C" int lpmm_rank1_stats(const float *x, int64_t rows, int64_t cols, floa
     return launch_status();
 }
 
+// row-wise kernels: columns a multiple of 8, 16-byte aligned operands, rows fit grid.y
+static bool rank1_rows_ok(const void *x, const void *colmax, const void *codes, int64_t rows, int64_t cols)
+{
+    return (cols % 8) == 0 && rows <= 65535 && aligned_to(x, 16) && aligned_to(colmax, 16) && aligned_to(codes, 4);
+}
+
 extern "C" int lpmm_quant_rank1(const float *x, int64_t rows, int64_t cols, const float *rowmax,
                                 const float *colmax, const float *qmap, uint8_t *codes, void *stream)
 {
@@ -446,8 +555,15 @@ extern "C" int lpmm_quant_rank1(const float *x, int64_t rows, int64_t cols, cons
     uint32_t tiles;
     if (!tiles_ok(n, kQTile, &tiles))
         return LPMM_ERR_SIZE;
-    hipLaunchKernelGGL(quant_rank1_kernel, dim3(tiles), dim3(kQThreads), 0, (hipStream_t)stream, x, n, cols,
-                       rowmax, colmax, qmap, codes, (int64_t)tiles * kQTile, aligned_to(x, 16));
+    const int64_t n_padded = (int64_t)tiles * kQTile;
+    if (rank1_rows_ok(x, colmax, codes, rows, cols)) {
+        const uint32_t gx = (uint32_t)((cols + kR1Cols - 1) / kR1Cols);
+        hipLaunchKernelGGL(quant_rank1_rows_kernel, dim3(gx, (uint32_t)rows), dim3(kQThreads), 0,
+                           (hipStream_t)stream, x, rows, cols, rowmax, colmax, qmap, codes, n_padded);
+    } else {
+        hipLaunchKernelGGL(quant_rank1_kernel, dim3(tiles), dim3(kQThreads), 0, (hipStream_t)stream, x, n, cols,
+                           rowmax, colmax, qmap, codes, n_padded, aligned_to(x, 16));
+    }
     return launch_status();
 }
 
@@ -469,8 +585,14 @@ extern "C" int lpmm_dequant_rank1(const uint8_t *codes, const float *rowmax, con
     uint32_t tiles;
     if (!tiles_ok(n, kQTile, &tiles))
         return LPMM_ERR_SIZE;
-    const bool vec = aligned_to(out, 16) && aligned_to(codes, 4);
-    hipLaunchKernelGGL(dequant_rank1_kernel, dim3(tiles), dim3(kQThreads), 0, (hipStream_t)stream, codes,
-                       rowmax, colmax, qmap, n, cols, out, vec);
+    if (rank1_rows_ok(out, colmax, codes, rows, cols)) {
+        const uint32_t gx = (uint32_t)((cols + kR1Cols - 1) / kR1Cols);
+        hipLaunchKernelGGL(dequant_rank1_rows_kernel, dim3(gx, (uint32_t)rows), dim3(kQThreads), 0,
+                           (hipStream_t)stream, codes, rowmax, colmax, qmap, cols, out);
+    } else {
+        const bool vec = aligned_to(out, 16) && aligned_to(codes, 4);
+        hipLaunchKernelGGL(dequant_rank1_kernel, dim3(tiles), dim3(kQThreads), 0, (hipStream_t)stream, codes,
+                           rowmax, colmax, qmap, n, cols, out, vec);
+    }
     return launch_status();
 }
