@@ -106,13 +106,20 @@ __global__ __launch_bounds__(kFThreads) void factored_partial_kernel(const float
     double cs[4] = {0.0, 0.0, 0.0, 0.0};
     for (int64_t rb = r0; rb < r1; rb += kSUnroll) {
         float u[kSUnroll][4];
+        if (lane_vec && rb + kSUnroll <= r1) {
+            // straight-line: all loads of the batch are in flight before the first use
+            float4 t[kSUnroll];
 #pragma unroll
-        for (int j = 0; j < kSUnroll; ++j) {
-            const int64_t r = rb + j;
-            if (r < r1 && lane_vec) {
-                const float4 t = load4(g + r * C + c0);
-                u[j][0] = t.x * t.x; u[j][1] = t.y * t.y; u[j][2] = t.z * t.z; u[j][3] = t.w * t.w;
-            } else {
+            for (int j = 0; j < kSUnroll; ++j)
+                t[j] = load4(g + (rb + j) * C + c0);
+#pragma unroll
+            for (int j = 0; j < kSUnroll; ++j) {
+                u[j][0] = t[j].x * t[j].x; u[j][1] = t[j].y * t[j].y; u[j][2] = t[j].z * t[j].z; u[j][3] = t[j].w * t[j].w;
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < kSUnroll; ++j) {
+                const int64_t r = rb + j;
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
                     const float t = (r < r1 && c0 + k < C) ? g[r * C + c0 + k] : 0.0f;

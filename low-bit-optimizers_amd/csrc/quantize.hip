@@ -235,13 +235,20 @@ __global__ __launch_bounds__(kQThreads) void rank1_stats_kernel(const float *__r
     float cm[4] = {0.0f, 0.0f, 0.0f, 0.0f};
     for (int64_t rb = r0; rb < r1; rb += kStatUnroll) {
         float a[kStatUnroll][4];
+        if (lane_vec && rb + kStatUnroll <= r1) {
+            // straight-line: all loads of the batch are in flight before the first use
+            float4 t[kStatUnroll];
 #pragma unroll
-        for (int u = 0; u < kStatUnroll; ++u) {
-            const int64_t r = rb + u;
-            if (r < r1 && lane_vec) {
-                const float4 t = load4(x + r * C + c0);
-                a[u][0] = fabsf(t.x); a[u][1] = fabsf(t.y); a[u][2] = fabsf(t.z); a[u][3] = fabsf(t.w);
-            } else {
+            for (int u = 0; u < kStatUnroll; ++u)
+                t[u] = load4(x + (rb + u) * C + c0);
+#pragma unroll
+            for (int u = 0; u < kStatUnroll; ++u) {
+                a[u][0] = fabsf(t[u].x); a[u][1] = fabsf(t[u].y); a[u][2] = fabsf(t[u].z); a[u][3] = fabsf(t[u].w);
+            }
+        } else {
+#pragma unroll
+            for (int u = 0; u < kStatUnroll; ++u) {
+                const int64_t r = rb + u;
 #pragma unroll
                 for (int k = 0; k < 4; ++k)
                     a[u][k] = (r < r1 && c0 + k < C) ? fabsf(x[r * C + c0 + k]) : 0.0f;

@@ -1,0 +1,124 @@
+"""Parity at the benchmark configurations' real tensor sizes: every distinct LLaMA-7B shape
+through the fused step, 2^26 values through the stand-alone quantisers, a 4096 x 11008
+tensor through the factored step -- each compared with the CPU oracle on seeded inputs, plus
+size-independent properties (quantise -> dequantise -> quantise is idempotent; the largest
+element of every group decodes to its scale)."""
+import numpy as np
+import pytest
+import torch
+
+from util import assert_codes, assert_rel, nibbles, to_dev, to_np
+
+pytestmark = pytest.mark.gpu
+
+HO = (0.9, 0.999, 1e-3, 0.01, 1e-8)
+
+
+def _student_t(rng, n):
+    z = rng.standard_normal((4, n), dtype=np.float32)
+    return (z[0] / np.sqrt((z[1] ** 2 + z[2] ** 2 + z[3] ** 2) / 3.0) * 1e-3).astype(np.float32)
+
+
+@pytest.mark.parametrize("shape", [(32000, 4096), (4096, 4096), (11008, 4096), (4096, 11008)])
+def test_fused_step_llama_shapes(oracle, qmaps, shape):
+    from lpmm import _native
+
+    lib = _native.lib()
+    qm, qv = qmaps
+    n = shape[0] * shape[1]
+    rng = np.random.default_rng(shape[0] + 3 * shape[1])
+    p_ref = (rng.standard_normal(n, dtype=np.float32) * 0.02).astype(np.float32)
+    mc_ref, vc_ref = np.zeros(n // 2, np.uint8), np.zeros(n // 2, np.uint8)
+    ms_ref, vs_ref = np.zeros(n // 128, np.float32), np.zeros(n // 128, np.float32)
+    p, mc, vc, ms, vs = (to_dev(a) for a in (p_ref, mc_ref, vc_ref, ms_ref, vs_ref))
+    dqm, dqv = to_dev(qm), to_dev(qv)
+    for step in (1, 2, 3):
+        g_np = _student_t(rng, n)
+        g = to_dev(g_np)
+        st = lib.lpmm_adamw4bit_step(p.data_ptr(), g.data_ptr(), mc.data_ptr(), vc.data_ptr(), ms.data_ptr(),
+                                     vs.data_ptr(), dqm.data_ptr(), dqv.data_ptr(), n, *HO, float(step),
+                                     torch.cuda.current_stream().cuda_stream)
+        assert st == 0
+        p_before = p_ref.copy()
+        oracle.adamw4bit_step(p_ref, g_np, mc_ref, vc_ref, ms_ref, vs_ref, qm, qv, *HO, float(step))
+        torch.cuda.synchronize()
+        flips = assert_codes(to_np(mc), mc_ref, n, f"m codes step {step}")
+        flips += assert_codes(to_np(vc), vc_ref, n, f"v codes step {step}")
+        assert_rel(to_np(ms), ms_ref, "m scales")
+        assert_rel(to_np(vs), vs_ref, "v scales")
+        assert_rel(to_np(p), p_ref, "p", scale=p_before)
+        if flips:
+            for d, h in ((mc, mc_ref), (vc, vc_ref), (ms, ms_ref), (vs, vs_ref), (p, p_ref)):
+                d.copy_(torch.from_numpy(h))
+    # property: the group maximum decodes to the scale (code 15 on the v map)
+    cv = nibbles(to_np(vc), n).reshape(-1, 128)
+    assert np.all(cv.max(axis=1) == 15)
+
+
+def test_quant_roundtrip_64m(oracle, qmaps):
+    import lpmm.functional as F
+
+    n = 1 << 26
+    rng = np.random.default_rng(1)
+    signed = rng.standard_normal(n, dtype=np.float32)
+    signed[rng.permutation(n)[: n // 1000]] *= 50.0
+    unsigned = (rng.standard_normal(n, dtype=np.float32) ** 2).astype(np.float32)
+    qm, qv = to_dev(qmaps[0]), to_dev(qmaps[1])
+    md_m = dict(b=4, scale_type="group", quant_type="nonlinear", round_type="real-nearest", gp_sz=128, signed=True)
+    md_vg = dict(b=4, scale_type="group", quant_type="power-1", round_type="real-nearest", gp_sz=128, signed=False)
+    md_vr = dict(md_vg, scale_type="rank1")
+    for name, x, dq, hq, md in (("signed", signed, qm, qmaps[0], md_m), ("unsigned", unsigned, qv, qmaps[1], md_vg)):
+        dx = to_dev(x)
+        qx, gen = F.vectorwise_quant(dx, qmap=dq, shape=dx.shape, **md)
+        want_codes, want_max1 = oracle.quant_group(x, hq, 128)
+        np.testing.assert_array_equal(to_np(gen["max1"]).reshape(-1), want_max1)
+        np.testing.assert_array_equal(to_np(qx).view(np.uint8), want_codes)
+        back = F.vectorwise_dequant(qx, qmap=dq, shape=dx.shape, **{**gen, **md})
+        want_back = oracle.dequant_group(want_codes, want_max1, hq, n)
+        np.testing.assert_array_equal(to_np(back), want_back)
+        # round-trip error equals the oracle's (lpmm/utils.py:84-87 formula)
+        rel = np.linalg.norm(x.astype(np.float64) - want_back) / np.linalg.norm(x.astype(np.float64))
+        got = float((dx.double() - back.double()).norm() / dx.double().norm())
+        assert abs(got - rel) <= 1e-9 * rel
+        if name == "unsigned":
+            # idempotence on the unsigned map (its largest element decodes to exactly the scale;
+            # on the signed map a negative maximum decodes to -0.8875 * scale, so the scale shrinks)
+            qx2, gen2 = F.vectorwise_quant(back, qmap=dq, shape=dx.shape, **md)
+            assert torch.equal(gen2["max1"], gen["max1"]) and torch.equal(qx2, qx)
+    # rank-1 on the unsigned data viewed 8192 x 8192
+    x2 = unsigned.reshape(8192, 8192)
+    dx = to_dev(x2)
+    qx, gen = F.vectorwise_quant(dx, qmap=qv, shape=dx.shape, **md_vr)
+    row, col = oracle.rank1_stats(x2)
+    np.testing.assert_array_equal(to_np(gen["max_dims"][0]).reshape(-1), row)
+    np.testing.assert_array_equal(to_np(gen["max_dims"][1]).reshape(-1), col)
+    want_codes = oracle.quant_rank1(x2, row, col, qmaps[1])
+    np.testing.assert_array_equal(to_np(qx).view(np.uint8), want_codes)
+    back = F.vectorwise_dequant(qx, qmap=qv, shape=dx.shape, **{**gen, **md_vr})
+    np.testing.assert_array_equal(to_np(back), oracle.dequant_rank1(want_codes, row, col, qmaps[1], 8192, 8192))
+
+
+def test_factored_step_llama_mlp_shape(oracle, qmaps):
+    import lpmm
+
+    qm, qv = qmaps
+    shape = (4096, 11008)
+    rng = np.random.default_rng(9)
+    host = (rng.standard_normal(shape, dtype=np.float32) * 0.02).astype(np.float32)
+    param = torch.nn.Parameter(to_dev(host))
+    opt = lpmm.optim.AdamW([param], lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01,
+                           factor_second_moment=True, fused=True)
+    state = oracle.NonFusedState(shape, factored=True)
+    for step in range(1, 4):
+        g = (rng.standard_normal(shape, dtype=np.float32) * 1e-3).astype(np.float32)
+        param.grad = to_dev(g)
+        before = host.copy()
+        opt.step()
+        oracle.nonfused_step(host, g, state, qm, qv, 1e-3, 0.9, 0.999, 1e-8, 0.01)
+        torch.cuda.synchronize()
+        s = opt.state[param]
+        assert_rel(to_np(s["exp_avg_sq_row"]), state.row, "row", tol=1e-6)
+        assert_rel(to_np(s["exp_avg_sq_col"]), state.col, "col", tol=1e-6)
+        np.testing.assert_array_equal(to_np(s["exp_avg"]).view(np.uint8), state.m[0])
+        np.testing.assert_array_equal(to_np(s["exp_avg_qstate"]["overhead"]["max1"]).reshape(-1), state.m[1])
+        assert_rel(to_np(param), host, "p", scale=before)
