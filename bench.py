@@ -29,9 +29,9 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 BYTES_PER_PARAM_4BIT = 14.125  # p r/w 8 + g 4 + m codes 1 + v codes 1 + scales 16/128
 BYTES_PER_PARAM_FP32 = 28.0    # p, m, v r/w + g r
 MULTI_MAX = 48                 # tensors per launch record (LPMM_MULTI_MAX)
-# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
-# script (each counter scaled by what it reads for a plain 1 GiB copy, --copy-probe):
-# profiles/fused_adamw4bit_llama7b_pmc.md.  Algorithmic bytes per launch for that workload: 19.035e9.
+# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
+# script (each counter scaled by what it reads for a plain 1 GiB copy, --copy-probe; the summary is
+# kept under profiles/).  Algorithmic bytes per launch for that workload: 19.035e9.
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"llama7b": 19.12e9}
 
 
@@ -220,7 +220,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; --gpus N with N > 1 is not supported "
-                 "(the step is rank-local; see DESIGN.md for how it would shard).")
+                 "(the optimizer step is rank-local: each GPU would run this same kernel on its own shard).")
 
     import torch
 

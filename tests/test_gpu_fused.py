@@ -17,7 +17,7 @@ def _native():
     return _native
 
 
-def _run_fused_steps(oracle, qmaps, n, steps, seed, grad_fn=None, p_scale=0.02, offset=0):
+def _run_fused_steps(oracle, qmaps, n, steps, seed, grad_fn=None, p_scale=0.02, offset=0, exact_p=False):
     """Runs `steps` fused steps on GPU and oracle from zero state; compares after every step."""
     nat = _native()
     lib = nat.lib()
@@ -160,3 +160,26 @@ def test_multi_tensor_matches_single(oracle, qmaps):
         assert_rel(to_np(d["ms"]), h["ms"], "m scale")
         assert_rel(to_np(d["vs"]), h["vs"], "v scale")
         assert_rel(to_np(d["p"]), h["p"], "p")
+
+
+def test_fused_step_extreme_scales(oracle, qmaps):
+    """Group maxima outside [2^-60, 2^60] leave the reciprocal-based division for the plain one;
+    gradients small enough that g*g underflows give all-zero v groups (code 15, scale 0)."""
+    for scale in (1e-12, 1e-22, 1e12, 3e-10):
+        def grad_fn(rng, n, s, scale=scale):
+            g = (rng.standard_normal(n) * scale).astype(np.float32)
+            g[:128] *= 1e-6
+            return g
+
+        _run_fused_steps(oracle, qmaps, 128 * 40 + 30, steps=3, seed=int(abs(np.log10(scale))), grad_fn=grad_fn)
+
+
+def test_fused_step_other_maps(oracle):
+    """Maps other than the two standard ones take the generic search in the same kernel:
+    a signed linear map for m (create_pow_map(4, True, 1)) and a quadratic map for v."""
+    qm = oracle.create_pow_map(4, True, 1)
+    qv = (oracle.qmap_v() ** 2).astype(np.float32)
+    _run_fused_steps(oracle, (qm, qv), 128 * 300 + 64, steps=4, seed=77)
+    # one standard, one not
+    _run_fused_steps(oracle, (oracle.qmap_m(), qv), 128 * 50, steps=3, seed=78)
+    _run_fused_steps(oracle, (qm, oracle.qmap_v()), 128 * 50, steps=3, seed=79)

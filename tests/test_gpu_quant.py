@@ -183,3 +183,41 @@ def test_shim_pack_unpack_signatures(oracle, qmaps):
         ext.pack_nonlinear(to_dev(x).reshape(-1), dq, 4, False)  # wrong dimension
     with pytest.raises(RuntimeError):
         ext.unpack_nonlinear(packed.to(torch.uint8), dq, 4, 3, 2048)  # not int8
+
+
+def test_quant_group_other_map(oracle):
+    """A non-standard map goes through the generic search of the same kernels."""
+    lib = _lib()
+    rng = np.random.default_rng(12)
+    qmap = oracle.create_pow_map(4, True, 1)
+    n = 2048 * 3 + 700
+    x = _signed(rng, n)
+    want_codes, want_max1 = oracle.quant_group(x, qmap, 128)
+    dx, dq = to_dev(x), to_dev(qmap)
+    codes = torch.empty(want_codes.size, dtype=torch.uint8, device="cuda")
+    max1 = torch.empty(want_max1.size, dtype=torch.float32, device="cuda")
+    assert lib.lpmm_quant_group(dx.data_ptr(), n, 128, dq.data_ptr(), codes.data_ptr(), max1.data_ptr(), _stream()) == 0
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(to_np(codes), want_codes)
+    np.testing.assert_array_equal(to_np(max1), want_max1)
+    normed = np.clip(rng.standard_normal(2048) * 0.5, -1.5, 1.5).astype(np.float32)
+    out = torch.empty(1025, dtype=torch.uint8, device="cuda")
+    assert lib.lpmm_pack_nonlinear_4bit(to_dev(normed).data_ptr(), dq.data_ptr(), 2048, out.data_ptr(), _stream()) == 0
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(to_np(out), oracle.pack_nonlinear_4bit(normed, qmap))
+
+
+def test_quant_group_extreme_scales(oracle, qmaps):
+    lib = _lib()
+    rng = np.random.default_rng(13)
+    for scale in (1e-30, 1e-20, 1e20, 1e30):
+        for qmap, x in ((qmaps[0], (rng.standard_normal(4096) * scale).astype(np.float32)),
+                        (qmaps[1], (rng.random(4096) * scale).astype(np.float32))):
+            want_codes, want_max1 = oracle.quant_group(x, qmap, 128)
+            dx, dq = to_dev(x), to_dev(qmap)
+            codes = torch.empty(want_codes.size, dtype=torch.uint8, device="cuda")
+            max1 = torch.empty(want_max1.size, dtype=torch.float32, device="cuda")
+            assert lib.lpmm_quant_group(dx.data_ptr(), 4096, 128, dq.data_ptr(), codes.data_ptr(), max1.data_ptr(), _stream()) == 0
+            torch.cuda.synchronize()
+            np.testing.assert_array_equal(to_np(codes), want_codes)
+            np.testing.assert_array_equal(to_np(max1), want_max1)
