@@ -326,6 +326,77 @@ __global__ __launch_bounds__(kFThreads) void factored_update_kernel(
     }
 }
 
+// The same pass when the column count is a multiple of 128: every 128-element group of the
+// flattened tensor is a 128-column piece of one row, the grid is (column chunks, rows), the
+// 16 lanes of a DPP row own one group in the row layout of the fused step (lane l: columns
+// [4l, 4l+4) and [64+4l, 64+4l+4) of the piece; whole cache lines per store), and no index
+// division is needed.  Workgroup (0,0) also writes the pad codes past the tensor.
+__global__ __launch_bounds__(kFThreads) void factored_update_rows128_kernel(
+    float *__restrict__ p, const float *__restrict__ g, uint8_t *__restrict__ m_codes,
+    float *__restrict__ m_max1, const float *__restrict__ qmap_m, const float *__restrict__ row,
+    const float *__restrict__ col, const float *__restrict__ row_mean_all, int64_t R, int64_t C,
+    int64_t n_padded, NfHyper h, bool first_step)
+{
+    __shared__ __align__(16) uint32_t lds[kLdsBytes / 4];
+    lds_fill(lds, qmap_m, nullptr);
+    const int kind = classify_map(qmap_m);
+    __syncthreads();
+    const int64_t n = R * C;
+    if (blockIdx.x == 0 && blockIdx.y == 0) {
+        const float z[kFElts] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+        const uint32_t wz = kind == kMapStdM ? encode8_std_m(lds, z)
+                                             : encode8_generic(make_mids(reinterpret_cast<const float *>(lds) + kLdsQ0 / 4), z);
+        for (int64_t i = n + (int64_t)threadIdx.x * kFElts; i < n_padded; i += kFTile)
+            *reinterpret_cast<uint32_t *>(m_codes + (i >> 1)) = wz;
+        if (threadIdx.x == 0)
+            m_codes[n_padded / 2] = 0;
+    }
+    const int lane16 = threadIdx.x & 15;
+    const int64_t r = blockIdx.y;
+    const int64_t c0 = (int64_t)blockIdx.x * kFTile + (int64_t)(threadIdx.x >> 4) * kGroup;  // first column of the group
+    if (c0 >= C)
+        return;  // uniform over the 16 lanes of the group
+    const int64_t gbase = r * C + c0;
+    const int64_t grp = gbase / kGroup;
+    float *pp = p + gbase + lane16 * 4;
+    const float *gp = g + gbase + lane16 * 4;
+    const float *cp = col + c0 + lane16 * 4;
+    const float4 a0 = load4(pp), a1 = load4(pp + 64), b0 = load4(gp), b1 = load4(gp + 64);
+    const float4 c_lo = *reinterpret_cast<const float4 *>(cp), c_hi = *reinterpret_cast<const float4 *>(cp + 64);
+    uint16_t *mcp = reinterpret_cast<uint16_t *>(m_codes + (gbase >> 1)) + lane16;
+    uint32_t wm = 0;
+    float sm = 0.0f;
+    if (!first_step) {
+        wm = load_u16(mcp) | (load_u16(mcp + 16) << 16);
+        sm = m_max1[grp];
+    }
+    const Nibbles nm = split_nibbles(wm);
+    const float rf = row[r] / *row_mean_all;
+    float pv[kFElts] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+    const float gv[kFElts] = {b0.x, b0.y, b0.z, b0.w, b1.x, b1.y, b1.z, b1.w};
+    const float cv[kFElts] = {c_lo.x, c_lo.y, c_lo.z, c_lo.w, c_hi.x, c_hi.y, c_hi.z, c_hi.w};
+    float m[kFElts];
+    float amax = 0.0f;
+#pragma unroll
+    for (int k = 0; k < kFElts; ++k) {
+        const float m_old = first_step ? 0.0f : decode_nibble(lds, kLdsQ0, nm, k) * sm;
+        const float pi = pv[k] * h.decay;
+        m[k] = lerp_w(m_old, gv[k], h.w1);
+        const float vi = rf * cv[k];
+        const float denom = div_by_rc(sqrt_fast(vi), h.bc2_sqrt, h.rbc2_sqrt) + h.eps;
+        pv[k] = pi + div_fast(h.neg_step_size * m[k], denom);
+        amax = fmaxf(amax, fabsf(m[k]));
+    }
+    amax = row16_max(amax);
+    const uint32_t om = encode8_scaled(lds, kLdsQ0, kind, m, amax);
+    store4(pp, make_float4(pv[0], pv[1], pv[2], pv[3]));
+    store4(pp + 64, make_float4(pv[4], pv[5], pv[6], pv[7]));
+    store_u16(mcp, om & 0xFFFFu);
+    store_u16(mcp + 16, om >> 16);
+    if (lane16 == 0)
+        m_max1[grp] = amax;
+}
+
 // The same update with an fp32 first moment (tensors at or under the quantisation threshold,
 // or first-moment quantisation disabled): m is read and written as floats.
 __global__ __launch_bounds__(kFThreads) void factored_update_fp32m_kernel(
@@ -460,7 +531,12 @@ extern "C" int lpmm_factored_update(float *p, const float *g, uint8_t *m_codes, 
         return LPMM_ERR_SIZE;
     const bool vec = aligned_to(p, 16) && aligned_to(g, 16);
     const NfHyper h = make_nf_hyper(beta1, beta2, lr, weight_decay, eps, step);
-    if ((cols % 8) == 0 && aligned_to(col, 16))
+    if ((cols % kGroup) == 0 && rows <= 65535 && vec && aligned_to(col, 16) && aligned_to(m_codes, 4)) {
+        const uint32_t gx = (uint32_t)((cols + kFTile - 1) / kFTile);
+        hipLaunchKernelGGL(factored_update_rows128_kernel, dim3(gx, (uint32_t)rows), dim3(kFThreads), 0,
+                           (hipStream_t)stream, p, g, m_codes, m_max1, qmap_m, row, col, row_mean_all, rows, cols,
+                           n_padded, h, first_step != 0);
+    } else if ((cols % 8) == 0 && aligned_to(col, 16))
         hipLaunchKernelGGL(factored_update_kernel<true>, dim3((uint32_t)tiles), dim3(kFThreads), 0,
                            (hipStream_t)stream, p, g, m_codes, m_max1, qmap_m, row, col, row_mean_all, n, cols,
                            n_groups, n_padded, h, first_step != 0, vec);

@@ -200,6 +200,35 @@ __global__ __launch_bounds__(kQThreads) void dequant_group_kernel(const uint8_t 
     store8(out, base, n, vec, v);
 }
 
+// Row layout (as in the fused step): 16 lanes own one 128-value group, lane l owns values
+// [4l, 4l+4) and [64+4l, 64+4l+4), so that every 16-byte store of a row covers whole cache
+// lines.  Handles the groups that lie fully inside the tensor; n must be >= 128.
+__global__ __launch_bounds__(kQThreads) void dequant_group_rows_kernel(const uint8_t *__restrict__ codes,
+                                                                       const float *__restrict__ max1,
+                                                                       const float *__restrict__ qmap,
+                                                                       int64_t full_groups, int rows_per_group,
+                                                                       float *__restrict__ out)
+{
+    __shared__ __align__(16) uint32_t lds[32];
+    if (threadIdx.x < 16)
+        lds[threadIdx.x] = __float_as_uint(qmap[threadIdx.x]);
+    __syncthreads();
+    const int lane16 = threadIdx.x & 15;
+    const int64_t row = (int64_t)blockIdx.x * (kQThreads / 16) + (threadIdx.x >> 4);
+    if (row >= full_groups)
+        return;
+    const uint16_t *cp = reinterpret_cast<const uint16_t *>(codes + row * 64) + lane16;
+    const Nibbles nb = split_nibbles(load_u16(cp) | (load_u16(cp + 16) << 16));
+    const float s = max1[row / rows_per_group];
+    float v[kQElts];
+#pragma unroll
+    for (int k = 0; k < kQElts; ++k)
+        v[k] = decode_nibble(lds, kLdsQ0, nb, k) * s;
+    float *o = out + row * kGroup + lane16 * 4;
+    store4(o, make_float4(v[0], v[1], v[2], v[3]));
+    store4(o + 64, make_float4(v[4], v[5], v[6], v[7]));
+}
+
 // ---------------------------------------------------------------------------------------
 // 'rank1' scaling of a row-major R x C tensor.
 // ---------------------------------------------------------------------------------------
@@ -413,6 +442,40 @@ __global__ __launch_bounds__(kQThreads) void dequant_rank1_rows_kernel(const uin
     store4(o + 4, make_float4(v[4], v[5], v[6], v[7]));
 }
 
+// Row layout variant for column counts that are a multiple of 128: 16 lanes own 128
+// consecutive columns of one row, lane l the columns [4l, 4l+4) and [64+4l, 64+4l+4), so that
+// every 16-byte store covers whole cache lines.
+__global__ __launch_bounds__(kQThreads) void dequant_rank1_rows128_kernel(const uint8_t *__restrict__ codes,
+                                                                          const float *__restrict__ rowmax,
+                                                                          const float *__restrict__ colmax,
+                                                                          const float *__restrict__ qmap, int64_t C,
+                                                                          float *__restrict__ out)
+{
+    __shared__ __align__(16) uint32_t lds[32];
+    if (threadIdx.x < 16)
+        lds[threadIdx.x] = __float_as_uint(qmap[threadIdx.x]);
+    __syncthreads();
+    const int lane16 = threadIdx.x & 15;
+    const int64_t r = blockIdx.y;
+    const int64_t c0 = (int64_t)blockIdx.x * kR1Cols + (int64_t)(threadIdx.x >> 4) * kGroup;
+    if (c0 >= C)
+        return;
+    const int64_t gbase = r * C + c0;
+    const float rm = rowmax[r];
+    const uint16_t *cp = reinterpret_cast<const uint16_t *>(codes + (gbase >> 1)) + lane16;
+    const Nibbles nb = split_nibbles(load_u16(cp) | (load_u16(cp + 16) << 16));
+    const float *cmp = colmax + c0 + lane16 * 4;
+    const float4 ca = *reinterpret_cast<const float4 *>(cmp), cb = *reinterpret_cast<const float4 *>(cmp + 64);
+    const float cmx[kQElts] = {ca.x, ca.y, ca.z, ca.w, cb.x, cb.y, cb.z, cb.w};
+    float v[kQElts];
+#pragma unroll
+    for (int k = 0; k < kQElts; ++k)
+        v[k] = decode_nibble(lds, kLdsQ0, nb, k) * ((cmx[k] < rm) ? cmx[k] : rm);
+    float *o = out + gbase + lane16 * 4;
+    store4(o, make_float4(v[0], v[1], v[2], v[3]));
+    store4(o + 64, make_float4(v[4], v[5], v[6], v[7]));
+}
+
 inline bool tiles_ok(int64_t n, int64_t tile, uint32_t *tiles)
 {
     const int64_t t = (n + tile - 1) / tile;
@@ -509,6 +572,17 @@ extern "C" int lpmm_dequant_group(const uint8_t *codes, const float *max1, const
     if (!tiles_ok(n, kQTile, &tiles))
         return LPMM_ERR_SIZE;
     const bool vec = aligned_to(out, 16) && aligned_to(codes, 4);
+    const int64_t full_groups = n / kGroup;
+    if (vec && full_groups > 0 && full_groups <= 0x7fffffffLL * 16) {
+        // whole 128-value rows in the row layout, the ragged tail (< 128 values) element-wise
+        hipLaunchKernelGGL(dequant_group_rows_kernel, dim3((uint32_t)((full_groups + 15) / 16)), dim3(kQThreads), 0,
+                           (hipStream_t)stream, codes, max1, qmap, full_groups, (int)(gp_sz / kGroup), out);
+        const int64_t done = full_groups * kGroup;
+        if (done < n)
+            hipLaunchKernelGGL(dequant_group_kernel, dim3(1), dim3(kQThreads), 0, (hipStream_t)stream,
+                               codes + done / 2, max1 + done / gp_sz, qmap, n - done, gp_sz, out + done, false);
+        return launch_status();
+    }
     hipLaunchKernelGGL(dequant_group_kernel, dim3(tiles), dim3(kQThreads), 0, (hipStream_t)stream, codes,
                        max1, qmap, n, gp_sz, out, vec);
     return launch_status();
@@ -592,7 +666,11 @@ extern "C" int lpmm_dequant_rank1(const uint8_t *codes, const float *rowmax, con
     uint32_t tiles;
     if (!tiles_ok(n, kQTile, &tiles))
         return LPMM_ERR_SIZE;
-    if (rank1_rows_ok(out, colmax, codes, rows, cols)) {
+    if (rank1_rows_ok(out, colmax, codes, rows, cols) && (cols % kGroup) == 0) {
+        const uint32_t gx = (uint32_t)((cols + kR1Cols - 1) / kR1Cols);
+        hipLaunchKernelGGL(dequant_rank1_rows128_kernel, dim3(gx, (uint32_t)rows), dim3(kQThreads), 0,
+                           (hipStream_t)stream, codes, rowmax, colmax, qmap, cols, out);
+    } else if (rank1_rows_ok(out, colmax, codes, rows, cols)) {
         const uint32_t gx = (uint32_t)((cols + kR1Cols - 1) / kR1Cols);
         hipLaunchKernelGGL(dequant_rank1_rows_kernel, dim3(gx, (uint32_t)rows), dim3(kQThreads), 0,
                            (hipStream_t)stream, codes, rowmax, colmax, qmap, cols, out);
