@@ -34,9 +34,10 @@ __device__ __forceinline__ void store_u32(uint32_t *p, uint32_t v) { __builtin_n
 // Near-exact arithmetic: hardware approximation + one fma correction of the exact residual.
 // ---------------------------------------------------------------------------------------
 
-// sqrt(x) for x >= 0: correctly rounded except for a vanishing fraction of inputs (1 ulp
-// there).  Inputs below the smallest normal are treated as that value (their square root is
-// far below any eps it is added to).
+// sqrt(x) for x >= 0: correctly rounded for x >= 2^-100 (no difference from sqrtf on every
+// 16th float on the device); below that the residual underflows and the result may be 1 ulp
+// off, and inputs below the smallest normal are treated as that value -- the square root of
+// such a second moment is far below any eps it is added to.
 __device__ __forceinline__ float sqrt_fast(float x)
 {
     const float y = __builtin_amdgcn_rsqf(fmaxf(x, 0x1p-126f));
@@ -46,7 +47,7 @@ __device__ __forceinline__ float sqrt_fast(float x)
     return __builtin_fmaf(r, h, s);
 }
 
-// x / d (same remark).
+// x / d: no difference from the correctly rounded quotient on 2^30 random pairs on the device.
 __device__ __forceinline__ float div_fast(float x, float d)
 {
     const float rc = __builtin_amdgcn_rcpf(d);

@@ -37,6 +37,7 @@ PROTOTYPES = {
     "lpmm_factored_stats": (_int, [_vp, _i64, _i64, _vp, _vp, _vp, _d, _vp, _vp]),
     "lpmm_factored_update": (_int, [_vp] * 8 + [_i64, _i64] + [_d] * 6 + [_int, _vp]),
     "lpmm_factored_update_fp32m": (_int, [_vp] * 6 + [_i64, _i64] + [_d] * 6 + [_vp]),
+    "lpmm_selftest_arithmetic": (_int, [_vp, ctypes.c_uint32, ctypes.c_uint64, ctypes.c_uint32, _vp]),
 }
 
 # numpy mirrors of the multi-tensor records (lpmm_adamw4bit_tensor / lpmm_adamw_fp32_tensor)
