@@ -125,6 +125,19 @@ def test_optimizer_argument_validation():
     assert md == dict(b=4, scale_type="group", quant_type="power-1", round_type="real-nearest", gp_sz=128, signed=False)
 
 
+def test_sgd_argument_validation():
+    import lpmm
+
+    p = [torch.nn.Parameter(torch.zeros(4))]
+    for kw in (dict(lr=-1.0), dict(lr=0.1, momentum=-0.5), dict(lr=0.1, weight_decay=-1.0), dict(lr=0.1, fused=True)):
+        with pytest.raises(ValueError):
+            lpmm.optim.SGD(p, **kw)
+    opt = lpmm.optim.SGD(p, lr=0.1, momentum=0.9)
+    assert opt.get_qmetadata_by_state_name("momentum_buffer")["quant_type"] == "nonlinear"
+    with pytest.raises(ValueError):
+        opt.get_subqconfig("exp_avg")
+
+
 def test_state_init_threshold_and_override():
     """State layout on first use (lpmm/optim/adamw.py:114-129) and the numel > 4096 rule
     (lpmm/optim/optimizer.py:156-163); needs no GPU because only the bookkeeping runs."""
