@@ -163,6 +163,24 @@ int lpmm_nonfused_update(float *p, const float *g, float *m, float *v, int64_t n
                          double beta2, double lr, double weight_decay, double eps, double step,
                          void *stream);
 
+/* The whole non-fused step on 4-bit states in one pass, for the configuration the reference
+ * uses by default when fused=False is combined with block-wise second-moment scaling (both
+ * moments 4-bit, 'group' scaling, gp_sz 128, real-nearest): dequantise m and v, the update
+ * above, re-quantise, for a list of tensors in one launch per LPMM_MULTI_MAX tensors.
+ * Replaces the body of _single_tensor_adamw4bit for such tensors
+ *   (lpmm/optim/adamw.py:394-436: vectorwise_dequant x2, the op sequence, vectorwise_quant x2).
+ * Records are lpmm_adamw4bit_tensor with the non-fused state layout:
+ *   m_codes, v_codes: ceil(n/2048)*1024 + 1 bytes each (lpmm/functional.py:503-509), written
+ *                     in full by every call, padding included;
+ *   m_scale, v_scale: the (ceil(n/128), 1) "max1" tensors.
+ * Before the first step the scales must be zero and the codes those of 0.0 (0x77 bytes for
+ * the standard first-moment map, 0x00 for the second): that state decodes to the all-zero
+ * moments the reference starts from. */
+int lpmm_nonfused_adamw4bit_step_multi(const lpmm_adamw4bit_tensor *tensors, int64_t count,
+                                       const float *qmap_m, const float *qmap_v, double beta1,
+                                       double beta2, double lr, double weight_decay, double eps,
+                                       void *stream);
+
 /* ---------------------------------------------------------------------------------------
  * (c) Factored second moment on a row-major R x C tensor.
  * Replaces _single_quantized_factored_update (lpmm/optim/adamw.py:579-627) and

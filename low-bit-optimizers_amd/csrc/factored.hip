@@ -8,52 +8,13 @@
 // the hardware approximations with one fma correction of the residual (correctly rounded
 // except for a vanishing fraction of inputs; the parameter never feeds back into a state).
 // Row/column means of g*g are summed in double in a fixed order and rounded once.
-#include "lpmm_codec.hpp"
-
-#include <math.h>
+#include "lpmm_update.hpp"
 
 namespace lpmm {
 
 constexpr int kFThreads = 256;
 constexpr int kFElts = 8;
 constexpr int kFTile = kFThreads * kFElts;  // 2048
-
-struct NfHyper {
-    float decay, w1, b2, w2, neg_step_size, bc2_sqrt, rbc2_sqrt, eps;  // rbc2_sqrt = 1 / bc2_sqrt, correctly rounded
-};
-
-inline NfHyper make_nf_hyper(double beta1, double beta2, double lr, double wd, double eps, double step)
-{
-    NfHyper h;
-    h.decay = (float)(1.0 - lr * wd);
-    h.w1 = (float)(1.0 - beta1);
-    h.b2 = (float)beta2;
-    h.w2 = (float)(1.0 - beta2);
-    const double bc1 = 1.0 - pow(beta1, step);
-    const double bc2 = 1.0 - pow(beta2, step);
-    h.neg_step_size = (float)(-(lr / bc1));
-    h.bc2_sqrt = (float)sqrt(bc2);
-    h.rbc2_sqrt = 1.0f / h.bc2_sqrt;
-    h.eps = (float)eps;
-    return h;
-}
-
-__device__ __forceinline__ float lerp_w(float a, float b, float w)
-{
-    return (fabsf(w) < 0.5f) ? __builtin_fmaf(w, b - a, a) : __builtin_fmaf(w - 1.0f, b - a, b);
-}
-
-// One lane: 4 consecutive elements per iteration (16-byte accesses), grid-stride.
-__device__ __forceinline__ void nonfused_elt(float &p, float g, float &m, float &v, const NfHyper &h)
-{
-    const float pi = p * h.decay;
-    m = lerp_w(m, g, h.w1);
-    float vi = v * h.b2;
-    vi = vi + (h.w2 * g) * g;
-    v = vi;
-    const float denom = div_by_rc(sqrt_fast(vi), h.bc2_sqrt, h.rbc2_sqrt) + h.eps;
-    p = pi + div_fast(h.neg_step_size * m, denom);
-}
 
 __global__ __launch_bounds__(kFThreads) void nonfused_update_kernel(float *__restrict__ p,
                                                                     const float *__restrict__ g,

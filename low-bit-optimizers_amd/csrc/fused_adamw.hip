@@ -18,7 +18,7 @@
 // use the correctly rounded reciprocal plus one fma correction step; both give the same
 // results as the generic search and the plain division, which remain as the fallback for
 // any other map.
-#include "lpmm_codec.hpp"
+#include "lpmm_update.hpp"
 
 #include <math.h>
 
@@ -46,39 +46,52 @@ struct Multi4 {
     Tensor4 t[LPMM_MULTI_MAX];
     uint32_t tile_start[LPMM_MULTI_MAX + 1];  // prefix sum of tiles per tensor
     int count;
-    float beta1, beta2, omb1, omb2, lr, wd, eps;  // omb = 1 - beta, subtracted in float on the host
+    float s[7];  // scalars shared by all tensors, in the order the arithmetic below reads them
+};
+
+// The two arithmetics the kernel is instantiated with.  Both read the shared scalars from
+// Multi4::s and three per-tensor ones from Tensor4::{c1, c2s, rc2s}.
+struct FusedArith {
+    // code buffers hold exactly ceil(n/2) bytes; a last odd element leaves its high nibble 0
+    static constexpr bool kPadded = false;
+    Hyper h;
+    __device__ __forceinline__ FusedArith(const Multi4 &a, const Tensor4 &t)
+    {
+        h.beta1 = a.s[0];
+        h.beta2 = a.s[1];
+        h.omb1 = a.s[2];
+        h.omb2 = a.s[3];
+        h.lr = a.s[4];
+        h.wd = a.s[5];
+        h.eps = a.s[6];
+        h.c1 = t.c1;
+        h.c2s = t.c2s;
+        h.rc2s = t.rc2s;
+    }
+    __device__ __forceinline__ void elt(float &p, float g, float &m, float &v) const { p = adamw_elt(p, g, m, v, h); }
+};
+
+struct NonFusedArith {
+    // code buffers are padded to whole tiles plus one byte, as the reference's packing
+    // operator lays them out: every nibble of an existing group is written, groups past the
+    // tensor hold the code of 0.0
+    static constexpr bool kPadded = true;
+    NfHyper h;
+    __device__ __forceinline__ NonFusedArith(const Multi4 &a, const Tensor4 &t)
+    {
+        h.decay = a.s[0];
+        h.w1 = a.s[1];
+        h.b2 = a.s[2];
+        h.w2 = a.s[3];
+        h.eps = a.s[4];
+        h.neg_step_size = t.c1;
+        h.bc2_sqrt = t.c2s;
+        h.rbc2_sqrt = t.rc2s;
+    }
+    __device__ __forceinline__ void elt(float &p, float g, float &m, float &v) const { nonfused_elt(p, g, m, v, h); }
 };
 
 static_assert(sizeof(Multi4) + 2 * sizeof(void *) <= 4096, "kernel arguments exceed 4 KB");
-
-struct Hyper {
-    float beta1, beta2, omb1, omb2, lr, wd, eps, c1, c2s, rc2s;
-};
-
-#ifndef LPMM_P_MODE
-#define LPMM_P_MODE 1  // 0: IEEE sqrt/div, 1: approximation + residual correction, 2: approximation only
-#endif
-
-// AdamW on one element; returns the new parameter, updates m and v in place.
-__device__ __forceinline__ float adamw_elt(float p, float g, float &m, float &v, const Hyper &h)
-{
-    m = h.beta1 * m + h.omb1 * g;
-    v = h.beta2 * v + h.omb2 * g * g;
-#if LPMM_P_MODE == 0
-    const float denom = (sqrtf(v) / h.c2s + h.eps) * h.c1;
-    const float update = (m / denom) + (h.wd * p);
-#elif LPMM_P_MODE == 1
-    const float s = sqrt_fast(v);
-    const float q = s * h.rc2s;
-    const float sq = __builtin_fmaf(__builtin_fmaf(-q, h.c2s, s), h.rc2s, q);
-    const float denom = (sq + h.eps) * h.c1;
-    const float update = div_fast(m, denom) + (h.wd * p);
-#else
-    const float denom = (__builtin_amdgcn_sqrtf(v) * h.rc2s + h.eps) * h.c1;
-    const float update = m * __builtin_amdgcn_rcpf(denom) + (h.wd * p);
-#endif
-    return p - (h.lr * update);
-}
 
 // element k (0..7) of a lane sits at this offset inside the lane's group
 __device__ __forceinline__ int elt_offset(int lane16, int k) { return lane16 * 4 + (k & 3) + (k >> 2) * 64; }
@@ -86,8 +99,8 @@ __device__ __forceinline__ int elt_offset(int lane16, int k) { return lane16 * 4
 // One 128-element group, handled by the 16 lanes of a DPP row.  FULL: the whole group lies
 // inside the tensor and the pointers allow vector access; otherwise every access is
 // guarded per element.  All 16 lanes take the same instantiation.
-template <bool FULL>
-__device__ __forceinline__ void group_step(const Tensor4 &t, const Hyper &h, const uint32_t *lds,
+template <bool FULL, class Arith>
+__device__ __forceinline__ void group_step(const Tensor4 &t, const Arith &h, const uint32_t *lds,
                                            bool std_maps, int64_t grp, int lane16)
 {
     const int64_t n = t.n;
@@ -95,7 +108,8 @@ __device__ __forceinline__ void group_step(const Tensor4 &t, const Hyper &h, con
     float pv[kEltsPerLane], gv[kEltsPerLane], m[kEltsPerLane], v[kEltsPerLane];
     uint32_t wm = 0, wv = 0;  // 8 nibbles each: elements 0..3 in the low half-word, 4..7 in the high
     float sm = 0.0f, sv = 0.0f;
-    const bool any = FULL || (gbase + lane16 * 4 < n);  // the lane's first element exists
+    // does the lane store anything: its first element exists, or the buffers are padded
+    const bool any = FULL || Arith::kPadded || (gbase + lane16 * 4 < n);
 
     if (FULL) {
         const float *pp = t.p + gbase + lane16 * 4;
@@ -138,7 +152,7 @@ __device__ __forceinline__ void group_step(const Tensor4 &t, const Hyper &h, con
         m[k] = decode_nibble(lds, kLdsQ0, nm, k) * sm;
         v[k] = decode_nibble(lds, kLdsQ1, nv, k) * sv;
         if (FULL || (gbase + elt_offset(lane16, k) < n)) {
-            pv[k] = adamw_elt(pv[k], gv[k], m[k], v[k], h);
+            h.elt(pv[k], gv[k], m[k], v[k]);
             amax_m = fmaxf(amax_m, fabsf(m[k]));
             amax_v = fmaxf(amax_v, v[k]);
         } else {
@@ -175,9 +189,9 @@ __device__ __forceinline__ void group_step(const Tensor4 &t, const Hyper &h, con
 #pragma unroll
         for (int k = 0; k < kEltsPerLane; k += 2) {
             const int64_t i = gbase + elt_offset(lane16, k);
-            if (i < n) {
-                // a last odd element leaves the high nibble of its byte 0
-                const uint32_t keep = (i + 1 < n) ? 0xFFu : 0x0Fu;
+            if (Arith::kPadded || i < n) {
+                // unpadded buffers: a last odd element leaves the high nibble of its byte 0
+                const uint32_t keep = (Arith::kPadded || i + 1 < n) ? 0xFFu : 0x0Fu;
                 t.mc[i >> 1] = (uint8_t)((cm >> (4 * k)) & keep);
                 t.vc[i >> 1] = (uint8_t)((cv >> (4 * k)) & keep);
             }
@@ -189,7 +203,7 @@ __device__ __forceinline__ void group_step(const Tensor4 &t, const Hyper &h, con
     }
 }
 
-template <bool ALIGNED>
+template <bool ALIGNED, class Arith>
 __global__ __launch_bounds__(kThreads) void adamw4bit_kernel(const Multi4 args,
                                                              const float *__restrict__ qmap_m,
                                                              const float *__restrict__ qmap_v)
@@ -209,19 +223,25 @@ __global__ __launch_bounds__(kThreads) void adamw4bit_kernel(const Multi4 args,
     const int lane16 = threadIdx.x & 15;
     const int64_t grp = (int64_t)(blockIdx.x - args.tile_start[lo]) * (kTile / kGroup) + (threadIdx.x >> 4);
 
-    Hyper h;
-    h.beta1 = args.beta1;
-    h.beta2 = args.beta2;
-    h.omb1 = args.omb1;
-    h.omb2 = args.omb2;
-    h.lr = args.lr;
-    h.wd = args.wd;
-    h.eps = args.eps;
-    h.c1 = t.c1;
-    h.c2s = t.c2s;
-    h.rc2s = t.rc2s;
+    const Arith h(args, t);
     __syncthreads();
 
+    if (Arith::kPadded && threadIdx.x == 0 && blockIdx.x + 1 == args.tile_start[lo + 1]) {
+        // the tensor's last tile also owns the extra byte at the end of each code buffer
+        const int64_t end = (int64_t)(args.tile_start[lo + 1] - args.tile_start[lo]) * (kTile / 2);
+        t.mc[end] = 0;
+        t.vc[end] = 0;
+    }
+    if (Arith::kPadded && grp * kGroup >= t.n) {
+        // a group the padding to whole tiles added: codes of 0.0 (m: 7, v: 0)
+        const int64_t b = (grp * kGroup >> 1) + lane16 * 4;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            t.mc[b + k] = 0x77;
+            t.vc[b + k] = 0;
+        }
+        return;
+    }
     if (ALIGNED && (grp + 1) * kGroup <= t.n)
         group_step<true>(t, h, lds, std_maps, grp, lane16);
     else
@@ -286,22 +306,15 @@ __global__ __launch_bounds__(kThreads) void adamw_fp32_kernel(const MultiF args)
     }
 }
 
-// bias corrections exactly as the reference computes them per thread
-// (fused_adamw_kernel.cu:103-104), done once on the host
-inline void bias_corrections(float beta1, float beta2, float step, float *c1, float *c2s)
-{
-    *c1 = 1.0f - powf(beta1, step);
-    *c2s = sqrtf(1.0f - powf(beta2, step));
-}
-
 }  // namespace lpmm
 
 using namespace lpmm;
 
-extern "C" int lpmm_adamw4bit_step_multi(const lpmm_adamw4bit_tensor *tensors, int64_t count,
-                                         const float *qmap_m, const float *qmap_v, float beta1,
-                                         float beta2, float lr, float weight_decay, float eps,
-                                         void *stream)
+// Validation, batching into launches of at most LPMM_MULTI_MAX tensors, and launch, shared
+// by the two arithmetics.  per_tensor(step, &c1, &c2s, &rc2s) fills the per-tensor scalars.
+template <class Arith, class PerTensor>
+static int step_multi4(const lpmm_adamw4bit_tensor *tensors, int64_t count, const float *qmap_m,
+                       const float *qmap_v, const float (&scalars)[7], PerTensor per_tensor, void *stream)
 {
     if (count < 0)
         return LPMM_ERR_SIZE;
@@ -336,13 +349,8 @@ extern "C" int lpmm_adamw4bit_step_multi(const lpmm_adamw4bit_tensor *tensors, i
     }
 
     Multi4 args;
-    args.beta1 = beta1;
-    args.beta2 = beta2;
-    args.omb1 = 1 - beta1;
-    args.omb2 = 1 - beta2;
-    args.lr = lr;
-    args.wd = weight_decay;
-    args.eps = eps;
+    for (int j = 0; j < 7; ++j)
+        args.s[j] = scalars[j];
     int64_t i = 0;
     while (i < count) {
         int k = 0;
@@ -365,8 +373,7 @@ extern "C" int lpmm_adamw4bit_step_multi(const lpmm_adamw4bit_tensor *tensors, i
             d.ms = t.m_scale;
             d.vs = t.v_scale;
             d.n = t.n;
-            bias_corrections(beta1, beta2, t.step, &d.c1, &d.c2s);
-            d.rc2s = 1.0f / d.c2s;
+            per_tensor(t.step, &d.c1, &d.c2s, &d.rc2s);
             d.pad = 0.0f;
             tiles += nt;
             args.tile_start[++k] = (uint32_t)tiles;
@@ -378,16 +385,48 @@ extern "C" int lpmm_adamw4bit_step_multi(const lpmm_adamw4bit_tensor *tensors, i
         for (int j = k + 1; j <= LPMM_MULTI_MAX; ++j)
             args.tile_start[j] = (uint32_t)tiles;
         if (aligned)
-            hipLaunchKernelGGL(adamw4bit_kernel<true>, dim3((uint32_t)tiles), dim3(kThreads), 0,
+            hipLaunchKernelGGL((adamw4bit_kernel<true, Arith>), dim3((uint32_t)tiles), dim3(kThreads), 0,
                                (hipStream_t)stream, args, qmap_m, qmap_v);
         else
-            hipLaunchKernelGGL(adamw4bit_kernel<false>, dim3((uint32_t)tiles), dim3(kThreads), 0,
+            hipLaunchKernelGGL((adamw4bit_kernel<false, Arith>), dim3((uint32_t)tiles), dim3(kThreads), 0,
                                (hipStream_t)stream, args, qmap_m, qmap_v);
         const int st = launch_status();
         if (st != LPMM_OK)
             return st;
     }
     return LPMM_OK;
+}
+
+extern "C" int lpmm_adamw4bit_step_multi(const lpmm_adamw4bit_tensor *tensors, int64_t count,
+                                         const float *qmap_m, const float *qmap_v, float beta1,
+                                         float beta2, float lr, float weight_decay, float eps,
+                                         void *stream)
+{
+    // 1 - beta is formed in float, as the reference kernel does
+    const float scalars[7] = {beta1, beta2, 1 - beta1, 1 - beta2, lr, weight_decay, eps};
+    return step_multi4<FusedArith>(tensors, count, qmap_m, qmap_v, scalars,
+                                   [=](float step, float *c1, float *c2s, float *rc2s) {
+                                       bias_corrections(beta1, beta2, step, c1, c2s);
+                                       *rc2s = 1.0f / *c2s;
+                                   },
+                                   stream);
+}
+
+extern "C" int lpmm_nonfused_adamw4bit_step_multi(const lpmm_adamw4bit_tensor *tensors, int64_t count,
+                                                  const float *qmap_m, const float *qmap_v, double beta1,
+                                                  double beta2, double lr, double weight_decay,
+                                                  double eps, void *stream)
+{
+    const NfHyper c = make_nf_hyper(beta1, beta2, lr, weight_decay, eps, 1.0);
+    const float scalars[7] = {c.decay, c.w1, c.b2, c.w2, c.eps, 0.0f, 0.0f};
+    return step_multi4<NonFusedArith>(tensors, count, qmap_m, qmap_v, scalars,
+                                      [=](float step, float *nss, float *bc2s, float *rbc2s) {
+                                          const NfHyper h = make_nf_hyper(beta1, beta2, lr, weight_decay, eps, step);
+                                          *nss = h.neg_step_size;
+                                          *bc2s = h.bc2_sqrt;
+                                          *rbc2s = h.rbc2_sqrt;
+                                      },
+                                      stream);
 }
 
 extern "C" int lpmm_adamw4bit_step(float *p, const float *g, uint8_t *m_codes, uint8_t *v_codes,

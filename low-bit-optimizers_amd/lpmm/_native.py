@@ -33,6 +33,7 @@ PROTOTYPES = {
     "lpmm_quant_rank1": (_int, [_vp, _i64, _i64, _vp, _vp, _vp, _vp, _vp]),
     "lpmm_dequant_rank1": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _vp, _vp]),
     "lpmm_nonfused_update": (_int, [_vp] * 4 + [_i64] + [_d] * 6 + [_vp]),
+    "lpmm_nonfused_adamw4bit_step_multi": (_int, [_vp, _i64, _vp, _vp] + [_d] * 5 + [_vp]),
     "lpmm_factored_workspace_bytes": (_i64, [_i64, _i64]),
     "lpmm_factored_stats": (_int, [_vp, _i64, _i64, _vp, _vp, _vp, _d, _vp, _vp]),
     "lpmm_factored_update": (_int, [_vp] * 8 + [_i64, _i64] + [_d] * 6 + [_int, _vp]),

@@ -33,6 +33,20 @@ def _is_placeholder(t):
     return t.numel() <= 1
 
 
+_ZERO_BYTE = {}
+
+
+def _zero_byte(qmap):
+    """int8 value of a packed byte whose two codes both select the map entry nearest 0.0
+    (what quantising a zero tensor stores); looked up once per map."""
+    key = (qmap.device, qmap.data_ptr(), qmap._version)
+    if key not in _ZERO_BYTE:
+        code = int(torch.argmin(qmap.abs()).item())
+        byte = code | (code << 4)
+        _ZERO_BYTE[key] = byte - 256 if byte > 127 else byte
+    return _ZERO_BYTE[key]
+
+
 class AdamW(LowBitOptimizer):
     def __init__(
         self,
@@ -215,6 +229,11 @@ class AdamW(LowBitOptimizer):
         md_m = self.get_qmetadata_by_state_name("exp_avg")
         md_v = self.get_qmetadata_by_state_name("exp_avg_sq")
         lib = _native.lib()
+        # both moments 4-bit with block-wise scaling over 128 values: dequantise, update and
+        # re-quantise in one kernel, all such tensors of the group in one launch
+        one_pass = all(md["scale_type"] == "group" and md["gp_sz"] == 128 and md["b"] == 4
+                       and md["round_type"] == "real-nearest" for md in (md_m, md_v))
+        batched = {}
         for p, grad, state, factored in work:
             state["step"] += 1
             step = state["step"].item()
@@ -223,6 +242,11 @@ class AdamW(LowBitOptimizer):
                 continue
             self._check_fp32_cuda(p, grad)
             en_m, en_v = self._enabled(p, state, "exp_avg"), self._enabled(p, state, "exp_avg_sq")
+            if one_pass and en_m and en_v:
+                key = (p.device, state["exp_avg_qstate"]["qmap"].data_ptr(),
+                       state["exp_avg_sq_qstate"]["qmap"].data_ptr())
+                batched.setdefault(key, []).append(self._nonfused_record(p, grad, state, step))
+                continue
             m = self._materialise(p, state, "exp_avg", en_m, md_m)
             v = self._materialise(p, state, "exp_avg_sq", en_v, md_v)
             with torch.cuda.device(p.device):
@@ -233,6 +257,32 @@ class AdamW(LowBitOptimizer):
                 self._requantise(p, state, "exp_avg", m, md_m)
             if en_v:
                 self._requantise(p, state, "exp_avg_sq", v, md_v)
+        for (dev, qm_ptr, qv_ptr), records in batched.items():
+            table = np.array(records, dtype=_native.ADAMW4BIT_TENSOR)
+            with torch.cuda.device(dev):
+                st = lib.lpmm_nonfused_adamw4bit_step_multi(table.ctypes.data, len(records), qm_ptr, qv_ptr, beta1,
+                                                            beta2, lr, wd, eps, _native.current_stream(dev))
+            _native.check(st, "non-fused 4-bit AdamW step")
+
+    def _nonfused_record(self, p, grad, state, step):
+        """The tensor's record for the one-pass non-fused step; creates the quantised states
+        on first use: all-zero moments in the layout and with the metadata vectorwise_quant
+        gives them (lpmm/optim/adamw.py:425-434)."""
+        n = p.numel()
+        groups = (n + 127) // 128
+        ptrs = []
+        for name in ("exp_avg", "exp_avg_sq"):
+            qstate = state[f"{name}_qstate"]
+            if _is_placeholder(state[name]):
+                state[name] = torch.full((packed_nbytes(groups * 128),), _zero_byte(qstate["qmap"]),
+                                         dtype=torch.int8, device=p.device)
+                oh = qstate["overhead"]
+                oh.clear()
+                oh.update({"dtype": p.dtype, "stride": p.stride(),
+                           "max1": torch.zeros((groups, 1), dtype=torch.float32, device=p.device),
+                           "scaled_shape": torch.Size((groups, 128))})
+            ptrs.append((state[name].data_ptr(), qstate["overhead"]["max1"].data_ptr()))
+        return (p.data_ptr(), grad.data_ptr(), ptrs[0][0], ptrs[1][0], ptrs[0][1], ptrs[1][1], n, step, 0.0)
 
     def _materialise(self, p, state, name, enabled, md):
         """fp32 view of a state for the update: zeros at the first step, the dequantised
