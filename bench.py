@@ -11,7 +11,8 @@ sequence on the host cores, bounded sample).
 
 Two further workloads measure the other kernels of the path with the same JSON shape:
 `--workload quant64m` (stand-alone quantise/dequantise round trip on 2^26 values) and
-`--workload factored` (factored second moment on LLaMA-7B MLP/attention shapes).
+`--workload factored` (factored second moment on LLaMA-7B MLP/attention shapes) and
+`--workload nonfused_group|nonfused_rank1` (fused=False on the LLaMA-7B-shaped set).
 """
 import argparse
 import json
@@ -207,12 +208,48 @@ def run_factored(torch, args):
                      "traffic": None, "bytes_per_param": 17.0625}}))
 
 
+def run_nonfused(torch, args, v_scale):
+    """fused=False on the LLaMA-7B-shaped set.  v_scale 'group': both moments block-wise over
+    128 values, one kernel per launch group of tensors; 'rank1' (the reference's default
+    configuration): dequantise, update, statistics and re-quantise kernels per tensor."""
+    import lpmm
+
+    dev = torch.device("cuda:0")
+    params = make_params(torch, llama7b_shapes(), dev, heavy_tailed=True)
+    cfg = os.path.join(os.path.dirname(lpmm.config.__file__), "configs",
+                       "2nd_moment_group_128.yml" if v_scale == "group" else "default.yml")
+    opt = lpmm.optim.AdamW(params, lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01, fused=False,
+                           qconfig=cfg)
+    n_total = sum(p.numel() for p in params)
+    for _ in range(args.warmup):
+        opt.step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        opt.step()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / args.steps
+    # one pass: p, g read, p written, two 4-bit codes read and written, scales;
+    # rank-1 (two passes): + g and the v codes read a second time, v codes written in the second pass
+    bytes_per_param = BYTES_PER_PARAM_4BIT if v_scale == "group" else 18.5625
+    achieved = n_total * bytes_per_param / dt / 1e9
+    print(json.dumps({
+        "metric": "non-fused 4-bit AdamW step: params/sec, 1 MI355X", "value": n_total / dt,
+        "unit": "params/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": dt * 1e3,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"fused=False, second moment '{v_scale}' scaling, LLaMA-7B-shaped fp32 set",
+                   "tensors": len(params), "params": n_total},
+        "roofline": {"bound": "hbm", "kernel": "whole step", "achieved": achieved, "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "bytes_per_param": bytes_per_param}}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=2)
-    ap.add_argument("--workload", default="llama7b", choices=sorted(WORKLOADS) + ["quant64m", "factored"])
+    ap.add_argument("--workload", default="llama7b", choices=sorted(WORKLOADS) + ["quant64m", "factored", "nonfused_group", "nonfused_rank1"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run three plain 1 GiB device copies first (calibration dispatches for "
@@ -245,6 +282,8 @@ def main():
         return run_quant_roundtrip(torch, args)
     if args.workload == "factored":
         return run_factored(torch, args)
+    if args.workload.startswith("nonfused_"):
+        return run_nonfused(torch, args, args.workload.split("_")[1])
 
     desc, shape_fn = WORKLOADS[args.workload]
     shapes = shape_fn()
@@ -310,7 +349,7 @@ def main():
         / (elapsed / args.steps) / 1e9,
         "roofline": {
             "bound": "hbm",
-            "kernel": "lpmm::adamw4bit_kernel<true>",
+            "kernel": "lpmm::adamw4bit_kernel<true, lpmm::FusedArith>",
             "achieved": achieved,
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",

@@ -163,6 +163,11 @@ int lpmm_nonfused_update(float *p, const float *g, float *m, float *v, int64_t n
                          double beta2, double lr, double weight_decay, double eps, double step,
                          void *stream);
 
+/* The same update for a list of tensors in one launch per 64 tensors (the many small
+ * tensors that keep fp32 states); records as for lpmm_adamw_fp32_step_multi. */
+int lpmm_nonfused_update_multi(const lpmm_adamw_fp32_tensor *tensors, int64_t count, double beta1,
+                               double beta2, double lr, double weight_decay, double eps, void *stream);
+
 /* The whole non-fused step on 4-bit states in one pass, for the configuration the reference
  * uses by default when fused=False is combined with block-wise second-moment scaling (both
  * moments 4-bit, 'group' scaling, gp_sz 128, real-nearest): dequantise m and v, the update
@@ -180,6 +185,40 @@ int lpmm_nonfused_adamw4bit_step_multi(const lpmm_adamw4bit_tensor *tensors, int
                                        const float *qmap_m, const float *qmap_v, double beta1,
                                        double beta2, double lr, double weight_decay, double eps,
                                        void *stream);
+
+/* The whole non-fused step with the reference's default scalings (lpmm/configs/default.yml:
+ * first moment 4-bit 'group' gp_sz 128, second moment 4-bit 'rank1') on row-major R x C
+ * tensors whose column count is a multiple of 128, in two passes over HBM: update + first
+ * moment + statistics of the new second moment, then re-quantisation of the second moment.
+ * Replaces, for such tensors, the body of _single_tensor_adamw4bit
+ *   (lpmm/optim/adamw.py:394-436) including get_sm3_statistics (lpmm/functional.py:503-509
+ *   for the packed layout, :190-203 for the rank-1 scale).
+ * v_rowmax (R floats) / v_colmax (C floats) are the statistics the v codes are currently
+ * scaled by (max_dims of the reference's metadata); the call leaves the statistics of the
+ * new second moment in v_rowmax_next / v_colmax_next (cleared by the call, must not alias
+ * the current ones) and the v codes scaled by them: the caller swaps the two pairs.
+ * Code arrays: ceil(R*C/2048)*1024 + 1 bytes, 4-byte aligned, written in full.  Before the
+ * first step all scales and statistics must be zero and the codes those of 0.0. */
+typedef struct lpmm_nonfused_rank1_tensor {
+    float *p;
+    const float *g;
+    uint8_t *m_codes;
+    float *m_max1;
+    uint8_t *v_codes;
+    const float *v_rowmax;
+    const float *v_colmax;
+    float *v_rowmax_next;
+    float *v_colmax_next;
+    int64_t rows;
+    int64_t cols;
+    float step;
+    float reserved;
+} lpmm_nonfused_rank1_tensor;
+
+int lpmm_nonfused_adamw4bit_rank1_step_multi(const lpmm_nonfused_rank1_tensor *tensors, int64_t count,
+                                             const float *qmap_m, const float *qmap_v, double beta1,
+                                             double beta2, double lr, double weight_decay, double eps,
+                                             void *stream);
 
 /* ---------------------------------------------------------------------------------------
  * (c) Factored second moment on a row-major R x C tensor.

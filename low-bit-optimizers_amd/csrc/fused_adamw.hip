@@ -55,7 +55,8 @@ struct FusedArith {
     // code buffers hold exactly ceil(n/2) bytes; a last odd element leaves its high nibble 0
     static constexpr bool kPadded = false;
     Hyper h;
-    __device__ __forceinline__ FusedArith(const Multi4 &a, const Tensor4 &t)
+    template <class M, class T>
+    __device__ __forceinline__ FusedArith(const M &a, const T &t)
     {
         h.beta1 = a.s[0];
         h.beta2 = a.s[1];
@@ -77,7 +78,8 @@ struct NonFusedArith {
     // tensor hold the code of 0.0
     static constexpr bool kPadded = true;
     NfHyper h;
-    __device__ __forceinline__ NonFusedArith(const Multi4 &a, const Tensor4 &t)
+    template <class M, class T>
+    __device__ __forceinline__ NonFusedArith(const M &a, const T &t)
     {
         h.decay = a.s[0];
         h.w1 = a.s[1];
@@ -92,9 +94,6 @@ struct NonFusedArith {
 };
 
 static_assert(sizeof(Multi4) + 2 * sizeof(void *) <= 4096, "kernel arguments exceed 4 KB");
-
-// element k (0..7) of a lane sits at this offset inside the lane's group
-__device__ __forceinline__ int elt_offset(int lane16, int k) { return lane16 * 4 + (k & 3) + (k >> 2) * 64; }
 
 // One 128-element group, handled by the 16 lanes of a DPP row.  FULL: the whole group lies
 // inside the tensor and the pointers allow vector access; otherwise every access is
@@ -233,12 +232,15 @@ __global__ __launch_bounds__(kThreads) void adamw4bit_kernel(const Multi4 args,
         t.vc[end] = 0;
     }
     if (Arith::kPadded && grp * kGroup >= t.n) {
-        // a group the padding to whole tiles added: codes of 0.0 (m: 7, v: 0)
+        // a group the padding to whole tiles added: codes of a plain 0.0
+        const float z[kEltsPerLane] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+        const uint32_t zm = encode8_plain(lds, kLdsQ0, std_maps ? kMapStdM : kMapGeneric, z);
+        const uint32_t zv = encode8_plain(lds, kLdsQ1, std_maps ? kMapStdV : kMapGeneric, z);
         const int64_t b = (grp * kGroup >> 1) + lane16 * 4;
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
-            t.mc[b + k] = 0x77;
-            t.vc[b + k] = 0;
+            t.mc[b + k] = (uint8_t)zm;  // all eight codes are the same
+            t.vc[b + k] = (uint8_t)zv;
         }
         return;
     }
@@ -257,8 +259,8 @@ struct TensorF {
     float *m;
     float *v;
     int64_t n;
-    float c1;
-    float c2s;
+    float c1, c2s, rc2s;  // per-tensor scalars, as in Tensor4
+    float pad;
 };
 
 constexpr int kMultiFMax = 64;
@@ -268,9 +270,14 @@ struct MultiF {
     TensorF t[kMultiFMax];
     uint32_t tile_start[kMultiFMax + 1];
     int count;
-    float beta1, beta2, lr, wd, eps;
+    float s[7];
 };
 
+static_assert(sizeof(MultiF) <= 4096, "kernel arguments exceed 4 KB");
+
+// fp32 states, either arithmetic (the FusedArith / NonFusedArith constructors only read the
+// scalars, which Multi4 and MultiF name alike)
+template <class Arith>
 __global__ __launch_bounds__(kThreads) void adamw_fp32_kernel(const MultiF args)
 {
     int lo = 0, hi = args.count;
@@ -282,24 +289,15 @@ __global__ __launch_bounds__(kThreads) void adamw_fp32_kernel(const MultiF args)
             hi = mid;
     }
     const TensorF &t = args.t[lo];
-    Hyper h;
-    h.beta1 = args.beta1;
-    h.beta2 = args.beta2;
-    h.omb1 = 1 - args.beta1;
-    h.omb2 = 1 - args.beta2;
-    h.lr = args.lr;
-    h.wd = args.wd;
-    h.eps = args.eps;
-    h.c1 = t.c1;
-    h.c2s = t.c2s;
-    h.rc2s = 1.0f / t.c2s;
+    const Arith h(args, t);
     const int64_t tile0 = (int64_t)(blockIdx.x - args.tile_start[lo]) * kTileF;
 #pragma unroll
     for (int k = 0; k < kTileF / kThreads; ++k) {
         const int64_t i = tile0 + k * kThreads + threadIdx.x;
         if (i < t.n) {
-            float m = t.m[i], v = t.v[i];
-            t.p[i] = adamw_elt(t.p[i], t.g[i], m, v, h);
+            float p = t.p[i], m = t.m[i], v = t.v[i];
+            h.elt(p, t.g[i], m, v);
+            t.p[i] = p;
             t.m[i] = m;
             t.v[i] = v;
         }
@@ -447,9 +445,9 @@ extern "C" int lpmm_adamw4bit_step(float *p, const float *g, uint8_t *m_codes, u
     return lpmm_adamw4bit_step_multi(&t, 1, qmap_m, qmap_v, beta1, beta2, lr, weight_decay, eps, stream);
 }
 
-extern "C" int lpmm_adamw_fp32_step_multi(const lpmm_adamw_fp32_tensor *tensors, int64_t count,
-                                          float beta1, float beta2, float lr, float weight_decay,
-                                          float eps, void *stream)
+template <class Arith, class PerTensor>
+static int step_multi_fp32(const lpmm_adamw_fp32_tensor *tensors, int64_t count, const float (&scalars)[7],
+                           PerTensor per_tensor, void *stream)
 {
     if (count < 0)
         return LPMM_ERR_SIZE;
@@ -472,11 +470,8 @@ extern "C" int lpmm_adamw_fp32_step_multi(const lpmm_adamw_fp32_tensor *tensors,
         LPMM_REQUIRE_ALIGN(t.v, 4);
     }
     MultiF args;
-    args.beta1 = beta1;
-    args.beta2 = beta2;
-    args.lr = lr;
-    args.wd = weight_decay;
-    args.eps = eps;
+    for (int j = 0; j < 7; ++j)
+        args.s[j] = scalars[j];
     int64_t i = 0;
     while (i < count) {
         int k = 0;
@@ -497,7 +492,8 @@ extern "C" int lpmm_adamw_fp32_step_multi(const lpmm_adamw_fp32_tensor *tensors,
             d.m = t.m;
             d.v = t.v;
             d.n = t.n;
-            bias_corrections(beta1, beta2, t.step, &d.c1, &d.c2s);
+            per_tensor(t.step, &d.c1, &d.c2s, &d.rc2s);
+            d.pad = 0.0f;
             tiles += nt;
             args.tile_start[++k] = (uint32_t)tiles;
             ++i;
@@ -507,13 +503,42 @@ extern "C" int lpmm_adamw_fp32_step_multi(const lpmm_adamw_fp32_tensor *tensors,
         args.count = k;
         for (int j = k + 1; j <= kMultiFMax; ++j)
             args.tile_start[j] = (uint32_t)tiles;
-        hipLaunchKernelGGL(adamw_fp32_kernel, dim3((uint32_t)tiles), dim3(kThreads), 0,
+        hipLaunchKernelGGL(adamw_fp32_kernel<Arith>, dim3((uint32_t)tiles), dim3(kThreads), 0,
                            (hipStream_t)stream, args);
         const int st = launch_status();
         if (st != LPMM_OK)
             return st;
     }
     return LPMM_OK;
+}
+
+extern "C" int lpmm_adamw_fp32_step_multi(const lpmm_adamw_fp32_tensor *tensors, int64_t count,
+                                          float beta1, float beta2, float lr, float weight_decay,
+                                          float eps, void *stream)
+{
+    const float scalars[7] = {beta1, beta2, 1 - beta1, 1 - beta2, lr, weight_decay, eps};
+    return step_multi_fp32<FusedArith>(tensors, count, scalars,
+                                       [=](float step, float *c1, float *c2s, float *rc2s) {
+                                           bias_corrections(beta1, beta2, step, c1, c2s);
+                                           *rc2s = 1.0f / *c2s;
+                                       },
+                                       stream);
+}
+
+extern "C" int lpmm_nonfused_update_multi(const lpmm_adamw_fp32_tensor *tensors, int64_t count, double beta1,
+                                          double beta2, double lr, double weight_decay, double eps,
+                                          void *stream)
+{
+    const NfHyper c = make_nf_hyper(beta1, beta2, lr, weight_decay, eps, 1.0);
+    const float scalars[7] = {c.decay, c.w1, c.b2, c.w2, c.eps, 0.0f, 0.0f};
+    return step_multi_fp32<NonFusedArith>(tensors, count, scalars,
+                                          [=](float step, float *nss, float *bc2s, float *rbc2s) {
+                                              const NfHyper h = make_nf_hyper(beta1, beta2, lr, weight_decay, eps, step);
+                                              *nss = h.neg_step_size;
+                                              *bc2s = h.bc2_sqrt;
+                                              *rbc2s = h.rbc2_sqrt;
+                                          },
+                                          stream);
 }
 
 extern "C" int lpmm_adamw_fp32_step(float *p, const float *g, float *m, float *v, int64_t n,

@@ -173,6 +173,30 @@ __device__ __forceinline__ uint32_t encode8_scaled(const uint32_t *lds, uint32_t
     return encode8_generic(mids, x);
 }
 
+// Codes of 8 values that are already normalised (no division); `kind` says which map sits at
+// LDS offset `lds_map`.  NaN -> 15 like the reference.
+__device__ __forceinline__ uint32_t encode8_plain(const uint32_t *lds, uint32_t lds_map, int kind, const float (&x)[8])
+{
+    if (kind == kMapGeneric)
+        return encode8_generic(make_mids(reinterpret_cast<const float *>(lds) + lds_map / 4), x);
+    uint32_t w;
+    if (kind == kMapStdM) {
+        w = encode8_std_m(lds, x);
+    } else {
+        // the closed form needs x <= 1 for the upper clamp; larger inputs are legal here
+        float y[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k)
+            y[k] = fminf(x[k], 1.0f);
+        w = encode8_std_v(y);
+    }
+#pragma unroll
+    for (int k = 0; k < 8; ++k)
+        if (x[k] != x[k])
+            w |= 15u << (4 * k);
+    return w;
+}
+
 // Decode offsets: byte j of `even` / `odd` holds 4 * nibble (2j) / (2j+1) of the code word.
 struct Nibbles {
     uint32_t even, odd;

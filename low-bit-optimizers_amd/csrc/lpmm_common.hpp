@@ -52,6 +52,16 @@ __device__ __forceinline__ float row16_max(float v)
     return v;
 }
 
+// Row layout: the 16 lanes of a DPP row own one 128-element group, lane l the elements
+// [4l, 4l+4) and [64+4l, 64+4l+4); element k (0..7) of a lane sits at this offset in the group.
+__device__ __forceinline__ int elt_offset(int lane16, int k) { return lane16 * 4 + (k & 3) + (k >> 2) * 64; }
+
+// max of non-negative floats == max of their bit patterns as unsigned integers
+__device__ __forceinline__ void atomic_max_nonneg(float *addr, float v)
+{
+    atomicMax(reinterpret_cast<unsigned int *>(addr), __float_as_uint(v));
+}
+
 __device__ __forceinline__ float wave_max(float v)
 {
     v = row16_max(v);

@@ -76,15 +76,20 @@ __device__ __forceinline__ float lerp_w(float a, float b, float w)
     return (fabsf(w) < 0.5f) ? __builtin_fmaf(w, b - a, a) : __builtin_fmaf(w - 1.0f, b - a, b);
 }
 
+// v.mul_(beta2).addcmul_(g, g, value=1 - beta2)
+__device__ __forceinline__ void nonfused_second_moment(float &v, float g, const NfHyper &h)
+{
+    const float vi = v * h.b2;
+    v = vi + (h.w2 * g) * g;
+}
+
 // One element of the non-fused update; p, m and v are updated in place.
 __device__ __forceinline__ void nonfused_elt(float &p, float g, float &m, float &v, const NfHyper &h)
 {
     const float pi = p * h.decay;
     m = lerp_w(m, g, h.w1);
-    float vi = v * h.b2;
-    vi = vi + (h.w2 * g) * g;
-    v = vi;
-    const float denom = div_by_rc(sqrt_fast(vi), h.bc2_sqrt, h.rbc2_sqrt) + h.eps;
+    nonfused_second_moment(v, g, h);
+    const float denom = div_by_rc(sqrt_fast(v), h.bc2_sqrt, h.rbc2_sqrt) + h.eps;
     p = pi + div_fast(h.neg_step_size * m, denom);
 }
 

@@ -1,0 +1,449 @@
+// The non-fused AdamW step on 4-bit states with the reference's default scalings -- first
+// moment block-wise over 128 values, second moment rank-1 (scale[r, c] = min(rowmax[r],
+// colmax[c])) -- in two passes over HBM instead of the seven of the staged path
+// (lpmm/optim/adamw.py:394-436: two dequantisations, the update, the statistics of the new
+// second moment, two quantisations).
+//
+// The second moment cannot be re-quantised where it is computed, because its scales are
+// maxima over whole rows and columns of the new values.  So:
+//
+//   pass 1 (update):   reads p, g, both code arrays and the current statistics; updates p,
+//                      re-quantises m, and merges the row/column maxima of the new v into the
+//                      next statistics (atomic max on the bit patterns: exact, order-free);
+//   pass 2 (requant):  reads g, the old v codes and both sets of statistics, recomputes the
+//                      new v with the same operations (bit-identical), normalises by the next
+//                      statistics and overwrites the v codes in place.
+//
+// 18.5 bytes per parameter cross HBM instead of 50.  The column count must be a multiple of
+// 128, so that the 128-value groups of m never straddle rows: 16 lanes (one DPP row) own 128
+// consecutive columns of one tensor row.  A 256-thread workgroup covers 16 rows by
+// 128 << lg_wide columns, per pass (16 >> lg_wide) rows of (1 << lg_wide) adjacent groups, so
+// that its accesses to a row are contiguous runs of 512 << lg_wide bytes.  16 rows by 1024
+// columns measured best on the LLaMA-7B shapes: smaller tiles pay for the column atomics and
+// the per-workgroup set-up, larger ones leave too few workgroups to balance the last wave of
+// them over the chip.  lg_wide is chosen per tensor on the host.
+#include "lpmm_update.hpp"
+
+namespace lpmm {
+
+constexpr int kThreads = 256;
+constexpr int kEltsPerLane = 8;
+constexpr int kDppRows = kThreads / 16;  // 128-column groups a workgroup handles per pass
+constexpr int kTileRows = 16;            // tensor rows per workgroup
+constexpr int kR1Max = 32;               // tensors per launch
+constexpr int kMaxLgWide = 3;
+constexpr int kMaxWide = 1 << kMaxLgWide;
+// Per-column data of a tile lives in LDS, not in registers (occupancy): the current column
+// statistics in the unused bytes between the maps and the encode table, further arrays after
+// the table.
+constexpr uint32_t kColBytes = kMaxWide * kGroup * 4;
+constexpr uint32_t kColOld = kLdsQ1 + 64;
+static_assert(kColOld + kColBytes <= kEncLdsBegin, "column statistics overlap the encode table");
+constexpr uint32_t kColExtra = (kLdsBytes + 15) / 16 * 16;  // first byte after the table
+// Column maxima of the tile, one slot of 8 x 16 words (+16 words of skew, so that the DPP rows
+// of a wave hit different banks) per column group: word k * 16 + lane16 of a slot is element k
+// of lane lane16.
+constexpr uint32_t kRedSlotWords = kGroup + 16;
+
+struct TensorR1 {
+    float *p;
+    const float *g;
+    uint8_t *mc;
+    float *ms;
+    uint8_t *vc;
+    const float *row_old;
+    const float *col_old;
+    float *row_new;
+    float *col_new;
+    int64_t rows;
+    uint32_t col_blocks;  // columns / 128
+    float neg_step_size, bc2_sqrt, rbc2_sqrt;
+    // a workgroup covers kTileRows rows x (128 << lg_wide) columns: per pass, (16 >> lg_wide)
+    // rows of (1 << lg_wide) adjacent groups each
+    uint32_t lg_wide;
+    uint32_t col_tiles;  // ceil(col_blocks / (1 << lg_wide))
+};
+
+struct MultiR1 {
+    TensorR1 t[kR1Max];
+    uint32_t tile_start[kR1Max + 1];  // prefix sum of tiles per tensor; unused slots hold the total
+    int count;
+    float decay, w1, b2, w2, eps;
+};
+
+static_assert(sizeof(MultiR1) + 2 * sizeof(void *) <= 4096, "kernel arguments exceed 4 KB");
+static_assert(kR1Max <= kWave, "one tile_start entry per lane");
+
+// tensor of this workgroup (uniform): the number of later tensors whose first tile is not
+// after this one
+__device__ __forceinline__ int find_tensor(const MultiR1 &args)
+{
+    const int lane = threadIdx.x & (kWave - 1);
+    const bool started = lane + 1 < kR1Max && args.tile_start[lane + 1] <= blockIdx.x;
+    return __popcll(__ballot(started));
+}
+
+__device__ __forceinline__ void unpack8(const float4 &a, const float4 &b, float (&o)[kEltsPerLane])
+{
+    o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w;
+    o[4] = b.x; o[5] = b.y; o[6] = b.z; o[7] = b.w;
+}
+
+// Where a DPP row of this workgroup works: column group `cg` (fixed), rows row0, row0 + step, ...
+struct Geometry {
+    int64_t row0;
+    uint32_t cg, col_tile;
+    int step, passes, wide;
+};
+
+__device__ __forceinline__ Geometry geometry(const TensorR1 &t, uint32_t tile, int drow)
+{
+    Geometry q;
+    const uint32_t rb = tile / t.col_tiles;
+    q.col_tile = tile - rb * t.col_tiles;
+    q.wide = 1 << t.lg_wide;
+    q.cg = q.col_tile * q.wide + (drow & (q.wide - 1));
+    q.row0 = (int64_t)rb * kTileRows + (drow >> t.lg_wide);
+    q.step = kDppRows >> t.lg_wide;
+    q.passes = kTileRows / q.step;
+    return q;
+}
+
+// Codes of a plain 0.0 into the padding [n, n_padded) of a packed array and 0 into the extra
+// last byte; one workgroup.  n and n_padded are multiples of 8, the array is 4-byte aligned.
+__device__ __forceinline__ void write_padding(uint8_t *codes, int64_t n, int64_t n_padded, uint32_t zero_word)
+{
+    for (int64_t i = n + (int64_t)threadIdx.x * kEltsPerLane; i < n_padded; i += kThreads * kEltsPerLane)
+        *reinterpret_cast<uint32_t *>(codes + (i >> 1)) = zero_word;
+    if (threadIdx.x == 0)
+        codes[n_padded / 2] = 0;
+}
+
+__global__ __launch_bounds__(kThreads) void rank1_clear_kernel(const MultiR1 args)
+{
+    const TensorR1 &t = args.t[blockIdx.y];
+    const int64_t cols = (int64_t)t.col_blocks * kGroup;
+    for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < t.rows + cols; i += (int64_t)gridDim.x * kThreads) {
+        if (i < t.rows)
+            t.row_new[i] = 0.0f;
+        else
+            t.col_new[i - t.rows] = 0.0f;
+    }
+}
+
+// 6 waves per SIMD: at most 80 registers
+__global__ __launch_bounds__(kThreads, 6) void rank1_update_kernel(const MultiR1 args, const float *__restrict__ qmap_m,
+                                                                const float *__restrict__ qmap_v)
+{
+    __shared__ __align__(16) uint32_t lds[(kColExtra + kMaxWide * kRedSlotWords * 4) / 4];
+    uint32_t *colred = lds + kColExtra / 4;
+    lds_fill(lds, qmap_m, qmap_v);
+    for (int j = threadIdx.x; j < kMaxWide * (int)kRedSlotWords; j += kThreads)
+        colred[j] = 0u;
+    const int kind_m = classify_map(qmap_m);
+    const int lo = find_tensor(args);
+    const TensorR1 &t = args.t[lo];
+    const uint32_t tl = blockIdx.x - args.tile_start[lo];
+    const int lane16 = threadIdx.x & 15, drow = threadIdx.x >> 4;
+    const Geometry q = geometry(t, tl, drow);
+    const int64_t cols = (int64_t)t.col_blocks * kGroup;
+    const int64_t tile_c0 = (int64_t)q.col_tile * q.wide * kGroup;
+    for (int j = threadIdx.x; j < q.wide * kGroup; j += kThreads)
+        lds[kColOld / 4 + j] = (tile_c0 + j < cols) ? __float_as_uint(t.col_old[tile_c0 + j]) : 0u;
+    NfHyper h;
+    h.decay = args.decay;
+    h.w1 = args.w1;
+    h.b2 = args.b2;
+    h.w2 = args.w2;
+    h.eps = args.eps;
+    h.neg_step_size = t.neg_step_size;
+    h.bc2_sqrt = t.bc2_sqrt;
+    h.rbc2_sqrt = t.rbc2_sqrt;
+    __syncthreads();
+
+    if (tl == 0) {
+        const float z[kEltsPerLane] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+        const int64_t n = t.rows * cols;
+        write_padding(t.mc, n, (n + LPMM_PACK_GROUP - 1) / LPMM_PACK_GROUP * LPMM_PACK_GROUP,
+                      encode8_plain(lds, kLdsQ0, kind_m, z));
+    }
+
+    const int slot = drow & (q.wide - 1);
+    if (q.cg < t.col_blocks) {  // the whole DPP row
+        const uint32_t co_off = kColOld + (slot * kGroup + lane16 * 4) * 4;
+        uint32_t *red = colred + slot * kRedSlotWords + lane16;
+#pragma unroll 1
+        for (int it = 0; it < q.passes; ++it) {
+            const int64_t r = q.row0 + it * q.step;
+            if (r >= t.rows)
+                break;
+            const int64_t grp = r * t.col_blocks + q.cg;
+            const int64_t gbase = grp * kGroup;
+            float *pp = t.p + gbase + lane16 * 4;
+            const float *gp = t.g + gbase + lane16 * 4;
+            const float4 a0 = load4(pp), a1 = load4(pp + 64);
+            const float4 b0 = load4(gp), b1 = load4(gp + 64);
+            uint16_t *mcp = reinterpret_cast<uint16_t *>(t.mc + (gbase >> 1)) + lane16;
+            const uint16_t *vcp = reinterpret_cast<const uint16_t *>(t.vc + (gbase >> 1)) + lane16;
+            const uint32_t wm = load_u16(mcp) | (load_u16(mcp + 16) << 16);
+            const uint32_t wv = load_u16(vcp) | (load_u16(vcp + 16) << 16);
+            const float sm = t.ms[grp];
+            const float ro = t.row_old[r];
+            float pv[kEltsPerLane], gv[kEltsPerLane], m[kEltsPerLane], v[kEltsPerLane], co[kEltsPerLane];
+            unpack8(a0, a1, pv);
+            unpack8(b0, b1, gv);
+            unpack8(lds_read<float4>(lds, co_off), lds_read<float4>(lds, co_off + 256), co);
+
+            const Nibbles nm = split_nibbles(wm), nv = split_nibbles(wv);
+            float amax_m = 0.0f, vmax = 0.0f;
+#pragma unroll
+            for (int k = 0; k < kEltsPerLane; ++k) {
+                m[k] = decode_nibble(lds, kLdsQ0, nm, k) * sm;
+                v[k] = decode_nibble(lds, kLdsQ1, nv, k) * ((co[k] < ro) ? co[k] : ro);
+                nonfused_elt(pv[k], gv[k], m[k], v[k], h);
+                amax_m = fmaxf(amax_m, fabsf(m[k]));
+                vmax = fmaxf(vmax, v[k]);
+                atomicMax(red + k * 16, __float_as_uint(v[k]));
+            }
+            amax_m = row16_max(amax_m);
+            vmax = row16_max(vmax);
+            const uint32_t cm = encode8_scaled(lds, kLdsQ0, kind_m, m, amax_m);
+
+            store4(pp, make_float4(pv[0], pv[1], pv[2], pv[3]));
+            store4(pp + 64, make_float4(pv[4], pv[5], pv[6], pv[7]));
+            store_u16(mcp, cm & 0xFFFFu);
+            store_u16(mcp + 16, cm >> 16);
+            if (lane16 == 0) {
+                t.ms[grp] = amax_m;
+                atomic_max_nonneg(t.row_new + r, vmax);
+            }
+        }
+    }
+    __syncthreads();
+    // column j of the tile = element k of lane l of slot s
+    for (int j = threadIdx.x; j < q.wide * kGroup; j += kThreads) {
+        const int w = j & (kGroup - 1);
+        const int k = ((w >> 6) << 2) | (w & 3), l = (w >> 2) & 15;
+        if (tile_c0 + j < cols)
+            atomic_max_nonneg(t.col_new + tile_c0 + j, __uint_as_float(colred[(j >> 7) * kRedSlotWords + k * 16 + l]));
+    }
+}
+
+__global__ __launch_bounds__(kThreads) void rank1_requant_kernel(const MultiR1 args, const float *__restrict__ qmap_v)
+{
+    __shared__ __align__(16) uint32_t lds[(kColExtra + 2 * kColBytes) / 4];
+    constexpr uint32_t kColNew = kColExtra, kColRcp = kColExtra + kColBytes;
+    lds_fill(lds, qmap_v, nullptr);
+    const int kind = classify_map(qmap_v);
+    const int lo = find_tensor(args);
+    const TensorR1 &t = args.t[lo];
+    const uint32_t tl = blockIdx.x - args.tile_start[lo];
+    const int lane16 = threadIdx.x & 15, drow = threadIdx.x >> 4;
+    const Geometry q = geometry(t, tl, drow);
+    const int64_t cols = (int64_t)t.col_blocks * kGroup;
+    const int64_t tile_c0 = (int64_t)q.col_tile * q.wide * kGroup;
+    for (int j = threadIdx.x; j < q.wide * kGroup; j += kThreads) {
+        const bool in = tile_c0 + j < cols;
+        const float cn = in ? t.col_new[tile_c0 + j] : 0.0f;
+        lds[kColOld / 4 + j] = in ? __float_as_uint(t.col_old[tile_c0 + j]) : 0u;
+        lds[kColNew / 4 + j] = __float_as_uint(cn);
+        lds[kColRcp / 4 + j] = __float_as_uint(1.0f / cn);
+    }
+    NfHyper h;
+    h.b2 = args.b2;
+    h.w2 = args.w2;
+    __syncthreads();
+
+    if (tl == 0) {
+        const float z[kEltsPerLane] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+        const int64_t n = t.rows * cols;
+        write_padding(t.vc, n, (n + LPMM_PACK_GROUP - 1) / LPMM_PACK_GROUP * LPMM_PACK_GROUP,
+                      encode8_plain(lds, kLdsQ0, kind, z));
+    }
+    if (q.cg >= t.col_blocks)
+        return;
+
+    const uint32_t col_off = ((drow & (q.wide - 1)) * kGroup + lane16 * 4) * 4;
+#pragma unroll 1
+    for (int it = 0; it < q.passes; ++it) {
+        const int64_t r = q.row0 + it * q.step;
+        if (r >= t.rows)
+            break;
+        const int64_t gbase = (r * t.col_blocks + q.cg) * kGroup;
+        const float *gp = t.g + gbase + lane16 * 4;
+        const float4 b0 = load4(gp), b1 = load4(gp + 64);
+        uint16_t *vcp = reinterpret_cast<uint16_t *>(t.vc + (gbase >> 1)) + lane16;
+        const uint32_t wv = load_u16(vcp) | (load_u16(vcp + 16) << 16);
+        const float ro = t.row_old[r], rn = t.row_new[r];
+        float gv[kEltsPerLane], v[kEltsPerLane], s[kEltsPerLane], x[kEltsPerLane], co[kEltsPerLane], cn[kEltsPerLane];
+        unpack8(b0, b1, gv);
+        unpack8(lds_read<float4>(lds, kColOld + col_off), lds_read<float4>(lds, kColOld + col_off + 256), co);
+        unpack8(lds_read<float4>(lds, kColNew + col_off), lds_read<float4>(lds, kColNew + col_off + 256), cn);
+        const Nibbles nv = split_nibbles(wv);
+        bool safe = true;
+#pragma unroll
+        for (int k = 0; k < kEltsPerLane; ++k) {
+            v[k] = decode_nibble(lds, kLdsQ0, nv, k) * ((co[k] < ro) ? co[k] : ro);
+            nonfused_second_moment(v[k], gv[k], h);
+            s[k] = (cn[k] < rn) ? cn[k] : rn;
+            safe = safe && rc_safe(s[k]);
+        }
+        uint32_t w;
+        if (kind == kMapStdV && __all(safe)) {
+            // the correctly rounded reciprocal of whichever statistic is the scale, then one
+            // multiply and two fmas: the correctly rounded quotient (v <= scale by construction)
+            const float rcr = 1.0f / rn;
+            float rcn[kEltsPerLane];
+            unpack8(lds_read<float4>(lds, kColRcp + col_off), lds_read<float4>(lds, kColRcp + col_off + 256), rcn);
+#pragma unroll
+            for (int k = 0; k < kEltsPerLane; ++k)
+                x[k] = div_by_rc(v[k], s[k], (cn[k] < rn) ? rcn[k] : rcr);
+            w = encode8_std_v(x);
+        } else {
+#pragma unroll
+            for (int k = 0; k < kEltsPerLane; ++k)
+                x[k] = v[k] / s[k];
+            w = encode8_plain(lds, kLdsQ0, kind, x);
+        }
+        store_u16(vcp, w & 0xFFFFu);
+        store_u16(vcp + 16, w >> 16);
+    }
+}
+
+}  // namespace lpmm
+
+using namespace lpmm;
+
+// The widest tile (longest contiguous runs) that leaves at most 5 % of the DPP rows of a
+// tensor's tiles without a column group; otherwise the width that wastes least.
+static uint32_t choose_lg_wide(uint32_t col_blocks)
+{
+    uint32_t best = 0;
+    double best_use = 0.0;
+    for (int lg = kMaxLgWide; lg >= 0; --lg) {
+        const uint32_t wide = 1u << lg;
+        const double use = (double)col_blocks / (double)((col_blocks + wide - 1) / wide * wide);
+        if (use >= 0.95)
+            return (uint32_t)lg;
+        if (use > best_use) {
+            best_use = use;
+            best = (uint32_t)lg;
+        }
+    }
+    return best;
+}
+
+extern "C" int lpmm_nonfused_adamw4bit_rank1_step_multi(const lpmm_nonfused_rank1_tensor *tensors, int64_t count,
+                                                        const float *qmap_m, const float *qmap_v, double beta1,
+                                                        double beta2, double lr, double weight_decay,
+                                                        double eps, void *stream)
+{
+    if (count < 0)
+        return LPMM_ERR_SIZE;
+    if (count == 0)
+        return LPMM_OK;
+    LPMM_REQUIRE_PTR(tensors);
+    LPMM_REQUIRE_PTR(qmap_m);
+    LPMM_REQUIRE_PTR(qmap_v);
+    LPMM_REQUIRE_ALIGN(qmap_m, 4);
+    LPMM_REQUIRE_ALIGN(qmap_v, 4);
+    for (int64_t i = 0; i < count; ++i) {
+        const lpmm_nonfused_rank1_tensor &t = tensors[i];
+        if (t.rows < 0 || t.cols < 0 || t.cols % kGroup != 0)
+            return LPMM_ERR_SIZE;
+        if (t.rows == 0 || t.cols == 0)
+            continue;
+        const int64_t col_blocks = t.cols / kGroup;
+        const int64_t row_blocks = (t.rows + kTileRows - 1) / kTileRows;
+        if (col_blocks > 0x7fffffffLL / 2 || row_blocks > 0x7fffffffLL / col_blocks ||
+            t.rows > INT64_MAX / t.cols)
+            return LPMM_ERR_SIZE;
+        LPMM_REQUIRE_PTR(t.p);
+        LPMM_REQUIRE_PTR(t.g);
+        LPMM_REQUIRE_PTR(t.m_codes);
+        LPMM_REQUIRE_PTR(t.m_max1);
+        LPMM_REQUIRE_PTR(t.v_codes);
+        LPMM_REQUIRE_PTR(t.v_rowmax);
+        LPMM_REQUIRE_PTR(t.v_colmax);
+        LPMM_REQUIRE_PTR(t.v_rowmax_next);
+        LPMM_REQUIRE_PTR(t.v_colmax_next);
+        LPMM_REQUIRE_ALIGN(t.p, 16);
+        LPMM_REQUIRE_ALIGN(t.g, 16);
+        LPMM_REQUIRE_ALIGN(t.m_codes, 4);
+        LPMM_REQUIRE_ALIGN(t.v_codes, 4);
+        LPMM_REQUIRE_ALIGN(t.m_max1, 4);
+        LPMM_REQUIRE_ALIGN(t.v_rowmax, 4);
+        LPMM_REQUIRE_ALIGN(t.v_colmax, 16);
+        LPMM_REQUIRE_ALIGN(t.v_rowmax_next, 4);
+        LPMM_REQUIRE_ALIGN(t.v_colmax_next, 16);
+        if (t.v_rowmax == t.v_rowmax_next || t.v_colmax == t.v_colmax_next)
+            return LPMM_ERR_ARG;
+    }
+
+    const NfHyper c = make_nf_hyper(beta1, beta2, lr, weight_decay, eps, 1.0);
+    MultiR1 args;
+    args.decay = c.decay;
+    args.w1 = c.w1;
+    args.b2 = c.b2;
+    args.w2 = c.w2;
+    args.eps = c.eps;
+    int64_t i = 0;
+    while (i < count) {
+        int k = 0;
+        uint64_t tiles = 0;
+        int64_t longest = 0;
+        args.tile_start[0] = 0;
+        while (i < count && k < kR1Max) {
+            const lpmm_nonfused_rank1_tensor &t = tensors[i];
+            if (t.rows == 0 || t.cols == 0) {
+                ++i;
+                continue;
+            }
+            const uint32_t col_blocks = (uint32_t)(t.cols / kGroup);
+            const uint32_t lg_wide = choose_lg_wide(col_blocks);
+            const uint32_t col_tiles = (col_blocks + (1u << lg_wide) - 1) >> lg_wide;
+            const uint64_t nt = (uint64_t)((t.rows + kTileRows - 1) / kTileRows) * col_tiles;
+            if (tiles + nt > 0x7fffffffULL)
+                break;
+            TensorR1 &d = args.t[k];
+            d.p = t.p;
+            d.g = t.g;
+            d.mc = t.m_codes;
+            d.ms = t.m_max1;
+            d.vc = t.v_codes;
+            d.row_old = t.v_rowmax;
+            d.col_old = t.v_colmax;
+            d.row_new = t.v_rowmax_next;
+            d.col_new = t.v_colmax_next;
+            d.rows = t.rows;
+            d.col_blocks = col_blocks;
+            d.lg_wide = lg_wide;
+            d.col_tiles = col_tiles;
+            const NfHyper h = make_nf_hyper(beta1, beta2, lr, weight_decay, eps, t.step);
+            d.neg_step_size = h.neg_step_size;
+            d.bc2_sqrt = h.bc2_sqrt;
+            d.rbc2_sqrt = h.rbc2_sqrt;
+            longest = t.rows + t.cols > longest ? t.rows + t.cols : longest;
+            tiles += nt;
+            args.tile_start[++k] = (uint32_t)tiles;
+            ++i;
+        }
+        if (k == 0)
+            continue;
+        args.count = k;
+        for (int j = k + 1; j <= kR1Max; ++j)
+            args.tile_start[j] = (uint32_t)tiles;
+        int64_t clear_blocks = (longest + kThreads - 1) / kThreads;
+        clear_blocks = clear_blocks > 64 ? 64 : clear_blocks;
+        hipLaunchKernelGGL(rank1_clear_kernel, dim3((uint32_t)clear_blocks, (uint32_t)k), dim3(kThreads), 0,
+                           (hipStream_t)stream, args);
+        hipLaunchKernelGGL(rank1_update_kernel, dim3((uint32_t)tiles), dim3(kThreads), 0, (hipStream_t)stream, args,
+                           qmap_m, qmap_v);
+        hipLaunchKernelGGL(rank1_requant_kernel, dim3((uint32_t)tiles), dim3(kThreads), 0, (hipStream_t)stream, args,
+                           qmap_v);
+        const int st = launch_status();
+        if (st != LPMM_OK)
+            return st;
+    }
+    return LPMM_OK;
+}

@@ -58,29 +58,6 @@ __device__ __forceinline__ uint32_t load_codes8(const uint8_t *__restrict__ code
     return w;
 }
 
-// Codes of 8 values that are already normalised (no division): NaN -> 15 like the reference.
-__device__ __forceinline__ uint32_t encode8_plain(const uint32_t *lds, int kind, const float (&x)[kQElts])
-{
-    if (kind == kMapGeneric)
-        return encode8_generic(make_mids(reinterpret_cast<const float *>(lds) + kLdsQ0 / 4), x);
-    uint32_t w;
-    if (kind == kMapStdM) {
-        w = encode8_std_m(lds, x);
-    } else {
-        // the closed form needs x <= 1 for the upper clamp; larger inputs are legal here
-        float y[kQElts];
-#pragma unroll
-        for (int k = 0; k < kQElts; ++k)
-            y[k] = fminf(x[k], 1.0f);
-        w = encode8_std_v(y);
-    }
-#pragma unroll
-    for (int k = 0; k < kQElts; ++k)
-        if (x[k] != x[k])
-            w |= 15u << (4 * k);
-    return w;
-}
-
 // ---------------------------------------------------------------------------------------
 // pack_nonlinear / unpack_nonlinear (values already normalised)
 // ---------------------------------------------------------------------------------------
@@ -100,7 +77,7 @@ __global__ __launch_bounds__(kQThreads) void pack4_kernel(const float *__restric
         return;
     float v[kQElts];
     load8(x, base, n_padded, vec, v);
-    const uint32_t w = encode8_plain(lds, kind, v);
+    const uint32_t w = encode8_plain(lds, kLdsQ0, kind, v);
     if (vec) {
         store_u32(reinterpret_cast<uint32_t *>(out + (base >> 1)), w);
     } else {
@@ -173,7 +150,7 @@ __global__ __launch_bounds__(kQThreads) void quant_group_kernel(const float *__r
     } else {
         // padding added by the re-grouping to 2048: plain zeros, not divided by anything
         const float z[kQElts] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
-        w = encode8_plain(lds, kind, z);
+        w = encode8_plain(lds, kLdsQ0, kind, z);
     }
     store_u32(reinterpret_cast<uint32_t *>(codes + (base >> 1)), w);
 }
@@ -244,12 +221,6 @@ __global__ void fill_zero_kernel(float *__restrict__ a, int64_t na, float *__res
 constexpr int kStatRows = 32;
 constexpr int kStatCols = 1024;  // 256 threads x 4 columns
 constexpr int kStatUnroll = 8;   // rows in flight per lane
-
-// max of non-negative floats == max of their bit patterns as unsigned integers
-__device__ __forceinline__ void atomic_max_nonneg(float *addr, float v)
-{
-    atomicMax(reinterpret_cast<unsigned int *>(addr), __float_as_uint(v));
-}
 
 // Tile of kStatRows x kStatCols; a lane keeps 4 column maxima in registers, row maxima are
 // reduced over the wave and merged with atomics (max is exact and order-independent).
@@ -335,7 +306,7 @@ __global__ __launch_bounds__(kQThreads) void quant_rank1_kernel(const float *__r
             }
         }
     }
-    store_u32(reinterpret_cast<uint32_t *>(codes + (base >> 1)), encode8_plain(lds, kind, xs));
+    store_u32(reinterpret_cast<uint32_t *>(codes + (base >> 1)), encode8_plain(lds, kLdsQ0, kind, xs));
 }
 
 // The same when C is a multiple of 8: a lane's 8 values lie in one row, the grid is
@@ -356,7 +327,7 @@ __global__ __launch_bounds__(kQThreads) void quant_rank1_rows_kernel(const float
     const int64_t n = R * C;
     if (blockIdx.x == 0 && blockIdx.y == 0) {
         const float z[kQElts] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
-        const uint32_t wz = encode8_plain(lds, kind, z);
+        const uint32_t wz = encode8_plain(lds, kLdsQ0, kind, z);
         for (int64_t i = n + (int64_t)threadIdx.x * kQElts; i < n_padded; i += kR1Cols)
             *reinterpret_cast<uint32_t *>(codes + (i >> 1)) = wz;
         if (threadIdx.x == 0)
@@ -377,7 +348,7 @@ __global__ __launch_bounds__(kQThreads) void quant_rank1_rows_kernel(const float
         const float st = (cmx[k] < rm) ? cmx[k] : rm;
         xs[k] = v[k] / st;
     }
-    store_u32(reinterpret_cast<uint32_t *>(codes + ((r * C + c) >> 1)), encode8_plain(lds, kind, xs));
+    store_u32(reinterpret_cast<uint32_t *>(codes + ((r * C + c) >> 1)), encode8_plain(lds, kLdsQ0, kind, xs));
 }
 
 __global__ __launch_bounds__(kQThreads) void dequant_rank1_kernel(const uint8_t *__restrict__ codes,

@@ -33,7 +33,9 @@ PROTOTYPES = {
     "lpmm_quant_rank1": (_int, [_vp, _i64, _i64, _vp, _vp, _vp, _vp, _vp]),
     "lpmm_dequant_rank1": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _vp, _vp]),
     "lpmm_nonfused_update": (_int, [_vp] * 4 + [_i64] + [_d] * 6 + [_vp]),
+    "lpmm_nonfused_update_multi": (_int, [_vp, _i64] + [_d] * 5 + [_vp]),
     "lpmm_nonfused_adamw4bit_step_multi": (_int, [_vp, _i64, _vp, _vp] + [_d] * 5 + [_vp]),
+    "lpmm_nonfused_adamw4bit_rank1_step_multi": (_int, [_vp, _i64, _vp, _vp] + [_d] * 5 + [_vp]),
     "lpmm_factored_workspace_bytes": (_i64, [_i64, _i64]),
     "lpmm_factored_stats": (_int, [_vp, _i64, _i64, _vp, _vp, _vp, _d, _vp, _vp]),
     "lpmm_factored_update": (_int, [_vp] * 8 + [_i64, _i64] + [_d] * 6 + [_int, _vp]),
@@ -45,6 +47,10 @@ PROTOTYPES = {
 ADAMW4BIT_TENSOR = np.dtype([("p", "<u8"), ("g", "<u8"), ("m_codes", "<u8"), ("v_codes", "<u8"),
                              ("m_scale", "<u8"), ("v_scale", "<u8"), ("n", "<i8"), ("step", "<f4"),
                              ("reserved", "<f4")])
+NONFUSED_RANK1_TENSOR = np.dtype([("p", "<u8"), ("g", "<u8"), ("m_codes", "<u8"), ("m_max1", "<u8"),
+                                  ("v_codes", "<u8"), ("v_rowmax", "<u8"), ("v_colmax", "<u8"),
+                                  ("v_rowmax_next", "<u8"), ("v_colmax_next", "<u8"), ("rows", "<i8"),
+                                  ("cols", "<i8"), ("step", "<f4"), ("reserved", "<f4")])
 ADAMW_FP32_TENSOR = np.dtype([("p", "<u8"), ("g", "<u8"), ("m", "<u8"), ("v", "<u8"), ("n", "<i8"),
                               ("step", "<f4"), ("reserved", "<f4")])
 

@@ -229,11 +229,16 @@ class AdamW(LowBitOptimizer):
         md_m = self.get_qmetadata_by_state_name("exp_avg")
         md_v = self.get_qmetadata_by_state_name("exp_avg_sq")
         lib = _native.lib()
-        # both moments 4-bit with block-wise scaling over 128 values: dequantise, update and
-        # re-quantise in one kernel, all such tensors of the group in one launch
-        one_pass = all(md["scale_type"] == "group" and md["gp_sz"] == 128 and md["b"] == 4
-                       and md["round_type"] == "real-nearest" for md in (md_m, md_v))
-        batched = {}
+        # both moments 4-bit, first moment block-wise over 128 values, second moment either the
+        # same or rank-1 on a 2-D tensor with a multiple of 128 columns: dequantise, update and
+        # re-quantise in one kernel (two for rank-1), all such tensors of the group per launch
+        def fits(md):
+            return md["b"] == 4 and md["round_type"] == "real-nearest"
+
+        m_group128 = fits(md_m) and md_m["scale_type"] == "group" and md_m["gp_sz"] == 128
+        v_group128 = fits(md_v) and md_v["scale_type"] == "group" and md_v["gp_sz"] == 128
+        v_rank1 = fits(md_v) and md_v["scale_type"] == "rank1"
+        batched, batched_rank1, plain = {}, {}, {}
         for p, grad, state, factored in work:
             state["step"] += 1
             step = state["step"].item()
@@ -242,13 +247,22 @@ class AdamW(LowBitOptimizer):
                 continue
             self._check_fp32_cuda(p, grad)
             en_m, en_v = self._enabled(p, state, "exp_avg"), self._enabled(p, state, "exp_avg_sq")
-            if one_pass and en_m and en_v:
+            if m_group128 and en_m and en_v:
                 key = (p.device, state["exp_avg_qstate"]["qmap"].data_ptr(),
                        state["exp_avg_sq_qstate"]["qmap"].data_ptr())
-                batched.setdefault(key, []).append(self._nonfused_record(p, grad, state, step))
-                continue
+                if v_group128:
+                    batched.setdefault(key, []).append(self._nonfused_record(p, grad, state, step))
+                    continue
+                if v_rank1 and p.dim() == 2 and p.shape[1] % 128 == 0:
+                    batched_rank1.setdefault(key, []).append(self._nonfused_rank1_record(p, grad, state, step))
+                    continue
             m = self._materialise(p, state, "exp_avg", en_m, md_m)
             v = self._materialise(p, state, "exp_avg_sq", en_v, md_v)
+            if not en_m and not en_v and p.is_contiguous() and m.is_contiguous() and v.is_contiguous():
+                # fp32 states (small tensors): all of them in one launch
+                plain.setdefault(p.device, []).append(
+                    (p.data_ptr(), grad.data_ptr(), m.data_ptr(), v.data_ptr(), p.numel(), step, 0.0))
+                continue
             with torch.cuda.device(p.device):
                 st = lib.lpmm_nonfused_update(p.data_ptr(), grad.data_ptr(), m.data_ptr(), v.data_ptr(), p.numel(),
                                               beta1, beta2, lr, wd, eps, step, _native.current_stream(p.device))
@@ -257,12 +271,25 @@ class AdamW(LowBitOptimizer):
                 self._requantise(p, state, "exp_avg", m, md_m)
             if en_v:
                 self._requantise(p, state, "exp_avg_sq", v, md_v)
+        for dev, records in plain.items():
+            table = np.array(records, dtype=_native.ADAMW_FP32_TENSOR)
+            with torch.cuda.device(dev):
+                st = lib.lpmm_nonfused_update_multi(table.ctypes.data, len(records), beta1, beta2, lr, wd, eps,
+                                                    _native.current_stream(dev))
+            _native.check(st, "non-fused AdamW update")
         for (dev, qm_ptr, qv_ptr), records in batched.items():
             table = np.array(records, dtype=_native.ADAMW4BIT_TENSOR)
             with torch.cuda.device(dev):
                 st = lib.lpmm_nonfused_adamw4bit_step_multi(table.ctypes.data, len(records), qm_ptr, qv_ptr, beta1,
                                                             beta2, lr, wd, eps, _native.current_stream(dev))
             _native.check(st, "non-fused 4-bit AdamW step")
+        for (dev, qm_ptr, qv_ptr), records in batched_rank1.items():
+            table = np.array(records, dtype=_native.NONFUSED_RANK1_TENSOR)
+            with torch.cuda.device(dev):
+                st = lib.lpmm_nonfused_adamw4bit_rank1_step_multi(table.ctypes.data, len(records), qm_ptr, qv_ptr,
+                                                                  beta1, beta2, lr, wd, eps,
+                                                                  _native.current_stream(dev))
+            _native.check(st, "non-fused 4-bit AdamW step (rank-1 second moment)")
 
     def _nonfused_record(self, p, grad, state, step):
         """The tensor's record for the one-pass non-fused step; creates the quantised states
@@ -283,6 +310,50 @@ class AdamW(LowBitOptimizer):
                            "scaled_shape": torch.Size((groups, 128))})
             ptrs.append((state[name].data_ptr(), qstate["overhead"]["max1"].data_ptr()))
         return (p.data_ptr(), grad.data_ptr(), ptrs[0][0], ptrs[1][0], ptrs[0][1], ptrs[1][1], n, step, 0.0)
+
+    def _nonfused_rank1_record(self, p, grad, state, step):
+        """The tensor's record for the two-pass step with a rank-1 second moment.  The kernels
+        leave the statistics of the new second moment in a second pair of buffers; the pairs
+        trade places here, so that the state's `max_dims` always are the statistics its codes
+        are scaled by."""
+        rows, cols = p.shape
+        n = p.numel()
+        groups = n // 128
+        dev = p.device
+        qs_m, qs_v = state["exp_avg_qstate"], state["exp_avg_sq_qstate"]
+        if _is_placeholder(state["exp_avg"]):
+            state["exp_avg"] = torch.full((packed_nbytes(n),), _zero_byte(qs_m["qmap"]), dtype=torch.int8, device=dev)
+            qs_m["overhead"].clear()
+            qs_m["overhead"].update({"dtype": p.dtype, "stride": p.stride(),
+                                     "max1": torch.zeros((groups, 1), dtype=torch.float32, device=dev),
+                                     "scaled_shape": torch.Size((groups, 128))})
+        if _is_placeholder(state["exp_avg_sq"]):
+            state["exp_avg_sq"] = torch.full((packed_nbytes(n),), _zero_byte(qs_v["qmap"]), dtype=torch.int8,
+                                             device=dev)
+            qs_v["overhead"].clear()
+            qs_v["overhead"].update({"dtype": p.dtype, "stride": p.stride(), "dim": 2, "max1": None,
+                                     "max_dims": [torch.zeros((rows, 1), dtype=torch.float32, device=dev),
+                                                  torch.zeros((1, cols), dtype=torch.float32, device=dev)],
+                                     "scaled_shape": p.shape})
+        oh = qs_v["overhead"]
+        cur = oh["max_dims"]
+        nxt = self._spare_stats.pop(p, None)
+        if nxt is None or nxt[0].device != dev:
+            nxt = [torch.empty_like(cur[0]), torch.empty_like(cur[1])]
+        self._spare_stats[p] = cur
+        oh["max_dims"] = nxt
+        return (p.data_ptr(), grad.data_ptr(), state["exp_avg"].data_ptr(), qs_m["overhead"]["max1"].data_ptr(),
+                state["exp_avg_sq"].data_ptr(), cur[0].data_ptr(), cur[1].data_ptr(), nxt[0].data_ptr(),
+                nxt[1].data_ptr(), rows, cols, step, 0.0)
+
+    @property
+    def _spare_stats(self):
+        # second pair of row/column statistics per parameter; not part of the optimizer state
+        # (its contents are only meaningful during a step)
+        d = self.__dict__.get("_spare_stats_by_param")
+        if d is None:
+            d = self.__dict__["_spare_stats_by_param"] = {}
+        return d
 
     def _materialise(self, p, state, name, enabled, md):
         """fp32 view of a state for the update: zeros at the first step, the dequantised

@@ -48,6 +48,34 @@ def test_nonfused_update_matches_oracle(oracle):
         assert mismatches <= max(1, n // 100000), mismatches
 
 
+def test_nonfused_update_multi_matches_oracle(oracle):
+    """Many small fp32-state tensors in one call (more than one launch holds), each with its
+    own step count."""
+    from lpmm import _native
+
+    lib = _lib()
+    rng = np.random.default_rng(6)
+    sizes = [int(n) for n in rng.integers(1, 5000, size=70)] + [4096 * 3 + 1]
+    host, dev = [], []
+    for n in sizes:
+        arrs = [(rng.standard_normal(n) * 0.02).astype(np.float32), (rng.standard_normal(n) * 1e-3).astype(np.float32),
+                (rng.standard_normal(n) * 1e-3).astype(np.float32), (rng.standard_normal(n) ** 2 * 1e-6).astype(np.float32)]
+        host.append(arrs)
+        dev.append([to_dev(a) for a in arrs])
+    steps = [float(1 + i % 9) for i in range(len(sizes))]
+    table = np.array([(d[0].data_ptr(), d[1].data_ptr(), d[2].data_ptr(), d[3].data_ptr(), n, st, 0.0)
+                      for d, n, st in zip(dev, sizes, steps)], dtype=_native.ADAMW_FP32_TENSOR)
+    st = lib.lpmm_nonfused_update_multi(table.ctypes.data, len(sizes), H["beta1"], H["beta2"], H["lr"], H["wd"],
+                                        H["eps"], _stream())
+    assert st == 0
+    torch.cuda.synchronize()
+    for (p, g, m, v), d, step in zip(host, dev, steps):
+        oracle.nonfused_update(p, g, m, v, H["beta1"], H["beta2"], H["lr"], H["wd"], H["eps"], step)
+        np.testing.assert_array_equal(to_np(d[2]), m)
+        np.testing.assert_array_equal(to_np(d[3]), v)
+        assert_rel(to_np(d[0]), p, "p", scale=p)
+
+
 @pytest.mark.parametrize("shape", [(64, 128), (100, 70), (513, 1025), (1024, 2752), (2752, 1024)])
 def test_factored_step_matches_oracle(oracle, qmaps, shape):
     lib = _lib()

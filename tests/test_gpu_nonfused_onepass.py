@@ -134,14 +134,19 @@ def test_onepass_zero_groups_and_outliers(oracle, qmaps):
     assert np.all(t.ref[1][3:5] == 0.0) and t.ref[0][128 * 3 // 2] == 0xFF
 
 
-def test_onepass_other_maps(oracle):
-    """Maps other than the two standard ones take the search fallback."""
-    qm = oracle.create_pow_map(4, True, 1)  # a signed linear map
+@pytest.mark.parametrize("which", ["linear", "shifted"])
+def test_onepass_other_maps(oracle, which):
+    """Maps other than the two standard ones take the search fallback; the padding holds the
+    code of 0.0 under the map in use."""
+    if which == "linear":
+        qm = oracle.create_pow_map(4, True, 1)  # a signed linear map
+    else:
+        qm = np.linspace(-0.2, 1.0, 16).astype(np.float32)  # the code of 0.0 is not 7
     qv = (oracle.qmap_v() ** 2).astype(np.float32)
     assert qm.size == 16 and qv.size == 16
     dqm, dqv = to_dev(qm), to_dev(qv)
     rng = np.random.default_rng(14)
-    zero_code = int(np.argmin(np.abs(qm)))
+    zero_code = int(np.sum((qm[:-1] + qm[1:]) * np.float32(0.5) < 0))
     tensors = [_Tensor(n, rng, zero_byte_m=zero_code | (zero_code << 4)) for n in (300, 5000, 2048 * 3)]
     for step in range(1, 4):
         grads = [(rng.standard_normal(t.n) * 1e-3).astype(np.float32) for t in tensors]
