@@ -244,6 +244,30 @@ int lpmm_factored_update(float *p, const float *g, uint8_t *m_codes, float *m_ma
                          double beta2, double lr, double weight_decay, double eps, double step,
                          int first_step, void *stream);
 
+/* Both passes for a list of row-major R x C tensors whose column count is a multiple of 128
+ * and whose first moment is quantised (4-bit, 'group', gp_sz 128): statistics and update of
+ * all tensors in four launches per 24 tensors instead of four per tensor.  Same results as
+ * lpmm_factored_stats followed by lpmm_factored_update.  workspace: device scratch of
+ * lpmm_factored_workspace_bytes(rows, cols) bytes per tensor, 8-byte aligned, not shared
+ * between the tensors of one call; p, g and col 16-byte aligned. */
+typedef struct lpmm_factored_tensor {
+    float *p;
+    const float *g;
+    uint8_t *m_codes;
+    float *m_max1;
+    float *row;
+    float *col;
+    void *workspace;
+    int64_t rows;
+    int64_t cols;
+    float step;
+    int32_t first_step;
+} lpmm_factored_tensor;
+
+int lpmm_factored_step_multi(const lpmm_factored_tensor *tensors, int64_t count, const float *qmap_m,
+                             double beta1, double beta2, double lr, double weight_decay, double eps,
+                             void *stream);
+
 /* The same pass with an fp32 first moment (m read and written as floats): tensors at or
  * under the quantisation threshold, or first-moment quantisation disabled
  * (the `else: exp_avg = q_exp_avg` branch, lpmm/optim/adamw.py:603-604). */

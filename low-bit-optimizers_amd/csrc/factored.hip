@@ -54,16 +54,16 @@ constexpr int kSRows = 32;
 constexpr int kSCols = 1024;  // 256 threads x 4 columns
 constexpr int kSUnroll = 8;   // rows in flight per lane
 
-__global__ __launch_bounds__(kFThreads) void factored_partial_kernel(const float *__restrict__ g, int64_t R,
-                                                                     int64_t C, double *__restrict__ colpart,
-                                                                     double *__restrict__ rowpart, bool vec)
+__device__ __forceinline__ void partial_body(const float *__restrict__ g, int64_t R, int64_t C,
+                                             double *__restrict__ colpart, double *__restrict__ rowpart, bool vec,
+                                             uint32_t bx, uint32_t by)
 {
-    const int64_t c0 = (int64_t)blockIdx.x * kSCols + (int64_t)threadIdx.x * 4;
-    const int64_t r0 = (int64_t)blockIdx.y * kSRows;
+    const int64_t c0 = (int64_t)bx * kSCols + (int64_t)threadIdx.x * 4;
+    const int64_t r0 = (int64_t)by * kSRows;
     const int64_t r1 = (r0 + kSRows < R) ? r0 + kSRows : R;
     const bool lane_vec = vec && c0 + 4 <= C;
     __shared__ double s_part[kFThreads / kWave][kSUnroll];
-    double *rp = rowpart + (int64_t)blockIdx.x * R;  // one row partial per workgroup
+    double *rp = rowpart + (int64_t)bx * R;  // one row partial per workgroup
     double cs[4] = {0.0, 0.0, 0.0, 0.0};
     for (int64_t rb = r0; rb < r1; rb += kSUnroll) {
         float u[kSUnroll][4];
@@ -107,25 +107,30 @@ __global__ __launch_bounds__(kFThreads) void factored_partial_kernel(const float
 #pragma unroll
     for (int k = 0; k < 4; ++k)
         if (c0 + k < C)
-            colpart[(int64_t)blockIdx.y * C + c0 + k] = cs[k];
+            colpart[(int64_t)by * C + c0 + k] = cs[k];
+}
+
+__global__ __launch_bounds__(kFThreads) void factored_partial_kernel(const float *__restrict__ g, int64_t R,
+                                                                     int64_t C, double *__restrict__ colpart,
+                                                                     double *__restrict__ rowpart, bool vec)
+{
+    partial_body(g, R, C, colpart, rowpart, vec, blockIdx.x, blockIdx.y);
 }
 
 // Pass B: fold the partials in a fixed order and update the EMAs
 // (row.mul_(beta2).add_(mean, alpha=1-beta2): fma(mean, 1-beta2, row*beta2)).
 // Workgroups [0, row_blocks) take 256 rows each and leave the sum of their new row values in
 // rowblock[b]; the remaining workgroups take 64 columns each.
-__global__ __launch_bounds__(kFThreads) void factored_finalize_kernel(const double *__restrict__ colpart,
-                                                                      const double *__restrict__ rowpart,
-                                                                      double *__restrict__ rowblock, int64_t R,
-                                                                      int64_t C, int tiles_y, int tiles_x,
-                                                                      int row_blocks, float *__restrict__ row,
-                                                                      float *__restrict__ col, float b2, float w2)
+__device__ __forceinline__ void finalize_body(const double *__restrict__ colpart, const double *__restrict__ rowpart,
+                                              double *__restrict__ rowblock, int64_t R, int64_t C, int tiles_y,
+                                              int tiles_x, int row_blocks, float *__restrict__ row,
+                                              float *__restrict__ col, float b2, float w2, uint32_t bx)
 {
-    if ((int)blockIdx.x >= row_blocks) {
+    if ((int)bx >= row_blocks) {
         // 64 columns per workgroup; the partials of a column are split over 4 threads, each
         // summing its contiguous quarter 8 loads at a time, and folded in a fixed order
         __shared__ double s_col[kFThreads];
-        const int64_t c = (int64_t)(blockIdx.x - row_blocks) * 64 + (threadIdx.x & 63);
+        const int64_t c = (int64_t)(bx - row_blocks) * 64 + (threadIdx.x & 63);
         const int quarter = threadIdx.x >> 6;
         const int per = (tiles_y + 3) / 4;
         const int t0 = quarter * per, t1 = (t0 + per < tiles_y) ? t0 + per : tiles_y;
@@ -153,7 +158,7 @@ __global__ __launch_bounds__(kFThreads) void factored_finalize_kernel(const doub
         return;
     }
     __shared__ double s_sum[kFThreads];
-    const int64_t r = (int64_t)blockIdx.x * kFThreads + threadIdx.x;
+    const int64_t r = (int64_t)bx * kFThreads + threadIdx.x;
     double mine = 0.0;
     if (r < R) {
         double s = 0.0;
@@ -172,7 +177,17 @@ __global__ __launch_bounds__(kFThreads) void factored_finalize_kernel(const doub
         __syncthreads();
     }
     if (threadIdx.x == 0)
-        rowblock[blockIdx.x] = s_sum[0];
+        rowblock[bx] = s_sum[0];
+}
+
+__global__ __launch_bounds__(kFThreads) void factored_finalize_kernel(const double *__restrict__ colpart,
+                                                                      const double *__restrict__ rowpart,
+                                                                      double *__restrict__ rowblock, int64_t R,
+                                                                      int64_t C, int tiles_y, int tiles_x,
+                                                                      int row_blocks, float *__restrict__ row,
+                                                                      float *__restrict__ col, float b2, float w2)
+{
+    finalize_body(colpart, rowpart, rowblock, R, C, tiles_y, tiles_x, row_blocks, row, col, b2, w2, blockIdx.x);
 }
 
 // Pass C: mean(row) from the per-workgroup sums, in order.
@@ -292,18 +307,18 @@ __global__ __launch_bounds__(kFThreads) void factored_update_kernel(
 // 16 lanes of a DPP row own one group in the row layout of the fused step (lane l: columns
 // [4l, 4l+4) and [64+4l, 64+4l+4) of the piece; whole cache lines per store), and no index
 // division is needed.  Workgroup (0,0) also writes the pad codes past the tensor.
-__global__ __launch_bounds__(kFThreads) void factored_update_rows128_kernel(
+__device__ __forceinline__ void update_rows128_body(
     float *__restrict__ p, const float *__restrict__ g, uint8_t *__restrict__ m_codes,
     float *__restrict__ m_max1, const float *__restrict__ qmap_m, const float *__restrict__ row,
     const float *__restrict__ col, const float *__restrict__ row_mean_all, int64_t R, int64_t C,
-    int64_t n_padded, NfHyper h, bool first_step)
+    int64_t n_padded, const NfHyper &h, bool first_step, uint32_t bx, int64_t by)
 {
     __shared__ __align__(16) uint32_t lds[kLdsBytes / 4];
     lds_fill(lds, qmap_m, nullptr);
     const int kind = classify_map(qmap_m);
     __syncthreads();
     const int64_t n = R * C;
-    if (blockIdx.x == 0 && blockIdx.y == 0) {
+    if (bx == 0 && by == 0) {
         const float z[kFElts] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
         const uint32_t wz = kind == kMapStdM ? encode8_std_m(lds, z)
                                              : encode8_generic(make_mids(reinterpret_cast<const float *>(lds) + kLdsQ0 / 4), z);
@@ -313,8 +328,8 @@ __global__ __launch_bounds__(kFThreads) void factored_update_rows128_kernel(
             m_codes[n_padded / 2] = 0;
     }
     const int lane16 = threadIdx.x & 15;
-    const int64_t r = blockIdx.y;
-    const int64_t c0 = (int64_t)blockIdx.x * kFTile + (int64_t)(threadIdx.x >> 4) * kGroup;  // first column of the group
+    const int64_t r = by;
+    const int64_t c0 = (int64_t)bx * kFTile + (int64_t)(threadIdx.x >> 4) * kGroup;  // first column of the group
     if (c0 >= C)
         return;  // uniform over the 16 lanes of the group
     const int64_t gbase = r * C + c0;
@@ -358,6 +373,16 @@ __global__ __launch_bounds__(kFThreads) void factored_update_rows128_kernel(
         m_max1[grp] = amax;
 }
 
+__global__ __launch_bounds__(kFThreads) void factored_update_rows128_kernel(
+    float *__restrict__ p, const float *__restrict__ g, uint8_t *__restrict__ m_codes,
+    float *__restrict__ m_max1, const float *__restrict__ qmap_m, const float *__restrict__ row,
+    const float *__restrict__ col, const float *__restrict__ row_mean_all, int64_t R, int64_t C,
+    int64_t n_padded, NfHyper h, bool first_step)
+{
+    update_rows128_body(p, g, m_codes, m_max1, qmap_m, row, col, row_mean_all, R, C, n_padded, h, first_step,
+                        blockIdx.x, blockIdx.y);
+}
+
 // The same update with an fp32 first moment (tensors at or under the quantisation threshold,
 // or first-moment quantisation disabled): m is read and written as floats.
 __global__ __launch_bounds__(kFThreads) void factored_update_fp32m_kernel(
@@ -375,6 +400,100 @@ __global__ __launch_bounds__(kFThreads) void factored_update_fp32m_kernel(
         p[i] = pi + div_fast(h.neg_step_size * mi, denom);
         m[i] = mi;
     }
+}
+
+// ---------------------------------------------------------------------------------------
+// The whole factored step for a list of tensors: the three statistics kernels and the update
+// run once per launch group instead of once per tensor.  Each workgroup finds its tensor in
+// a prefix sum of workgroup counts kept in the kernel arguments and then does exactly what
+// the single-tensor kernels above do.
+// ---------------------------------------------------------------------------------------
+constexpr int kFaMax = 24;  // tensors per launch group
+
+struct TensorFa {
+    float *p;
+    const float *g;
+    uint8_t *mc;
+    float *ms;
+    float *row;
+    float *col;
+    double *colpart;
+    double *rowpart;
+    double *rowblock;
+    float *mean;
+    int64_t R, C;
+    int64_t n_padded;
+    uint32_t tiles_x, tiles_y;  // statistics tiles
+    uint32_t row_blocks;        // finalize: workgroups that take rows; the rest take 64 columns each
+    uint32_t upd_x;             // update: 2048-column chunks per row
+    uint32_t first_step;
+    float neg_step_size, bc2_sqrt, rbc2_sqrt;
+};
+
+struct MultiFa {
+    TensorFa t[kFaMax];
+    // prefix sums of workgroups per tensor for the three big kernels; unused slots hold the total
+    uint32_t start_stats[kFaMax + 1], start_fin[kFaMax + 1], start_upd[kFaMax + 1];
+    int count;
+    float decay, w1, b2, w2, eps;
+};
+
+static_assert(sizeof(MultiFa) + sizeof(void *) <= 4096, "kernel arguments exceed 4 KB");
+static_assert(kFaMax <= kWave, "one prefix-sum entry per lane");
+
+__device__ __forceinline__ int find_slot(const uint32_t (&start)[kFaMax + 1])
+{
+    const int lane = threadIdx.x & (kWave - 1);
+    const bool started = lane + 1 < kFaMax && start[lane + 1] <= blockIdx.x;
+    return __popcll(__ballot(started));
+}
+
+__global__ __launch_bounds__(kFThreads) void factored_partial_multi_kernel(const MultiFa args)
+{
+    const int i = find_slot(args.start_stats);
+    const TensorFa &t = args.t[i];
+    const uint32_t local = blockIdx.x - args.start_stats[i];
+    const uint32_t by = local / t.tiles_x, bx = local - by * t.tiles_x;
+    partial_body(t.g, t.R, t.C, t.colpart, t.rowpart, true, bx, by);
+}
+
+__global__ __launch_bounds__(kFThreads) void factored_finalize_multi_kernel(const MultiFa args)
+{
+    const int i = find_slot(args.start_fin);
+    const TensorFa &t = args.t[i];
+    finalize_body(t.colpart, t.rowpart, t.rowblock, t.R, t.C, (int)t.tiles_y, (int)t.tiles_x, (int)t.row_blocks,
+                  t.row, t.col, args.b2, args.w2, blockIdx.x - args.start_fin[i]);
+}
+
+__global__ void factored_mean_multi_kernel(const MultiFa args)
+{
+    const TensorFa &t = args.t[blockIdx.x];
+    if (threadIdx.x == 0) {
+        double s = 0.0;
+        for (uint32_t b = 0; b < t.row_blocks; ++b)
+            s += t.rowblock[b];
+        *t.mean = (float)(s / (double)t.R);
+    }
+}
+
+__global__ __launch_bounds__(kFThreads) void factored_update_multi_kernel(const MultiFa args,
+                                                                          const float *__restrict__ qmap_m)
+{
+    const int i = find_slot(args.start_upd);
+    const TensorFa &t = args.t[i];
+    const uint32_t local = blockIdx.x - args.start_upd[i];
+    const uint32_t by = local / t.upd_x, bx = local - by * t.upd_x;
+    NfHyper h;
+    h.decay = args.decay;
+    h.w1 = args.w1;
+    h.b2 = args.b2;
+    h.w2 = args.w2;
+    h.eps = args.eps;
+    h.neg_step_size = t.neg_step_size;
+    h.bc2_sqrt = t.bc2_sqrt;
+    h.rbc2_sqrt = t.rbc2_sqrt;
+    update_rows128_body(t.p, t.g, t.mc, t.ms, qmap_m, t.row, t.col, t.mean, t.R, t.C, t.n_padded, h,
+                        t.first_step != 0, bx, by);
 }
 
 inline int64_t round_up(int64_t a, int64_t b) { return (a + b - 1) / b * b; }
@@ -415,7 +534,9 @@ extern "C" int64_t lpmm_factored_workspace_bytes(int64_t rows, int64_t cols)
         return 0;
     const int64_t ty = (rows + kSRows - 1) / kSRows, tx = (cols + kSCols - 1) / kSCols;
     const int64_t row_blocks = (rows + kFThreads - 1) / kFThreads;
-    return (ty * cols + tx * rows + row_blocks) * (int64_t)sizeof(double);
+    // column partials, row partials, per-workgroup sums of the new row statistics, and (used by
+    // the multi-tensor step only) mean(row)
+    return (ty * cols + tx * rows + row_blocks + 1) * (int64_t)sizeof(double);
 }
 
 extern "C" int lpmm_factored_stats(const float *g, int64_t rows, int64_t cols, float *row, float *col,
@@ -535,4 +656,114 @@ extern "C" int lpmm_factored_update_fp32m(float *p, const float *g, float *m, co
                        (hipStream_t)stream, p, g, m, row, col, row_mean_all, n, cols,
                        make_nf_hyper(beta1, beta2, lr, weight_decay, eps, step));
     return launch_status();
+}
+
+extern "C" int lpmm_factored_step_multi(const lpmm_factored_tensor *tensors, int64_t count, const float *qmap_m,
+                                        double beta1, double beta2, double lr, double weight_decay, double eps,
+                                        void *stream)
+{
+    if (count < 0)
+        return LPMM_ERR_SIZE;
+    if (count == 0)
+        return LPMM_OK;
+    LPMM_REQUIRE_PTR(tensors);
+    LPMM_REQUIRE_PTR(qmap_m);
+    LPMM_REQUIRE_ALIGN(qmap_m, 4);
+    for (int64_t i = 0; i < count; ++i) {
+        const lpmm_factored_tensor &t = tensors[i];
+        if (t.rows <= 0 || t.cols <= 0 || t.cols % kGroup != 0 || t.rows > INT64_MAX / t.cols)
+            return LPMM_ERR_SIZE;
+        const int64_t ty = (t.rows + kSRows - 1) / kSRows, tx = (t.cols + kSCols - 1) / kSCols;
+        const int64_t ux = (t.cols + kFTile - 1) / kFTile;
+        if (tx > 0x7fffffffLL / ty || ux > 0x7fffffffLL / t.rows ||
+            (t.rows + kFThreads - 1) / kFThreads + (t.cols + 63) / 64 > 0x7fffffffLL)
+            return LPMM_ERR_SIZE;
+        LPMM_REQUIRE_PTR(t.p);
+        LPMM_REQUIRE_PTR(t.g);
+        LPMM_REQUIRE_PTR(t.m_codes);
+        LPMM_REQUIRE_PTR(t.m_max1);
+        LPMM_REQUIRE_PTR(t.row);
+        LPMM_REQUIRE_PTR(t.col);
+        LPMM_REQUIRE_PTR(t.workspace);
+        LPMM_REQUIRE_ALIGN(t.p, 16);
+        LPMM_REQUIRE_ALIGN(t.g, 16);
+        LPMM_REQUIRE_ALIGN(t.m_codes, 4);
+        LPMM_REQUIRE_ALIGN(t.m_max1, 4);
+        LPMM_REQUIRE_ALIGN(t.row, 4);
+        LPMM_REQUIRE_ALIGN(t.col, 16);
+        LPMM_REQUIRE_ALIGN(t.workspace, 8);
+    }
+
+    const NfHyper c = make_nf_hyper(beta1, beta2, lr, weight_decay, eps, 1.0);
+    MultiFa args;
+    args.decay = c.decay;
+    args.w1 = c.w1;
+    args.b2 = c.b2;
+    args.w2 = c.w2;
+    args.eps = c.eps;
+    int64_t i = 0;
+    while (i < count) {
+        int k = 0;
+        uint64_t n_stats = 0, n_fin = 0, n_upd = 0;
+        args.start_stats[0] = args.start_fin[0] = args.start_upd[0] = 0;
+        while (i < count && k < kFaMax) {
+            const lpmm_factored_tensor &t = tensors[i];
+            const uint64_t ty = (uint64_t)((t.rows + kSRows - 1) / kSRows), tx = (uint64_t)((t.cols + kSCols - 1) / kSCols);
+            const uint64_t row_blocks = (uint64_t)((t.rows + kFThreads - 1) / kFThreads);
+            const uint64_t fin = row_blocks + (uint64_t)((t.cols + 63) / 64);
+            const uint64_t ux = (uint64_t)((t.cols + kFTile - 1) / kFTile);
+            if (n_stats + tx * ty > 0x7fffffffULL || n_fin + fin > 0x7fffffffULL ||
+                n_upd + ux * (uint64_t)t.rows > 0x7fffffffULL) {
+                if (k == 0)
+                    return LPMM_ERR_SIZE;  // cannot happen after the checks above
+                break;
+            }
+            TensorFa &d = args.t[k];
+            d.p = t.p;
+            d.g = t.g;
+            d.mc = t.m_codes;
+            d.ms = t.m_max1;
+            d.row = t.row;
+            d.col = t.col;
+            d.colpart = static_cast<double *>(t.workspace);
+            d.rowpart = d.colpart + ty * (uint64_t)t.cols;
+            d.rowblock = d.rowpart + tx * (uint64_t)t.rows;
+            d.mean = reinterpret_cast<float *>(d.rowblock + row_blocks);
+            d.R = t.rows;
+            d.C = t.cols;
+            d.n_padded = round_up(t.rows * t.cols, kFTile);
+            d.tiles_x = (uint32_t)tx;
+            d.tiles_y = (uint32_t)ty;
+            d.row_blocks = (uint32_t)row_blocks;
+            d.upd_x = (uint32_t)ux;
+            d.first_step = t.first_step != 0;
+            const NfHyper h = make_nf_hyper(beta1, beta2, lr, weight_decay, eps, t.step);
+            d.neg_step_size = h.neg_step_size;
+            d.bc2_sqrt = h.bc2_sqrt;
+            d.rbc2_sqrt = h.rbc2_sqrt;
+            n_stats += tx * ty;
+            n_fin += fin;
+            n_upd += ux * (uint64_t)t.rows;
+            ++k;
+            args.start_stats[k] = (uint32_t)n_stats;
+            args.start_fin[k] = (uint32_t)n_fin;
+            args.start_upd[k] = (uint32_t)n_upd;
+            ++i;
+        }
+        args.count = k;
+        for (int j = k + 1; j <= kFaMax; ++j) {
+            args.start_stats[j] = (uint32_t)n_stats;
+            args.start_fin[j] = (uint32_t)n_fin;
+            args.start_upd[j] = (uint32_t)n_upd;
+        }
+        hipStream_t s = (hipStream_t)stream;
+        hipLaunchKernelGGL(factored_partial_multi_kernel, dim3((uint32_t)n_stats), dim3(kFThreads), 0, s, args);
+        hipLaunchKernelGGL(factored_finalize_multi_kernel, dim3((uint32_t)n_fin), dim3(kFThreads), 0, s, args);
+        hipLaunchKernelGGL(factored_mean_multi_kernel, dim3((uint32_t)k), dim3(kWave), 0, s, args);
+        hipLaunchKernelGGL(factored_update_multi_kernel, dim3((uint32_t)n_upd), dim3(kFThreads), 0, s, args, qmap_m);
+        const int st = launch_status();
+        if (st != LPMM_OK)
+            return st;
+    }
+    return LPMM_OK;
 }

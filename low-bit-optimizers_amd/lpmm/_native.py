@@ -39,6 +39,7 @@ PROTOTYPES = {
     "lpmm_factored_workspace_bytes": (_i64, [_i64, _i64]),
     "lpmm_factored_stats": (_int, [_vp, _i64, _i64, _vp, _vp, _vp, _d, _vp, _vp]),
     "lpmm_factored_update": (_int, [_vp] * 8 + [_i64, _i64] + [_d] * 6 + [_int, _vp]),
+    "lpmm_factored_step_multi": (_int, [_vp, _i64, _vp] + [_d] * 5 + [_vp]),
     "lpmm_factored_update_fp32m": (_int, [_vp] * 6 + [_i64, _i64] + [_d] * 6 + [_vp]),
     "lpmm_selftest_arithmetic": (_int, [_vp, ctypes.c_uint32, ctypes.c_uint64, ctypes.c_uint32, _vp]),
 }
@@ -51,6 +52,9 @@ NONFUSED_RANK1_TENSOR = np.dtype([("p", "<u8"), ("g", "<u8"), ("m_codes", "<u8")
                                   ("v_codes", "<u8"), ("v_rowmax", "<u8"), ("v_colmax", "<u8"),
                                   ("v_rowmax_next", "<u8"), ("v_colmax_next", "<u8"), ("rows", "<i8"),
                                   ("cols", "<i8"), ("step", "<f4"), ("reserved", "<f4")])
+FACTORED_TENSOR = np.dtype([("p", "<u8"), ("g", "<u8"), ("m_codes", "<u8"), ("m_max1", "<u8"), ("row", "<u8"),
+                            ("col", "<u8"), ("workspace", "<u8"), ("rows", "<i8"), ("cols", "<i8"), ("step", "<f4"),
+                            ("first_step", "<i4")])
 ADAMW_FP32_TENSOR = np.dtype([("p", "<u8"), ("g", "<u8"), ("m", "<u8"), ("v", "<u8"), ("n", "<i8"),
                               ("step", "<f4"), ("reserved", "<f4")])
 

@@ -150,12 +150,13 @@ class AdamW(LowBitOptimizer):
         md_m = self.get_qmetadata_by_state_name("exp_avg")
         md_v = self.get_qmetadata_by_state_name("exp_avg_sq")
         quant, plain = {}, {}  # device -> list of records
+        factored_work = []
         for p, grad, state, factored in work:
             state["step"] += 1
             step = state["step"].item()
             if factored:
                 # the fused kernel does not cover the factored case (adamw.py:472-495)
-                self._factored_step(group, p, grad, state, step)
+                factored_work.append((p, grad, state, step))
                 continue
             en_m, en_v = self._enabled(p, state, "exp_avg"), self._enabled(p, state, "exp_avg_sq")
             if en_m != en_v:
@@ -198,6 +199,7 @@ class AdamW(LowBitOptimizer):
                     (p.data_ptr(), grad.data_ptr(), state["exp_avg"].data_ptr(), state["exp_avg_sq"].data_ptr(),
                      p.numel(), step, 0.0))
 
+        self._factored_steps(group, factored_work)
         lib = _native.lib()
         for (dev, qm_ptr, qv_ptr), records in quant.items():
             table = np.array(records, dtype=_native.ADAMW4BIT_TENSOR)
@@ -239,11 +241,12 @@ class AdamW(LowBitOptimizer):
         v_group128 = fits(md_v) and md_v["scale_type"] == "group" and md_v["gp_sz"] == 128
         v_rank1 = fits(md_v) and md_v["scale_type"] == "rank1"
         batched, batched_rank1, plain = {}, {}, {}
+        factored_work = []
         for p, grad, state, factored in work:
             state["step"] += 1
             step = state["step"].item()
             if factored:
-                self._factored_step(group, p, grad, state, step)
+                factored_work.append((p, grad, state, step))
                 continue
             self._check_fp32_cuda(p, grad)
             en_m, en_v = self._enabled(p, state, "exp_avg"), self._enabled(p, state, "exp_avg_sq")
@@ -271,6 +274,7 @@ class AdamW(LowBitOptimizer):
                 self._requantise(p, state, "exp_avg", m, md_m)
             if en_v:
                 self._requantise(p, state, "exp_avg_sq", v, md_v)
+        self._factored_steps(group, factored_work)
         for dev, records in plain.items():
             table = np.array(records, dtype=_native.ADAMW_FP32_TENSOR)
             with torch.cuda.device(dev):
@@ -378,6 +382,51 @@ class AdamW(LowBitOptimizer):
         qstate["overhead"].update(gen)
 
     # ---- factored second moment (lpmm/optim/adamw.py:579-627) ---------------------------
+    def _factored_steps(self, group, items):
+        """Factored tensors of a parameter group: 2-D tensors with a multiple of 128 columns and a
+        4-bit block-wise first moment go to the multi-tensor kernels together, the others one
+        by one."""
+        if not items:
+            return
+        beta1, beta2 = group["betas"]
+        lr, wd, eps = group["lr"], group["weight_decay"], group["eps"]
+        md_m = self.get_qmetadata_by_state_name("exp_avg")
+        m_fits = (md_m["scale_type"] == "group" and md_m["gp_sz"] == 128 and md_m["b"] == 4
+                  and md_m["round_type"] == "real-nearest")
+        lib = _native.lib()
+        batched = {}
+        for p, grad, state, step in items:
+            if not (m_fits and p.dim() == 2 and p.shape[1] % 128 == 0 and self._enabled(p, state, "exp_avg")):
+                self._factored_step(group, p, grad, state, step)
+                continue
+            self._check_fp32_cuda(p, grad)
+            rows, cols = p.shape
+            qstate = state["exp_avg_qstate"]
+            first = _is_placeholder(state["exp_avg"])
+            if first:
+                groups = p.numel() // 128
+                state["exp_avg"] = torch.empty((packed_nbytes(p.numel()),), dtype=torch.int8, device=p.device)
+                qstate["overhead"].clear()
+                qstate["overhead"].update({"dtype": p.dtype, "stride": p.stride(),
+                                           "max1": torch.empty((groups, 1), dtype=torch.float32, device=p.device),
+                                           "scaled_shape": torch.Size((groups, 128))})
+            key = (p.device, qstate["qmap"].data_ptr())
+            ws = (lib.lpmm_factored_workspace_bytes(rows, cols) + 255) // 256 * 256
+            batched.setdefault(key, []).append(
+                [p.data_ptr(), grad.data_ptr(), state["exp_avg"].data_ptr(), qstate["overhead"]["max1"].data_ptr(),
+                 state["exp_avg_sq_row"].data_ptr(), state["exp_avg_sq_col"].data_ptr(), ws, rows, cols, step,
+                 1 if first else 0])
+        for (dev, qm_ptr), records in batched.items():
+            with torch.cuda.device(dev):
+                work = torch.empty((sum(r[6] for r in records),), dtype=torch.uint8, device=dev)
+                offset = work.data_ptr()
+                for r in records:
+                    r[6], offset = offset, offset + r[6]
+                table = np.array([tuple(r) for r in records], dtype=_native.FACTORED_TENSOR)
+                st = lib.lpmm_factored_step_multi(table.ctypes.data, len(records), qm_ptr, beta1, beta2, lr, wd, eps,
+                                                  _native.current_stream(dev))
+            _native.check(st, "factored step")
+
     def _factored_step(self, group, p, grad, state, step):
         beta1, beta2 = group["betas"]
         lr, wd, eps = group["lr"], group["weight_decay"], group["eps"]

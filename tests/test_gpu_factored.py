@@ -124,6 +124,59 @@ def test_factored_step_matches_oracle(oracle, qmaps, shape):
         drow.copy_(torch.from_numpy(row)); dcol.copy_(torch.from_numpy(col)); dp.copy_(torch.from_numpy(p))
 
 
+def test_factored_step_multi_matches_oracle(oracle, qmaps):
+    """Statistics + update of many tensors per call (more than one launch group holds), each
+    with its own step count, against the oracle."""
+    from lpmm import _native
+
+    lib = _lib()
+    qm = qmaps[0]
+    dqm = to_dev(qm)
+    rng = np.random.default_rng(9)
+    shapes = [(64, 128), (1, 128), (33, 256), (513, 1024), (100, 2176), (300, 4224)]
+    shapes += [(int(r), 128 * int(cb)) for r, cb in zip(rng.integers(1, 120, 24), rng.integers(1, 4, 24))]
+    tensors = []
+    for r, c in shapes:
+        n = r * c
+        t = dict(r=r, c=c, n=n, p=(rng.standard_normal((r, c)) * 0.02).astype(np.float32),
+                 row=np.zeros(r, np.float32), col=np.zeros(c, np.float32), m_state=None,
+                 step0=int(rng.integers(0, 5)))
+        t["dp"], t["drow"], t["dcol"] = to_dev(t["p"]), to_dev(t["row"]), to_dev(t["col"])
+        t["codes"] = torch.full(((n + 2047) // 2048 * 1024 + 1,), 0x55, dtype=torch.uint8, device="cuda")
+        t["max1"] = torch.zeros(n // 128, dtype=torch.float32, device="cuda")
+        t["work"] = torch.empty(lib.lpmm_factored_workspace_bytes(r, c), dtype=torch.uint8, device="cuda")
+        tensors.append(t)
+    for it in range(1, 4):
+        grads, recs = [], []
+        for t in tensors:
+            g = (rng.standard_normal((t["r"], t["c"])) * 1e-3 * (1 + rng.random((t["r"], 1)) * 3)).astype(np.float32)
+            t["g"], t["dg"] = g, to_dev(g)
+            recs.append((t["dp"].data_ptr(), t["dg"].data_ptr(), t["codes"].data_ptr(), t["max1"].data_ptr(),
+                         t["drow"].data_ptr(), t["dcol"].data_ptr(), t["work"].data_ptr(), t["r"], t["c"],
+                         float(t["step0"] + it), 1 if it == 1 else 0))
+        table = np.array(recs, dtype=_native.FACTORED_TENSOR)
+        st = lib.lpmm_factored_step_multi(table.ctypes.data, len(recs), dqm.data_ptr(), H["beta1"], H["beta2"],
+                                          H["lr"], H["wd"], H["eps"], _stream())
+        assert st == 0, lib.lpmm_status_string(st)
+        torch.cuda.synchronize()
+        for t in tensors:
+            what = f'{t["r"]}x{t["c"]} iteration {it}'
+            row_mean, col_mean = oracle.factored_stats(t["g"])
+            mean_ref = oracle.factored_ema(t["row"], t["col"], row_mean, col_mean, H["beta2"])
+            m = (np.zeros(t["n"], np.float32) if t["m_state"] is None
+                 else oracle.dequant_group(t["m_state"][0], t["m_state"][1], qm, t["n"]))
+            oracle.factored_update(t["p"], t["g"], m, t["row"], t["col"], mean_ref, H["beta1"], H["beta2"], H["lr"],
+                                   H["wd"], H["eps"], float(t["step0"] + it))
+            t["m_state"] = oracle.quant_group(m, qm)
+            assert_rel(to_np(t["drow"]), t["row"], f"row {what}", tol=2e-7)
+            assert_rel(to_np(t["dcol"]), t["col"], f"col {what}", tol=2e-7)
+            assert_rel(to_np(t["dp"]), t["p"], f"p {what}")
+            np.testing.assert_array_equal(to_np(t["max1"]), t["m_state"][1], err_msg=what)
+            np.testing.assert_array_equal(to_np(t["codes"]), t["m_state"][0], err_msg=what)
+            t["drow"].copy_(torch.from_numpy(t["row"])); t["dcol"].copy_(torch.from_numpy(t["col"]))
+            t["dp"].copy_(torch.from_numpy(t["p"]))
+
+
 def test_factored_fp32m_matches_oracle(oracle):
     lib = _lib()
     r, c = 48, 64
