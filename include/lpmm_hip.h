@@ -126,8 +126,7 @@ int lpmm_unpack_nonlinear_4bit(const uint8_t *codes, const float *qmap, int64_t 
 
 /* vectorwise_quant with scale_type 'group' in one pass: per-group max|x| -> max1, x/max1,
  * code search, pack.  Replaces lpmm/functional.py:184-189 + :359-369 (abs, max, div, cat,
- * pack_nonlinear as separate passes).  gp_sz must be a multiple of 128 and a divisor of
- * 2048 or a multiple of it; codes: ceil(G*gp_sz/2048)*1024 + 1 bytes; max1: fp32[G],
+ * pack_nonlinear as separate passes).  gp_sz = 128 * 2^k, at most 4096; codes: ceil(G*gp_sz/2048)*1024 + 1 bytes; max1: fp32[G],
  * G = ceil(n/gp_sz). */
 int lpmm_quant_group(const float *x, int64_t n, int64_t gp_sz, const float *qmap, uint8_t *codes,
                      float *max1, void *stream);
@@ -152,6 +151,29 @@ int lpmm_quant_rank1(const float *x, int64_t rows, int64_t cols, const float *ro
 /* out[r,c] = qmap[code] * min(rowmax[r], colmax[c]).  Replaces lpmm/functional.py:97-106. */
 int lpmm_dequant_rank1(const uint8_t *codes, const float *rowmax, const float *colmax,
                        const float *qmap, int64_t rows, int64_t cols, float *out, void *stream);
+
+/* ---------------------------------------------------------------------------------------
+ * The same six operations for any code width 1..8 (lpmm/configs/default_{5,6,7,8}b.yml use
+ * 5..8).  Storage follows lpmm/cpp_extension/quantization_kernel.cu:592-601, :695-705:
+ * widths 1, 2, 4 pack 8/bits codes per byte (code j of a byte at bit j*bits), every other
+ * width stores one code per byte; arrays hold n_padded*storage_bits/8 + 1 bytes and must be
+ * 8-byte aligned.  qmap: 2^bits ascending floats.  Codes come from the reference's search
+ * (:397-427); for NaN it stores the all-ones code (packed) or 255 (one code per byte), which
+ * decodes here as map entry 2^bits - 1 (the reference would read past a shorter map).
+ * ------------------------------------------------------------------------------------- */
+int lpmm_pack_nonlinear(const float *x, const float *qmap, int bits, int64_t n_padded, uint8_t *out,
+                        void *stream);
+int lpmm_unpack_nonlinear(const uint8_t *codes, const float *qmap, int bits, int64_t n, float *out,
+                          void *stream);
+int lpmm_quant_group_bits(const float *x, int64_t n, int64_t gp_sz, const float *qmap, int bits,
+                          uint8_t *codes, float *max1, void *stream);
+int lpmm_dequant_group_bits(const uint8_t *codes, const float *max1, const float *qmap, int bits,
+                            int64_t n, int64_t gp_sz, float *out, void *stream);
+int lpmm_quant_rank1_bits(const float *x, int64_t rows, int64_t cols, const float *rowmax,
+                          const float *colmax, const float *qmap, int bits, uint8_t *codes, void *stream);
+int lpmm_dequant_rank1_bits(const uint8_t *codes, const float *rowmax, const float *colmax,
+                            const float *qmap, int bits, int64_t rows, int64_t cols, float *out,
+                            void *stream);
 
 /* ---------------------------------------------------------------------------------------
  * Non-fused step, elementwise part on fp32 m and v (already dequantised):

@@ -108,20 +108,22 @@ __global__ __launch_bounds__(kQThreads) void unpack4_kernel(const uint8_t *__res
 
 // ---------------------------------------------------------------------------------------
 // 'group' scaling: max|x| per gp_sz values, x / max, search, pack -- one pass.
-// rows_per_group = gp_sz / 128 in {1, 2, 4, 8, 16}.
+// rows_per_group = gp_sz / 128 in {1, 2, 4, 8, 16, 32}.
 // ---------------------------------------------------------------------------------------
-__global__ __launch_bounds__(kQThreads) void quant_group_kernel(const float *__restrict__ x, int64_t n,
-                                                                int rows_per_group,
-                                                                const float *__restrict__ qmap,
-                                                                uint8_t *__restrict__ codes,
-                                                                float *__restrict__ max1, int64_t n_groups,
-                                                                int64_t n_padded, bool vec)
+// THREADS: 256 (a workgroup covers one 2048-value pack group) or, for gp_sz 4096, 512.
+template <int THREADS>
+__global__ __launch_bounds__(THREADS) void quant_group_kernel(const float *__restrict__ x, int64_t n,
+                                                              int rows_per_group,
+                                                              const float *__restrict__ qmap,
+                                                              uint8_t *__restrict__ codes,
+                                                              float *__restrict__ max1, int64_t n_groups,
+                                                              int64_t n_padded, bool vec)
 {
     __shared__ __align__(16) uint32_t lds[kLdsBytes / 4];
-    __shared__ float s_row[kQThreads / 16];
+    __shared__ float s_row[THREADS / 16];
     lds_fill(lds, qmap, nullptr);
     const int kind = classify_map(qmap);
-    const int64_t base = ((int64_t)blockIdx.x * kQThreads + threadIdx.x) * kQElts;
+    const int64_t base = ((int64_t)blockIdx.x * THREADS + threadIdx.x) * kQElts;
     if (base == 0)
         codes[n_padded / 2] = 0;
     float v[kQElts];
@@ -152,7 +154,8 @@ __global__ __launch_bounds__(kQThreads) void quant_group_kernel(const float *__r
         const float z[kQElts] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
         w = encode8_plain(lds, kLdsQ0, kind, z);
     }
-    store_u32(reinterpret_cast<uint32_t *>(codes + (base >> 1)), w);
+    if (base < n_padded)  // a 512-thread workgroup may reach past the last pack group
+        store_u32(reinterpret_cast<uint32_t *>(codes + (base >> 1)), w);
 }
 
 __global__ __launch_bounds__(kQThreads) void dequant_group_kernel(const uint8_t *__restrict__ codes,
@@ -507,7 +510,7 @@ extern "C" int lpmm_quant_group(const float *x, int64_t n, int64_t gp_sz, const 
 {
     if (n <= 0)
         return LPMM_ERR_SIZE;
-    if (gp_sz < kGroup || gp_sz > kQTile || (gp_sz & (gp_sz - 1)) != 0)
+    if (gp_sz < kGroup || gp_sz > 2 * kQTile || (gp_sz & (gp_sz - 1)) != 0)
         return LPMM_ERR_SIZE;
     LPMM_REQUIRE_PTR(x);
     LPMM_REQUIRE_PTR(qmap);
@@ -522,8 +525,13 @@ extern "C" int lpmm_quant_group(const float *x, int64_t n, int64_t gp_sz, const 
     if (!tiles_ok(n_groups * gp_sz, kQTile, &tiles))
         return LPMM_ERR_SIZE;
     const int64_t n_padded = (int64_t)tiles * kQTile;
-    hipLaunchKernelGGL(quant_group_kernel, dim3(tiles), dim3(kQThreads), 0, (hipStream_t)stream, x, n,
-                       (int)(gp_sz / kGroup), qmap, codes, max1, n_groups, n_padded, aligned_to(x, 16));
+    if (gp_sz > kQTile)
+        hipLaunchKernelGGL(quant_group_kernel<2 * kQThreads>, dim3((tiles + 1) / 2), dim3(2 * kQThreads), 0,
+                           (hipStream_t)stream, x, n, (int)(gp_sz / kGroup), qmap, codes, max1, n_groups, n_padded,
+                           aligned_to(x, 16));
+    else
+        hipLaunchKernelGGL(quant_group_kernel<kQThreads>, dim3(tiles), dim3(kQThreads), 0, (hipStream_t)stream, x, n,
+                           (int)(gp_sz / kGroup), qmap, codes, max1, n_groups, n_padded, aligned_to(x, 16));
     return launch_status();
 }
 

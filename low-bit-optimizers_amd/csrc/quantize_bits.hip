@@ -1,0 +1,473 @@
+// Quantise / dequantise for every code width the reference's operators accept (1..8 bits),
+// non-stochastic.  lpmm/cpp_extension/quantization_kernel.cu:592-601, :695-705 choose the
+// storage: widths that divide 8 and are below 8 (1, 2, 4) pack 8/bits codes per byte, code j
+// of a byte at bit j*bits (:430-459, :604-628); every other width (3, 5, 6, 7, 8) stores one
+// code per byte (:516-533, :656-669).  Either way the packed array has one extra last byte
+// (:476, :550), written as 0 here.
+//
+// The 4-bit kernels of quantize.hip stay the fast path for the width the optimizers use by
+// default; these kernels serve the other widths (lpmm/configs/default_{5,6,7,8}b.yml) with the
+// same flattened work layout: a lane owns 8 consecutive values, a 256-thread workgroup one
+// 2048-value pack group.  The map (2^bits entries) sits in LDS and the code is found by the
+// reference's own search (upper bound, then the midpoint test, :397-427), so maps with
+// repeated entries behave as there.
+#include "lpmm_codec.hpp"
+
+namespace lpmm {
+
+constexpr int kBThreads = 256;
+constexpr int kBElts = 8;
+constexpr int kBTile = kBThreads * kBElts;  // 2048
+
+__device__ __forceinline__ int codes_per_byte(int bits) { return (bits == 1 || bits == 2 || bits == 4) ? 8 / bits : 1; }
+
+// the map, 2^bits floats, into LDS; the caller synchronises
+__device__ __forceinline__ void fill_map(float *lds_map, const float *__restrict__ qmap, int bits)
+{
+    for (int j = threadIdx.x; j < (1 << bits); j += blockDim.x)
+        lds_map[j] = qmap[j];
+}
+
+// quantize_bsearch<false> (quantization_kernel.cu:397-427) as the stored code: the reference
+// casts the int to uint8_t (one code per byte) or masks it (packed), so NaN (-1) becomes 255
+// or the all-ones code.
+__device__ __forceinline__ uint32_t search_code(const float *lds_map, int bits, float x)
+{
+    int lo = 0, hi = 1 << bits;
+    if (x <= lds_map[0])
+        return 0u;
+    if (lds_map[hi - 1] <= x)
+        return (uint32_t)(hi - 1);
+    while (lo < hi) {
+        const int mi = (lo + hi) >> 1;
+        if (lds_map[mi] <= x)
+            lo = mi + 1;
+        else
+            hi = mi;
+    }
+    if (lo == 0)  // only NaN gets here; the reference's read of qmap[-1] does not change its result
+        return codes_per_byte(bits) == 1 ? 255u : (1u << bits) - 1u;
+    const float mid = (lds_map[lo - 1] + lds_map[lo]) * 0.5f;
+    return (uint32_t)((mid < x) ? lo : lo - 1);
+}
+
+// codes of the lane's 8 values (base = index of the first, a multiple of 8) into the array
+__device__ __forceinline__ void store_codes(uint8_t *__restrict__ codes, int64_t base, int bits,
+                                            const uint32_t (&c)[kBElts])
+{
+    const int per = codes_per_byte(bits);
+    if (per == 1) {
+        uint2 w;
+        w.x = c[0] | (c[1] << 8) | (c[2] << 16) | (c[3] << 24);
+        w.y = c[4] | (c[5] << 8) | (c[6] << 16) | (c[7] << 24);
+        *reinterpret_cast<uint2 *>(codes + base) = w;
+    } else {
+        uint32_t w = 0;
+#pragma unroll
+        for (int k = 0; k < kBElts; ++k)
+            w |= c[k] << (k * bits);  // 8, 16 or 32 bits in all
+        if (per == 8)
+            codes[base >> 3] = (uint8_t)w;
+        else if (per == 4)
+            *reinterpret_cast<uint16_t *>(codes + (base >> 2)) = (uint16_t)w;
+        else
+            *reinterpret_cast<uint32_t *>(codes + (base >> 1)) = w;
+    }
+}
+
+// map entries of the lane's 8 codes.  One code per byte: the reference indexes the map with
+// the whole byte (quantization_kernel.cu:666-667), which for a 255 stored for NaN reads past a
+// map of fewer than 256 entries; here the index is reduced to the map's range.
+__device__ __forceinline__ void load_decode(const uint8_t *__restrict__ codes, int64_t base, int bits,
+                                            const float *lds_map, float (&v)[kBElts])
+{
+    const int per = codes_per_byte(bits);
+    const uint32_t mask = (1u << bits) - 1u;
+    if (per == 1) {
+        const uint2 w = *reinterpret_cast<const uint2 *>(codes + base);
+#pragma unroll
+        for (int k = 0; k < kBElts; ++k)
+            v[k] = lds_map[(((k < 4 ? w.x : w.y) >> (8 * (k & 3))) & 0xFFu) & mask];
+    } else {
+        uint32_t w;
+        if (per == 8)
+            w = codes[base >> 3];
+        else if (per == 4)
+            w = *reinterpret_cast<const uint16_t *>(codes + (base >> 2));
+        else
+            w = *reinterpret_cast<const uint32_t *>(codes + (base >> 1));
+#pragma unroll
+        for (int k = 0; k < kBElts; ++k)
+            v[k] = lds_map[(w >> (k * bits)) & mask];
+    }
+}
+
+__device__ __forceinline__ void load_values(const float *__restrict__ x, int64_t base, int64_t n, bool vec,
+                                            float (&v)[kBElts])
+{
+    if (vec && base + kBElts <= n) {
+        const float4 a = load4(x + base), b = load4(x + base + 4);
+        v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+        v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+    } else {
+#pragma unroll
+        for (int k = 0; k < kBElts; ++k)
+            v[k] = (base + k < n) ? x[base + k] : 0.0f;
+    }
+}
+
+__device__ __forceinline__ void store_values(float *__restrict__ out, int64_t base, int64_t n, bool vec,
+                                             const float (&v)[kBElts])
+{
+    if (vec && base + kBElts <= n) {
+        store4(out + base, make_float4(v[0], v[1], v[2], v[3]));
+        store4(out + base + 4, make_float4(v[4], v[5], v[6], v[7]));
+    } else {
+#pragma unroll
+        for (int k = 0; k < kBElts; ++k)
+            if (base + k < n)
+                out[base + k] = v[k];
+    }
+}
+
+// index of the extra last byte of an array of n_padded codes
+__device__ __forceinline__ int64_t last_byte(int64_t n_padded, int bits) { return n_padded / codes_per_byte(bits); }
+
+// pack_nonlinear: x holds n_padded values that are already normalised.
+__global__ __launch_bounds__(kBThreads) void pack_bits_kernel(const float *__restrict__ x,
+                                                              const float *__restrict__ qmap, int bits,
+                                                              int64_t n_padded, uint8_t *__restrict__ out, bool vec)
+{
+    __shared__ float lds_map[256];
+    fill_map(lds_map, qmap, bits);
+    __syncthreads();
+    const int64_t base = ((int64_t)blockIdx.x * kBThreads + threadIdx.x) * kBElts;
+    if (base == 0)
+        out[last_byte(n_padded, bits)] = 0;
+    if (base >= n_padded)
+        return;
+    float v[kBElts];
+    load_values(x, base, n_padded, vec, v);
+    uint32_t c[kBElts];
+#pragma unroll
+    for (int k = 0; k < kBElts; ++k)
+        c[k] = search_code(lds_map, bits, v[k]);
+    store_codes(out, base, bits, c);
+}
+
+// unpack_nonlinear: out[i] = qmap[code_i] for i < n (n a multiple of 8).
+__global__ __launch_bounds__(kBThreads) void unpack_bits_kernel(const uint8_t *__restrict__ codes,
+                                                                const float *__restrict__ qmap, int bits, int64_t n,
+                                                                float *__restrict__ out, bool vec)
+{
+    __shared__ float lds_map[256];
+    fill_map(lds_map, qmap, bits);
+    __syncthreads();
+    const int64_t base = ((int64_t)blockIdx.x * kBThreads + threadIdx.x) * kBElts;
+    if (base >= n)
+        return;
+    float v[kBElts];
+    load_decode(codes, base, bits, lds_map, v);
+    store_values(out, base, n, vec, v);
+}
+
+// 'group' scaling in one pass, any width.  THREADS as in quantize.hip's 4-bit kernel.
+template <int THREADS>
+__global__ __launch_bounds__(THREADS) void quant_group_bits_kernel(const float *__restrict__ x, int64_t n,
+                                                                   int rows_per_group,
+                                                                   const float *__restrict__ qmap, int bits,
+                                                                   uint8_t *__restrict__ codes,
+                                                                   float *__restrict__ max1, int64_t n_groups,
+                                                                   int64_t n_padded, bool vec)
+{
+    __shared__ float lds_map[256];
+    __shared__ float s_row[THREADS / 16];
+    fill_map(lds_map, qmap, bits);
+    const int64_t base = ((int64_t)blockIdx.x * THREADS + threadIdx.x) * kBElts;
+    if (base == 0)
+        codes[last_byte(n_padded, bits)] = 0;
+    float v[kBElts];
+    load_values(x, base, n, vec, v);  // zero beyond n: the reference's zero padding
+    float amax = 0.0f;
+#pragma unroll
+    for (int k = 0; k < kBElts; ++k)
+        amax = fmaxf(amax, fabsf(v[k]));
+    amax = row16_max(amax);
+    if ((threadIdx.x & 15) == 0)
+        s_row[threadIdx.x >> 4] = amax;
+    __syncthreads();
+    if (rows_per_group > 1) {
+        const int first = (threadIdx.x >> 4) & ~(rows_per_group - 1);
+        amax = s_row[first];
+        for (int r = 1; r < rows_per_group; ++r)
+            amax = fmaxf(amax, s_row[first + r]);
+    }
+    if (base >= n_padded)
+        return;
+    const int64_t gp_sz = (int64_t)rows_per_group * kGroup;
+    const int64_t grp = base / gp_sz;
+    uint32_t c[kBElts];
+    if (grp < n_groups) {
+        if ((base % gp_sz) == 0)
+            max1[grp] = amax;
+#pragma unroll
+        for (int k = 0; k < kBElts; ++k)
+            c[k] = search_code(lds_map, bits, v[k] / amax);
+    } else {
+        // padding added by the re-grouping to 2048: plain zeros, not divided by anything
+        const uint32_t z = search_code(lds_map, bits, 0.0f);
+#pragma unroll
+        for (int k = 0; k < kBElts; ++k)
+            c[k] = z;
+    }
+    store_codes(codes, base, bits, c);
+}
+
+__global__ __launch_bounds__(kBThreads) void dequant_group_bits_kernel(const uint8_t *__restrict__ codes,
+                                                                       const float *__restrict__ max1,
+                                                                       const float *__restrict__ qmap, int bits,
+                                                                       int64_t n, int64_t gp_sz,
+                                                                       float *__restrict__ out, bool vec)
+{
+    __shared__ float lds_map[256];
+    fill_map(lds_map, qmap, bits);
+    __syncthreads();
+    const int64_t base = ((int64_t)blockIdx.x * kBThreads + threadIdx.x) * kBElts;
+    if (base >= n)
+        return;
+    float v[kBElts];
+    load_decode(codes, base, bits, lds_map, v);  // the array is padded: a whole word is always there
+    const float s = max1[base / gp_sz];          // gp_sz is a multiple of 128, so uniform over the lane's 8
+#pragma unroll
+    for (int k = 0; k < kBElts; ++k)
+        v[k] *= s;
+    store_values(out, base, n, vec, v);
+}
+
+// 'rank1' scaling of a row-major R x C tensor: normalise by min(rowmax[r], colmax[c]), search,
+// store.  A lane's 8 values may straddle rows.
+__global__ __launch_bounds__(kBThreads) void quant_rank1_bits_kernel(const float *__restrict__ x, int64_t n,
+                                                                     int64_t C, const float *__restrict__ rowmax,
+                                                                     const float *__restrict__ colmax,
+                                                                     const float *__restrict__ qmap, int bits,
+                                                                     uint8_t *__restrict__ codes, int64_t n_padded,
+                                                                     bool vec)
+{
+    __shared__ float lds_map[256];
+    fill_map(lds_map, qmap, bits);
+    __syncthreads();
+    const int64_t base = ((int64_t)blockIdx.x * kBThreads + threadIdx.x) * kBElts;
+    if (base == 0)
+        codes[last_byte(n_padded, bits)] = 0;
+    if (base >= n_padded)
+        return;
+    float v[kBElts];
+    load_values(x, base, n, vec, v);
+    int64_t r = base / C;
+    int64_t c = base - r * C;
+    float rm = (base < n) ? rowmax[r] : 0.0f;
+    uint32_t code[kBElts];
+#pragma unroll
+    for (int k = 0; k < kBElts; ++k) {
+        float xs = 0.0f;  // padding added by the re-grouping to 2048
+        if (base + k < n) {
+            const float cmx = colmax[c];
+            xs = v[k] / ((cmx < rm) ? cmx : rm);
+            if (++c == C) {
+                c = 0;
+                ++r;
+                rm = (base + k + 1 < n) ? rowmax[r] : 0.0f;
+            }
+        }
+        code[k] = search_code(lds_map, bits, xs);
+    }
+    store_codes(codes, base, bits, code);
+}
+
+__global__ __launch_bounds__(kBThreads) void dequant_rank1_bits_kernel(const uint8_t *__restrict__ codes,
+                                                                       const float *__restrict__ rowmax,
+                                                                       const float *__restrict__ colmax,
+                                                                       const float *__restrict__ qmap, int bits,
+                                                                       int64_t n, int64_t C, float *__restrict__ out,
+                                                                       bool vec)
+{
+    __shared__ float lds_map[256];
+    fill_map(lds_map, qmap, bits);
+    __syncthreads();
+    const int64_t base = ((int64_t)blockIdx.x * kBThreads + threadIdx.x) * kBElts;
+    if (base >= n)
+        return;
+    float v[kBElts];
+    load_decode(codes, base, bits, lds_map, v);
+    int64_t r = base / C;
+    int64_t c = base - r * C;
+    float rm = rowmax[r];
+#pragma unroll
+    for (int k = 0; k < kBElts; ++k) {
+        if (base + k < n) {
+            const float cmx = colmax[c];
+            v[k] *= (cmx < rm) ? cmx : rm;
+            if (++c == C) {
+                c = 0;
+                ++r;
+                rm = (base + k + 1 < n) ? rowmax[r] : 0.0f;
+            }
+        }
+    }
+    store_values(out, base, n, vec, v);
+}
+
+inline bool bits_ok(int bits) { return bits >= 1 && bits <= 8; }
+
+inline bool tiles_for(int64_t n, uint32_t *tiles)
+{
+    const int64_t t = (n + kBTile - 1) / kBTile;
+    if (t > 0x7fffffffLL)
+        return false;
+    *tiles = (uint32_t)t;
+    return true;
+}
+
+}  // namespace lpmm
+
+using namespace lpmm;
+
+extern "C" int lpmm_pack_nonlinear(const float *x, const float *qmap, int bits, int64_t n_padded, uint8_t *out,
+                                   void *stream)
+{
+    if (!bits_ok(bits) || n_padded <= 0 || (n_padded % 8) != 0)
+        return LPMM_ERR_SIZE;
+    LPMM_REQUIRE_PTR(x);
+    LPMM_REQUIRE_PTR(qmap);
+    LPMM_REQUIRE_PTR(out);
+    LPMM_REQUIRE_ALIGN(x, 4);
+    LPMM_REQUIRE_ALIGN(qmap, 4);
+    LPMM_REQUIRE_ALIGN(out, 8);
+    uint32_t tiles;
+    if (!tiles_for(n_padded, &tiles))
+        return LPMM_ERR_SIZE;
+    hipLaunchKernelGGL(pack_bits_kernel, dim3(tiles), dim3(kBThreads), 0, (hipStream_t)stream, x, qmap, bits,
+                       n_padded, out, aligned_to(x, 16));
+    return launch_status();
+}
+
+extern "C" int lpmm_unpack_nonlinear(const uint8_t *codes, const float *qmap, int bits, int64_t n, float *out,
+                                     void *stream)
+{
+    if (!bits_ok(bits) || n <= 0 || (n % 8) != 0)
+        return LPMM_ERR_SIZE;
+    LPMM_REQUIRE_PTR(codes);
+    LPMM_REQUIRE_PTR(qmap);
+    LPMM_REQUIRE_PTR(out);
+    LPMM_REQUIRE_ALIGN(codes, 8);
+    LPMM_REQUIRE_ALIGN(qmap, 4);
+    LPMM_REQUIRE_ALIGN(out, 4);
+    uint32_t tiles;
+    if (!tiles_for(n, &tiles))
+        return LPMM_ERR_SIZE;
+    hipLaunchKernelGGL(unpack_bits_kernel, dim3(tiles), dim3(kBThreads), 0, (hipStream_t)stream, codes, qmap, bits,
+                       n, out, aligned_to(out, 16));
+    return launch_status();
+}
+
+extern "C" int lpmm_quant_group_bits(const float *x, int64_t n, int64_t gp_sz, const float *qmap, int bits,
+                                     uint8_t *codes, float *max1, void *stream)
+{
+    if (!bits_ok(bits) || n <= 0)
+        return LPMM_ERR_SIZE;
+    if (gp_sz < kGroup || gp_sz > 2 * kBTile || (gp_sz & (gp_sz - 1)) != 0)
+        return LPMM_ERR_SIZE;
+    LPMM_REQUIRE_PTR(x);
+    LPMM_REQUIRE_PTR(qmap);
+    LPMM_REQUIRE_PTR(codes);
+    LPMM_REQUIRE_PTR(max1);
+    LPMM_REQUIRE_ALIGN(x, 4);
+    LPMM_REQUIRE_ALIGN(qmap, 4);
+    LPMM_REQUIRE_ALIGN(max1, 4);
+    LPMM_REQUIRE_ALIGN(codes, 8);
+    const int64_t n_groups = (n + gp_sz - 1) / gp_sz;
+    uint32_t tiles;
+    if (!tiles_for(n_groups * gp_sz, &tiles))
+        return LPMM_ERR_SIZE;
+    const int64_t n_padded = (int64_t)tiles * kBTile;
+    if (gp_sz > kBTile)
+        hipLaunchKernelGGL(quant_group_bits_kernel<2 * kBThreads>, dim3((tiles + 1) / 2), dim3(2 * kBThreads), 0,
+                           (hipStream_t)stream, x, n, (int)(gp_sz / kGroup), qmap, bits, codes, max1, n_groups,
+                           n_padded, aligned_to(x, 16));
+    else
+        hipLaunchKernelGGL(quant_group_bits_kernel<kBThreads>, dim3(tiles), dim3(kBThreads), 0, (hipStream_t)stream,
+                           x, n, (int)(gp_sz / kGroup), qmap, bits, codes, max1, n_groups, n_padded,
+                           aligned_to(x, 16));
+    return launch_status();
+}
+
+extern "C" int lpmm_dequant_group_bits(const uint8_t *codes, const float *max1, const float *qmap, int bits,
+                                       int64_t n, int64_t gp_sz, float *out, void *stream)
+{
+    if (!bits_ok(bits) || n <= 0 || gp_sz < kGroup || (gp_sz % kGroup) != 0)
+        return LPMM_ERR_SIZE;
+    LPMM_REQUIRE_PTR(codes);
+    LPMM_REQUIRE_PTR(max1);
+    LPMM_REQUIRE_PTR(qmap);
+    LPMM_REQUIRE_PTR(out);
+    LPMM_REQUIRE_ALIGN(codes, 8);
+    LPMM_REQUIRE_ALIGN(max1, 4);
+    LPMM_REQUIRE_ALIGN(qmap, 4);
+    LPMM_REQUIRE_ALIGN(out, 4);
+    uint32_t tiles;
+    if (!tiles_for(n, &tiles))
+        return LPMM_ERR_SIZE;
+    hipLaunchKernelGGL(dequant_group_bits_kernel, dim3(tiles), dim3(kBThreads), 0, (hipStream_t)stream, codes, max1,
+                       qmap, bits, n, gp_sz, out, aligned_to(out, 16));
+    return launch_status();
+}
+
+extern "C" int lpmm_quant_rank1_bits(const float *x, int64_t rows, int64_t cols, const float *rowmax,
+                                     const float *colmax, const float *qmap, int bits, uint8_t *codes,
+                                     void *stream)
+{
+    if (!bits_ok(bits) || rows <= 0 || cols <= 0 || rows > INT64_MAX / cols)
+        return LPMM_ERR_SIZE;
+    LPMM_REQUIRE_PTR(x);
+    LPMM_REQUIRE_PTR(rowmax);
+    LPMM_REQUIRE_PTR(colmax);
+    LPMM_REQUIRE_PTR(qmap);
+    LPMM_REQUIRE_PTR(codes);
+    LPMM_REQUIRE_ALIGN(x, 4);
+    LPMM_REQUIRE_ALIGN(rowmax, 4);
+    LPMM_REQUIRE_ALIGN(colmax, 4);
+    LPMM_REQUIRE_ALIGN(qmap, 4);
+    LPMM_REQUIRE_ALIGN(codes, 8);
+    const int64_t n = rows * cols;
+    uint32_t tiles;
+    if (!tiles_for(n, &tiles))
+        return LPMM_ERR_SIZE;
+    hipLaunchKernelGGL(quant_rank1_bits_kernel, dim3(tiles), dim3(kBThreads), 0, (hipStream_t)stream, x, n, cols,
+                       rowmax, colmax, qmap, bits, codes, (int64_t)tiles * kBTile, aligned_to(x, 16));
+    return launch_status();
+}
+
+extern "C" int lpmm_dequant_rank1_bits(const uint8_t *codes, const float *rowmax, const float *colmax,
+                                       const float *qmap, int bits, int64_t rows, int64_t cols, float *out,
+                                       void *stream)
+{
+    if (!bits_ok(bits) || rows <= 0 || cols <= 0 || rows > INT64_MAX / cols)
+        return LPMM_ERR_SIZE;
+    LPMM_REQUIRE_PTR(codes);
+    LPMM_REQUIRE_PTR(rowmax);
+    LPMM_REQUIRE_PTR(colmax);
+    LPMM_REQUIRE_PTR(qmap);
+    LPMM_REQUIRE_PTR(out);
+    LPMM_REQUIRE_ALIGN(codes, 8);
+    LPMM_REQUIRE_ALIGN(rowmax, 4);
+    LPMM_REQUIRE_ALIGN(colmax, 4);
+    LPMM_REQUIRE_ALIGN(qmap, 4);
+    LPMM_REQUIRE_ALIGN(out, 4);
+    const int64_t n = rows * cols;
+    uint32_t tiles;
+    if (!tiles_for(n, &tiles))
+        return LPMM_ERR_SIZE;
+    hipLaunchKernelGGL(dequant_rank1_bits_kernel, dim3(tiles), dim3(kBThreads), 0, (hipStream_t)stream, codes, rowmax,
+                       colmax, qmap, bits, n, cols, out, aligned_to(out, 16));
+    return launch_status();
+}

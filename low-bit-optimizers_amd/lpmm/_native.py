@@ -32,6 +32,12 @@ PROTOTYPES = {
     "lpmm_rank1_stats": (_int, [_vp, _i64, _i64, _vp, _vp, _vp]),
     "lpmm_quant_rank1": (_int, [_vp, _i64, _i64, _vp, _vp, _vp, _vp, _vp]),
     "lpmm_dequant_rank1": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _vp, _vp]),
+    "lpmm_pack_nonlinear": (_int, [_vp, _vp, _int, _i64, _vp, _vp]),
+    "lpmm_unpack_nonlinear": (_int, [_vp, _vp, _int, _i64, _vp, _vp]),
+    "lpmm_quant_group_bits": (_int, [_vp, _i64, _i64, _vp, _int, _vp, _vp, _vp]),
+    "lpmm_dequant_group_bits": (_int, [_vp, _vp, _vp, _int, _i64, _i64, _vp, _vp]),
+    "lpmm_quant_rank1_bits": (_int, [_vp, _i64, _i64, _vp, _vp, _vp, _int, _vp, _vp]),
+    "lpmm_dequant_rank1_bits": (_int, [_vp, _vp, _vp, _vp, _int, _i64, _i64, _vp, _vp]),
     "lpmm_nonfused_update": (_int, [_vp] * 4 + [_i64] + [_d] * 6 + [_vp]),
     "lpmm_nonfused_update_multi": (_int, [_vp, _i64] + [_d] * 5 + [_vp]),
     "lpmm_nonfused_adamw4bit_step_multi": (_int, [_vp, _i64, _vp, _vp] + [_d] * 5 + [_vp]),

@@ -1,5 +1,5 @@
 """lpmm.cpp_extension.quantization: pack_nonlinear / unpack_nonlinear of the reference's
-pybind module (lpmm/cpp_extension/quantization.cc:54-83) for 4-bit, round-to-nearest codes.
+pybind module (lpmm/cpp_extension/quantization.cc:54-83) for round-to-nearest codes of 1..8 bits.
 Both allocate and return a new tensor on the input's device and leave the inputs untouched."""
 import torch
 
@@ -9,33 +9,44 @@ from ._checks import check_cuda_tensor_dim_float, check_cuda_tensor_dim_type, sa
 __all__ = ["pack_nonlinear", "unpack_nonlinear"]
 
 
-def _require_4bit(bits):
+def _check_bits(bits, qmap):
     if bits > 8:
         raise RuntimeError("Expected bits <= 8 to be true, but got false.")
-    if bits != 4:
-        raise NotImplementedError(f"this build packs 4-bit codes only, got bits={bits}")
+    if bits < 1:
+        raise RuntimeError(f"bits must be at least 1, got {bits}")
+    if qmap.numel() < 2 ** bits:
+        raise RuntimeError(f"{bits}-bit quantisation maps must have {2 ** bits} entries, got {qmap.numel()}")
+
+
+def _storage_bits(bits):
+    # widths that divide 8 are packed, the others take a byte per code
+    # (lpmm/cpp_extension/quantization_kernel.cu:592-601)
+    return bits if bits in (1, 2, 4) else 8
 
 
 def pack_nonlinear(data, qmap, bits, stochastic):
     """data: float32 (num_groups, group_size), already normalised.  Returns int8 of
-    bits*numel/8 + 1 bytes (lpmm/cpp_extension/quantization_kernel.cu:475-477); the final byte,
+    storage_bits*numel/8 + 1 bytes (lpmm/cpp_extension/quantization_kernel.cu:475-477, :549-550; storage_bits
+    is `bits` for 1, 2 and 4 and 8 otherwise); the final byte,
     left uninitialised by the reference, is 0.  Unlike the reference this does not touch
     torch's default random generator."""
-    _require_4bit(bits)
     check_cuda_tensor_dim_float(data, "data", 2)
     check_cuda_tensor_dim_float(qmap, "qmap", 1)
+    _check_bits(bits, qmap)
     if stochastic:
         raise NotImplementedError("stochastic rounding is not part of this build")
-    if data.size(1) % 8 != 0:
+    if data.size(1) % (4 * (8 // _storage_bits(bits))) != 0 or data.numel() % 8 != 0:
         raise RuntimeError("Expected group_size % work_per_thread == 0 to be true, but got false.")
-    if qmap.numel() != 16:
-        raise RuntimeError("4-bit quantisation maps must have 16 entries")
     dev = same_device(data, qmap)
     n = data.numel()
-    out = torch.empty((n // 2 + 1,), dtype=torch.int8, device=dev)
+    out = torch.empty((n * _storage_bits(bits) // 8 + 1,), dtype=torch.int8, device=dev)
     with torch.cuda.device(dev):
-        st = _native.lib().lpmm_pack_nonlinear_4bit(data.data_ptr(), qmap.data_ptr(), n, out.data_ptr(),
-                                                    _native.current_stream(dev))
+        if bits == 4:
+            st = _native.lib().lpmm_pack_nonlinear_4bit(data.data_ptr(), qmap.data_ptr(), n, out.data_ptr(),
+                                                        _native.current_stream(dev))
+        else:
+            st = _native.lib().lpmm_pack_nonlinear(data.data_ptr(), qmap.data_ptr(), bits, n, out.data_ptr(),
+                                                   _native.current_stream(dev))
     _native.check(st, "pack_nonlinear")
     return out
 
@@ -43,18 +54,23 @@ def pack_nonlinear(data, qmap, bits, stochastic):
 def unpack_nonlinear(data, qmap, bits, num_groups, group_size):
     """data: int8 1-D packed codes.  Returns float32 (num_groups, group_size) of qmap[code]
     (lpmm/cpp_extension/quantization_kernel.cu:604-653)."""
-    _require_4bit(bits)
     check_cuda_tensor_dim_type(data, "data", 1, torch.int8)
     check_cuda_tensor_dim_float(qmap, "qmap", 1)
+    _check_bits(bits, qmap)
     n = int(num_groups) * int(group_size)
-    if data.numel() * 2 < n:
-        raise RuntimeError(f"packed data holds {data.numel() * 2} codes, fewer than the {n} requested")
-    if qmap.numel() != 16:
-        raise RuntimeError("4-bit quantisation maps must have 16 entries")
+    held = data.numel() * 8 // _storage_bits(bits)
+    if held < n:
+        raise RuntimeError(f"packed data holds {held} codes, fewer than the {n} requested")
+    if n % 8 != 0:
+        raise RuntimeError("Expected group_size % work_per_thread == 0 to be true, but got false.")
     dev = same_device(data, qmap)
     out = torch.empty((int(num_groups), int(group_size)), dtype=qmap.dtype, device=dev)
     with torch.cuda.device(dev):
-        st = _native.lib().lpmm_unpack_nonlinear_4bit(data.data_ptr(), qmap.data_ptr(), n, out.data_ptr(),
-                                                      _native.current_stream(dev))
+        if bits == 4:
+            st = _native.lib().lpmm_unpack_nonlinear_4bit(data.data_ptr(), qmap.data_ptr(), n, out.data_ptr(),
+                                                          _native.current_stream(dev))
+        else:
+            st = _native.lib().lpmm_unpack_nonlinear(data.data_ptr(), qmap.data_ptr(), bits, n, out.data_ptr(),
+                                                     _native.current_stream(dev))
     _native.check(st, "unpack_nonlinear")
     return out

@@ -3,10 +3,11 @@
 Same functions and keyword protocol as the slice of lpmm/functional.py the optimizer uses:
 `vectorwise_quant(x, **kw) -> (packed int8, metadata)` (lpmm/functional.py:26-59),
 `vectorwise_dequant(qx, **kw) -> x` (:62-151) and `create_general_qmap` (:244-268), for
-4-bit codes, 'real-nearest' rounding and the scale types 'group' and 'rank1'.  The packed
-layout and the metadata dict are the reference's: int8[NG*1024 + 1] with two codes per byte
-(low nibble = even index), `max1` of shape (G, 1) for 'group', `max_dims` for 'rank1',
-`scaled_shape`, `dtype`, `stride`.
+1..8-bit codes (4-bit is the optimizers' default and the fast path), 'real-nearest' rounding
+and the scale types 'group' and 'rank1'.  The packed layout and the metadata dict are the
+reference's: for 4 bits int8[NG*1024 + 1] with two codes per byte (low nibble = even index),
+for widths that do not divide 8 one code per byte; `max1` of shape (G, 1) for 'group',
+`max_dims` for 'rank1', `scaled_shape`, `dtype`, `stride`.
 
 Where the reference chains abs / max / div / cat / pack (and unpack / mul) as separate
 passes, each call here is one HIP kernel (two for rank-1 quantisation: statistics, then
@@ -171,8 +172,8 @@ def _select_qmap(kwargs):
 def _require_supported(kwargs, x):
     if kwargs["quant_type"] not in _NONLINEAR_TYPES:
         raise ValueError(f"Not support {kwargs['quant_type']} quant type.")
-    if kwargs["b"] != 4:
-        raise NotImplementedError(f"{kwargs['b']}-bit states: this build implements the 4-bit path only")
+    if not 1 <= kwargs["b"] <= 8:
+        raise ValueError(f"code width must be 1..8 bits, got {kwargs['b']}")
     if not kwargs["round_type"].startswith("real-nearest"):
         raise NotImplementedError(
             f"round_type {kwargs['round_type']!r}: this build implements 'real-nearest' only")
@@ -180,42 +181,59 @@ def _require_supported(kwargs, x):
         raise RuntimeError("x must be a CUDA tensor! (the quantised optimizer path has no CPU implementation)")
 
 
-def packed_nbytes(numel_scaled):
-    """Bytes of the packed tensor for numel_scaled normalised values."""
-    return (numel_scaled + PACK_GROUP - 1) // PACK_GROUP * (PACK_GROUP // 2) + 1
+def storage_bits(b):
+    """Bits a code occupies in the packed tensor: widths that divide 8 (1, 2, 4) are packed,
+    every other width takes a whole byte (lpmm/cpp_extension/quantization_kernel.cu:592-601)."""
+    return b if b in (1, 2, 4) else 8
+
+
+def packed_nbytes(numel_scaled, b=4):
+    """Bytes of the packed tensor for numel_scaled normalised values of b-bit codes."""
+    return (numel_scaled + PACK_GROUP - 1) // PACK_GROUP * (PACK_GROUP * storage_bits(b) // 8) + 1
 
 
 def _group_gp_sz_ok(gp_sz):
-    return gp_sz in (128, 256, 512, 1024, 2048)
+    return gp_sz in (128, 256, 512, 1024, 2048, 4096)
 
 
-def quant_group_(x, qmap, gp_sz, codes=None, max1=None):
+def quant_group_(x, qmap, gp_sz, codes=None, max1=None, b=4):
     """'group' scaling in one kernel.  x: contiguous float32 CUDA tensor.  Optionally writes
     into caller-owned `codes` / `max1` buffers of the right size."""
     n = x.numel()
     groups = (n + gp_sz - 1) // gp_sz
     if codes is None:
-        codes = torch.empty((packed_nbytes(groups * gp_sz),), dtype=torch.int8, device=x.device)
+        codes = torch.empty((packed_nbytes(groups * gp_sz, b),), dtype=torch.int8, device=x.device)
     if max1 is None:
         max1 = torch.empty((groups, 1), dtype=torch.float32, device=x.device)
+    lib = _native.lib()
     with torch.cuda.device(x.device):
-        st = _native.lib().lpmm_quant_group(x.data_ptr(), n, gp_sz, qmap.data_ptr(), codes.data_ptr(),
-                                            max1.data_ptr(), _native.current_stream(x.device))
+        stream = _native.current_stream(x.device)
+        if b == 4:
+            st = lib.lpmm_quant_group(x.data_ptr(), n, gp_sz, qmap.data_ptr(), codes.data_ptr(), max1.data_ptr(),
+                                      stream)
+        else:
+            st = lib.lpmm_quant_group_bits(x.data_ptr(), n, gp_sz, qmap.data_ptr(), b, codes.data_ptr(),
+                                           max1.data_ptr(), stream)
     _native.check(st, "quant_group")
     return codes, max1
 
 
-def quant_rank1_(x, qmap, codes=None):
+def quant_rank1_(x, qmap, codes=None, b=4):
     """'rank1' scaling of a contiguous 2-D float32 CUDA tensor: statistics kernel, then
     normalise + search + pack kernel."""
     rows, cols = x.shape
     max_dims = get_sm3_statistics(x)
     if codes is None:
-        codes = torch.empty((packed_nbytes(rows * cols),), dtype=torch.int8, device=x.device)
+        codes = torch.empty((packed_nbytes(rows * cols, b),), dtype=torch.int8, device=x.device)
+    lib = _native.lib()
     with torch.cuda.device(x.device):
-        st = _native.lib().lpmm_quant_rank1(x.data_ptr(), rows, cols, max_dims[0].data_ptr(),
-                                            max_dims[1].data_ptr(), qmap.data_ptr(), codes.data_ptr(),
-                                            _native.current_stream(x.device))
+        stream = _native.current_stream(x.device)
+        if b == 4:
+            st = lib.lpmm_quant_rank1(x.data_ptr(), rows, cols, max_dims[0].data_ptr(), max_dims[1].data_ptr(),
+                                      qmap.data_ptr(), codes.data_ptr(), stream)
+        else:
+            st = lib.lpmm_quant_rank1_bits(x.data_ptr(), rows, cols, max_dims[0].data_ptr(), max_dims[1].data_ptr(),
+                                           qmap.data_ptr(), b, codes.data_ptr(), stream)
     _native.check(st, "quant_rank1")
     return codes, max_dims
 
@@ -231,25 +249,26 @@ def vectorwise_quant(x, **kwargs):
         raise NotImplementedError(f"{src.dtype} states: this build implements the fp32 path only")
     src = src.contiguous()
     scale_type = kwargs["scale_type"]
+    b = kwargs["b"]
     as_group = scale_type == "group" or (scale_type == "rank1" and src.dim() == 1)
     if scale_type == "rank1":
         md["dim"] = src.dim()
     if as_group:
         gp_sz = kwargs["gp_sz"] if scale_type == "group" else 128
         if _group_gp_sz_ok(gp_sz):
-            codes, max1 = quant_group_(src, qmap, gp_sz)
+            codes, max1 = quant_group_(src, qmap, gp_sz, b=b)
         else:  # any other group size: PyTorch reductions, HIP search + pack
             grouped = group_tensor(src, gp_sz)
             max1 = _max_reduce_except_dim(grouped.abs(), 0)
-            codes = nonlinear_quant(grouped.div(max1), qmap, 4, round_type="real-nearest")
+            codes = nonlinear_quant(grouped.div(max1), qmap, b, round_type="real-nearest")
         md["max1"] = max1
         md["scaled_shape"] = torch.Size((max1.shape[0], gp_sz))
     elif scale_type == "rank1":
         if src.dim() == 2:
-            codes, max_dims = quant_rank1_(src, qmap)
+            codes, max_dims = quant_rank1_(src, qmap, b=b)
         else:
             max_dims = get_sm3_statistics(src.abs())
-            codes = nonlinear_quant(src.div(_compute_sm3_scale_tensor(max_dims)), qmap, 4,
+            codes = nonlinear_quant(src.div(_compute_sm3_scale_tensor(max_dims)), qmap, b,
                                     round_type="real-nearest")
         md["max_dims"] = max_dims
         md["max1"] = None
@@ -269,9 +288,11 @@ def vectorwise_dequant(qx, denormalized=True, **kwargs):
     scale_type = kwargs["scale_type"]
     codes = qx.detach()
     dev = codes.device
+    b = kwargs["b"]
+    lib = _native.lib()
     as_group = scale_type == "group" or (scale_type == "rank1" and kwargs["dim"] == 1)
     if not denormalized:
-        return nonlinear_dequant(codes, qmap, 4, shape=scaled_shape, round_type=kwargs["round_type"])
+        return nonlinear_dequant(codes, qmap, b, shape=scaled_shape, round_type=kwargs["round_type"])
     if as_group:
         shape = kwargs["shape"]
         gp_sz = scaled_shape[1]
@@ -279,12 +300,16 @@ def vectorwise_dequant(qx, denormalized=True, **kwargs):
         if gp_sz % 128 == 0:
             x = torch.empty(shape, dtype=torch.float32, device=dev)
             with torch.cuda.device(dev):
-                st = _native.lib().lpmm_dequant_group(codes.data_ptr(), kwargs["max1"].data_ptr(),
-                                                      qmap.data_ptr(), n, gp_sz, x.data_ptr(),
-                                                      _native.current_stream(dev))
+                stream = _native.current_stream(dev)
+                if b == 4:
+                    st = lib.lpmm_dequant_group(codes.data_ptr(), kwargs["max1"].data_ptr(), qmap.data_ptr(), n,
+                                                gp_sz, x.data_ptr(), stream)
+                else:
+                    st = lib.lpmm_dequant_group_bits(codes.data_ptr(), kwargs["max1"].data_ptr(), qmap.data_ptr(),
+                                                     b, n, gp_sz, x.data_ptr(), stream)
             _native.check(st, "dequant_group")
         else:
-            x = nonlinear_dequant(codes, qmap, 4, shape=scaled_shape, round_type=kwargs["round_type"])
+            x = nonlinear_dequant(codes, qmap, b, shape=scaled_shape, round_type=kwargs["round_type"])
             x = recon_grouped_tensor(x.mul(kwargs["max1"]), shape)
     elif scale_type == "rank1":
         max_dims = kwargs["max_dims"]
@@ -292,12 +317,17 @@ def vectorwise_dequant(qx, denormalized=True, **kwargs):
             rows, cols = scaled_shape
             x = torch.empty(scaled_shape, dtype=torch.float32, device=dev)
             with torch.cuda.device(dev):
-                st = _native.lib().lpmm_dequant_rank1(codes.data_ptr(), max_dims[0].data_ptr(),
-                                                      max_dims[1].data_ptr(), qmap.data_ptr(), rows, cols,
-                                                      x.data_ptr(), _native.current_stream(dev))
+                stream = _native.current_stream(dev)
+                if b == 4:
+                    st = lib.lpmm_dequant_rank1(codes.data_ptr(), max_dims[0].data_ptr(), max_dims[1].data_ptr(),
+                                                qmap.data_ptr(), rows, cols, x.data_ptr(), stream)
+                else:
+                    st = lib.lpmm_dequant_rank1_bits(codes.data_ptr(), max_dims[0].data_ptr(),
+                                                     max_dims[1].data_ptr(), qmap.data_ptr(), b, rows, cols,
+                                                     x.data_ptr(), stream)
             _native.check(st, "dequant_rank1")
         else:
-            x = nonlinear_dequant(codes, qmap, 4, shape=scaled_shape, round_type=kwargs["round_type"])
+            x = nonlinear_dequant(codes, qmap, b, shape=scaled_shape, round_type=kwargs["round_type"])
             x = x.mul(_compute_sm3_scale_tensor(max_dims))
     else:
         raise NotImplementedError(f"scale_type {scale_type!r}: this build implements 'group' and 'rank1'")

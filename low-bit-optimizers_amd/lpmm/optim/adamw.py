@@ -164,6 +164,11 @@ class AdamW(LowBitOptimizer):
                                  f"unquantized simultaneously, but get ({en_m} {en_v})")
             self._check_fp32_cuda(p, grad)
             if en_m:
+                if md_m["b"] != 4 or md_v["b"] != 4:
+                    # the reference's fused kernel reads and writes 4-bit codes whatever the
+                    # configuration says (fused_adamw_kernel.cu:113, :157); refuse instead
+                    raise ValueError("fused=True supports 4-bit states only; use fused=False for "
+                                     f"{md_m['b']}-bit exp_avg / {md_v['b']}-bit exp_avg_sq")
                 if md_m["scale_type"] != "group":
                     print("Warning: fused_adamw4bit only support block-wise scaling, but get exp_avg "
                           f"scale_type {md_m['scale_type']}.")

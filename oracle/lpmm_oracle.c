@@ -17,7 +17,9 @@
  * Parity status (what pins each function, apart from the HIP kernels being compared to it):
  *   qmapping            brute force against the closed form "number of fp32 midpoints < x",
  *                       every map point, every midpoint and its two neighbours, NaN, +-0.
- *   pack/unpack         exhaustive 256-byte round trip, length formulas, pad codes.
+ *   pack/unpack         exhaustive 256-byte round trip, length formulas, pad codes; the
+ *                       any-width versions additionally against the 4-bit ones at width 4
+ *                       and against a bit-by-bit Python restatement for widths 1..8.
  *   adamw_fp32_step     torch.optim.AdamW (library routine) over 100 steps.
  *   adamw4bit_step      closed form of the first step from zero state; equals
  *                       adamw_fp32_step when the state is representable; one-cell bound.
@@ -101,6 +103,61 @@ void lpmm_oracle_unpack_nonlinear_4bit(const uint8_t *codes, const float *qmap, 
 #pragma omp parallel for schedule(static)
     for (int64_t i = 0; i < n; ++i)
         out[i] = qmap[(codes[i >> 1] >> ((i & 1) * 4)) & 0xF];
+}
+
+/* ------------------------------------------------------------------------------------ */
+/* pack_nonlinear / unpack_nonlinear for any width 1..8, non-stochastic.                 */
+/* lpmm/cpp_extension/quantization_kernel.cu:592-601, :695-705 (dispatch on the width):  */
+/* widths that divide 8 and are below 8 go to the packing kernels (:430-459, :604-628:   */
+/* 8/bits codes per byte, code j masked and shifted by j*bits), every other width to the */
+/* one-code-per-byte kernels (:516-533: the int result cast to uint8_t, so -1 for NaN    */
+/* becomes 255; :656-669: qmap[byte]).  out holds n_padded*storage_bits/8 + 1 bytes, the */
+/* last one (uninitialised in the reference) written as 0.                               */
+/* The reference's unpack reads qmap[255] for a NaN code of a width below 8, past the    */
+/* end of the map; that read is undefined there and restated here as the map's last      */
+/* entry (index masked to the width).                                                    */
+/* ------------------------------------------------------------------------------------ */
+static inline int width_is_packed(int bits)
+{
+    return 8 % bits == 0 && bits < 8;
+}
+
+void lpmm_oracle_pack_nonlinear(const float *x, const float *qmap, int bits, int64_t n_padded,
+                                uint8_t *out)
+{
+    if (width_is_packed(bits)) {
+        const int per = 8 / bits;
+        const int mask = (1 << bits) - 1;
+#pragma omp parallel for schedule(static)
+        for (int64_t b = 0; b < n_padded / per; ++b) {
+            uint8_t byte = 0;
+            for (int j = 0; j < per; ++j)
+                byte |= (uint8_t)((lpmm_oracle_qmapping(qmap, bits, x[b * per + j]) & mask) << (j * bits));
+            out[b] = byte;
+        }
+        out[n_padded / per] = 0;
+    } else {
+#pragma omp parallel for schedule(static)
+        for (int64_t i = 0; i < n_padded; ++i)
+            out[i] = (uint8_t)lpmm_oracle_qmapping(qmap, bits, x[i]);
+        out[n_padded] = 0;
+    }
+}
+
+void lpmm_oracle_unpack_nonlinear(const uint8_t *codes, const float *qmap, int bits, int64_t n,
+                                  float *out)
+{
+    const int mask = (1 << bits) - 1;
+    if (width_is_packed(bits)) {
+        const int per = 8 / bits;
+#pragma omp parallel for schedule(static)
+        for (int64_t i = 0; i < n; ++i)
+            out[i] = qmap[(codes[i / per] >> ((i % per) * bits)) & mask];
+    } else {
+#pragma omp parallel for schedule(static)
+        for (int64_t i = 0; i < n; ++i)
+            out[i] = qmap[codes[i] & mask];
+    }
 }
 
 /* ------------------------------------------------------------------------------------ */

@@ -53,6 +53,8 @@ _qmapping = _sig("lpmm_oracle_qmapping", ctypes.c_int, _f32p, ctypes.c_int, _f)
 _qmapping_many = _sig("lpmm_oracle_qmapping_many", None, _f32p, _f32p, _i64, _u8p)
 _pack = _sig("lpmm_oracle_pack_nonlinear_4bit", None, _f32p, _f32p, _i64, _u8p)
 _unpack = _sig("lpmm_oracle_unpack_nonlinear_4bit", None, _u8p, _f32p, _i64, _f32p)
+_pack_bits = _sig("lpmm_oracle_pack_nonlinear", None, _f32p, _f32p, ctypes.c_int, _i64, _u8p)
+_unpack_bits = _sig("lpmm_oracle_unpack_nonlinear", None, _u8p, _f32p, ctypes.c_int, _i64, _f32p)
 _adamw_fp32 = _sig("lpmm_oracle_adamw_fp32_step", None, _f32p, _f32p, _f32p, _f32p, _i64,
                    _f, _f, _f, _f, _f, _f)
 _adamw4bit = _sig("lpmm_oracle_adamw4bit_step", None, _f32p, _f32p, _u8p, _u8p, _f32p, _f32p,
@@ -201,6 +203,64 @@ def unpack_nonlinear_4bit(codes, qmap, n):
     return out
 
 
+def storage_bits(bits):
+    """quantization_kernel.cu:592-601: widths 1, 2, 4 are packed, the others take a byte."""
+    return bits if bits in (1, 2, 4) else 8
+
+
+def pack_nonlinear(x, qmap, bits):
+    """Codes of already-normalised values, any width; x.size a multiple of 8."""
+    x = _c(x, np.float32).reshape(-1)
+    assert x.size % 8 == 0 and len(qmap) == 2 ** bits
+    out = np.empty(x.size * storage_bits(bits) // 8 + 1, dtype=np.uint8)
+    _pack_bits(x, _c(qmap, np.float32), bits, x.size, out)
+    return out
+
+
+def unpack_nonlinear(codes, qmap, bits, n):
+    out = np.empty(n, dtype=np.float32)
+    _unpack_bits(_c(codes, np.uint8), _c(qmap, np.float32), bits, n, out)
+    return out
+
+
+def _pad_to(x, multiple):
+    rem = (-x.size) % multiple
+    return np.concatenate([x, np.zeros(rem, np.float32)]) if rem else x
+
+
+def quant_group_bits(x, qmap, bits, gp_sz=GROUP):
+    """vectorwise_quant with 'group' scaling for any width, composed as the reference composes
+    it (lpmm/functional.py:184-189, :404-422, :359-369): zero-pad to whole groups, max|x| per
+    group, true division (0/0 -> NaN), zero-pad to whole 2048-value pack groups, pack."""
+    x = _c(x, np.float32).reshape(-1)
+    grouped = _pad_to(x, gp_sz).reshape(-1, gp_sz)
+    max1 = np.abs(grouped).max(axis=1).astype(np.float32)
+    with np.errstate(invalid="ignore", divide="ignore"):
+        normed = (grouped / max1[:, None]).astype(np.float32).reshape(-1)
+    return pack_nonlinear(_pad_to(normed, PACK_GROUP), qmap, bits), max1
+
+
+def dequant_group_bits(codes, max1, qmap, bits, n, gp_sz=GROUP):
+    """lpmm/functional.py:393-400, :115-118."""
+    g = max1.size
+    vals = unpack_nonlinear(codes, qmap, bits, g * gp_sz).reshape(g, gp_sz)
+    return (vals * _c(max1, np.float32).reshape(-1, 1)).astype(np.float32).reshape(-1)[:n]
+
+
+def quant_rank1_bits(x, rowmax, colmax, qmap, bits):
+    """lpmm/functional.py:190-203, :503-509 for any width."""
+    x = _c(x, np.float32)
+    st = np.where(colmax[None, :] < rowmax[:, None], colmax[None, :], rowmax[:, None]).astype(np.float32)
+    with np.errstate(invalid="ignore", divide="ignore"):
+        normed = (x / st).astype(np.float32).reshape(-1)
+    return pack_nonlinear(_pad_to(normed, PACK_GROUP), qmap, bits)
+
+
+def dequant_rank1_bits(codes, rowmax, colmax, qmap, bits, r, c):
+    st = np.where(colmax[None, :] < rowmax[:, None], colmax[None, :], rowmax[:, None]).astype(np.float32)
+    return (unpack_nonlinear(codes, qmap, bits, r * c).reshape(r, c) * st).astype(np.float32)
+
+
 def adamw_fp32_step(p, g, m, v, beta1, beta2, lr, wd, eps, step):
     _adamw_fp32(p, g, m, v, p.size, beta1, beta2, lr, wd, eps, step)
 
@@ -290,7 +350,8 @@ class NonFusedState:
     functional.py:32-34, :240): packed codes of NG*1024+1 bytes plus max1 (G,) for 'group'
     scaling or (rowmax, colmax) for 'rank1' on a 2-D tensor."""
 
-    def __init__(self, shape, v_scale_type="group", factored=False):
+    def __init__(self, shape, v_scale_type="group", factored=False, bits=4):
+        self.bits = bits  # code width of both moments (lpmm/configs/default_{5,6,7,8}b.yml)
         self.shape = tuple(shape)
         self.n = int(np.prod(self.shape))
         self.step = 0
@@ -314,23 +375,34 @@ def nonfused_step(p, g, state, qm, qv, lr, beta1, beta2, eps, wd):
     pf, gf = p.reshape(-1), np.ascontiguousarray(g, dtype=np.float32).reshape(-1)
     if state.factored:
         return _factored_step(p, g, state, qm, lr, beta1, beta2, eps, wd)
-    m = np.zeros(n, np.float32) if state.m is None else dequant_group(state.m[0], state.m[1], qm, n)
+    b = state.bits
+    if b == 4:
+        deq_g = lambda s, q: dequant_group(s[0], s[1], q, n)
+        deq_r = lambda s, q, r, c: dequant_rank1(s[0], s[1], s[2], q, r, c)
+        q_g = quant_group
+        q_r = quant_rank1
+    else:
+        deq_g = lambda s, q: dequant_group_bits(s[0], s[1], q, b, n)
+        deq_r = lambda s, q, r, c: dequant_rank1_bits(s[0], s[1], s[2], q, b, r, c)
+        q_g = lambda x, q: quant_group_bits(x, q, b)
+        q_r = lambda x, rm, cm, q: quant_rank1_bits(x, rm, cm, q, b)
+    m = np.zeros(n, np.float32) if state.m is None else deq_g(state.m, qm)
     if state.v is None:
         v = np.zeros(n, np.float32)
     elif _v_is_rank1(state):
         r, c = state.shape
-        v = dequant_rank1(state.v[0], state.v[1], state.v[2], qv, r, c).reshape(-1)
+        v = np.ascontiguousarray(deq_r(state.v, qv, r, c)).reshape(-1)
     else:
-        v = dequant_group(state.v[0], state.v[1], qv, n)
+        v = deq_g(state.v, qv)
     nonfused_update(pf, gf, m, v, beta1, beta2, lr, wd, eps, float(state.step))
-    state.m = quant_group(m, qm)
+    state.m = q_g(m, qm)
     if _v_is_rank1(state):
         r, c = state.shape
         v2 = v.reshape(r, c)
         rowmax, colmax = rank1_stats(v2)
-        state.v = (quant_rank1(v2, rowmax, colmax, qv), rowmax, colmax)
+        state.v = (q_r(v2, rowmax, colmax, qv), rowmax, colmax)
     else:
-        state.v = quant_group(v, qv)
+        state.v = q_g(v, qv)
     return m, v
 
 

@@ -54,7 +54,8 @@ def test_pack_unpack_match_oracle(oracle, qmaps, n):
 
 
 @pytest.mark.parametrize("n,gp_sz", [(4097, 128), (128 * 33, 128), (2048 * 7 + 100, 128), (4096 * 4096 // 16, 128),
-                                     (10000, 256), (2048 * 5 + 3, 512), (70000, 1024), (50000, 2048)])
+                                     (10000, 256), (2048 * 5 + 3, 512), (70000, 1024), (50000, 2048), (50000, 4096),
+                                     (4096 * 3, 4096), (100, 4096)])
 def test_quant_dequant_group(oracle, qmaps, n, gp_sz):
     lib = _lib()
     rng = np.random.default_rng(n + gp_sz)

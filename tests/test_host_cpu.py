@@ -62,7 +62,7 @@ def test_argument_errors_without_gpu():
     assert lib.lpmm_pack_nonlinear_4bit(None, ptr, 16, ptr, None) == NULL
     assert lib.lpmm_unpack_nonlinear_4bit(ptr, ptr, -5, ptr, None) == SIZE
     assert lib.lpmm_quant_group(ptr, 64, 100, ptr, ptr, ptr, None) == SIZE  # group size not 128 * 2^k
-    assert lib.lpmm_quant_group(ptr, 64, 4096, ptr, ptr, ptr, None) == SIZE
+    assert lib.lpmm_quant_group(ptr, 64, 8192, ptr, ptr, ptr, None) == SIZE
     assert lib.lpmm_quant_group(ptr, 0, 128, ptr, ptr, ptr, None) == SIZE
     assert lib.lpmm_dequant_group(ptr, ptr, ptr, 64, 64, ptr, None) == SIZE
     assert lib.lpmm_rank1_stats(ptr, 0, 8, ptr, ptr, None) == SIZE
