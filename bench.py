@@ -15,6 +15,8 @@ Two further workloads measure the other kernels of the path with the same JSON s
 `--workload nonfused_group|nonfused_rank1` (fused=False on the LLaMA-7B-shaped set).
 """
 import argparse
+import contextlib
+import gc
 import json
 import math
 import os
@@ -115,16 +117,29 @@ def cpu_baseline(torch, steps=3):
     }
 
 
+@contextlib.contextmanager
+def _gc_paused():
+    """A full collection of the interpreter's cyclic garbage collector takes 70-80 ms of host time
+    with torch loaded, several optimizer steps: collect first, keep it off inside a timed region."""
+    gc.collect()
+    gc.disable()
+    try:
+        yield
+    finally:
+        gc.enable()
+
+
 def _time_events(torch, fn, iters):
     for _ in range(2):
         fn()
     torch.cuda.synchronize()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for _ in range(iters):
-        fn()
-    e1.record()
-    torch.cuda.synchronize()
+    with _gc_paused():
+        e0.record()
+        for _ in range(iters):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
     return e0.elapsed_time(e1) / iters  # ms
 
 
@@ -191,11 +206,12 @@ def run_factored(torch, args):
     for _ in range(args.warmup):
         opt.step()
     torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        opt.step()
-    torch.cuda.synchronize()
-    dt = (time.perf_counter() - t0) / args.steps
+    with _gc_paused():
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            opt.step()
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - t0) / args.steps
     achieved = n_2d * 17.0625 / dt / 1e9
     print(json.dumps({
         "metric": "factored-second-moment 4-bit AdamW step: params/sec, 1 MI355X", "value": n_total / dt,
@@ -224,11 +240,12 @@ def run_nonfused(torch, args, v_scale):
     for _ in range(args.warmup):
         opt.step()
     torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        opt.step()
-    torch.cuda.synchronize()
-    dt = (time.perf_counter() - t0) / args.steps
+    with _gc_paused():
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            opt.step()
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - t0) / args.steps
     # one pass: p, g read, p written, two 4-bit codes read and written, scales;
     # rank-1 (two passes): + g and the v codes read a second time, v codes written in the second pass
     bytes_per_param = BYTES_PER_PARAM_4BIT if v_scale == "group" else 18.5625
@@ -316,11 +333,12 @@ def main():
         opt.step()
     torch.cuda.synchronize()
     recording["on"] = True
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        opt.step()
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
+    with _gc_paused():
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            opt.step()
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
     recording["on"] = False
 
     ms_per_step = elapsed * 1e3 / args.steps

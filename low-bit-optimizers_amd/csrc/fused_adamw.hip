@@ -28,6 +28,16 @@ constexpr int kThreads = 256;
 constexpr int kEltsPerLane = 8;
 constexpr int kTile = kThreads * kEltsPerLane;  // 2048 elements = 16 groups
 
+// LDS per workgroup.  The tables need kLdsBytes; the allocation is larger on purpose, so that
+// at most 5 workgroups (20 waves) are resident on a CU (160 KB of LDS).  With the 7 that the
+// registers would allow, the waves that are not computing all sit in the memory queues, and
+// the HBM system of MI355X sustains less with deeper queues: the bare access pattern of this
+// kernel runs at 5.9 TB/s with 8 resident workgroups per CU and at 6.2-6.4 TB/s with 3-5; the
+// kernel itself gains 3 % with 5 and loses with 4 (too few waves to cover the arithmetic).
+constexpr uint32_t kFusedLdsBytes = 30 * 1024;
+static_assert(kFusedLdsBytes >= kLdsBytes, "tables do not fit");
+static_assert(160 * 1024 / kFusedLdsBytes == 5, "residency cap");
+
 struct Tensor4 {
     float *p;
     const float *g;
@@ -98,9 +108,37 @@ static_assert(sizeof(Multi4) + 2 * sizeof(void *) <= 4096, "kernel arguments exc
 // One 128-element group, handled by the 16 lanes of a DPP row.  FULL: the whole group lies
 // inside the tensor and the pointers allow vector access; otherwise every access is
 // guarded per element.  All 16 lanes take the same instantiation.
+// The operands of a lane whose group lies wholly inside the tensor, as loaded from HBM.  The
+// loads are issued at the top of the kernel, before the LDS tables are set up, so that their
+// latency overlaps the prologue.
+struct GroupRegs {
+    float4 a0, a1, b0, b1;   // p, g
+    uint32_t m0, m1, v0, v1; // code half-words
+    float sm, sv;
+};
+
+__device__ __forceinline__ void group_load(const Tensor4 &t, int64_t grp, int lane16, GroupRegs &r)
+{
+    const int64_t gbase = grp * kGroup;
+    const float *pp = t.p + gbase + lane16 * 4;
+    const float *gp = t.g + gbase + lane16 * 4;
+    r.a0 = load4(pp);
+    r.a1 = load4(pp + 64);
+    r.b0 = load4(gp);
+    r.b1 = load4(gp + 64);
+    const uint16_t *mcp = reinterpret_cast<const uint16_t *>(t.mc + (gbase >> 1)) + lane16;
+    const uint16_t *vcp = reinterpret_cast<const uint16_t *>(t.vc + (gbase >> 1)) + lane16;
+    r.m0 = load_u16(mcp);
+    r.m1 = load_u16(mcp + 16);
+    r.v0 = load_u16(vcp);
+    r.v1 = load_u16(vcp + 16);
+    r.sm = t.ms[grp];
+    r.sv = t.vs[grp];
+}
+
 template <bool FULL, class Arith>
 __device__ __forceinline__ void group_step(const Tensor4 &t, const Arith &h, const uint32_t *lds,
-                                           bool std_maps, int64_t grp, int lane16)
+                                           bool std_maps, int64_t grp, int lane16, const GroupRegs &r)
 {
     const int64_t n = t.n;
     const int64_t gbase = grp * kGroup;
@@ -111,20 +149,14 @@ __device__ __forceinline__ void group_step(const Tensor4 &t, const Arith &h, con
     const bool any = FULL || Arith::kPadded || (gbase + lane16 * 4 < n);
 
     if (FULL) {
-        const float *pp = t.p + gbase + lane16 * 4;
-        const float *gp = t.g + gbase + lane16 * 4;
-        const float4 a0 = load4(pp), a1 = load4(pp + 64);
-        const float4 b0 = load4(gp), b1 = load4(gp + 64);
-        const uint16_t *mcp = reinterpret_cast<const uint16_t *>(t.mc + (gbase >> 1)) + lane16;
-        const uint16_t *vcp = reinterpret_cast<const uint16_t *>(t.vc + (gbase >> 1)) + lane16;
-        wm = load_u16(mcp) | (load_u16(mcp + 16) << 16);
-        wv = load_u16(vcp) | (load_u16(vcp + 16) << 16);
-        sm = t.ms[grp];
-        sv = t.vs[grp];
-        pv[0] = a0.x; pv[1] = a0.y; pv[2] = a0.z; pv[3] = a0.w;
-        pv[4] = a1.x; pv[5] = a1.y; pv[6] = a1.z; pv[7] = a1.w;
-        gv[0] = b0.x; gv[1] = b0.y; gv[2] = b0.z; gv[3] = b0.w;
-        gv[4] = b1.x; gv[5] = b1.y; gv[6] = b1.z; gv[7] = b1.w;
+        wm = r.m0 | (r.m1 << 16);
+        wv = r.v0 | (r.v1 << 16);
+        sm = r.sm;
+        sv = r.sv;
+        pv[0] = r.a0.x; pv[1] = r.a0.y; pv[2] = r.a0.z; pv[3] = r.a0.w;
+        pv[4] = r.a1.x; pv[5] = r.a1.y; pv[6] = r.a1.z; pv[7] = r.a1.w;
+        gv[0] = r.b0.x; gv[1] = r.b0.y; gv[2] = r.b0.z; gv[3] = r.b0.w;
+        gv[4] = r.b1.x; gv[5] = r.b1.y; gv[6] = r.b1.z; gv[7] = r.b1.w;
     } else if (any) {
         sm = t.ms[grp];
         sv = t.vs[grp];
@@ -207,23 +239,38 @@ __global__ __launch_bounds__(kThreads) void adamw4bit_kernel(const Multi4 args,
                                                              const float *__restrict__ qmap_m,
                                                              const float *__restrict__ qmap_v)
 {
-    __shared__ __align__(16) uint32_t lds[kLdsBytes / 4];
-    lds_fill(lds, qmap_m, qmap_v);
-    const bool std_maps = classify_map(qmap_m) == kMapStdM && classify_map(qmap_v) == kMapStdV;
+    __shared__ __align__(16) uint32_t lds[kFusedLdsBytes / 4];
+    // the small loads first: maps and encode table for LDS
+    const LdsFill fill = lds_fill_load(qmap_m, qmap_v);
 
     // which tensor does this tile belong to (uniform over the workgroup): the number of
     // later tensors whose first tile is not after this one; unused slots hold the total
     // (one entry per lane, one ballot per wave)
     static_assert(LPMM_MULTI_MAX <= kWave, "one tile_start entry per lane");
     const int lane = threadIdx.x & (kWave - 1);
-    const bool started = lane + 1 < LPMM_MULTI_MAX && args.tile_start[lane + 1] <= blockIdx.x;
+    // lanes past the last slot read the total, which no block index reaches
+    const int slot = lane + 1 < LPMM_MULTI_MAX ? lane + 1 : LPMM_MULTI_MAX;
+    const uint32_t first_tile = args.tile_start[slot];
+    // one wait covers the three small loads; the streaming loads below are issued after it
+    lds_fill_store(lds, fill);
+    const bool started = first_tile <= blockIdx.x;
     const int lo = __popcll(__ballot(started));
     const Tensor4 &t = args.t[lo];
     const int lane16 = threadIdx.x & 15;
     const int64_t grp = (int64_t)(blockIdx.x - args.tile_start[lo]) * (kTile / kGroup) + (threadIdx.x >> 4);
 
+    // a group that lies wholly inside its tensor starts its loads now; the waves wait only
+    // for their LDS writes at the barrier (no global access is ordered by it)
+    const bool full = ALIGNED && (grp + 1) * kGroup <= t.n;
+    GroupRegs regs;
+    regs.m0 = regs.m1 = regs.v0 = regs.v1 = 0;
+    if (full)
+        group_load(t, grp, lane16, regs);
+    const bool std_maps = classify_map(qmap_m) == kMapStdM && classify_map(qmap_v) == kMapStdV;
     const Arith h(args, t);
-    __syncthreads();
+    lds_barrier();
+    // the loaded words stay as they are until here, so that nothing above waits for them
+    asm volatile("" : "+v"(regs.m0), "+v"(regs.m1), "+v"(regs.v0), "+v"(regs.v1));
 
     if (Arith::kPadded && threadIdx.x == 0 && blockIdx.x + 1 == args.tile_start[lo + 1]) {
         // the tensor's last tile also owns the extra byte at the end of each code buffer
@@ -244,10 +291,10 @@ __global__ __launch_bounds__(kThreads) void adamw4bit_kernel(const Multi4 args,
         }
         return;
     }
-    if (ALIGNED && (grp + 1) * kGroup <= t.n)
-        group_step<true>(t, h, lds, std_maps, grp, lane16);
+    if (full)
+        group_step<true>(t, h, lds, std_maps, grp, lane16, regs);
     else
-        group_step<false>(t, h, lds, std_maps, grp, lane16);
+        group_step<false>(t, h, lds, std_maps, grp, lane16, regs);
 }
 
 // ---------------------------------------------------------------------------------------

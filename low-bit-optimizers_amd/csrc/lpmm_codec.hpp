@@ -94,6 +94,13 @@ constexpr uint32_t kLdsBytes = kEncLdsEnd;
 constexpr uint32_t kLdsQ0 = 0, kLdsQ1 = 64;
 static_assert(kLdsQ1 + 64 <= kEncLdsBegin, "maps overlap the encode table");
 
+// Workgroup barrier that orders LDS accesses only: the waves wait for their own LDS
+// operations, not for global loads that are still in flight.
+__device__ __forceinline__ void lds_barrier()
+{
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
 template <typename T>
 __device__ __forceinline__ T lds_read(const uint32_t *lds, uint32_t byte_off)
 {
@@ -113,6 +120,34 @@ __device__ __forceinline__ void lds_fill(uint32_t *lds, const float *__restrict_
         *reinterpret_cast<uint4 *>(reinterpret_cast<char *>(lds) + e.w) = e;  // e.w: the entry's LDS offset
     }
 }
+
+// The same in two halves, so that a kernel can issue these small loads first, start its
+// streaming loads, and write LDS once the small ones have arrived (loads return in order).
+struct LdsFill {
+    uint32_t q;
+    uint4 e;
+};
+
+__device__ __forceinline__ LdsFill lds_fill_load(const float *__restrict__ q0, const float *__restrict__ q1)
+{
+    // every thread loads (from a clamped index), so that no branch surrounds the loads
+    LdsFill f;
+    const uint32_t t = threadIdx.x;
+    const float *qp = (t < 16) ? q0 + t : q1 + (t & 15);
+    f.q = __float_as_uint(*qp);
+    const uint32_t te = t < 2 * kEncBuckets ? t : 2 * kEncBuckets - 1;
+    f.e = *reinterpret_cast<const uint4 *>(kEncTableM[te]);
+    return f;
+}
+
+__device__ __forceinline__ void lds_fill_store(uint32_t *lds, const LdsFill &f)
+{
+    if (threadIdx.x < 32)
+        lds[threadIdx.x] = f.q;  // kLdsQ0 = 0, kLdsQ1 = 64: the two maps are adjacent
+    if (threadIdx.x < 2 * kEncBuckets)
+        *reinterpret_cast<uint4 *>(reinterpret_cast<char *>(lds) + f.e.w) = f.e;
+}
+static_assert(kLdsQ0 == 0 && kLdsQ1 == 64, "lds_fill_store writes the maps back to back");
 
 // Codes of 8 already divided values with the standard first-moment map: nibble k = code of x[k].
 __device__ __forceinline__ uint32_t encode8_std_m(const uint32_t *lds, const float (&x)[8])
