@@ -110,8 +110,15 @@ __global__ __launch_bounds__(kQThreads) void unpack4_kernel(const uint8_t *__res
 // 'group' scaling: max|x| per gp_sz values, x / max, search, pack -- one pass.
 // rows_per_group = gp_sz / 128 in {1, 2, 4, 8, 16, 32}.
 // ---------------------------------------------------------------------------------------
-// THREADS: 256 (a workgroup covers one 2048-value pack group) or, for gp_sz 4096, 512.
-template <int THREADS>
+// THREADS: 256 (a tile is one 2048-value pack group) or, for gp_sz 4096, 512; a workgroup
+// handles T consecutive tiles, so that the set-up of the LDS tables is paid once per T tiles.
+// A workgroup whose values all lie inside the tensor (and whose operands allow vector access)
+// works in the row layout of the fused step: 16 lanes own 128 consecutive values, lane l the
+// values [4l, 4l+4) and [64+4l, 64+4l+4), so every 16-byte load of a row covers whole cache
+// lines; the loads of all its tiles are issued before the LDS tables are set up.  Other
+// workgroups (the ragged end, the padding) let every lane own 8 consecutive values and guard
+// each access.
+template <int THREADS, int T>
 __global__ __launch_bounds__(THREADS) void quant_group_kernel(const float *__restrict__ x, int64_t n,
                                                               int rows_per_group,
                                                               const float *__restrict__ qmap,
@@ -119,43 +126,94 @@ __global__ __launch_bounds__(THREADS) void quant_group_kernel(const float *__res
                                                               float *__restrict__ max1, int64_t n_groups,
                                                               int64_t n_padded, bool vec)
 {
+    constexpr int kTileElts = THREADS * kQElts;
     __shared__ __align__(16) uint32_t lds[kLdsBytes / 4];
-    __shared__ float s_row[THREADS / 16];
+    __shared__ float s_row[T][THREADS / 16];
+    const int64_t tile0 = (int64_t)blockIdx.x * T * kTileElts;
+    const int lane16 = threadIdx.x & 15;
+    const int wrow = threadIdx.x >> 4;
+    const int64_t gp_sz = (int64_t)rows_per_group * kGroup;
+    const int first = wrow & ~(rows_per_group - 1);
+
+    if (vec && tile0 + (int64_t)T * kTileElts <= n) {  // uniform over the workgroup
+        float v[T][kQElts];
+#pragma unroll
+        for (int t = 0; t < T; ++t) {
+            const float *p = x + tile0 + (int64_t)t * kTileElts + wrow * kGroup + lane16 * 4;
+            const float4 a = load4(p), b = load4(p + 64);
+            v[t][0] = a.x; v[t][1] = a.y; v[t][2] = a.z; v[t][3] = a.w;
+            v[t][4] = b.x; v[t][5] = b.y; v[t][6] = b.z; v[t][7] = b.w;
+        }
+        lds_fill(lds, qmap, nullptr);
+        const int kind = classify_map(qmap);
+        if (tile0 == 0 && threadIdx.x == 0)
+            codes[n_padded / 2] = 0;
+        float amax[T];
+#pragma unroll
+        for (int t = 0; t < T; ++t) {
+            float m = 0.0f;
+#pragma unroll
+            for (int k = 0; k < kQElts; ++k)
+                m = fmaxf(m, fabsf(v[t][k]));
+            amax[t] = row16_max(m);
+            if (lane16 == 0)
+                s_row[t][wrow] = amax[t];
+        }
+        lds_barrier();
+#pragma unroll
+        for (int t = 0; t < T; ++t) {
+            if (rows_per_group > 1) {
+                amax[t] = s_row[t][first];
+                for (int r = 1; r < rows_per_group; ++r)
+                    amax[t] = fmaxf(amax[t], s_row[t][first + r]);
+            }
+            const int64_t base = tile0 + (int64_t)t * kTileElts + wrow * kGroup;
+            if ((base % gp_sz) == 0 && lane16 == 0)
+                max1[base / gp_sz] = amax[t];
+            const uint32_t w = encode8_scaled(lds, kLdsQ0, kind, v[t], amax[t]);
+            uint16_t *cp = reinterpret_cast<uint16_t *>(codes + (base >> 1)) + lane16;
+            store_u16(cp, w & 0xFFFFu);
+            store_u16(cp + 16, w >> 16);
+        }
+        return;
+    }
+
     lds_fill(lds, qmap, nullptr);
     const int kind = classify_map(qmap);
-    const int64_t base = ((int64_t)blockIdx.x * THREADS + threadIdx.x) * kQElts;
-    if (base == 0)
+    if (tile0 == 0 && threadIdx.x == 0)
         codes[n_padded / 2] = 0;
-    float v[kQElts];
-    load8(x, base, n, vec, v);  // zero beyond n: the reference's zero padding
-    float amax = 0.0f;
+    for (int t = 0; t < T; ++t) {  // uniform trip count: the barriers below are reached by all
+        const int64_t base = tile0 + (int64_t)t * kTileElts + (int64_t)threadIdx.x * kQElts;
+        float v[kQElts];
+        load8(x, base, n, vec, v);  // zero beyond n: the reference's zero padding
+        float amax = 0.0f;
 #pragma unroll
-    for (int k = 0; k < kQElts; ++k)
-        amax = fmaxf(amax, fabsf(v[k]));
-    amax = row16_max(amax);
-    if ((threadIdx.x & 15) == 0)
-        s_row[threadIdx.x >> 4] = amax;
-    __syncthreads();
-    if (rows_per_group > 1) {
-        const int first = (threadIdx.x >> 4) & ~(rows_per_group - 1);
-        amax = s_row[first];
-        for (int r = 1; r < rows_per_group; ++r)
-            amax = fmaxf(amax, s_row[first + r]);
+        for (int k = 0; k < kQElts; ++k)
+            amax = fmaxf(amax, fabsf(v[k]));
+        amax = row16_max(amax);
+        __syncthreads();  // the previous tile's readers are done (and, first, the tables are in)
+        if (lane16 == 0)
+            s_row[0][wrow] = amax;
+        __syncthreads();
+        if (rows_per_group > 1) {
+            amax = s_row[0][first];
+            for (int r = 1; r < rows_per_group; ++r)
+                amax = fmaxf(amax, s_row[0][first + r]);
+        }
+        const int64_t grp = base / gp_sz;
+        uint32_t w;
+        if (grp < n_groups) {
+            if ((base % gp_sz) == 0)
+                max1[grp] = amax;
+            w = encode8_scaled(lds, kLdsQ0, kind, v, amax);
+        } else {
+            // padding added by the re-grouping to 2048: plain zeros, not divided by anything
+            const float z[kQElts] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+            w = encode8_plain(lds, kLdsQ0, kind, z);
+        }
+        if (base < n_padded)  // the last workgroup may reach past the last pack group
+            store_u32(reinterpret_cast<uint32_t *>(codes + (base >> 1)), w);
     }
-    const int64_t gp_sz = (int64_t)rows_per_group * kGroup;
-    const int64_t grp = base / gp_sz;
-    uint32_t w;
-    if (grp < n_groups) {
-        if ((base % gp_sz) == 0)
-            max1[grp] = amax;
-        w = encode8_scaled(lds, kLdsQ0, kind, v, amax);
-    } else {
-        // padding added by the re-grouping to 2048: plain zeros, not divided by anything
-        const float z[kQElts] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
-        w = encode8_plain(lds, kLdsQ0, kind, z);
-    }
-    if (base < n_padded)  // a 512-thread workgroup may reach past the last pack group
-        store_u32(reinterpret_cast<uint32_t *>(codes + (base >> 1)), w);
 }
 
 __global__ __launch_bounds__(kQThreads) void dequant_group_kernel(const uint8_t *__restrict__ codes,
@@ -183,6 +241,7 @@ __global__ __launch_bounds__(kQThreads) void dequant_group_kernel(const uint8_t 
 // Row layout (as in the fused step): 16 lanes own one 128-value group, lane l owns values
 // [4l, 4l+4) and [64+4l, 64+4l+4), so that every 16-byte store of a row covers whole cache
 // lines.  Handles the groups that lie fully inside the tensor; n must be >= 128.
+template <int T>
 __global__ __launch_bounds__(kQThreads) void dequant_group_rows_kernel(const uint8_t *__restrict__ codes,
                                                                        const float *__restrict__ max1,
                                                                        const float *__restrict__ qmap,
@@ -190,23 +249,40 @@ __global__ __launch_bounds__(kQThreads) void dequant_group_rows_kernel(const uin
                                                                        float *__restrict__ out)
 {
     __shared__ __align__(16) uint32_t lds[32];
+    const int lane16 = threadIdx.x & 15;
+    // T passes of 16 rows each; the loads of all passes first, the map afterwards
+    const int64_t row0 = (int64_t)blockIdx.x * T * (kQThreads / 16) + (threadIdx.x >> 4);
+    uint32_t c0[T], c1[T];
+    float s[T];
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+        const int64_t row = row0 + t * (kQThreads / 16);
+        c0[t] = c1[t] = 0;
+        s[t] = 0.0f;
+        if (row < full_groups) {
+            const uint16_t *cp = reinterpret_cast<const uint16_t *>(codes + row * 64) + lane16;
+            c0[t] = load_u16(cp);
+            c1[t] = load_u16(cp + 16);
+            s[t] = max1[row / rows_per_group];
+        }
+    }
     if (threadIdx.x < 16)
         lds[threadIdx.x] = __float_as_uint(qmap[threadIdx.x]);
-    __syncthreads();
-    const int lane16 = threadIdx.x & 15;
-    const int64_t row = (int64_t)blockIdx.x * (kQThreads / 16) + (threadIdx.x >> 4);
-    if (row >= full_groups)
-        return;
-    const uint16_t *cp = reinterpret_cast<const uint16_t *>(codes + row * 64) + lane16;
-    const Nibbles nb = split_nibbles(load_u16(cp) | (load_u16(cp + 16) << 16));
-    const float s = max1[row / rows_per_group];
-    float v[kQElts];
+    lds_barrier();
 #pragma unroll
-    for (int k = 0; k < kQElts; ++k)
-        v[k] = decode_nibble(lds, kLdsQ0, nb, k) * s;
-    float *o = out + row * kGroup + lane16 * 4;
-    store4(o, make_float4(v[0], v[1], v[2], v[3]));
-    store4(o + 64, make_float4(v[4], v[5], v[6], v[7]));
+    for (int t = 0; t < T; ++t) {
+        const int64_t row = row0 + t * (kQThreads / 16);
+        if (row >= full_groups)
+            continue;
+        const Nibbles nb = split_nibbles(c0[t] | (c1[t] << 16));
+        float v[kQElts];
+#pragma unroll
+        for (int k = 0; k < kQElts; ++k)
+            v[k] = decode_nibble(lds, kLdsQ0, nb, k) * s[t];
+        float *o = out + row * kGroup + lane16 * 4;
+        store4(o, make_float4(v[0], v[1], v[2], v[3]));
+        store4(o + 64, make_float4(v[4], v[5], v[6], v[7]));
+    }
 }
 
 // ---------------------------------------------------------------------------------------
@@ -221,7 +297,7 @@ __global__ void fill_zero_kernel(float *__restrict__ a, int64_t na, float *__res
         b[i] = 0.0f;
 }
 
-constexpr int kStatRows = 32;
+constexpr int kStatRows = 64;
 constexpr int kStatCols = 1024;  // 256 threads x 4 columns
 constexpr int kStatUnroll = 8;   // rows in flight per lane
 
@@ -317,17 +393,39 @@ __global__ __launch_bounds__(kQThreads) void quant_rank1_kernel(const float *__r
 // pad codes past the tensor.
 constexpr int kR1Cols = kQThreads * kQElts;  // columns per workgroup
 
+constexpr int kR1RowsPerWg = 4;  // rows of one column chunk per workgroup: the column maxima are loaded once
+
 __global__ __launch_bounds__(kQThreads) void quant_rank1_rows_kernel(const float *__restrict__ x, int64_t R,
                                                                      int64_t C, const float *__restrict__ rowmax,
                                                                      const float *__restrict__ colmax,
                                                                      const float *__restrict__ qmap,
                                                                      uint8_t *__restrict__ codes, int64_t n_padded)
 {
+    constexpr int T = kR1RowsPerWg;
     __shared__ __align__(16) uint32_t lds[kLdsBytes / 4];
+    const int64_t n = R * C;
+    const int64_t r0 = (int64_t)blockIdx.y * T;
+    const int64_t c = (int64_t)blockIdx.x * kR1Cols + (int64_t)threadIdx.x * kQElts;
+    const bool live = c < C;
+    // the lane's loads first, the LDS tables afterwards
+    float4 a[T], b[T], ca, cb;
+    float rm[T];
+    if (live) {
+        ca = *reinterpret_cast<const float4 *>(colmax + c);
+        cb = *reinterpret_cast<const float4 *>(colmax + c + 4);
+#pragma unroll
+        for (int t = 0; t < T; ++t) {
+            if (r0 + t < R) {
+                const float *p = x + (r0 + t) * C + c;
+                a[t] = load4(p);
+                b[t] = load4(p + 4);
+                rm[t] = rowmax[r0 + t];
+            }
+        }
+    }
     lds_fill(lds, qmap, nullptr);
     const int kind = classify_map(qmap);
-    __syncthreads();
-    const int64_t n = R * C;
+    lds_barrier();
     if (blockIdx.x == 0 && blockIdx.y == 0) {
         const float z[kQElts] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
         const uint32_t wz = encode8_plain(lds, kLdsQ0, kind, z);
@@ -336,22 +434,23 @@ __global__ __launch_bounds__(kQThreads) void quant_rank1_rows_kernel(const float
         if (threadIdx.x == 0)
             codes[n_padded / 2] = 0;
     }
-    const int64_t r = blockIdx.y;
-    const int64_t c = (int64_t)blockIdx.x * kR1Cols + (int64_t)threadIdx.x * kQElts;
-    if (c >= C)
+    if (!live)
         return;
-    const float rm = rowmax[r];
-    const float4 a = load4(x + r * C + c), b = load4(x + r * C + c + 4);
-    const float4 ca = *reinterpret_cast<const float4 *>(colmax + c), cb = *reinterpret_cast<const float4 *>(colmax + c + 4);
-    const float v[kQElts] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
     const float cmx[kQElts] = {ca.x, ca.y, ca.z, ca.w, cb.x, cb.y, cb.z, cb.w};
-    float xs[kQElts];
 #pragma unroll
-    for (int k = 0; k < kQElts; ++k) {
-        const float st = (cmx[k] < rm) ? cmx[k] : rm;
-        xs[k] = v[k] / st;
+    for (int t = 0; t < T; ++t) {
+        if (r0 + t >= R)
+            break;
+        const float v[kQElts] = {a[t].x, a[t].y, a[t].z, a[t].w, b[t].x, b[t].y, b[t].z, b[t].w};
+        float xs[kQElts];
+#pragma unroll
+        for (int k = 0; k < kQElts; ++k) {
+            const float st = (cmx[k] < rm[t]) ? cmx[k] : rm[t];
+            xs[k] = v[k] / st;
+        }
+        store_u32(reinterpret_cast<uint32_t *>(codes + (((r0 + t) * C + c) >> 1)),
+                  encode8_plain(lds, kLdsQ0, kind, xs));
     }
-    store_u32(reinterpret_cast<uint32_t *>(codes + ((r * C + c) >> 1)), encode8_plain(lds, kLdsQ0, kind, xs));
 }
 
 __global__ __launch_bounds__(kQThreads) void dequant_rank1_kernel(const uint8_t *__restrict__ codes,
@@ -392,28 +491,47 @@ __global__ __launch_bounds__(kQThreads) void dequant_rank1_kernel(const uint8_t 
 __global__ __launch_bounds__(kQThreads) void dequant_rank1_rows_kernel(const uint8_t *__restrict__ codes,
                                                                        const float *__restrict__ rowmax,
                                                                        const float *__restrict__ colmax,
-                                                                       const float *__restrict__ qmap, int64_t C,
-                                                                       float *__restrict__ out)
+                                                                       const float *__restrict__ qmap, int64_t R,
+                                                                       int64_t C, float *__restrict__ out)
 {
+    constexpr int T = kR1RowsPerWg;
     __shared__ __align__(16) uint32_t lds[32];
+    const int64_t r0 = (int64_t)blockIdx.y * T;
+    const int64_t c = (int64_t)blockIdx.x * kR1Cols + (int64_t)threadIdx.x * kQElts;
+    const bool live = c < C;
+    uint32_t w[T];
+    float rm[T];
+    float4 ca, cb;
+    if (live) {
+        ca = *reinterpret_cast<const float4 *>(colmax + c);
+        cb = *reinterpret_cast<const float4 *>(colmax + c + 4);
+#pragma unroll
+        for (int t = 0; t < T; ++t) {
+            if (r0 + t < R) {
+                w[t] = load_u32(reinterpret_cast<const uint32_t *>(codes + (((r0 + t) * C + c) >> 1)));
+                rm[t] = rowmax[r0 + t];
+            }
+        }
+    }
     if (threadIdx.x < 16)
         lds[threadIdx.x] = __float_as_uint(qmap[threadIdx.x]);
-    __syncthreads();
-    const int64_t r = blockIdx.y;
-    const int64_t c = (int64_t)blockIdx.x * kR1Cols + (int64_t)threadIdx.x * kQElts;
-    if (c >= C)
+    lds_barrier();
+    if (!live)
         return;
-    const float rm = rowmax[r];
-    const Nibbles nb = split_nibbles(load_u32(reinterpret_cast<const uint32_t *>(codes + ((r * C + c) >> 1))));
-    const float4 ca = *reinterpret_cast<const float4 *>(colmax + c), cb = *reinterpret_cast<const float4 *>(colmax + c + 4);
     const float cmx[kQElts] = {ca.x, ca.y, ca.z, ca.w, cb.x, cb.y, cb.z, cb.w};
-    float v[kQElts];
 #pragma unroll
-    for (int k = 0; k < kQElts; ++k)
-        v[k] = decode_nibble(lds, kLdsQ0, nb, k) * ((cmx[k] < rm) ? cmx[k] : rm);
-    float *o = out + r * C + c;
-    store4(o, make_float4(v[0], v[1], v[2], v[3]));
-    store4(o + 4, make_float4(v[4], v[5], v[6], v[7]));
+    for (int t = 0; t < T; ++t) {
+        if (r0 + t >= R)
+            break;
+        const Nibbles nb = split_nibbles(w[t]);
+        float v[kQElts];
+#pragma unroll
+        for (int k = 0; k < kQElts; ++k)
+            v[k] = decode_nibble(lds, kLdsQ0, nb, k) * ((cmx[k] < rm[t]) ? cmx[k] : rm[t]);
+        float *o = out + (r0 + t) * C + c;
+        store4(o, make_float4(v[0], v[1], v[2], v[3]));
+        store4(o + 4, make_float4(v[4], v[5], v[6], v[7]));
+    }
 }
 
 // Row layout variant for column counts that are a multiple of 128: 16 lanes own 128
@@ -422,32 +540,51 @@ __global__ __launch_bounds__(kQThreads) void dequant_rank1_rows_kernel(const uin
 __global__ __launch_bounds__(kQThreads) void dequant_rank1_rows128_kernel(const uint8_t *__restrict__ codes,
                                                                           const float *__restrict__ rowmax,
                                                                           const float *__restrict__ colmax,
-                                                                          const float *__restrict__ qmap, int64_t C,
-                                                                          float *__restrict__ out)
+                                                                          const float *__restrict__ qmap, int64_t R,
+                                                                          int64_t C, float *__restrict__ out)
 {
+    constexpr int T = kR1RowsPerWg;
     __shared__ __align__(16) uint32_t lds[32];
+    const int lane16 = threadIdx.x & 15;
+    const int64_t r0 = (int64_t)blockIdx.y * T;
+    const int64_t c0 = (int64_t)blockIdx.x * kR1Cols + (int64_t)(threadIdx.x >> 4) * kGroup;
+    const bool live = c0 < C;
+    uint32_t w0[T], w1[T];
+    float rm[T];
+    float4 ca, cb;
+    if (live) {
+        const float *cmp = colmax + c0 + lane16 * 4;
+        ca = *reinterpret_cast<const float4 *>(cmp);
+        cb = *reinterpret_cast<const float4 *>(cmp + 64);
+#pragma unroll
+        for (int t = 0; t < T; ++t) {
+            if (r0 + t < R) {
+                const uint16_t *cp = reinterpret_cast<const uint16_t *>(codes + (((r0 + t) * C + c0) >> 1)) + lane16;
+                w0[t] = load_u16(cp);
+                w1[t] = load_u16(cp + 16);
+                rm[t] = rowmax[r0 + t];
+            }
+        }
+    }
     if (threadIdx.x < 16)
         lds[threadIdx.x] = __float_as_uint(qmap[threadIdx.x]);
-    __syncthreads();
-    const int lane16 = threadIdx.x & 15;
-    const int64_t r = blockIdx.y;
-    const int64_t c0 = (int64_t)blockIdx.x * kR1Cols + (int64_t)(threadIdx.x >> 4) * kGroup;
-    if (c0 >= C)
+    lds_barrier();
+    if (!live)
         return;
-    const int64_t gbase = r * C + c0;
-    const float rm = rowmax[r];
-    const uint16_t *cp = reinterpret_cast<const uint16_t *>(codes + (gbase >> 1)) + lane16;
-    const Nibbles nb = split_nibbles(load_u16(cp) | (load_u16(cp + 16) << 16));
-    const float *cmp = colmax + c0 + lane16 * 4;
-    const float4 ca = *reinterpret_cast<const float4 *>(cmp), cb = *reinterpret_cast<const float4 *>(cmp + 64);
     const float cmx[kQElts] = {ca.x, ca.y, ca.z, ca.w, cb.x, cb.y, cb.z, cb.w};
-    float v[kQElts];
 #pragma unroll
-    for (int k = 0; k < kQElts; ++k)
-        v[k] = decode_nibble(lds, kLdsQ0, nb, k) * ((cmx[k] < rm) ? cmx[k] : rm);
-    float *o = out + gbase + lane16 * 4;
-    store4(o, make_float4(v[0], v[1], v[2], v[3]));
-    store4(o + 64, make_float4(v[4], v[5], v[6], v[7]));
+    for (int t = 0; t < T; ++t) {
+        if (r0 + t >= R)
+            break;
+        const Nibbles nb = split_nibbles(w0[t] | (w1[t] << 16));
+        float v[kQElts];
+#pragma unroll
+        for (int k = 0; k < kQElts; ++k)
+            v[k] = decode_nibble(lds, kLdsQ0, nb, k) * ((cmx[k] < rm[t]) ? cmx[k] : rm[t]);
+        float *o = out + (r0 + t) * C + c0 + lane16 * 4;
+        store4(o, make_float4(v[0], v[1], v[2], v[3]));
+        store4(o + 64, make_float4(v[4], v[5], v[6], v[7]));
+    }
 }
 
 inline bool tiles_ok(int64_t n, int64_t tile, uint32_t *tiles)
@@ -525,13 +662,15 @@ extern "C" int lpmm_quant_group(const float *x, int64_t n, int64_t gp_sz, const 
     if (!tiles_ok(n_groups * gp_sz, kQTile, &tiles))
         return LPMM_ERR_SIZE;
     const int64_t n_padded = (int64_t)tiles * kQTile;
+    constexpr int kT = 4;  // tiles per workgroup
     if (gp_sz > kQTile)
-        hipLaunchKernelGGL(quant_group_kernel<2 * kQThreads>, dim3((tiles + 1) / 2), dim3(2 * kQThreads), 0,
+        hipLaunchKernelGGL((quant_group_kernel<2 * kQThreads, 1>), dim3((tiles + 1) / 2), dim3(2 * kQThreads), 0,
                            (hipStream_t)stream, x, n, (int)(gp_sz / kGroup), qmap, codes, max1, n_groups, n_padded,
                            aligned_to(x, 16));
     else
-        hipLaunchKernelGGL(quant_group_kernel<kQThreads>, dim3(tiles), dim3(kQThreads), 0, (hipStream_t)stream, x, n,
-                           (int)(gp_sz / kGroup), qmap, codes, max1, n_groups, n_padded, aligned_to(x, 16));
+        hipLaunchKernelGGL((quant_group_kernel<kQThreads, kT>), dim3((tiles + kT - 1) / kT), dim3(kQThreads), 0,
+                           (hipStream_t)stream, x, n, (int)(gp_sz / kGroup), qmap, codes, max1, n_groups, n_padded,
+                           aligned_to(x, 16));
     return launch_status();
 }
 
@@ -554,8 +693,10 @@ extern "C" int lpmm_dequant_group(const uint8_t *codes, const float *max1, const
     const int64_t full_groups = n / kGroup;
     if (vec && full_groups > 0 && full_groups <= 0x7fffffffLL * 16) {
         // whole 128-value rows in the row layout, the ragged tail (< 128 values) element-wise
-        hipLaunchKernelGGL(dequant_group_rows_kernel, dim3((uint32_t)((full_groups + 15) / 16)), dim3(kQThreads), 0,
-                           (hipStream_t)stream, codes, max1, qmap, full_groups, (int)(gp_sz / kGroup), out);
+        constexpr int kT = 4;  // passes of 16 rows per workgroup
+        hipLaunchKernelGGL(dequant_group_rows_kernel<kT>, dim3((uint32_t)((full_groups + 16 * kT - 1) / (16 * kT))),
+                           dim3(kQThreads), 0, (hipStream_t)stream, codes, max1, qmap, full_groups,
+                           (int)(gp_sz / kGroup), out);
         const int64_t done = full_groups * kGroup;
         if (done < n)
             hipLaunchKernelGGL(dequant_group_kernel, dim3(1), dim3(kQThreads), 0, (hipStream_t)stream,
@@ -593,7 +734,7 @@ extern "C" int lpmm_rank1_stats(const float *x, int64_t rows, int64_t cols, floa
 // row-wise kernels: columns a multiple of 8, 16-byte aligned operands, rows fit grid.y
 static bool rank1_rows_ok(const void *x, const void *colmax, const void *codes, int64_t rows, int64_t cols)
 {
-    return (cols % 8) == 0 && rows <= 65535 && aligned_to(x, 16) && aligned_to(colmax, 16) && aligned_to(codes, 4);
+    return (cols % 8) == 0 && rows <= 65535LL * kR1RowsPerWg && aligned_to(x, 16) && aligned_to(colmax, 16) && aligned_to(codes, 4);
 }
 
 extern "C" int lpmm_quant_rank1(const float *x, int64_t rows, int64_t cols, const float *rowmax,
@@ -618,7 +759,8 @@ extern "C" int lpmm_quant_rank1(const float *x, int64_t rows, int64_t cols, cons
     const int64_t n_padded = (int64_t)tiles * kQTile;
     if (rank1_rows_ok(x, colmax, codes, rows, cols)) {
         const uint32_t gx = (uint32_t)((cols + kR1Cols - 1) / kR1Cols);
-        hipLaunchKernelGGL(quant_rank1_rows_kernel, dim3(gx, (uint32_t)rows), dim3(kQThreads), 0,
+        const uint32_t gy = (uint32_t)((rows + kR1RowsPerWg - 1) / kR1RowsPerWg);
+        hipLaunchKernelGGL(quant_rank1_rows_kernel, dim3(gx, gy), dim3(kQThreads), 0,
                            (hipStream_t)stream, x, rows, cols, rowmax, colmax, qmap, codes, n_padded);
     } else {
         hipLaunchKernelGGL(quant_rank1_kernel, dim3(tiles), dim3(kQThreads), 0, (hipStream_t)stream, x, n, cols,
@@ -647,12 +789,14 @@ extern "C" int lpmm_dequant_rank1(const uint8_t *codes, const float *rowmax, con
         return LPMM_ERR_SIZE;
     if (rank1_rows_ok(out, colmax, codes, rows, cols) && (cols % kGroup) == 0) {
         const uint32_t gx = (uint32_t)((cols + kR1Cols - 1) / kR1Cols);
-        hipLaunchKernelGGL(dequant_rank1_rows128_kernel, dim3(gx, (uint32_t)rows), dim3(kQThreads), 0,
-                           (hipStream_t)stream, codes, rowmax, colmax, qmap, cols, out);
+        const uint32_t gy = (uint32_t)((rows + kR1RowsPerWg - 1) / kR1RowsPerWg);
+        hipLaunchKernelGGL(dequant_rank1_rows128_kernel, dim3(gx, gy), dim3(kQThreads), 0,
+                           (hipStream_t)stream, codes, rowmax, colmax, qmap, rows, cols, out);
     } else if (rank1_rows_ok(out, colmax, codes, rows, cols)) {
         const uint32_t gx = (uint32_t)((cols + kR1Cols - 1) / kR1Cols);
-        hipLaunchKernelGGL(dequant_rank1_rows_kernel, dim3(gx, (uint32_t)rows), dim3(kQThreads), 0,
-                           (hipStream_t)stream, codes, rowmax, colmax, qmap, cols, out);
+        const uint32_t gy = (uint32_t)((rows + kR1RowsPerWg - 1) / kR1RowsPerWg);
+        hipLaunchKernelGGL(dequant_rank1_rows_kernel, dim3(gx, gy), dim3(kQThreads), 0,
+                           (hipStream_t)stream, codes, rowmax, colmax, qmap, rows, cols, out);
     } else {
         const bool vec = aligned_to(out, 16) && aligned_to(codes, 4);
         hipLaunchKernelGGL(dequant_rank1_kernel, dim3(tiles), dim3(kQThreads), 0, (hipStream_t)stream, codes,
