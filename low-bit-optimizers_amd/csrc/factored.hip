@@ -50,9 +50,9 @@ __global__ __launch_bounds__(kFThreads) void nonfused_update_kernel(float *__res
 // kSRows x kSCols, accumulated in double.  Partials go to the workspace:
 //   colpart[ty][c]  (ty = row-tile index)   rowpart[tx][r]  (tx = column-tile index)
 // ---------------------------------------------------------------------------------------
-constexpr int kSRows = 32;
+constexpr int kSRows = 64;
 constexpr int kSCols = 1024;  // 256 threads x 4 columns
-constexpr int kSUnroll = 8;   // rows in flight per lane
+constexpr int kSUnroll = 8;   // rows in flight per lane (wave_sum8_f64 reduces 8 rows at once)
 
 __device__ __forceinline__ void partial_body(const float *__restrict__ g, int64_t R, int64_t C,
                                              double *__restrict__ colpart, double *__restrict__ rowpart, bool vec,
@@ -62,9 +62,10 @@ __device__ __forceinline__ void partial_body(const float *__restrict__ g, int64_
     const int64_t r0 = (int64_t)by * kSRows;
     const int64_t r1 = (r0 + kSRows < R) ? r0 + kSRows : R;
     const bool lane_vec = vec && c0 + 4 <= C;
-    __shared__ double s_part[kFThreads / kWave][kSUnroll];
+    __shared__ double s_part[kFThreads / kWave][kSRows];  // row sums of the tile, per wave
     double *rp = rowpart + (int64_t)bx * R;  // one row partial per workgroup
     double cs[4] = {0.0, 0.0, 0.0, 0.0};
+    const int lane = threadIdx.x & (kWave - 1);
     for (int64_t rb = r0; rb < r1; rb += kSUnroll) {
         float u[kSUnroll][4];
         if (lane_vec && rb + kSUnroll <= r1) {
@@ -88,22 +89,23 @@ __device__ __forceinline__ void partial_body(const float *__restrict__ g, int64_
                 }
             }
         }
+        double rs[kSUnroll];
 #pragma unroll
         for (int j = 0; j < kSUnroll; ++j) {
-            double rs = ((double)u[j][0] + (double)u[j][1]) + ((double)u[j][2] + (double)u[j][3]);
+            rs[j] = ((double)u[j][0] + (double)u[j][1]) + ((double)u[j][2] + (double)u[j][3]);
 #pragma unroll
             for (int k = 0; k < 4; ++k)
                 cs[k] += (double)u[j][k];
-            rs = wave_sum_f64(rs);
-            if ((threadIdx.x & 63) == 0)
-                s_part[threadIdx.x >> 6][j] = rs;
         }
-        __syncthreads();
-        if (threadIdx.x < kSUnroll && rb + threadIdx.x < r1)
-            rp[rb + threadIdx.x] = (s_part[0][threadIdx.x] + s_part[1][threadIdx.x]) +
-                                   (s_part[2][threadIdx.x] + s_part[3][threadIdx.x]);
-        __syncthreads();
+        // the wave's 8 row sums at once: lane 8j ends up with the sum of row j
+        const double tot = wave_sum8_f64(rs, lane);
+        if ((lane & 7) == 0)
+            s_part[threadIdx.x >> 6][(int)(rb - r0) + (lane >> 3)] = tot;
     }
+    __syncthreads();
+    if (threadIdx.x < kSRows && r0 + threadIdx.x < r1)
+        rp[r0 + threadIdx.x] = (s_part[0][threadIdx.x] + s_part[1][threadIdx.x]) +
+                               (s_part[2][threadIdx.x] + s_part[3][threadIdx.x]);
 #pragma unroll
     for (int k = 0; k < 4; ++k)
         if (c0 + k < C)

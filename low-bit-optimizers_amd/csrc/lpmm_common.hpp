@@ -78,6 +78,70 @@ __device__ __forceinline__ double wave_sum_f64(double v)
     return v;
 }
 
+// Eight wave-wide sums at once.  Three halving exchanges (lane ^ 32, ^ 16, ^ 8) in each of
+// which a lane keeps half of its values and hands the other half over, then three steps on
+// the one value left: lane 8j (and the seven lanes after it) holds the sum of v[j] over the
+// wave.  7 value exchanges through the LDS crossbar instead of 48, the order of the additions
+// is fixed.
+template <int CTRL>
+__device__ __forceinline__ double dpp_f64(double v)
+{
+    const uint64_t u = (uint64_t)__double_as_longlong(v);
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(uint32_t)u, CTRL, 0xF, 0xF, false);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(uint32_t)(u >> 32), CTRL, 0xF, 0xF, false);
+    return __longlong_as_double((long long)(((uint64_t)hi << 32) | lo));
+}
+
+__device__ __forceinline__ double wave_sum8_f64(const double (&v)[8], int lane)
+{
+    double a[4], b[2], c;
+    const bool h32 = (lane & 32) != 0, h16 = (lane & 16) != 0, h8 = (lane & 8) != 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const double keep = h32 ? v[4 + i] : v[i], give = h32 ? v[i] : v[4 + i];
+        a[i] = keep + __shfl_xor(give, 32, 64);
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const double keep = h16 ? a[2 + i] : a[i], give = h16 ? a[i] : a[2 + i];
+        b[i] = keep + __shfl_xor(give, 16, 64);
+    }
+    {
+        const double keep = h8 ? b[1] : b[0], give = h8 ? b[0] : b[1];
+        c = keep + __shfl_xor(give, 8, 64);
+    }
+    c += dpp_f64<0xB1>(c);   // quad_perm [1,0,3,2]
+    c += dpp_f64<0x4E>(c);   // quad_perm [2,3,0,1]
+    c += dpp_f64<0x141>(c);  // row_half_mirror: the other quad of the same eight lanes
+    return c;
+}
+
+// The same for eight wave-wide maxima of floats: lane 8j (and the seven lanes after it) ends
+// up with the maximum of v[j] over the wave.
+__device__ __forceinline__ float wave_max8(const float (&v)[8], int lane)
+{
+    float a[4], b[2], c;
+    const bool h32 = (lane & 32) != 0, h16 = (lane & 16) != 0, h8 = (lane & 8) != 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const float keep = h32 ? v[4 + i] : v[i], give = h32 ? v[i] : v[4 + i];
+        a[i] = fmaxf(keep, __shfl_xor(give, 32, 64));
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const float keep = h16 ? a[2 + i] : a[i], give = h16 ? a[i] : a[2 + i];
+        b[i] = fmaxf(keep, __shfl_xor(give, 16, 64));
+    }
+    {
+        const float keep = h8 ? b[1] : b[0], give = h8 ? b[0] : b[1];
+        c = fmaxf(keep, __shfl_xor(give, 8, 64));
+    }
+    c = fmaxf(c, dpp_f32<0xB1>(c));   // quad_perm [1,0,3,2]
+    c = fmaxf(c, dpp_f32<0x4E>(c));   // quad_perm [2,3,0,1]
+    c = fmaxf(c, dpp_f32<0x141>(c));  // row_half_mirror: the other quad of the same eight lanes
+    return c;
+}
+
 // ---------------------------------------------------------------------------------------
 // Code assignment for an ascending 16-entry map given its 15 fp32 midpoints:
 // code = number of midpoints strictly below x.  Identical to the reference's upper-bound

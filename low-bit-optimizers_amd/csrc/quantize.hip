@@ -333,16 +333,20 @@ __global__ __launch_bounds__(kQThreads) void rank1_stats_kernel(const float *__r
                     a[u][k] = (r < r1 && c0 + k < C) ? fabsf(x[r * C + c0 + k]) : 0.0f;
             }
         }
+        float rm[kStatUnroll];
 #pragma unroll
         for (int u = 0; u < kStatUnroll; ++u) {
-            float rm = fmaxf(fmaxf(a[u][0], a[u][1]), fmaxf(a[u][2], a[u][3]));
+            rm[u] = fmaxf(fmaxf(a[u][0], a[u][1]), fmaxf(a[u][2], a[u][3]));
 #pragma unroll
             for (int k = 0; k < 4; ++k)
                 cm[k] = fmaxf(cm[k], a[u][k]);
-            rm = wave_max(rm);
-            if ((threadIdx.x & 63) == 0 && rb + u < r1)
-                atomic_max_nonneg(rowmax + rb + u, rm);
         }
+        // the wave's 8 row maxima at once: lane 8u holds the maximum of row rb + u
+        static_assert(kStatUnroll == 8, "wave_max8 reduces eight rows");
+        const int lane = threadIdx.x & 63;
+        const float m = wave_max8(rm, lane);
+        if ((lane & 7) == 0 && rb + (lane >> 3) < r1)
+            atomic_max_nonneg(rowmax + rb + (lane >> 3), m);
     }
 #pragma unroll
     for (int k = 0; k < 4; ++k)
