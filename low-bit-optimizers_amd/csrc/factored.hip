@@ -316,10 +316,39 @@ __device__ __forceinline__ void update_rows128_body(
     int64_t n_padded, const NfHyper &h, bool first_step, uint32_t bx, int64_t by)
 {
     __shared__ __align__(16) uint32_t lds[kLdsBytes / 4];
+    const int64_t n = R * C;
+    const int lane16 = threadIdx.x & 15;
+    const int64_t r = by;
+    const int64_t c0 = (int64_t)bx * kFTile + (int64_t)(threadIdx.x >> 4) * kGroup;  // first column of the group
+    const bool live = c0 < C;  // uniform over the 16 lanes of the group
+    const int64_t gbase = r * C + c0;
+    const int64_t grp = gbase / kGroup;
+    float *pp = p + gbase + lane16 * 4;
+    uint16_t *mcp = reinterpret_cast<uint16_t *>(m_codes + (gbase >> 1)) + lane16;
+    // the group's loads first, the LDS tables afterwards
+    float4 a0, a1, b0, b1, c_lo, c_hi;
+    uint32_t w0 = 0, w1 = 0;
+    float sm = 0.0f, row_r = 0.0f, mean_all = 1.0f;
+    if (live) {
+        const float *gp = g + gbase + lane16 * 4;
+        const float *cp = col + c0 + lane16 * 4;
+        a0 = load4(pp);
+        a1 = load4(pp + 64);
+        b0 = load4(gp);
+        b1 = load4(gp + 64);
+        c_lo = *reinterpret_cast<const float4 *>(cp);
+        c_hi = *reinterpret_cast<const float4 *>(cp + 64);
+        if (!first_step) {
+            w0 = load_u16(mcp);
+            w1 = load_u16(mcp + 16);
+            sm = m_max1[grp];
+        }
+        row_r = row[r];
+        mean_all = *row_mean_all;
+    }
     lds_fill(lds, qmap_m, nullptr);
     const int kind = classify_map(qmap_m);
-    __syncthreads();
-    const int64_t n = R * C;
+    lds_barrier();
     if (bx == 0 && by == 0) {
         const float z[kFElts] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
         const uint32_t wz = kind == kMapStdM ? encode8_std_m(lds, z)
@@ -329,27 +358,11 @@ __device__ __forceinline__ void update_rows128_body(
         if (threadIdx.x == 0)
             m_codes[n_padded / 2] = 0;
     }
-    const int lane16 = threadIdx.x & 15;
-    const int64_t r = by;
-    const int64_t c0 = (int64_t)bx * kFTile + (int64_t)(threadIdx.x >> 4) * kGroup;  // first column of the group
-    if (c0 >= C)
-        return;  // uniform over the 16 lanes of the group
-    const int64_t gbase = r * C + c0;
-    const int64_t grp = gbase / kGroup;
-    float *pp = p + gbase + lane16 * 4;
-    const float *gp = g + gbase + lane16 * 4;
-    const float *cp = col + c0 + lane16 * 4;
-    const float4 a0 = load4(pp), a1 = load4(pp + 64), b0 = load4(gp), b1 = load4(gp + 64);
-    const float4 c_lo = *reinterpret_cast<const float4 *>(cp), c_hi = *reinterpret_cast<const float4 *>(cp + 64);
-    uint16_t *mcp = reinterpret_cast<uint16_t *>(m_codes + (gbase >> 1)) + lane16;
-    uint32_t wm = 0;
-    float sm = 0.0f;
-    if (!first_step) {
-        wm = load_u16(mcp) | (load_u16(mcp + 16) << 16);
-        sm = m_max1[grp];
-    }
+    if (!live)
+        return;
+    const uint32_t wm = w0 | (w1 << 16);
     const Nibbles nm = split_nibbles(wm);
-    const float rf = row[r] / *row_mean_all;
+    const float rf = row_r / mean_all;
     float pv[kFElts] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
     const float gv[kFElts] = {b0.x, b0.y, b0.z, b0.w, b1.x, b1.y, b1.z, b1.w};
     const float cv[kFElts] = {c_lo.x, c_lo.y, c_lo.z, c_lo.w, c_hi.x, c_hi.y, c_hi.z, c_hi.w};

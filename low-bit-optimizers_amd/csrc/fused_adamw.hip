@@ -52,12 +52,17 @@ struct Tensor4 {
     float pad;
 };
 
+constexpr int kStartSlots = LPMM_MULTI_MAX + 8;   // tile_start is read 8 entries at a time
+constexpr int kCoarseSlots = LPMM_MULTI_MAX / 8;  // every eighth entry of tile_start
+
 struct Multi4 {
     Tensor4 t[LPMM_MULTI_MAX];
-    uint32_t tile_start[LPMM_MULTI_MAX + 1];  // prefix sum of tiles per tensor
+    uint32_t tile_start[kStartSlots];  // prefix sum of tiles per tensor; unused slots hold the total
+    uint32_t coarse[kCoarseSlots];     // tile_start[8], tile_start[16], ...
     int count;
     float s[7];  // scalars shared by all tensors, in the order the arithmetic below reads them
 };
+static_assert(LPMM_MULTI_MAX % 8 == 0, "coarse table");
 
 // The two arithmetics the kernel is instantiated with.  Both read the shared scalars from
 // Multi4::s and three per-tensor ones from Tensor4::{c1, c2s, rc2s}.
@@ -234,7 +239,10 @@ __device__ __forceinline__ void group_step(const Tensor4 &t, const Arith &h, con
     }
 }
 
-template <bool ALIGNED, class Arith>
+// ALIGNED: every pointer allows vector access.  ALLFULL (implies ALIGNED): every tensor of the
+// launch is a whole number of tiles, so no access needs a guard and the loads are straight-line
+// code.
+template <bool ALIGNED, bool ALLFULL, class Arith>
 __global__ __launch_bounds__(kThreads) void adamw4bit_kernel(const Multi4 args,
                                                              const float *__restrict__ qmap_m,
                                                              const float *__restrict__ qmap_v)
@@ -243,31 +251,36 @@ __global__ __launch_bounds__(kThreads) void adamw4bit_kernel(const Multi4 args,
     // the small loads first: maps and encode table for LDS
     const LdsFill fill = lds_fill_load(qmap_m, qmap_v);
 
-    // which tensor does this tile belong to (uniform over the workgroup): the number of
-    // later tensors whose first tile is not after this one; unused slots hold the total
-    // (one entry per lane, one ballot per wave)
-    static_assert(LPMM_MULTI_MAX <= kWave, "one tile_start entry per lane");
-    const int lane = threadIdx.x & (kWave - 1);
-    // lanes past the last slot read the total, which no block index reaches
-    const int slot = lane + 1 < LPMM_MULTI_MAX ? lane + 1 : LPMM_MULTI_MAX;
-    const uint32_t first_tile = args.tile_start[slot];
-    // one wait covers the three small loads; the streaming loads below are issued after it
-    lds_fill_store(lds, fill);
-    const bool started = first_tile <= blockIdx.x;
-    const int lo = __popcll(__ballot(started));
+    // Which tensor does this tile belong to (uniform over the workgroup): the number of later
+    // tensors whose first tile is not after this one; unused slots hold the total, which no
+    // block index reaches.  Two rounds of scalar loads from the kernel arguments (every eighth
+    // entry, then the seven in between) and scalar compares: nothing here queues behind the
+    // streaming traffic of the vector memory path.
+    const uint32_t bid = blockIdx.x;
+    int base = 0;
+#pragma unroll
+    for (int j = 0; j < kCoarseSlots; ++j)
+        base += (args.coarse[j] <= bid) ? 8 : 0;
+    int lo = base;
+#pragma unroll
+    for (int i = 1; i < 8; ++i)
+        lo += (args.tile_start[base + i] <= bid) ? 1 : 0;
     const Tensor4 &t = args.t[lo];
     const int lane16 = threadIdx.x & 15;
-    const int64_t grp = (int64_t)(blockIdx.x - args.tile_start[lo]) * (kTile / kGroup) + (threadIdx.x >> 4);
+    const int64_t grp = (int64_t)(bid - args.tile_start[lo]) * (kTile / kGroup) + (threadIdx.x >> 4);
 
-    // a group that lies wholly inside its tensor starts its loads now; the waves wait only
-    // for their LDS writes at the barrier (no global access is ordered by it)
-    const bool full = ALIGNED && (grp + 1) * kGroup <= t.n;
+    // a group that lies wholly inside its tensor starts its loads now; the small loads were
+    // issued before them and return first
+    const bool full = ALLFULL || (ALIGNED && (grp + 1) * kGroup <= t.n);
     GroupRegs regs;
-    regs.m0 = regs.m1 = regs.v0 = regs.v1 = 0;
+    if (!ALLFULL)
+        regs.m0 = regs.m1 = regs.v0 = regs.v1 = 0;
     if (full)
         group_load(t, grp, lane16, regs);
+    lds_fill_store(lds, fill);
     const bool std_maps = classify_map(qmap_m) == kMapStdM && classify_map(qmap_v) == kMapStdV;
     const Arith h(args, t);
+    // the waves wait only for their LDS writes at the barrier (no global access is ordered by it)
     lds_barrier();
     // the loaded words stay as they are until here, so that nothing above waits for them
     asm volatile("" : "+v"(regs.m0), "+v"(regs.m1), "+v"(regs.v0), "+v"(regs.v1));
@@ -278,7 +291,7 @@ __global__ __launch_bounds__(kThreads) void adamw4bit_kernel(const Multi4 args,
         t.mc[end] = 0;
         t.vc[end] = 0;
     }
-    if (Arith::kPadded && grp * kGroup >= t.n) {
+    if (!ALLFULL && Arith::kPadded && grp * kGroup >= t.n) {
         // a group the padding to whole tiles added: codes of a plain 0.0
         const float z[kEltsPerLane] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
         const uint32_t zm = encode8_plain(lds, kLdsQ0, std_maps ? kMapStdM : kMapGeneric, z);
@@ -370,7 +383,7 @@ static int step_multi4(const lpmm_adamw4bit_tensor *tensors, int64_t count, cons
     LPMM_REQUIRE_PTR(qmap_v);
     LPMM_REQUIRE_ALIGN(qmap_m, 4);
     LPMM_REQUIRE_ALIGN(qmap_v, 4);
-    bool aligned = true;
+    bool aligned = true, allfull = true;
     for (int64_t i = 0; i < count; ++i) {
         const lpmm_adamw4bit_tensor &t = tensors[i];
         if (t.n < 0)
@@ -389,6 +402,7 @@ static int step_multi4(const lpmm_adamw4bit_tensor *tensors, int64_t count, cons
         LPMM_REQUIRE_ALIGN(t.v_scale, 4);
         if ((t.n + kTile - 1) / kTile > 0x7fffffffLL)
             return LPMM_ERR_SIZE;
+        allfull = allfull && (t.n % kTile) == 0;
         aligned = aligned && aligned_to(t.p, 16) && aligned_to(t.g, 16) && aligned_to(t.m_codes, 2) &&
                   aligned_to(t.v_codes, 2);
     }
@@ -427,14 +441,20 @@ static int step_multi4(const lpmm_adamw4bit_tensor *tensors, int64_t count, cons
         if (k == 0)
             continue;
         args.count = k;
-        for (int j = k + 1; j <= LPMM_MULTI_MAX; ++j)
+        for (int j = k + 1; j < kStartSlots; ++j)
             args.tile_start[j] = (uint32_t)tiles;
-        if (aligned)
-            hipLaunchKernelGGL((adamw4bit_kernel<true, Arith>), dim3((uint32_t)tiles), dim3(kThreads), 0,
-                               (hipStream_t)stream, args, qmap_m, qmap_v);
+        for (int j = 0; j < kCoarseSlots; ++j)
+            args.coarse[j] = args.tile_start[8 * (j + 1)];
+        const dim3 grid((uint32_t)tiles), block(kThreads);
+        if (aligned && allfull)
+            hipLaunchKernelGGL((adamw4bit_kernel<true, true, Arith>), grid, block, 0, (hipStream_t)stream, args,
+                               qmap_m, qmap_v);
+        else if (aligned)
+            hipLaunchKernelGGL((adamw4bit_kernel<true, false, Arith>), grid, block, 0, (hipStream_t)stream, args,
+                               qmap_m, qmap_v);
         else
-            hipLaunchKernelGGL((adamw4bit_kernel<false, Arith>), dim3((uint32_t)tiles), dim3(kThreads), 0,
-                               (hipStream_t)stream, args, qmap_m, qmap_v);
+            hipLaunchKernelGGL((adamw4bit_kernel<false, false, Arith>), grid, block, 0, (hipStream_t)stream, args,
+                               qmap_m, qmap_v);
         const int st = launch_status();
         if (st != LPMM_OK)
             return st;

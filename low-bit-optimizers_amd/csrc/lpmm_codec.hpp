@@ -123,6 +123,9 @@ __device__ __forceinline__ void lds_fill(uint32_t *lds, const float *__restrict_
 
 // The same in two halves, so that a kernel can issue these small loads first, start its
 // streaming loads, and write LDS once the small ones have arrived (loads return in order).
+// Every thread loads and every thread stores (threads past the tables repeat an entry, so some
+// addresses are written several times with the same value): no branch surrounds either half,
+// and the wait before the stores counts exactly the loads issued in between.
 struct LdsFill {
     uint32_t q;
     uint4 e;
@@ -130,10 +133,9 @@ struct LdsFill {
 
 __device__ __forceinline__ LdsFill lds_fill_load(const float *__restrict__ q0, const float *__restrict__ q1)
 {
-    // every thread loads (from a clamped index), so that no branch surrounds the loads
     LdsFill f;
     const uint32_t t = threadIdx.x;
-    const float *qp = (t < 16) ? q0 + t : q1 + (t & 15);
+    const float *qp = ((t & 16) == 0) ? q0 + (t & 15) : q1 + (t & 15);
     f.q = __float_as_uint(*qp);
     const uint32_t te = t < 2 * kEncBuckets ? t : 2 * kEncBuckets - 1;
     f.e = *reinterpret_cast<const uint4 *>(kEncTableM[te]);
@@ -142,10 +144,8 @@ __device__ __forceinline__ LdsFill lds_fill_load(const float *__restrict__ q0, c
 
 __device__ __forceinline__ void lds_fill_store(uint32_t *lds, const LdsFill &f)
 {
-    if (threadIdx.x < 32)
-        lds[threadIdx.x] = f.q;  // kLdsQ0 = 0, kLdsQ1 = 64: the two maps are adjacent
-    if (threadIdx.x < 2 * kEncBuckets)
-        *reinterpret_cast<uint4 *>(reinterpret_cast<char *>(lds) + f.e.w) = f.e;
+    lds[threadIdx.x & 31] = f.q;  // kLdsQ0 = 0, kLdsQ1 = 64: the two maps are adjacent
+    *reinterpret_cast<uint4 *>(reinterpret_cast<char *>(lds) + f.e.w) = f.e;
 }
 static_assert(kLdsQ0 == 0 && kLdsQ1 == 64, "lds_fill_store writes the maps back to back");
 
