@@ -35,7 +35,7 @@ MULTI_MAX = 48                 # tensors per launch record (LPMM_MULTI_MAX)
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
 # script (each counter scaled by what it reads for a plain 1 GiB copy, --copy-probe; the summary is
 # kept under profiles/).  Algorithmic bytes per launch for that workload: 19.035e9.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"llama7b": 19.12e9}
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"llama7b": 19.125e9}
 
 
 def llama7b_shapes():
@@ -367,7 +367,9 @@ def main():
         / (elapsed / args.steps) / 1e9,
         "roofline": {
             "bound": "hbm",
-            "kernel": "lpmm::adamw4bit_kernel<true, lpmm::FusedArith>",
+            # second template argument: every quantised tensor is a whole number of 2048-element tiles
+            "kernel": "lpmm::adamw4bit_kernel<true, %s, lpmm::FusedArith>" % (
+                "true" if all(p.numel() % 2048 == 0 for p in params if p.numel() > 4096) else "false"),
             "achieved": achieved,
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
