@@ -72,7 +72,7 @@ def test_argument_errors_without_gpu():
     assert lib.lpmm_factored_stats(ptr, 8, 8, ptr, ptr, ptr, 0.999, None, None) == NULL
     assert lib.lpmm_factored_update(ptr, ptr, ptr, ptr, ptr, ptr, ptr, ptr, 0, 8, 0.9, 0.999, 1e-3, 0.01, 1e-8, 1.0,
                                     0, None) == SIZE
-    assert lib.lpmm_factored_workspace_bytes(4096, 11008) == (128 * 11008 + 11 * 4096 + 16 + 1) * 8
+    assert lib.lpmm_factored_workspace_bytes(4096, 11008) == (64 * 11008 + 11 * 4096 + 16 + 1) * 8  # 64-row tiles
     assert lib.lpmm_status_string(NULL).decode().startswith("a required pointer")
     with pytest.raises(RuntimeError, match="status 3"):
         _native.check(SIZE, "probe")
@@ -239,3 +239,21 @@ def test_oracle_under_sanitizers(tmp_path):
     out = subprocess.run([exe], capture_output=True, text=True)
     assert out.returncode == 0, out.stderr[-2000:]
     assert "ok" in out.stdout
+
+
+def test_utils_metrics_and_bookkeeping():
+    """lpmm.utils: closed forms of the error metrics, byte counting, rank helpers."""
+    from lpmm import utils
+
+    x = torch.tensor([3.0, 4.0])
+    qx = torch.tensor([3.0, 3.0])
+    assert utils.relerr(x, qx).item() == pytest.approx(1.0 / 5.0)
+    assert utils.abserr(x, qx).item() == pytest.approx(0.5)
+    assert utils.sqnr(x, qx).item() == pytest.approx(20 * np.log10(5.0), rel=1e-6)
+    assert utils.compute_tensor_bytes([torch.zeros(10), torch.zeros(6, dtype=torch.int8),
+                                       torch.zeros(4, dtype=torch.bfloat16)]) == 40 + 6 + 8
+    assert utils.compute_tensor_bytes(torch.zeros(3, dtype=torch.float64)) == 0  # a type the reference does not list
+    assert utils.get_rank() == 0 and utils.get_world_size() == 1
+    assert utils.get_metric_fn("min")(1, 2) and utils.get_metric_fn("max")(2, 1)
+    with pytest.raises(NotImplementedError):
+        utils.get_metric_fn("median")
