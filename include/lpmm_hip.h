@@ -163,6 +163,15 @@ int lpmm_dequant_rank1(const uint8_t *codes, const float *rowmax, const float *c
  * ------------------------------------------------------------------------------------- */
 int lpmm_pack_nonlinear(const float *x, const float *qmap, int bits, int64_t n_padded, uint8_t *out,
                         void *stream);
+/* pack_nonlinear(..., stochastic=True): lpmm/cpp_extension/quantization.cc:54-63 with
+ * quantize_bsearch<true> (quantization_kernel.cu:418-421): between map entries q[lo-1] <= x <
+ * q[lo] the code is lo with probability (x - q[lo-1]) / (q[lo] - q[lo-1]).  The random numbers
+ * are the ones the reference draws (:443-451, :526-531): Philox4x32-10 keyed by `seed`, one
+ * subsequence per reference thread (4 * codes-per-byte consecutive values), starting `offset`
+ * outputs into each subsequence -- the (seed, offset) pair the reference takes from torch's
+ * default device generator (:480-487).  n_padded: a multiple of 32. */
+int lpmm_pack_nonlinear_sr(const float *x, const float *qmap, int bits, int64_t n_padded, uint64_t seed,
+                           uint64_t offset, uint8_t *out, void *stream);
 int lpmm_unpack_nonlinear(const uint8_t *codes, const float *qmap, int bits, int64_t n, float *out,
                           void *stream);
 int lpmm_quant_group_bits(const float *x, int64_t n, int64_t gp_sz, const float *qmap, int bits,

@@ -155,6 +155,111 @@ __global__ __launch_bounds__(kBThreads) void pack_bits_kernel(const float *__res
     store_codes(out, base, bits, c);
 }
 
+// ---------------------------------------------------------------------------------------
+// Stochastic rounding: pack_nonlinear(..., stochastic=True) of the reference
+// (quantization_kernel.cu:418-421 for the rounding, :443-451 and :526-531 for the random
+// stream).  The reference draws one curand_uniform per value from a Philox4x32-10 state that
+// curand_init(seed, thread id, offset) sets up per thread, a thread handling
+// work_per_thread = 4 * codes_per_byte consecutive values.  Philox is counter-based, so value i
+// gets its number directly: subsequence i / work_per_thread, output number
+// offset + i % work_per_thread of it -- counter {block lo, block hi, subsequence lo,
+// subsequence hi} with block = output number / 4, key = the two halves of the seed, the four
+// outputs of a block taken in the order x, y, z, w.
+// ---------------------------------------------------------------------------------------
+struct Philox4 {
+    uint32_t v[4];
+};
+
+__device__ __forceinline__ Philox4 philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, uint32_t k0,
+                                                 uint32_t k1)
+{
+#pragma unroll
+    for (int r = 0; r < 10; ++r) {
+        const uint32_t hi0 = __umulhi(0xD2511F53u, c0), lo0 = 0xD2511F53u * c0;
+        const uint32_t hi1 = __umulhi(0xCD9E8D57u, c2), lo1 = 0xCD9E8D57u * c2;
+        c0 = hi1 ^ c1 ^ k0;
+        c1 = lo1;
+        c2 = hi0 ^ c3 ^ k1;
+        c3 = lo0;
+        k0 += 0x9E3779B9u;
+        k1 += 0xBB67AE85u;
+    }
+    Philox4 o;
+    o.v[0] = c0; o.v[1] = c1; o.v[2] = c2; o.v[3] = c3;
+    return o;
+}
+
+// curand_uniform: (0, 1]
+__device__ __forceinline__ float philox_uniform(uint32_t u) { return (float)u * 0x1p-32f + 0x1p-33f; }
+
+// quantize_bsearch<true>: the code as stored (NaN -> all ones, as in search_code)
+__device__ __forceinline__ uint32_t search_code_sr(const float *lds_map, int bits, float x, float noise)
+{
+    int lo = 0, hi = 1 << bits;
+    if (x <= lds_map[0])
+        return 0u;
+    if (lds_map[hi - 1] <= x)
+        return (uint32_t)(hi - 1);
+    while (lo < hi) {
+        const int mi = (lo + hi) >> 1;
+        if (lds_map[mi] <= x)
+            lo = mi + 1;
+        else
+            hi = mi;
+    }
+    if (lo == 0)
+        return codes_per_byte(bits) == 1 ? 255u : (1u << bits) - 1u;
+    const float proba = (x - lds_map[lo - 1]) / (lds_map[lo] - lds_map[lo - 1]);
+    const float t = (proba + noise) - 0.5f;
+    const int flag = (int)__builtin_rintf(t);  // __float2int_rn
+    return (uint32_t)(flag ? lo : lo - 1);
+}
+
+__global__ __launch_bounds__(kBThreads) void pack_bits_sr_kernel(const float *__restrict__ x,
+                                                                 const float *__restrict__ qmap, int bits,
+                                                                 int64_t n_padded, uint64_t seed, uint64_t offset,
+                                                                 uint8_t *__restrict__ out, bool vec)
+{
+    __shared__ float lds_map[256];
+    fill_map(lds_map, qmap, bits);
+    __syncthreads();
+    const int64_t base = ((int64_t)blockIdx.x * kBThreads + threadIdx.x) * kBElts;
+    if (base == 0)
+        out[last_byte(n_padded, bits)] = 0;
+    if (base >= n_padded)
+        return;
+    float v[kBElts];
+    load_values(x, base, n_padded, vec, v);
+    // the lane's 8 values are two runs of 4 consecutive outputs: work_per_thread is 4, 8, 16 or
+    // 32 and base a multiple of 8, so a run of 4 never straddles reference threads; it
+    // straddles Philox blocks only when offset is not a multiple of 4
+    const int wpt = 4 * codes_per_byte(bits);
+    uint32_t c[kBElts];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        const uint64_t i = (uint64_t)base + 4 * h;
+        const uint64_t sub = i / wpt;
+        const uint64_t pos = offset + (i - sub * wpt);  // output number of the run's first value
+        const uint64_t blk = pos >> 2;
+        const int ph = (int)(pos & 3);
+        const Philox4 a = philox4x32_10((uint32_t)blk, (uint32_t)(blk >> 32), (uint32_t)sub, (uint32_t)(sub >> 32),
+                                        (uint32_t)seed, (uint32_t)(seed >> 32));
+        uint32_t u[4] = {a.v[0], a.v[1], a.v[2], a.v[3]};
+        if (ph != 0) {  // uniform over the launch
+            const uint64_t nb = blk + 1;
+            const Philox4 b = philox4x32_10((uint32_t)nb, (uint32_t)(nb >> 32), (uint32_t)sub, (uint32_t)(sub >> 32),
+                                            (uint32_t)seed, (uint32_t)(seed >> 32));
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+                u[k] = (k + ph < 4) ? a.v[(k + ph) & 3] : b.v[(k + ph) & 3];
+        }
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+            c[4 * h + k] = search_code_sr(lds_map, bits, v[4 * h + k], philox_uniform(u[k]));
+    }
+    store_codes(out, base, bits, c);
+}
+
 // unpack_nonlinear: out[i] = qmap[code_i] for i < n (n a multiple of 8).
 __global__ __launch_bounds__(kBThreads) void unpack_bits_kernel(const uint8_t *__restrict__ codes,
                                                                 const float *__restrict__ qmap, int bits, int64_t n,
@@ -348,6 +453,26 @@ extern "C" int lpmm_pack_nonlinear(const float *x, const float *qmap, int bits, 
         return LPMM_ERR_SIZE;
     hipLaunchKernelGGL(pack_bits_kernel, dim3(tiles), dim3(kBThreads), 0, (hipStream_t)stream, x, qmap, bits,
                        n_padded, out, aligned_to(x, 16));
+    return launch_status();
+}
+
+extern "C" int lpmm_pack_nonlinear_sr(const float *x, const float *qmap, int bits, int64_t n_padded,
+                                      uint64_t seed, uint64_t offset, uint8_t *out, void *stream)
+{
+    // a reference thread handles up to 32 values (1-bit codes): whole threads only
+    if (!bits_ok(bits) || n_padded <= 0 || (n_padded % 32) != 0)
+        return LPMM_ERR_SIZE;
+    LPMM_REQUIRE_PTR(x);
+    LPMM_REQUIRE_PTR(qmap);
+    LPMM_REQUIRE_PTR(out);
+    LPMM_REQUIRE_ALIGN(x, 4);
+    LPMM_REQUIRE_ALIGN(qmap, 4);
+    LPMM_REQUIRE_ALIGN(out, 8);
+    uint32_t tiles;
+    if (!tiles_for(n_padded, &tiles))
+        return LPMM_ERR_SIZE;
+    hipLaunchKernelGGL(pack_bits_sr_kernel, dim3(tiles), dim3(kBThreads), 0, (hipStream_t)stream, x, qmap, bits,
+                       n_padded, seed, offset, out, aligned_to(x, 16));
     return launch_status();
 }
 

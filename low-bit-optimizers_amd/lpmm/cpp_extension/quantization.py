@@ -1,6 +1,7 @@
 """lpmm.cpp_extension.quantization: pack_nonlinear / unpack_nonlinear of the reference's
-pybind module (lpmm/cpp_extension/quantization.cc:54-83) for round-to-nearest codes of 1..8 bits.
-Both allocate and return a new tensor on the input's device and leave the inputs untouched."""
+pybind module (lpmm/cpp_extension/quantization.cc:54-83) for codes of 1..8 bits, rounded to
+nearest or stochastically.  Both allocate and return a new tensor on the input's device and
+leave the inputs untouched."""
 import torch
 
 from .. import _native
@@ -28,20 +29,32 @@ def pack_nonlinear(data, qmap, bits, stochastic):
     """data: float32 (num_groups, group_size), already normalised.  Returns int8 of
     storage_bits*numel/8 + 1 bytes (lpmm/cpp_extension/quantization_kernel.cu:475-477, :549-550; storage_bits
     is `bits` for 1, 2 and 4 and 8 otherwise); the final byte,
-    left uninitialised by the reference, is 0.  Unlike the reference this does not touch
-    torch's default random generator."""
+    left uninitialised by the reference, is 0.
+
+    stochastic=True draws its random numbers as the reference does
+    (lpmm/cpp_extension/quantization_kernel.cu:480-487): a (seed, offset) pair from torch's default
+    generator of the device, whose offset advances by group_size * work_per_thread rounded up
+    to a multiple of 4.  With stochastic=False the generator is left alone (the reference
+    advances it there too, although its kernel ignores the numbers)."""
     check_cuda_tensor_dim_float(data, "data", 2)
     check_cuda_tensor_dim_float(qmap, "qmap", 1)
     _check_bits(bits, qmap)
-    if stochastic:
-        raise NotImplementedError("stochastic rounding is not part of this build")
     if data.size(1) % (4 * (8 // _storage_bits(bits))) != 0 or data.numel() % 8 != 0:
         raise RuntimeError("Expected group_size % work_per_thread == 0 to be true, but got false.")
     dev = same_device(data, qmap)
     n = data.numel()
     out = torch.empty((n * _storage_bits(bits) // 8 + 1,), dtype=torch.int8, device=dev)
     with torch.cuda.device(dev):
-        if bits == 4:
+        if stochastic:
+            if n % 32 != 0:
+                raise RuntimeError("stochastic rounding needs a multiple of 32 values")
+            work_per_thread = 4 * (8 // _storage_bits(bits))
+            gen = torch.cuda.default_generators[dev.index if dev.index is not None else torch.cuda.current_device()]
+            seed, offset = gen.initial_seed(), gen.get_offset()
+            gen.set_offset(offset + (data.size(1) * work_per_thread + 3) // 4 * 4)
+            st = _native.lib().lpmm_pack_nonlinear_sr(data.data_ptr(), qmap.data_ptr(), bits, n, seed, offset,
+                                                      out.data_ptr(), _native.current_stream(dev))
+        elif bits == 4:
             st = _native.lib().lpmm_pack_nonlinear_4bit(data.data_ptr(), qmap.data_ptr(), n, out.data_ptr(),
                                                         _native.current_stream(dev))
         else:

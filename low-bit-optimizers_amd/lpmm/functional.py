@@ -146,15 +146,18 @@ def _compute_sm3_scale_tensor(max_dims):
 # --------------------------------------------------------------------------------------
 # code search + packing on already-normalised values (lpmm/functional.py:359-400)
 # --------------------------------------------------------------------------------------
+_ROUND_TYPES = ("real-nearest", "real-sr")  # the two that go through the packing operator
+
+
 def nonlinear_quant(qx, qmap, b, round_type="sr"):
-    if round_type != "real-nearest":
-        raise NotImplementedError(f"round_type {round_type!r}: this build implements 'real-nearest' only")
-    return ext_quantization.pack_nonlinear(group_tensor(qx, PACK_GROUP), qmap, b, False)
+    if round_type not in _ROUND_TYPES:
+        raise NotImplementedError(f"round_type {round_type!r}: this build implements {_ROUND_TYPES} only")
+    return ext_quantization.pack_nonlinear(group_tensor(qx, PACK_GROUP), qmap, b, round_type == "real-sr")
 
 
 def nonlinear_dequant(qx, qmap, b, shape, round_type="sr"):
     if not round_type.startswith("real"):
-        raise NotImplementedError(f"round_type {round_type!r}: this build implements 'real-nearest' only")
+        raise NotImplementedError(f"round_type {round_type!r}: this build implements {_ROUND_TYPES} only")
     num_groups = (shape.numel() + PACK_GROUP - 1) // PACK_GROUP
     return recon_grouped_tensor(ext_quantization.unpack_nonlinear(qx, qmap, b, num_groups, PACK_GROUP), shape)
 
@@ -174,9 +177,9 @@ def _require_supported(kwargs, x):
         raise ValueError(f"Not support {kwargs['quant_type']} quant type.")
     if not 1 <= kwargs["b"] <= 8:
         raise ValueError(f"code width must be 1..8 bits, got {kwargs['b']}")
-    if not kwargs["round_type"].startswith("real-nearest"):
+    if kwargs["round_type"] not in _ROUND_TYPES:
         raise NotImplementedError(
-            f"round_type {kwargs['round_type']!r}: this build implements 'real-nearest' only")
+            f"round_type {kwargs['round_type']!r}: this build implements {_ROUND_TYPES} only")
     if not x.is_cuda:
         raise RuntimeError("x must be a CUDA tensor! (the quantised optimizer path has no CPU implementation)")
 
@@ -253,23 +256,26 @@ def vectorwise_quant(x, **kwargs):
     as_group = scale_type == "group" or (scale_type == "rank1" and src.dim() == 1)
     if scale_type == "rank1":
         md["dim"] = src.dim()
+    # stochastic rounding: scaling by PyTorch device ops as in the reference
+    # (lpmm/functional.py:184-203), the search and packing by the HIP operator
+    nearest = kwargs["round_type"] == "real-nearest"
     if as_group:
         gp_sz = kwargs["gp_sz"] if scale_type == "group" else 128
-        if _group_gp_sz_ok(gp_sz):
+        if nearest and _group_gp_sz_ok(gp_sz):
             codes, max1 = quant_group_(src, qmap, gp_sz, b=b)
         else:  # any other group size: PyTorch reductions, HIP search + pack
             grouped = group_tensor(src, gp_sz)
             max1 = _max_reduce_except_dim(grouped.abs(), 0)
-            codes = nonlinear_quant(grouped.div(max1), qmap, b, round_type="real-nearest")
+            codes = nonlinear_quant(grouped.div(max1), qmap, b, round_type=kwargs["round_type"])
         md["max1"] = max1
         md["scaled_shape"] = torch.Size((max1.shape[0], gp_sz))
     elif scale_type == "rank1":
-        if src.dim() == 2:
+        if nearest and src.dim() == 2:
             codes, max_dims = quant_rank1_(src, qmap, b=b)
         else:
             max_dims = get_sm3_statistics(src.abs())
             codes = nonlinear_quant(src.div(_compute_sm3_scale_tensor(max_dims)), qmap, b,
-                                    round_type="real-nearest")
+                                    round_type=kwargs["round_type"])
         md["max_dims"] = max_dims
         md["max1"] = None
         md["scaled_shape"] = src.shape

@@ -28,6 +28,11 @@
  *   nonfused_step       PyTorch CPU op sequence (library ops) of the reference's
  *                       _single_tensor_adamw4bit, to 1e-6 relative.
  *   factored_step       closed form v = row*col/mean(row) (Adafactor); rank-one g^2 case.
+ *   philox / SR pack    Random123's known-answer vectors for philox4x32-10; torch.randint on
+ *                       the GPU for cuRAND's state conventions; noise = 0.5 reduces the
+ *                       stochastic search to round-to-nearest on the linear scale; the
+ *                       empirical mean of the decoded codes equals x.  Against a real CUDA
+ *                       build: parity unpinned (no CUDA here).
  * The reference ships no tests, golden vectors or fixtures for any of these.
  */
 #include <math.h>
@@ -158,6 +163,118 @@ void lpmm_oracle_unpack_nonlinear(const uint8_t *codes, const float *qmap, int b
         for (int64_t i = 0; i < n; ++i)
             out[i] = qmap[codes[i] & mask];
     }
+}
+
+/* ------------------------------------------------------------------------------------ */
+/* Stochastic rounding (quantize_bsearch<true>, quantization_kernel.cu:418-421) with the   */
+/* random stream the reference draws it from: curandStatePhilox4_32_10_t initialised per   */
+/* thread with curand_init(seed, thread id, offset) and read with curand_uniform           */
+/* (quantization_kernel.cu:443-451, :526-531).  cuRAND itself is not part of the reference */
+/* tree; its generator is the published Philox4x32-10 of Salmon et al. (SC'11, Random123), */
+/* restated here, with cuRAND's documented conventions: key = the two halves of the seed,  */
+/* counter words {x, y} = block index within the subsequence (offset / 4), {z, w} = the    */
+/* subsequence, the four outputs of a block consumed in the order x, y, z, w starting at   */
+/* offset % 4, and uniform = u * 2^-32 + 2^-33 in float, i.e. (0, 1].                      */
+/* Pinned by: the three known-answer vectors of Random123 for philox4x32-10; PyTorch's     */
+/* device generator on the GPU (torch.randint, which draws the raw outputs from the same    */
+/* state layout) for the counter/subsequence/ordering conventions.  The uniform conversion  */
+/* is cuRAND's documented one; the device library under PyTorch-ROCm differs from it in the */
+/* last place, so it is compared to within that.                                            */
+/* ------------------------------------------------------------------------------------ */
+static inline void philox_round(uint32_t c[4], const uint32_t k[2])
+{
+    const uint64_t p0 = (uint64_t)0xD2511F53u * c[0];
+    const uint64_t p1 = (uint64_t)0xCD9E8D57u * c[2];
+    const uint32_t n0 = (uint32_t)(p1 >> 32) ^ c[1] ^ k[0];
+    const uint32_t n1 = (uint32_t)p1;
+    const uint32_t n2 = (uint32_t)(p0 >> 32) ^ c[3] ^ k[1];
+    const uint32_t n3 = (uint32_t)p0;
+    c[0] = n0; c[1] = n1; c[2] = n2; c[3] = n3;
+}
+
+void lpmm_oracle_philox4x32_10(const uint32_t ctr[4], const uint32_t key[2], uint32_t out[4])
+{
+    uint32_t c[4] = {ctr[0], ctr[1], ctr[2], ctr[3]};
+    uint32_t k[2] = {key[0], key[1]};
+    for (int r = 0; r < 10; ++r) {
+        if (r > 0) {
+            k[0] += 0x9E3779B9u;
+            k[1] += 0xBB67AE85u;
+        }
+        philox_round(c, k);
+    }
+    out[0] = c[0]; out[1] = c[1]; out[2] = c[2]; out[3] = c[3];
+}
+
+/* draw number j (0-based) of the state curand_init(seed, subsequence, offset) gives */
+uint32_t lpmm_oracle_philox_draw(uint64_t seed, uint64_t subsequence, uint64_t offset, uint64_t j)
+{
+    const uint64_t pos = offset + j;  /* position in the subsequence, in 32-bit outputs */
+    const uint64_t block = pos >> 2;
+    const uint32_t ctr[4] = {(uint32_t)block, (uint32_t)(block >> 32), (uint32_t)subsequence,
+                             (uint32_t)(subsequence >> 32)};
+    const uint32_t key[2] = {(uint32_t)seed, (uint32_t)(seed >> 32)};
+    uint32_t out[4];
+    lpmm_oracle_philox4x32_10(ctr, key, out);
+    return out[pos & 3];
+}
+
+float lpmm_oracle_philox_uniform(uint64_t seed, uint64_t subsequence, uint64_t offset, uint64_t j)
+{
+    const float u = (float)lpmm_oracle_philox_draw(seed, subsequence, offset, j);
+    return u * 0x1p-32f + 0x1p-33f;
+}
+
+/* quantize_bsearch<true> (quantization_kernel.cu:397-421).  NaN gives -1 as in the
+ * non-stochastic search (the reference reads qmap[-1] there; __float2int_rn(NaN) is 0, so it
+ * returns lo - 1 = -1 whatever that read yields). */
+int lpmm_oracle_qmapping_sr(const float *qmap, int bits, float x, float noise)
+{
+    int lo = 0;
+    int hi = 1 << bits;
+
+    if (x <= qmap[lo])
+        return lo;
+    if (qmap[hi - 1] <= x)
+        return hi - 1;
+    while (lo < hi) {
+        int mi = (lo + hi) >> 1;
+        if (qmap[mi] <= x)
+            lo = mi + 1;
+        else
+            hi = mi;
+    }
+    if (lo == 0)
+        return -1;
+    const float proba = (x - qmap[lo - 1]) / (qmap[lo] - qmap[lo - 1]);
+    const float t = (proba + noise) - 0.5f;
+    const int flag = (int)rintf(t); /* __float2int_rn: to nearest, ties to even */
+    return flag ? lo : lo - 1;
+}
+
+/* pack_nonlinear(..., stochastic=True) for any width: thread t of the reference's launch
+ * handles work_per_thread consecutive values (4 * 8/bits for the packing widths 1, 2, 4,
+ * quantization_kernel.cu:437-441; 4 for the one-code-per-byte widths, :525) and draws one
+ * uniform per value, in order, from subsequence t (:443-451, :526-531). */
+void lpmm_oracle_pack_nonlinear_sr(const float *x, const float *qmap, int bits, int64_t n_padded,
+                                   uint64_t seed, uint64_t offset, uint8_t *out)
+{
+    const int packed = width_is_packed(bits);
+    const int per = packed ? 8 / bits : 1;
+    const int wpt = 4 * per;
+    const int mask = (1 << bits) - 1;
+#pragma omp parallel for schedule(static)
+    for (int64_t b = 0; b < n_padded / per; ++b) {
+        uint8_t byte = 0;
+        for (int j = 0; j < per; ++j) {
+            const int64_t i = b * per + j;
+            const float noise = lpmm_oracle_philox_uniform(seed, (uint64_t)(i / wpt), offset, (uint64_t)(i % wpt));
+            const int q = lpmm_oracle_qmapping_sr(qmap, bits, x[i], noise);
+            byte |= packed ? (uint8_t)((q & mask) << (j * bits)) : (uint8_t)q;
+        }
+        out[b] = byte;
+    }
+    out[n_padded / per] = 0;
 }
 
 /* ------------------------------------------------------------------------------------ */

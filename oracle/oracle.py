@@ -55,6 +55,13 @@ _pack = _sig("lpmm_oracle_pack_nonlinear_4bit", None, _f32p, _f32p, _i64, _u8p)
 _unpack = _sig("lpmm_oracle_unpack_nonlinear_4bit", None, _u8p, _f32p, _i64, _f32p)
 _pack_bits = _sig("lpmm_oracle_pack_nonlinear", None, _f32p, _f32p, ctypes.c_int, _i64, _u8p)
 _unpack_bits = _sig("lpmm_oracle_unpack_nonlinear", None, _u8p, _f32p, ctypes.c_int, _i64, _f32p)
+_u32p = np.ctypeslib.ndpointer(dtype=np.uint32, flags="C_CONTIGUOUS")
+_u64 = ctypes.c_uint64
+_philox = _sig("lpmm_oracle_philox4x32_10", None, _u32p, _u32p, _u32p)
+_philox_draw = _sig("lpmm_oracle_philox_draw", ctypes.c_uint32, _u64, _u64, _u64, _u64)
+_philox_uniform = _sig("lpmm_oracle_philox_uniform", _f, _u64, _u64, _u64, _u64)
+_qmapping_sr = _sig("lpmm_oracle_qmapping_sr", ctypes.c_int, _f32p, ctypes.c_int, _f, _f)
+_pack_sr = _sig("lpmm_oracle_pack_nonlinear_sr", None, _f32p, _f32p, ctypes.c_int, _i64, _u64, _u64, _u8p)
 _adamw_fp32 = _sig("lpmm_oracle_adamw_fp32_step", None, _f32p, _f32p, _f32p, _f32p, _i64,
                    _f, _f, _f, _f, _f, _f)
 _adamw4bit = _sig("lpmm_oracle_adamw4bit_step", None, _f32p, _f32p, _u8p, _u8p, _f32p, _f32p,
@@ -214,6 +221,37 @@ def pack_nonlinear(x, qmap, bits):
     assert x.size % 8 == 0 and len(qmap) == 2 ** bits
     out = np.empty(x.size * storage_bits(bits) // 8 + 1, dtype=np.uint8)
     _pack_bits(x, _c(qmap, np.float32), bits, x.size, out)
+    return out
+
+
+def philox4x32_10(ctr, key):
+    """One Philox4x32-10 block: ctr 4 words, key 2 words -> 4 words."""
+    out = np.empty(4, np.uint32)
+    _philox(_c(ctr, np.uint32), _c(key, np.uint32), out)
+    return out
+
+
+def philox_draw(seed, subsequence, offset, j):
+    """32-bit output number j of the state curand_init(seed, subsequence, offset) gives."""
+    return int(_philox_draw(seed, subsequence, offset, j))
+
+
+def philox_uniform(seed, subsequence, offset, j):
+    """curand_uniform of that output: u * 2^-32 + 2^-33 in float, (0, 1]."""
+    return float(_philox_uniform(seed, subsequence, offset, j))
+
+
+def qmapping_sr(qmap, x, noise, bits=4):
+    """quantize_bsearch<true>: the int the reference returns (-1 for NaN)."""
+    return int(_qmapping_sr(_c(qmap, np.float32), bits, x, noise))
+
+
+def pack_nonlinear_sr(x, qmap, bits, seed, offset):
+    """pack_nonlinear(..., stochastic=True) with the Philox stream (seed, offset)."""
+    x = _c(x, np.float32).reshape(-1)
+    assert x.size % 32 == 0 and len(qmap) == 2 ** bits
+    out = np.empty(x.size * storage_bits(bits) // 8 + 1, dtype=np.uint8)
+    _pack_sr(x, _c(qmap, np.float32), bits, x.size, seed, offset, out)
     return out
 
 
