@@ -162,6 +162,42 @@ def test_multi_tensor_matches_single(oracle, qmaps):
         assert_rel(to_np(d["p"]), h["p"], "p")
 
 
+def test_multi_tensor_whole_tiles(oracle, qmaps):
+    """110 tensors, every one a whole number of 2048-element tiles (the straight-line variant of
+    the kernel), three launch records with tensors of 1 to 5 tiles: every tile finds its tensor
+    through the two-level lookup, also across the boundaries of its coarse table."""
+    nat = _native()
+    lib = nat.lib()
+    qm, qv = qmaps
+    dqm, dqv = to_dev(qm), to_dev(qv)
+    rng = np.random.default_rng(77)
+    sizes = [2048 * int(k) for k in rng.integers(1, 6, 110)]
+    host, devs, recs = [], [], []
+    for i, n in enumerate(sizes):
+        h = dict(p=(rng.standard_normal(n) * 0.02).astype(np.float32),
+                 g=(rng.standard_normal(n) * 1e-3).astype(np.float32),
+                 mc=rng.integers(0, 256, n // 2, dtype=np.uint8), vc=rng.integers(0, 256, n // 2, dtype=np.uint8),
+                 ms=np.abs(rng.standard_normal(n // 128) * 1e-3).astype(np.float32),
+                 vs=np.abs(rng.standard_normal(n // 128) * 1e-6).astype(np.float32), step=float(1 + i % 5))
+        d = {k: to_dev(v) for k, v in h.items() if k != "step"}
+        host.append(h); devs.append(d)
+        recs.append((d["p"].data_ptr(), d["g"].data_ptr(), d["mc"].data_ptr(), d["vc"].data_ptr(),
+                     d["ms"].data_ptr(), d["vs"].data_ptr(), n, h["step"], 0.0))
+    table = np.array(recs, dtype=nat.ADAMW4BIT_TENSOR)
+    st = lib.lpmm_adamw4bit_step_multi(table.ctypes.data, len(recs), dqm.data_ptr(), dqv.data_ptr(), 0.9, 0.999,
+                                       1e-3, 0.01, 1e-8, torch.cuda.current_stream().cuda_stream)
+    assert st == 0
+    torch.cuda.synchronize()
+    for i, (h, d, n) in enumerate(zip(host, devs, sizes)):
+        oracle.adamw4bit_step(h["p"], h["g"], h["mc"], h["vc"], h["ms"], h["vs"], qm, qv, 0.9, 0.999, 1e-3, 0.01,
+                              1e-8, h["step"])
+        assert_codes(to_np(d["mc"]), h["mc"], n, f"m codes of tensor {i}")
+        assert_codes(to_np(d["vc"]), h["vc"], n, f"v codes of tensor {i}")
+        assert_rel(to_np(d["ms"]), h["ms"], f"m scale of tensor {i}")
+        assert_rel(to_np(d["vs"]), h["vs"], f"v scale of tensor {i}")
+        assert_rel(to_np(d["p"]), h["p"], f"p of tensor {i}")
+
+
 def test_fused_step_extreme_scales(oracle, qmaps):
     """Group maxima outside [2^-60, 2^60] leave the reciprocal-based division for the plain one;
     gradients small enough that g*g underflows give all-zero v groups (code 15, scale 0)."""
