@@ -244,6 +244,44 @@ def test_golden_fixture_on_gpu(qmaps):
         fused_adamw.adamw4bit_single_tensor(p, g[:-2], mc, vc, ms, vs, qm, qv, 0.9, 0.999, 1e-3, 0.01, 1e-8, 4.0)
 
 
+@pytest.mark.parametrize("kind", ["group", "rank1", "factored"])
+def test_golden_nonfused_fixture_on_gpu(kind):
+    """The committed non-fused fixture (tests/golden/nonfused_steps_small.npz) through
+    lpmm.optim.AdamW(fused=False): block-wise second moment (one-pass kernel), rank-1 second
+    moment (two-pass kernels, the default configuration) and factored second moment."""
+    import lpmm
+
+    gold = np.load(os.path.join(HERE, "golden", "nonfused_steps_small.npz"))
+    cfg_dir = os.path.join(os.path.dirname(lpmm.config.__file__), "configs")
+    p = torch.nn.Parameter(to_dev(gold["p0"]))
+    if kind == "factored":
+        opt = lpmm.optim.AdamW([p], fused=False, factor_second_moment=True, **H)
+    else:
+        cfg = os.path.join(cfg_dir, "default.yml" if kind == "rank1" else "2nd_moment_group_128.yml")
+        opt = lpmm.optim.AdamW([p], fused=False, qconfig=cfg, **H)
+    for s in range(3):
+        p.grad = to_dev(gold["grads"][s])
+        opt.step()
+        torch.cuda.synchronize()
+        st = opt.state[p]
+        k = f"{kind}{s + 1}"
+        np.testing.assert_array_equal(to_np(st["exp_avg"]).view(np.uint8), gold[f"mc_{k}"], err_msg=f"m codes {k}")
+        np.testing.assert_array_equal(to_np(st["exp_avg_qstate"]["overhead"]["max1"]).reshape(-1), gold[f"ms_{k}"])
+        if kind == "factored":
+            # sums of squares in double, folded in another order than the oracle's loop
+            assert_rel(to_np(st["exp_avg_sq_row"]), gold[f"row_{k}"], f"row {k}", tol=2e-7)
+            assert_rel(to_np(st["exp_avg_sq_col"]), gold[f"col_{k}"], f"col {k}", tol=2e-7)
+            continue
+        np.testing.assert_array_equal(to_np(st["exp_avg_sq"]).view(np.uint8), gold[f"vc_{k}"], err_msg=f"v codes {k}")
+        oh = st["exp_avg_sq_qstate"]["overhead"]
+        if kind == "rank1":
+            np.testing.assert_array_equal(to_np(oh["max_dims"][0]).reshape(-1), gold[f"vs0_{k}"])
+            np.testing.assert_array_equal(to_np(oh["max_dims"][1]).reshape(-1), gold[f"vs1_{k}"])
+        else:
+            np.testing.assert_array_equal(to_np(oh["max1"]).reshape(-1), gold[f"vs0_{k}"])
+    assert_rel(to_np(p.detach()), gold[f"p_{kind}3"], f"p {kind}", scale=gold["p0"])
+
+
 def test_checkpoint_resume_on_gpu(oracle):
     """state_dict -> load_state_dict -> continue gives the same bytes as an uninterrupted run."""
     import lpmm

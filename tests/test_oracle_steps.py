@@ -291,3 +291,25 @@ def test_factored_c_follows_torch_cpu_ops(oracle, qmaps):
         state.row[...] = ts["row"].numpy()
         state.col[...] = ts["col"].numpy()
         p_c[...] = p_t.numpy()
+
+
+@pytest.mark.parametrize("kind", ["group", "rank1", "factored"])
+def test_golden_nonfused_fixture(oracle, qmaps, kind):
+    """The committed non-fused fixture (tests/golden/nonfused_steps_small.npz) is what the oracle
+    produces today: guards the oracle and the fixture against drifting apart."""
+    gold = np.load(os.path.join(HERE, "golden", "nonfused_steps_small.npz"))
+    p = gold["p0"].copy()
+    st = oracle.NonFusedState(p.shape, v_scale_type="rank1" if kind == "rank1" else "group", factored=kind == "factored")
+    for s in range(3):
+        oracle.nonfused_step(p, gold["grads"][s], st, qmaps[0], qmaps[1], 1e-3, 0.9, 0.999, 1e-8, 0.01)
+        k = f"{kind}{s + 1}"
+        np.testing.assert_array_equal(st.m[0], gold[f"mc_{k}"])
+        np.testing.assert_array_equal(st.m[1], gold[f"ms_{k}"])
+        if kind == "factored":
+            np.testing.assert_array_equal(st.row, gold[f"row_{k}"])
+            np.testing.assert_array_equal(st.col, gold[f"col_{k}"])
+        else:
+            np.testing.assert_array_equal(st.v[0], gold[f"vc_{k}"])
+            for j, a in enumerate(st.v[1:]):
+                np.testing.assert_array_equal(a, gold[f"vs{j}_{k}"])
+    np.testing.assert_array_equal(p, gold[f"p_{kind}3"])
