@@ -1,93 +1,113 @@
-"""Small helpers with the names and meanings of the reference's lpmm/utils.py: device-memory
-bookkeeping (lpmm/utils.py:12-45), rank helpers (:48-58) and quantisation-error metrics
-(:78-116)."""
-import torch
-import torch.nn.functional as F
+"""Helpers that users of lpmm import next to the optimizers: device-memory bookkeeping, rank
+queries and quantisation-error metrics.  Names, arguments and results follow the reference's
+lpmm/utils.py (memory: lines 12-45, ranks: 48-58, metrics: 61-116)."""
+import operator
 
-_ITEM_BYTES = {torch.float32: 4, torch.int32: 4, torch.bfloat16: 2, torch.float16: 2, torch.int16: 2, torch.int8: 1}
+import torch
+
+# element sizes the reference's byte counter knows (lpmm/utils.py:38-43); any other dtype counts as 0
+_COUNTED_ITEMSIZE = {
+    torch.float32: 4, torch.int32: 4,
+    torch.bfloat16: 2, torch.float16: 2, torch.int16: 2,
+    torch.int8: 1,
+}
+_MIB = float(1 << 20)
+
+
+def _device0_memory():
+    return torch.cuda.memory_allocated(0), torch.cuda.memory_reserved(0)
 
 
 def empty_cache(ratio):
-    """Release torch's cached device memory when less than `ratio` of it is in use."""
-    if ratio is None:
-        return
-    reserved = torch.cuda.memory_reserved(0)
-    if reserved > 0 and torch.cuda.memory_allocated(0) / reserved < ratio:
-        torch.cuda.empty_cache()
+    """Hand torch's cached blocks of device 0 back to the driver when less than `ratio` of the
+    reserved memory is in use; `None` switches the check off."""
+    if ratio is not None:
+        in_use, reserved = _device0_memory()
+        if reserved > 0 and in_use < ratio * reserved:
+            torch.cuda.empty_cache()
 
 
 def get_memory_usage(print_info=False):
-    """Bytes currently allocated by torch on device 0."""
-    allocated = torch.cuda.memory_allocated(0)
+    """Bytes torch has allocated on device 0 right now."""
+    in_use, reserved = _device0_memory()
     if print_info:
-        print("allocated: %.2f MB" % (allocated / 2 ** 20), flush=True)
-        print("reserved:  %.2f MB" % (torch.cuda.memory_reserved(0) / 2 ** 20), flush=True)
-    return allocated
+        print(f"allocated: {in_use / _MIB:.2f} MB", flush=True)
+        print(f"reserved:  {reserved / _MIB:.2f} MB", flush=True)
+    return in_use
 
 
 def compute_tensor_bytes(tensors):
-    """Bytes held by a tensor or a list of tensors; as in the reference only the 4-, 2- and
-    1-byte types it lists are counted (float32/int32, bf16/fp16/int16, int8), others as 0."""
-    if not isinstance(tensors, (list, tuple)):
-        tensors = [tensors]
-    return sum(x.numel() * _ITEM_BYTES.get(x.dtype, 0) for x in tensors)
+    """Bytes held by one tensor or by a list/tuple of tensors."""
+    seq = tensors if isinstance(tensors, (list, tuple)) else (tensors,)
+    return sum(t.numel() * _COUNTED_ITEMSIZE.get(t.dtype, 0) for t in seq)
+
+
+def _dist_query(name, single_process_value):
+    dist = torch.distributed
+    return getattr(dist, name)() if dist.is_available() and dist.is_initialized() else single_process_value
 
 
 def get_rank():
-    return torch.distributed.get_rank() if torch.distributed.is_initialized() else 0
+    return _dist_query("get_rank", 0)
 
 
 def get_world_size():
-    return torch.distributed.get_world_size() if torch.distributed.is_initialized() else 1
+    return _dist_query("get_world_size", 1)
 
 
 def print0(*args, **kwargs):
+    """print on rank 0 only."""
     if get_rank() == 0:
         print(*args, **kwargs)
 
 
-def min_fn(a, b):
-    return a < b
-
-
-def max_fn(a, b):
-    return a > b
+min_fn = operator.lt  # "a is better than b" when smaller is better
+max_fn = operator.gt  # ... when larger is better
 
 
 def get_metric_fn(metric_op):
-    if metric_op == "min":
-        return min_fn
-    if metric_op == "max":
-        return max_fn
-    raise NotImplementedError
+    try:
+        return {"min": min_fn, "max": max_fn}[metric_op]
+    except KeyError:
+        raise NotImplementedError(metric_op) from None
+
+
+def _err(x, qx):
+    return x - qx
 
 
 def sqnr(x, qx):
-    """Signal-to-quantisation-noise ratio in dB."""
-    return 20 * torch.log10(torch.norm(x) / torch.norm(x - qx))
+    """Signal-to-quantisation-noise ratio in dB: 20 log10(|x| / |x - qx|)."""
+    return 20 * torch.log10(torch.linalg.vector_norm(x) / torch.linalg.vector_norm(_err(x, qx)))
 
 
 def relerr(x, qx):
-    return torch.abs(x - qx).norm() / torch.abs(x).norm()
-
-
-def jsd(x, qx):
-    x, qx = x.flatten(), qx.flatten()
-    m = 0.5 * (x + qx)
-    return 0.5 * (F.kl_div(x, m) + F.kl_div(qx, m))
+    """|x - qx| / |x| in the Euclidean norm."""
+    return torch.linalg.vector_norm(_err(x, qx)) / torch.linalg.vector_norm(x)
 
 
 def abserr(x, qx):
-    return torch.abs(x - qx).mean()
+    """Mean absolute error."""
+    return _err(x, qx).abs().mean()
+
+
+def jsd(x, qx):
+    """Jensen-Shannon style divergence of two flattened tensors, built from torch's kl_div with
+    its default arguments as in the reference (lpmm/utils.py:90-95)."""
+    a, b = x.reshape(-1), qx.reshape(-1)
+    mid = (a + b) / 2
+    kl = torch.nn.functional.kl_div
+    return (kl(a, mid) + kl(b, mid)) / 2
 
 
 def get_metric_from_q_and_dq(x, op, average, **kwargs):
-    """Mean relative error of op(x) against op(dequantise(quantise(x))) over `average`
-    round trips (lpmm/utils.py:102-116 always measures 'relerr')."""
+    """Relative error of op(x) against op(dequantise(quantise(x))), averaged over `average`
+    round trips (the reference measures 'relerr' whatever else it lists, lpmm/utils.py:103-116)."""
     from .functional import vectorwise_dequant, vectorwise_quant
 
-    total = 0.0
+    target = op(x)
+    runs = []
     for _ in range(average):
-        qx, md = vectorwise_quant(x, **kwargs)
-        total += relerr(op(x), op(vectorwise_dequant(qx, **md)))
-    return total / average
+        codes, meta = vectorwise_quant(x, **kwargs)
+        runs.append(relerr(target, op(vectorwise_dequant(codes, **meta))))
+    return sum(runs) / average
