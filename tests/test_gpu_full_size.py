@@ -55,6 +55,41 @@ def test_fused_step_llama_shapes(oracle, qmaps, shape):
     assert np.all(cv.max(axis=1) == 15)
 
 
+def test_nonfused_default_config_4096x4096(oracle, qmaps):
+    """The first benchmark configuration as it is written: non-fused lpmm.optim.AdamW with the
+    default configuration file (m block-wise 128 with the signed map, v rank-1 with the linear
+    map), one 4096 x 4096 fp32 parameter ~ N(0, 0.02), gradients ~ N(0, 1e-3) reseeded each
+    step, lr 1e-3, betas (0.9, 0.999), wd 0.01, 10 steps -- against the oracle's staged
+    sequence on the same inputs."""
+    import os
+
+    import lpmm
+
+    qm, qv = qmaps
+    shape = (4096, 4096)
+    p_ref = (torch.randn(shape, generator=torch.Generator().manual_seed(0)) * 0.02).numpy()
+    p = torch.nn.Parameter(to_dev(p_ref))
+    cfg = os.path.join(os.path.dirname(lpmm.config.__file__), "configs", "default.yml")
+    opt = lpmm.optim.AdamW([p], lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01, fused=False, qconfig=cfg)
+    state = oracle.NonFusedState(shape, v_scale_type="rank1")
+    n = p_ref.size
+    for step in range(1, 11):
+        g_np = (torch.randn(shape, generator=torch.Generator().manual_seed(1000 + step)) * 1e-3).numpy()
+        p.grad = to_dev(g_np)
+        opt.step()
+        p_before = p_ref.copy()
+        oracle.nonfused_step(p_ref, g_np, state, qm, qv, 1e-3, 0.9, 0.999, 1e-8, 0.01)
+        torch.cuda.synchronize()
+        st = opt.state[p]
+        oh = st["exp_avg_sq_qstate"]["overhead"]
+        np.testing.assert_array_equal(to_np(oh["max_dims"][0]).reshape(-1), state.v[1], err_msg=f"row maxima step {step}")
+        np.testing.assert_array_equal(to_np(oh["max_dims"][1]).reshape(-1), state.v[2], err_msg=f"col maxima step {step}")
+        np.testing.assert_array_equal(to_np(st["exp_avg_qstate"]["overhead"]["max1"]).reshape(-1), state.m[1])
+        assert_codes(to_np(st["exp_avg"]), state.m[0], n, f"m codes step {step}")
+        assert_codes(to_np(st["exp_avg_sq"]), state.v[0], n, f"v codes step {step}")
+        assert_rel(to_np(p.detach()), p_ref, f"p step {step}", scale=p_before)
+
+
 def test_quant_roundtrip_64m(oracle, qmaps):
     import lpmm.functional as F
 
