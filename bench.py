@@ -367,9 +367,10 @@ def main():
         / (elapsed / args.steps) / 1e9,
         "roofline": {
             "bound": "hbm",
-            # second template argument: every quantised tensor is a whole number of 2048-element tiles
+            # second template argument, chosen per launch: every tensor of the launch is a whole
+            # number of 2048-element tiles
             "kernel": "lpmm::adamw4bit_kernel<true, %s, lpmm::FusedArith>" % (
-                "true" if all(p.numel() % 2048 == 0 for p in params if p.numel() > 4096) else "false"),
+                "true" if all(p.numel() % 2048 == 0 for p in params if p.numel() > 4096) else "true|false"),
             "achieved": achieved,
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",

@@ -383,7 +383,6 @@ static int step_multi4(const lpmm_adamw4bit_tensor *tensors, int64_t count, cons
     LPMM_REQUIRE_PTR(qmap_v);
     LPMM_REQUIRE_ALIGN(qmap_m, 4);
     LPMM_REQUIRE_ALIGN(qmap_v, 4);
-    bool aligned = true, allfull = true;
     for (int64_t i = 0; i < count; ++i) {
         const lpmm_adamw4bit_tensor &t = tensors[i];
         if (t.n < 0)
@@ -402,9 +401,6 @@ static int step_multi4(const lpmm_adamw4bit_tensor *tensors, int64_t count, cons
         LPMM_REQUIRE_ALIGN(t.v_scale, 4);
         if ((t.n + kTile - 1) / kTile > 0x7fffffffLL)
             return LPMM_ERR_SIZE;
-        allfull = allfull && (t.n % kTile) == 0;
-        aligned = aligned && aligned_to(t.p, 16) && aligned_to(t.g, 16) && aligned_to(t.m_codes, 2) &&
-                  aligned_to(t.v_codes, 2);
     }
 
     Multi4 args;
@@ -414,6 +410,8 @@ static int step_multi4(const lpmm_adamw4bit_tensor *tensors, int64_t count, cons
     while (i < count) {
         int k = 0;
         uint64_t tiles = 0;
+        // per launch: do all pointers allow vector access, is every tensor a whole number of tiles
+        bool aligned = true, allfull = true;
         args.tile_start[0] = 0;
         while (i < count && k < LPMM_MULTI_MAX) {
             const lpmm_adamw4bit_tensor &t = tensors[i];
@@ -424,6 +422,9 @@ static int step_multi4(const lpmm_adamw4bit_tensor *tensors, int64_t count, cons
             const uint64_t nt = (uint64_t)((t.n + kTile - 1) / kTile);
             if (tiles + nt > 0x7fffffffULL)
                 break;
+            allfull = allfull && (t.n % kTile) == 0;
+            aligned = aligned && aligned_to(t.p, 16) && aligned_to(t.g, 16) && aligned_to(t.m_codes, 2) &&
+                      aligned_to(t.v_codes, 2);
             Tensor4 &d = args.t[k];
             d.p = t.p;
             d.g = t.g;
