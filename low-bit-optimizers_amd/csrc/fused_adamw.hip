@@ -35,8 +35,9 @@ constexpr int kTile = kThreads * kEltsPerLane;  // 2048 elements = 16 groups
 // kernel runs at 5.9 TB/s with 8 resident workgroups per CU and at 6.2-6.4 TB/s with 3-5; the
 // kernel itself gains 3 % with 5 and loses with 4 (too few waves to cover the arithmetic).
 constexpr uint32_t kFusedLdsBytes = 30 * 1024;
-static_assert(kFusedLdsBytes >= kLdsBytes, "tables do not fit");
 static_assert(160 * 1024 / kFusedLdsBytes == 5, "residency cap");
+static_assert(kFusedLdsBytes >= kLdsBytes, "tables do not fit");
+
 
 struct Tensor4 {
     float *p;
@@ -122,27 +123,55 @@ struct GroupRegs {
     float sm, sv;
 };
 
-__device__ __forceinline__ void group_load(const Tensor4 &t, int64_t grp, int lane16, GroupRegs &r)
+// Where a lane's operands of a whole group live: the tile's base addresses (uniform over the
+// workgroup, so they stay in scalar registers) plus 32-bit lane offsets.
+struct TileView {
+    float *p;
+    const float *g;
+    uint8_t *mc, *vc;
+    float *ms, *vs;
+    uint32_t eoff;  // element offset of the lane's first four values in the tile
+    uint32_t coff;  // byte offset of its first code half-word
+    uint32_t soff;  // its group within the tile
+};
+
+__device__ __forceinline__ TileView tile_view(const Tensor4 &t, uint32_t tile_in_tensor)
 {
-    const int64_t gbase = grp * kGroup;
-    const float *pp = t.p + gbase + lane16 * 4;
-    const float *gp = t.g + gbase + lane16 * 4;
+    TileView w;
+    const int64_t e0 = (int64_t)tile_in_tensor * kTile;
+    w.p = t.p + e0;
+    w.g = t.g + e0;
+    w.mc = t.mc + (e0 >> 1);
+    w.vc = t.vc + (e0 >> 1);
+    w.ms = t.ms + e0 / kGroup;
+    w.vs = t.vs + e0 / kGroup;
+    const uint32_t row = threadIdx.x >> 4, lane16 = threadIdx.x & 15;
+    w.eoff = row * kGroup + lane16 * 4;
+    w.coff = row * (kGroup / 2) + lane16 * 2;
+    w.soff = row;
+    return w;
+}
+
+__device__ __forceinline__ void group_load(const TileView &w, GroupRegs &r)
+{
+    const float *pp = w.p + w.eoff;
+    const float *gp = w.g + w.eoff;
     r.a0 = load4(pp);
     r.a1 = load4(pp + 64);
     r.b0 = load4(gp);
     r.b1 = load4(gp + 64);
-    const uint16_t *mcp = reinterpret_cast<const uint16_t *>(t.mc + (gbase >> 1)) + lane16;
-    const uint16_t *vcp = reinterpret_cast<const uint16_t *>(t.vc + (gbase >> 1)) + lane16;
+    const uint16_t *mcp = reinterpret_cast<const uint16_t *>(w.mc + w.coff);
+    const uint16_t *vcp = reinterpret_cast<const uint16_t *>(w.vc + w.coff);
     r.m0 = load_u16(mcp);
     r.m1 = load_u16(mcp + 16);
     r.v0 = load_u16(vcp);
     r.v1 = load_u16(vcp + 16);
-    r.sm = t.ms[grp];
-    r.sv = t.vs[grp];
+    r.sm = w.ms[w.soff];
+    r.sv = w.vs[w.soff];
 }
 
 template <bool FULL, class Arith>
-__device__ __forceinline__ void group_step(const Tensor4 &t, const Arith &h, const uint32_t *lds,
+__device__ __forceinline__ void group_step(const Tensor4 &t, const TileView &w, const Arith &h, const uint32_t *lds,
                                            bool std_maps, int64_t grp, int lane16, const GroupRegs &r)
 {
     const int64_t n = t.n;
@@ -206,15 +235,20 @@ __device__ __forceinline__ void group_step(const Tensor4 &t, const Arith &h, con
     const uint32_t cv = encode8_scaled(lds, kLdsQ1, std_maps ? kMapStdV : kMapGeneric, v, amax_v);
 
     if (FULL) {
-        float *pp = t.p + gbase + lane16 * 4;
+        float *pp = w.p + w.eoff;
         store4(pp, make_float4(pv[0], pv[1], pv[2], pv[3]));
         store4(pp + 64, make_float4(pv[4], pv[5], pv[6], pv[7]));
-        uint16_t *mcp = reinterpret_cast<uint16_t *>(t.mc + (gbase >> 1)) + lane16;
-        uint16_t *vcp = reinterpret_cast<uint16_t *>(t.vc + (gbase >> 1)) + lane16;
+        uint16_t *mcp = reinterpret_cast<uint16_t *>(w.mc + w.coff);
+        uint16_t *vcp = reinterpret_cast<uint16_t *>(w.vc + w.coff);
         store_u16(mcp, cm & 0xFFFFu);
         store_u16(mcp + 16, cm >> 16);
         store_u16(vcp, cv & 0xFFFFu);
         store_u16(vcp + 16, cv >> 16);
+        if (lane16 == 0) {
+            w.ms[w.soff] = amax_m;
+            w.vs[w.soff] = amax_v;
+        }
+        return;
     } else {
 #pragma unroll
         for (int k = 0; k < kEltsPerLane; ++k) {
@@ -256,18 +290,22 @@ __global__ __launch_bounds__(kThreads) void adamw4bit_kernel(const Multi4 args,
     // block index reaches.  Two rounds of scalar loads from the kernel arguments (every eighth
     // entry, then the seven in between) and scalar compares: nothing here queues behind the
     // streaming traffic of the vector memory path.
+    // (start <= bid) as the sign bit of start - 1 - bid (tile counts stay below 2^31): plain
+    // scalar arithmetic, no compare masks
     const uint32_t bid = blockIdx.x;
-    int base = 0;
+    uint32_t base = 0;
 #pragma unroll
     for (int j = 0; j < kCoarseSlots; ++j)
-        base += (args.coarse[j] <= bid) ? 8 : 0;
-    int lo = base;
+        base += ((args.coarse[j] - 1u - bid) >> 31) * 8u;
+    uint32_t lo = base;
 #pragma unroll
     for (int i = 1; i < 8; ++i)
-        lo += (args.tile_start[base + i] <= bid) ? 1 : 0;
+        lo += (args.tile_start[base + i] - 1u - bid) >> 31;
     const Tensor4 &t = args.t[lo];
     const int lane16 = threadIdx.x & 15;
-    const int64_t grp = (int64_t)(bid - args.tile_start[lo]) * (kTile / kGroup) + (threadIdx.x >> 4);
+    const uint32_t tile_in_tensor = bid - args.tile_start[lo];
+    const int64_t grp = (int64_t)tile_in_tensor * (kTile / kGroup) + (threadIdx.x >> 4);
+    const TileView view = tile_view(t, tile_in_tensor);
 
     // a group that lies wholly inside its tensor starts its loads now; the small loads were
     // issued before them and return first
@@ -276,7 +314,7 @@ __global__ __launch_bounds__(kThreads) void adamw4bit_kernel(const Multi4 args,
     if (!ALLFULL)
         regs.m0 = regs.m1 = regs.v0 = regs.v1 = 0;
     if (full)
-        group_load(t, grp, lane16, regs);
+        group_load(view, regs);
     lds_fill_store(lds, fill);
     const bool std_maps = classify_map(qmap_m) == kMapStdM && classify_map(qmap_v) == kMapStdV;
     const Arith h(args, t);
@@ -305,9 +343,9 @@ __global__ __launch_bounds__(kThreads) void adamw4bit_kernel(const Multi4 args,
         return;
     }
     if (full)
-        group_step<true>(t, h, lds, std_maps, grp, lane16, regs);
+        group_step<true>(t, view, h, lds, std_maps, grp, lane16, regs);
     else
-        group_step<false>(t, h, lds, std_maps, grp, lane16, regs);
+        group_step<false>(t, view, h, lds, std_maps, grp, lane16, regs);
 }
 
 // ---------------------------------------------------------------------------------------
