@@ -310,13 +310,15 @@ int lpmm_factored_update_fp32m(float *p, const float *g, float *m, const float *
 /* ---------------------------------------------------------------------------------------
  * Diagnostic (no counterpart in the reference): compares the library's near-exact sqrt and
  * division sequences (hardware approximation + one fma correction of the residual) with the
- * correctly rounded operations on the device.  counts: 9 zero-initialised device uint64:
+ * correctly rounded operations on the device.  counts: 11 zero-initialised device uint64:
  *   [0] sqrt inputs tried (every sqrt_stride-th positive normal float), [1] results that
  *   differ from sqrtf, [2] of those, by more than 1 ulp, [3] of those, with an input of at
  *   least 2^-100 (below that the residual underflows; such a second moment is far below any
  *   eps); [4] division pairs tried, [5] results that differ from x/d, [6] of those, by more
  *   than 1 ulp; [7] pairs tried for the reciprocal-based group division, [8] results that
- *   differ from x/y (must stay 0).
+ *   differ from x/y (must stay 0); [9] floats tried for the Newton-corrected reciprocal of the
+ *   group maximum (every float in [2^-60, 2^60]), [10] results that differ from 1/y (must
+ *   stay 0).
  * ------------------------------------------------------------------------------------- */
 int lpmm_selftest_arithmetic(unsigned long long *counts, uint32_t sqrt_stride, uint64_t pairs,
                              uint32_t seed, void *stream);

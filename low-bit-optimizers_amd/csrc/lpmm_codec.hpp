@@ -40,7 +40,10 @@ __device__ __forceinline__ void store_u32(uint32_t *p, uint32_t v) { __builtin_n
 // such a second moment is far below any eps it is added to.
 __device__ __forceinline__ float sqrt_fast(float x)
 {
-    const float y = __builtin_amdgcn_rsqf(fmaxf(x, 0x1p-126f));
+    // max(x, 2^-126) on the bit patterns: the same as on the values for x >= +0 (a second moment is
+    // never negative and never -0), one instruction instead of a canonicalising float max
+    const uint32_t xb = __float_as_uint(x);
+    const float y = __builtin_amdgcn_rsqf(__uint_as_float(xb > 0x00800000u ? xb : 0x00800000u));
     const float s = x * y;
     const float h = 0.5f * y;
     const float r = __builtin_fmaf(-s, s, x);
@@ -67,6 +70,16 @@ __device__ __forceinline__ float div_by_rc(float x, float y, float rc)
 }
 
 __device__ __forceinline__ bool rc_safe(float y) { return y >= 0x1p-60f && y <= 0x1p60f; }
+
+// 1 / y for y in [2^-60, 2^60]: the hardware approximation and one Newton step.  Equal to the
+// correctly rounded reciprocal for every float of that range on gfx950 (all 1 006 632 961 of
+// them are compared by the device self-test), at 3 instructions instead of the 10 of the IEEE
+// division sequence.
+__device__ __forceinline__ float rcp_exact(float y)
+{
+    const float r = __builtin_amdgcn_rcpf(y);
+    return __builtin_fmaf(__builtin_fmaf(-y, r, 1.0f), r, r);
+}
 
 // ---------------------------------------------------------------------------------------
 // Which map is this?  Decided on the device from the 16 values themselves (scalar loads,
@@ -194,7 +207,7 @@ __device__ __forceinline__ uint32_t encode8_scaled(const uint32_t *lds, uint32_t
 {
     float x[8];
     if (kind != kMapGeneric && rc_safe(amax)) {
-        const float rc = 1.0f / amax;
+        const float rc = rcp_exact(amax);
 #pragma unroll
         for (int k = 0; k < 8; ++k)
             x[k] = div_by_rc(v[k], amax, rc);

@@ -292,7 +292,7 @@ __global__ __launch_bounds__(kThreads) void rank1_requant_kernel(const MultiR1 a
         if (kind == kMapStdV && __all(safe)) {
             // the correctly rounded reciprocal of whichever statistic is the scale, then one
             // multiply and two fmas: the correctly rounded quotient (v <= scale by construction)
-            const float rcr = 1.0f / rn;
+            const float rcr = rcp_exact(rn);  // used only where rn is the scale and in range
             float rcn[kEltsPerLane];
             unpack8(lds_read<float4>(lds, kColRcp + col_off), lds_read<float4>(lds, kColRcp + col_off + 256), rcn);
 #pragma unroll

@@ -7,11 +7,12 @@ namespace lpmm {
 // counts[0] sqrt inputs, [1] sqrt results that differ from sqrtf, [2] of those, more than 1 ulp apart,
 // [3] of those, with an input of at least 2^-100 (below that the residual underflows),
 // counts[4] div pairs, [5] div_fast != x/d, [6] of those, more than 1 ulp apart,
-// counts[7] div_by_rc pairs, [8] div_by_rc != x/y
+// counts[7] div_by_rc pairs, [8] div_by_rc != x/y,
+// counts[9] reciprocal inputs (every float in [2^-60, 2^60]), [10] rcp_exact != 1/y
 __global__ __launch_bounds__(256) void selftest_kernel(unsigned long long *counts, uint32_t sqrt_stride,
                                                        uint64_t pairs_per_thread, uint32_t seed)
 {
-    unsigned long long c[9] = {0, 0, 0, 0, 0, 0, 0, 0, 0};
+    unsigned long long c[11] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
     const uint64_t tid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const uint64_t nthreads = (uint64_t)gridDim.x * blockDim.x;
     // every sqrt_stride-th positive normal float (stride 1: all of them)
@@ -53,11 +54,18 @@ __global__ __launch_bounds__(256) void selftest_kernel(unsigned long long *count
             y2 = t;
         }
         ++c[7];
-        if (div_by_rc(x2, y2, 1.0f / y2) != x2 / y2)
+        if (div_by_rc(x2, y2, rcp_exact(y2)) != x2 / y2)
             ++c[8];
     }
+    // the reciprocal of the group maximum: every float it is used for
+    for (uint64_t b = 0x21800000ull + tid; b <= 0x5d800000ull; b += nthreads) {
+        const float y = __uint_as_float((uint32_t)b);
+        ++c[9];
+        if (rcp_exact(y) != 1.0f / y)
+            ++c[10];
+    }
 #pragma unroll
-    for (int k = 0; k < 9; ++k)
+    for (int k = 0; k < 11; ++k)
         if (c[k])
             atomicAdd(counts + k, c[k]);
 }

@@ -224,16 +224,18 @@ def test_fused_step_other_maps(oracle):
 def test_near_exact_arithmetic_selftest():
     """sqrt_fast / div_fast (parameter update only) against the correctly rounded device
     operations on every 16th positive normal float and 2^30 divisor pairs; the reciprocal-based
-    group division, which decides codes, must agree with IEEE division on every pair."""
+    group division, which decides codes, must agree with IEEE division on every pair, and the
+    Newton-corrected reciprocal it starts from with 1/y on every float of its range."""
     lib = _native().lib()
-    counts = torch.zeros(9, dtype=torch.int64, device="cuda")
+    counts = torch.zeros(11, dtype=torch.int64, device="cuda")
     st = lib.lpmm_selftest_arithmetic(counts.data_ptr(), 16, 1 << 30, 12345, torch.cuda.current_stream().cuda_stream)
     assert st == 0
     torch.cuda.synchronize()
     c = counts.cpu().tolist()
     print("sqrt: %d tried, %d differ, %d by > 1 ulp, %d at x >= 2^-100; div: %d tried, %d differ, %d by > 1 ulp; "
-          "group div: %d tried, %d differ" % tuple(c))
+          "group div: %d tried, %d differ; reciprocal: %d tried, %d differ" % tuple(c))
     assert c[0] > 1.3e8 and c[4] >= 1 << 30 and c[7] >= 1 << 30
     assert c[2] == 0 and c[3] == 0   # sqrt: never more than 1 ulp, exact from 2^-100 upwards
     assert c[5] == 0 and c[6] == 0   # division for the update: exact on this sample
     assert c[8] == 0                 # division by the group maximum: exact
+    assert c[9] == 0x5d800000 - 0x21800000 + 1 and c[10] == 0   # its reciprocal: exact on the whole range
