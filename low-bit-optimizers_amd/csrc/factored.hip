@@ -73,7 +73,7 @@ __device__ __forceinline__ void partial_body(const float *__restrict__ g, int64_
             float4 t[kSUnroll];
 #pragma unroll
             for (int j = 0; j < kSUnroll; ++j)
-                t[j] = load4(g + (rb + j) * C + c0);
+                t[j] = load4_keep(g + (rb + j) * C + c0);  // the update pass reads g again
 #pragma unroll
             for (int j = 0; j < kSUnroll; ++j) {
                 u[j][0] = t[j].x * t[j].x; u[j][1] = t[j].y * t[j].y; u[j][2] = t[j].z * t[j].z; u[j][3] = t[j].w * t[j].w;
@@ -445,6 +445,13 @@ struct TensorFa {
     float neg_step_size, bc2_sqrt, rbc2_sqrt;
 };
 
+// Gradient bytes per launch batch.  The update pass re-reads the gradient that the
+// statistics pass of the same batch has just read, and walks it back to front, so the part
+// that the 256 MB memory-side cache still holds is not fetched from HBM a second time.
+// Smaller batches hit more often but pay four launches each: 384 MB measured best on
+// LLaMA-7B MLP shapes (2 % faster than batches bounded by the tensor count alone).
+constexpr int64_t kFaBatchBytes = (int64_t)384 << 20;
+
 struct MultiFa {
     TensorFa t[kFaMax];
     // prefix sums of workgroups per tensor for the three big kernels; unused slots hold the total
@@ -456,16 +463,16 @@ struct MultiFa {
 static_assert(sizeof(MultiFa) + sizeof(void *) <= 4096, "kernel arguments exceed 4 KB");
 static_assert(kFaMax <= kWave, "one prefix-sum entry per lane");
 
-__device__ __forceinline__ int find_slot(const uint32_t (&start)[kFaMax + 1])
+__device__ __forceinline__ int find_slot(const uint32_t (&start)[kFaMax + 1], uint32_t block)
 {
     const int lane = threadIdx.x & (kWave - 1);
-    const bool started = lane + 1 < kFaMax && start[lane + 1] <= blockIdx.x;
+    const bool started = lane + 1 < kFaMax && start[lane + 1] <= block;
     return __popcll(__ballot(started));
 }
 
 __global__ __launch_bounds__(kFThreads) void factored_partial_multi_kernel(const MultiFa args)
 {
-    const int i = find_slot(args.start_stats);
+    const int i = find_slot(args.start_stats, blockIdx.x);
     const TensorFa &t = args.t[i];
     const uint32_t local = blockIdx.x - args.start_stats[i];
     const uint32_t by = local / t.tiles_x, bx = local - by * t.tiles_x;
@@ -474,7 +481,7 @@ __global__ __launch_bounds__(kFThreads) void factored_partial_multi_kernel(const
 
 __global__ __launch_bounds__(kFThreads) void factored_finalize_multi_kernel(const MultiFa args)
 {
-    const int i = find_slot(args.start_fin);
+    const int i = find_slot(args.start_fin, blockIdx.x);
     const TensorFa &t = args.t[i];
     finalize_body(t.colpart, t.rowpart, t.rowblock, t.R, t.C, (int)t.tiles_y, (int)t.tiles_x, (int)t.row_blocks,
                   t.row, t.col, args.b2, args.w2, blockIdx.x - args.start_fin[i]);
@@ -494,9 +501,12 @@ __global__ void factored_mean_multi_kernel(const MultiFa args)
 __global__ __launch_bounds__(kFThreads) void factored_update_multi_kernel(const MultiFa args,
                                                                           const float *__restrict__ qmap_m)
 {
-    const int i = find_slot(args.start_upd);
+    // last tile first: the statistics pass has just read g front to back, so its tail is what
+    // the memory-side cache still holds when the batch is larger than that cache
+    const uint32_t block = gridDim.x - 1u - blockIdx.x;
+    const int i = find_slot(args.start_upd, block);
     const TensorFa &t = args.t[i];
-    const uint32_t local = blockIdx.x - args.start_upd[i];
+    const uint32_t local = block - args.start_upd[i];
     const uint32_t by = local / t.upd_x, bx = local - by * t.upd_x;
     NfHyper h;
     h.decay = args.decay;
@@ -720,9 +730,14 @@ extern "C" int lpmm_factored_step_multi(const lpmm_factored_tensor *tensors, int
     while (i < count) {
         int k = 0;
         uint64_t n_stats = 0, n_fin = 0, n_upd = 0;
+        int64_t g_bytes = 0;
         args.start_stats[0] = args.start_fin[0] = args.start_upd[0] = 0;
         while (i < count && k < kFaMax) {
             const lpmm_factored_tensor &t = tensors[i];
+            const int64_t t_bytes = t.rows * t.cols * 4;  // the grid limits above keep rows * cols below 2^43
+            if (k > 0 && g_bytes + t_bytes > kFaBatchBytes)
+                break;
+            g_bytes += t_bytes;
             const uint64_t ty = (uint64_t)((t.rows + kSRows - 1) / kSRows), tx = (uint64_t)((t.cols + kSCols - 1) / kSCols);
             const uint64_t row_blocks = (uint64_t)((t.rows + kFThreads - 1) / kFThreads);
             const uint64_t fin = row_blocks + (uint64_t)((t.cols + 63) / 64);

@@ -204,3 +204,49 @@ def test_factored_fp32m_matches_oracle(oracle):
         assert_rel(to_np(dp), p, "p")
         np.testing.assert_array_equal(to_np(dm), m)
         drow.copy_(torch.from_numpy(row)); dcol.copy_(torch.from_numpy(col)); dp.copy_(torch.from_numpy(p))
+
+
+def test_factored_step_multi_large_batches_equal_single_tensor_calls(qmaps):
+    """Tensors whose gradients exceed the byte budget of one launch batch: the multi-tensor
+    call (several batches, update pass walking back to front) must leave exactly what
+    lpmm_factored_stats + lpmm_factored_update leave tensor by tensor."""
+    from lpmm import _native
+
+    lib = _lib()
+    dqm = to_dev(qmaps[0])
+    gen = torch.Generator(device="cuda").manual_seed(77)
+    shapes = [(4096, 8192), (2048, 11008), (4096, 8192), (8192, 4096), (4096, 8192), (1000, 1152), (4096, 8192)]
+    assert sum(r * c * 4 for r, c in shapes) > (384 << 20) * 3 // 2  # at least two batches
+
+    def fresh(r, c):
+        n = r * c
+        t = dict(r=r, c=c, p=torch.randn(r, c, device="cuda", generator=gen) * 0.02,
+                 row=torch.rand(r, device="cuda", generator=gen) * 1e-6,
+                 col=torch.rand(c, device="cuda", generator=gen) * 1e-6,
+                 codes=torch.randint(0, 256, (n // 2048 * 1024 + (1024 if n % 2048 else 0) + 1,), dtype=torch.uint8,
+                                     device="cuda", generator=gen),
+                 max1=torch.rand(n // 128, device="cuda", generator=gen) * 1e-3,
+                 g=torch.randn(r, c, device="cuda", generator=gen) * 1e-3,
+                 work=torch.empty(lib.lpmm_factored_workspace_bytes(r, c), dtype=torch.uint8, device="cuda"))
+        return t
+
+    a = [fresh(r, c) for r, c in shapes]
+    b = [{k: (v.clone() if torch.is_tensor(v) else v) for k, v in t.items()} for t in a]
+    recs = [(t["p"].data_ptr(), t["g"].data_ptr(), t["codes"].data_ptr(), t["max1"].data_ptr(), t["row"].data_ptr(),
+             t["col"].data_ptr(), t["work"].data_ptr(), t["r"], t["c"], 7.0, 0) for t in a]
+    table = np.array(recs, dtype=_native.FACTORED_TENSOR)
+    st = lib.lpmm_factored_step_multi(table.ctypes.data, len(recs), dqm.data_ptr(), H["beta1"], H["beta2"], H["lr"],
+                                      H["wd"], H["eps"], _stream())
+    assert st == 0, lib.lpmm_status_string(st)
+    mean_all = torch.zeros(1, dtype=torch.float32, device="cuda")
+    for t in b:
+        assert lib.lpmm_factored_stats(t["g"].data_ptr(), t["r"], t["c"], t["row"].data_ptr(), t["col"].data_ptr(),
+                                       mean_all.data_ptr(), H["beta2"], t["work"].data_ptr(), _stream()) == 0
+        assert lib.lpmm_factored_update(t["p"].data_ptr(), t["g"].data_ptr(), t["codes"].data_ptr(),
+                                        t["max1"].data_ptr(), dqm.data_ptr(), t["row"].data_ptr(), t["col"].data_ptr(),
+                                        mean_all.data_ptr(), t["r"], t["c"], H["beta1"], H["beta2"], H["lr"], H["wd"],
+                                        H["eps"], 7.0, 0, _stream()) == 0
+    torch.cuda.synchronize()
+    for x, y in zip(a, b):
+        for k in ("p", "row", "col", "codes", "max1"):
+            assert torch.equal(x[k], y[k]), f'{k} of {x["r"]}x{x["c"]}'
