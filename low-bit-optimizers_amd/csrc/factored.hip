@@ -66,41 +66,84 @@ __device__ __forceinline__ void partial_body(const float *__restrict__ g, int64_
     double *rp = rowpart + (int64_t)bx * R;  // one row partial per workgroup
     double cs[4] = {0.0, 0.0, 0.0, 0.0};
     const int lane = threadIdx.x & (kWave - 1);
-    for (int64_t rb = r0; rb < r1; rb += kSUnroll) {
-        float u[kSUnroll][4];
-        if (lane_vec && rb + kSUnroll <= r1) {
-            // straight-line: all loads of the batch are in flight before the first use
-            float4 t[kSUnroll];
-#pragma unroll
-            for (int j = 0; j < kSUnroll; ++j)
-                t[j] = load4_keep(g + (rb + j) * C + c0);  // the update pass reads g again
+    if (vec && r0 + kSRows <= R && (int64_t)(bx + 1) * kSCols <= C) {
+        // whole tile (uniform over the workgroup, so no load sits behind a branch): two register
+        // buffers of 8 rows; the loads of a batch are in flight while the batch before it is summed
+        float4 a[kSUnroll], b[kSUnroll];
+        // uniform row addresses plus a 32-bit lane offset: no 64-bit address per row in registers
+        const float *tile = g + r0 * C + (int64_t)bx * kSCols;
+        const uint32_t lane_off = threadIdx.x * 4u;
+        auto fetch = [&](float4(&t)[kSUnroll], int i) {
 #pragma unroll
             for (int j = 0; j < kSUnroll; ++j) {
-                u[j][0] = t[j].x * t[j].x; u[j][1] = t[j].y * t[j].y; u[j][2] = t[j].z * t[j].z; u[j][3] = t[j].w * t[j].w;
+                const float *row = tile + (int64_t)(i * kSUnroll + j) * C;
+                t[j] = load4_keep(row + lane_off);  // kept in the caches: the update pass reads g again
             }
-        } else {
+        };
+        auto sum = [&](const float4(&t)[kSUnroll], int i) {
+            double rs[kSUnroll];
 #pragma unroll
             for (int j = 0; j < kSUnroll; ++j) {
-                const int64_t r = rb + j;
+                const float u[4] = {t[j].x * t[j].x, t[j].y * t[j].y, t[j].z * t[j].z, t[j].w * t[j].w};
+                rs[j] = ((double)u[0] + (double)u[1]) + ((double)u[2] + (double)u[3]);
 #pragma unroll
-                for (int k = 0; k < 4; ++k) {
-                    const float t = (r < r1 && c0 + k < C) ? g[r * C + c0 + k] : 0.0f;
-                    u[j][k] = t * t;
+                for (int k = 0; k < 4; ++k)
+                    cs[k] += (double)u[k];
+            }
+            const double tot = wave_sum8_f64(rs, lane);
+            if ((lane & 7) == 0)
+                s_part[threadIdx.x >> 6][i * kSUnroll + (lane >> 3)] = tot;
+        };
+        constexpr int kBatches = kSRows / kSUnroll;
+        static_assert(kBatches % 2 == 0 && kBatches >= 4, "two batches per iteration, the last pair peeled");
+        fetch(a, 0);
+#pragma unroll 1
+        for (int i = 0; i < kBatches - 2; i += 2) {
+            fetch(b, i + 1);
+            sum(a, i);
+            fetch(a, i + 2);
+            sum(b, i + 1);
+        }
+        fetch(b, kBatches - 1);
+        sum(a, kBatches - 2);
+        sum(b, kBatches - 1);
+    } else {
+        for (int64_t rb = r0; rb < r1; rb += kSUnroll) {
+            float u[kSUnroll][4];
+            if (lane_vec && rb + kSUnroll <= r1) {
+                // straight-line: all loads of the batch are in flight before the first use
+                float4 t[kSUnroll];
+#pragma unroll
+                for (int j = 0; j < kSUnroll; ++j)
+                    t[j] = load4_keep(g + (rb + j) * C + c0);
+#pragma unroll
+                for (int j = 0; j < kSUnroll; ++j) {
+                    u[j][0] = t[j].x * t[j].x; u[j][1] = t[j].y * t[j].y; u[j][2] = t[j].z * t[j].z; u[j][3] = t[j].w * t[j].w;
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < kSUnroll; ++j) {
+                    const int64_t r = rb + j;
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        const float t = (r < r1 && c0 + k < C) ? g[r * C + c0 + k] : 0.0f;
+                        u[j][k] = t * t;
+                    }
                 }
             }
-        }
-        double rs[kSUnroll];
+            double rs[kSUnroll];
 #pragma unroll
-        for (int j = 0; j < kSUnroll; ++j) {
-            rs[j] = ((double)u[j][0] + (double)u[j][1]) + ((double)u[j][2] + (double)u[j][3]);
+            for (int j = 0; j < kSUnroll; ++j) {
+                rs[j] = ((double)u[j][0] + (double)u[j][1]) + ((double)u[j][2] + (double)u[j][3]);
 #pragma unroll
-            for (int k = 0; k < 4; ++k)
-                cs[k] += (double)u[j][k];
+                for (int k = 0; k < 4; ++k)
+                    cs[k] += (double)u[j][k];
+            }
+            // the wave's 8 row sums at once: lane 8j ends up with the sum of row j
+            const double tot = wave_sum8_f64(rs, lane);
+            if ((lane & 7) == 0)
+                s_part[threadIdx.x >> 6][(int)(rb - r0) + (lane >> 3)] = tot;
         }
-        // the wave's 8 row sums at once: lane 8j ends up with the sum of row j
-        const double tot = wave_sum8_f64(rs, lane);
-        if ((lane & 7) == 0)
-            s_part[threadIdx.x >> 6][(int)(rb - r0) + (lane >> 3)] = tot;
     }
     __syncthreads();
     if (threadIdx.x < kSRows && r0 + threadIdx.x < r1)
