@@ -366,3 +366,57 @@ def test_sgd_4bit_momentum(oracle, qmaps, nesterov):
             h[...] = to_np(params[i])
     with pytest.raises(ValueError):
         lpmm.optim.SGD(params, lr=0.1, fused=True)
+
+
+@pytest.mark.parametrize("mode", ["fused", "nonfused_group", "nonfused_rank1", "factored"])
+def test_steps_are_reproducible_bit_for_bit(mode):
+    """Two optimizers fed the same parameters and gradients end in identical parameters and
+    states: the row/column maxima of the rank-1 path are merged with an order-free integer
+    atomic max and the factored sums are folded in a fixed order, so nothing depends on the
+    order in which workgroups happen to run."""
+    import lpmm
+
+    cfg_dir = os.path.join(os.path.dirname(lpmm.config.__file__), "configs")
+    kw = dict(H)
+    if mode == "fused":
+        kw.update(fused=True)
+    elif mode == "nonfused_group":
+        kw.update(fused=False, qconfig=os.path.join(cfg_dir, "2nd_moment_group_128.yml"))
+    elif mode == "nonfused_rank1":
+        kw.update(fused=False, qconfig=os.path.join(cfg_dir, "default.yml"))
+    else:
+        kw.update(fused=True, factor_second_moment=True)
+    shapes = [(1024, 2048), (300, 4224), (2048, 1152), (6400,), (1600,)]
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    init = [torch.randn(s, device="cuda", generator=gen) * 0.02 for s in shapes]
+    grads = [[torch.randn(s, device="cuda", generator=gen) * 1e-3 * (1 + 10 * (i == 1)) for s in shapes]
+             for i in range(3)]
+
+    def run():
+        params = [torch.nn.Parameter(t.clone()) for t in init]
+        opt = lpmm.optim.AdamW(params, **kw)
+        for gs in grads:
+            for p, g in zip(params, gs):
+                p.grad = g.clone()
+            opt.step()
+        torch.cuda.synchronize()
+        out = []
+        for p in params:
+            st = opt.state[p]
+            out.append(p.detach().clone())
+            for name in sorted(st):
+                if name == "step":
+                    continue
+                v = st[name]
+                found = [v] if torch.is_tensor(v) else []
+                if isinstance(v, dict):  # a qstate: the scales live in its overhead
+                    for o in v.get("overhead", {}).values():
+                        found += [o] if torch.is_tensor(o) else [x for x in o if torch.is_tensor(x)] if isinstance(o, (list, tuple)) else []
+                out.extend(x.clone() for x in found)
+        return out
+
+    a, b = run(), run()
+    assert len(a) == len(b) and len(a) > len(shapes)
+    for x, y in zip(a, b):
+        assert x.dtype == y.dtype and x.shape == y.shape
+        assert torch.equal(x.view(torch.uint8) if x.dtype == torch.int8 else x, y.view(torch.uint8) if y.dtype == torch.int8 else y)
