@@ -420,3 +420,68 @@ def test_steps_are_reproducible_bit_for_bit(mode):
     for x, y in zip(a, b):
         assert x.dtype == y.dtype and x.shape == y.shape
         assert torch.equal(x.view(torch.uint8) if x.dtype == torch.int8 else x, y.view(torch.uint8) if y.dtype == torch.int8 else y)
+
+
+@pytest.mark.parametrize("fused", [True, False])
+def test_param_groups_missing_grads_and_closure(oracle, qmaps, fused):
+    """Two parameter groups with their own hyper-parameters, a parameter that gets its first
+    gradient two steps late (its own step count, lpmm/optim/adamw.py:119, :498) and a closure:
+    every tensor must follow the oracle run with its group's hyper-parameters and its own
+    step number."""
+    import lpmm
+
+    qm, qv = qmaps
+    rng = np.random.default_rng(21)
+    shapes = [(96, 128), (70, 256), (5000,)]  # all quantised (numel > 4096)
+    host, params = _params(shapes, rng)
+    groups = [dict(params=[params[0], params[2]], lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01),
+              dict(params=[params[1]], lr=3e-4, betas=(0.8, 0.99), eps=1e-6, weight_decay=0.0)]
+    hyper = [(0.9, 0.999, 1e-3, 0.01, 1e-8), (0.8, 0.99, 3e-4, 0.0, 1e-6), (0.9, 0.999, 1e-3, 0.01, 1e-8)]
+    kw = dict(fused=True) if fused else dict(
+        fused=False, qconfig=os.path.join(os.path.dirname(lpmm.config.__file__), "configs", "2nd_moment_group_128.yml"))
+    opt = lpmm.optim.AdamW(groups, **kw)
+    steps_done = [0, 0, 0]
+    if fused:
+        ref = [dict(mc=np.zeros((h.size + 1) // 2, np.uint8), vc=np.zeros((h.size + 1) // 2, np.uint8),
+                    ms=np.zeros((h.size + 127) // 128, np.float32), vs=np.zeros((h.size + 127) // 128, np.float32))
+               for h in host]
+    else:
+        ref = [dict(m=None, v=None) for _ in host]
+    calls = []
+    for it in range(4):
+        grads = [(rng.standard_normal(s) * 1e-3).astype(np.float32) for s in shapes]
+        for i, (p, g) in enumerate(zip(params, grads)):
+            p.grad = None if (i == 2 and it < 2) else to_dev(g)
+
+        def closure():
+            calls.append(it)
+            return torch.tensor(float(it))
+
+        loss = opt.step(closure)
+        assert float(loss) == float(it)
+        for i, (h, g, r) in enumerate(zip(host, grads, ref)):
+            if i == 2 and it < 2:
+                continue
+            steps_done[i] += 1
+            b1, b2, lr, wd, eps = hyper[i]
+            if fused:
+                oracle.adamw4bit_step(h.reshape(-1), g.reshape(-1), r["mc"], r["vc"], r["ms"], r["vs"], qm, qv,
+                                      b1, b2, lr, wd, eps, float(steps_done[i]))
+            else:
+                n = h.size
+                m = np.zeros(n, np.float32) if r["m"] is None else oracle.dequant_group(r["m"][0], r["m"][1], qm, n)
+                v = np.zeros(n, np.float32) if r["v"] is None else oracle.dequant_group(r["v"][0], r["v"][1], qv, n)
+                oracle.nonfused_update(h.reshape(-1), g.reshape(-1), m, v, b1, b2, lr, wd, eps, float(steps_done[i]))
+                r["m"], r["v"] = oracle.quant_group(m, qm), oracle.quant_group(v, qv)
+    torch.cuda.synchronize()
+    assert calls == [0, 1, 2, 3]
+    for i, (p, h, r) in enumerate(zip(params, host, ref)):
+        st = opt.state[p]
+        assert float(st["step"]) == float(steps_done[i]) == (2.0 if i == 2 else 4.0)
+        assert_rel(to_np(p), h, f"p of tensor {i}", scale=h)
+        if fused:
+            assert_codes(to_np(st["exp_avg"]), r["mc"], h.size, "m codes")
+            assert_codes(to_np(st["exp_avg_sq"]), r["vc"], h.size, "v codes")
+        else:
+            np.testing.assert_array_equal(to_np(st["exp_avg"]).view(np.uint8), r["m"][0])
+            np.testing.assert_array_equal(to_np(st["exp_avg_sq"]).view(np.uint8), r["v"][0])
