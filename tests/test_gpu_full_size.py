@@ -157,3 +157,81 @@ def test_factored_step_llama_mlp_shape(oracle, qmaps):
         np.testing.assert_array_equal(to_np(s["exp_avg"]).view(np.uint8), state.m[0])
         np.testing.assert_array_equal(to_np(s["exp_avg_qstate"]["overhead"]["max1"]).reshape(-1), state.m[1])
         assert_rel(to_np(param), host, "p", scale=before)
+
+
+def test_indexing_beyond_two_to_the_31_elements(qmaps):
+    """One tensor of 2^31 + 4160 elements (its byte offsets pass 2^33, its last group holds 64
+    values) must come out exactly as the same buffers processed as two tensors split at a
+    group boundary: groups are independent, and the two halves are indexed with small numbers,
+    the regime the oracle comparisons cover.  Fused step (two steps, the second from non-zero
+    states), then the block-wise quantiser and dequantiser on the same number of values."""
+    from lpmm import _native
+
+    lib = _native.lib()
+    stream = torch.cuda.current_stream().cuda_stream
+    dqm, dqv = to_dev(qmaps[0]), to_dev(qmaps[1])
+    n = (1 << 31) + 4160
+    cut = (1 << 30) + 128 * 5  # a group boundary that is not a tile boundary
+    gen = torch.Generator(device="cuda").manual_seed(31)
+    g = torch.empty(n, device="cuda")
+    p0 = torch.empty(n, device="cuda")
+    chunk = 1 << 28
+    for lo in range(0, n, chunk):  # filled in pieces: bounded temporaries
+        hi = min(n, lo + chunk)
+        p0[lo:hi] = torch.randn(hi - lo, device="cuda", generator=gen) * 0.02
+        g[lo:hi] = torch.randn(hi - lo, device="cuda", generator=gen) * 1e-3
+    groups = (n + 127) // 128
+
+    def fresh():
+        return dict(p=p0.clone(), mc=torch.zeros(n // 2, dtype=torch.uint8, device="cuda"),
+                    vc=torch.zeros(n // 2, dtype=torch.uint8, device="cuda"),
+                    ms=torch.zeros(groups, device="cuda"), vs=torch.zeros(groups, device="cuda"))
+
+    a, b = fresh(), fresh()
+    for step in (1.0, 2.0):
+        st = lib.lpmm_adamw4bit_step(a["p"].data_ptr(), g.data_ptr(), a["mc"].data_ptr(), a["vc"].data_ptr(),
+                                     a["ms"].data_ptr(), a["vs"].data_ptr(), dqm.data_ptr(), dqv.data_ptr(), n, *HO,
+                                     step, stream)
+        assert st == 0, lib.lpmm_status_string(st)
+        recs = []
+        for lo, hi in ((0, cut), (cut, n)):
+            recs.append((b["p"].data_ptr() + 4 * lo, g.data_ptr() + 4 * lo, b["mc"].data_ptr() + lo // 2,
+                         b["vc"].data_ptr() + lo // 2, b["ms"].data_ptr() + 4 * (lo // 128),
+                         b["vs"].data_ptr() + 4 * (lo // 128), hi - lo, step, 0.0))
+        table = np.array(recs, dtype=_native.ADAMW4BIT_TENSOR)
+        st = lib.lpmm_adamw4bit_step_multi(table.ctypes.data, 2, dqm.data_ptr(), dqv.data_ptr(), *HO, stream)
+        assert st == 0, lib.lpmm_status_string(st)
+        torch.cuda.synchronize()
+        for k in ("p", "mc", "vc", "ms", "vs"):
+            assert torch.equal(a[k], b[k]), f"{k} differs after step {step}"
+    # the states are non-trivial: the last (64-value) group has a scale and the codes of its missing half stay 0
+    assert float(a["vs"][-1]) > 0 and int(a["mc"][-1]) != 0
+    del a, b, p0
+    torch.cuda.empty_cache()
+
+    # block-wise quantiser / dequantiser in the non-fused layout, split at a 2048-value pack boundary
+    cutq = (1 << 30) + 2048 * 3
+    nbytes = (n + 2047) // 2048 * 1024 + 1
+    codes_a = torch.zeros(nbytes, dtype=torch.uint8, device="cuda")
+    codes_b = torch.zeros(nbytes, dtype=torch.uint8, device="cuda")
+    max_a, max_b = torch.zeros(groups, device="cuda"), torch.zeros(groups, device="cuda")
+    assert lib.lpmm_quant_group(g.data_ptr(), n, 128, dqm.data_ptr(), codes_a.data_ptr(), max_a.data_ptr(), stream) == 0
+    assert lib.lpmm_quant_group(g.data_ptr() + 4 * cutq, n - cutq, 128, dqm.data_ptr(), codes_b.data_ptr() + cutq // 2,
+                                max_b.data_ptr() + 4 * (cutq // 128), stream) == 0
+    # the first part second: its trailing byte (always written as 0) lands on the first code byte of the second part
+    tail = codes_b[cutq // 2].clone()
+    assert lib.lpmm_quant_group(g.data_ptr(), cutq, 128, dqm.data_ptr(), codes_b.data_ptr(), max_b.data_ptr(), stream) == 0
+    codes_b[cutq // 2] = tail
+    torch.cuda.synchronize()
+    assert torch.equal(codes_a, codes_b) and torch.equal(max_a, max_b)
+    out_a = torch.empty(n, device="cuda")
+    assert lib.lpmm_dequant_group(codes_a.data_ptr(), max_a.data_ptr(), dqm.data_ptr(), n, 128, out_a.data_ptr(), stream) == 0
+    out_b = torch.empty(n, device="cuda")
+    assert lib.lpmm_dequant_group(codes_a.data_ptr(), max_a.data_ptr(), dqm.data_ptr(), cutq, 128, out_b.data_ptr(), stream) == 0
+    assert lib.lpmm_dequant_group(codes_a.data_ptr() + cutq // 2, max_a.data_ptr() + 4 * (cutq // 128), dqm.data_ptr(),
+                                  n - cutq, 128, out_b.data_ptr() + 4 * cutq, stream) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(out_a, out_b)
+    # and the round trip is what quantisation promises: every value within its group's scale
+    err = (out_a[: 1 << 20] - g[: 1 << 20]).abs().max()
+    assert float(err) <= float(max_a[: 1 << 13].max())
