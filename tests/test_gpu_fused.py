@@ -239,3 +239,65 @@ def test_near_exact_arithmetic_selftest():
     assert c[5] == 0 and c[6] == 0   # division for the update: exact on this sample
     assert c[8] == 0                 # division by the group maximum: exact
     assert c[9] == 0x5d800000 - 0x21800000 + 1 and c[10] == 0   # its reciprocal: exact on the whole range
+
+
+def test_fused_multi_step_under_graph_capture(qmaps):
+    """The library only enqueues kernels on the stream it is given (no allocation, no memset, no
+    synchronisation), so a multi-tensor step can be recorded into a HIP graph.  Each of three
+    replays, with eager work and synchronisations in between, must leave exactly what the same
+    call leaves when it is issued eagerly on copies of the buffers."""
+    nat = _native()
+    lib = nat.lib()
+    dqm, dqv = to_dev(qmaps[0]), to_dev(qmaps[1])
+    gen = torch.Generator(device="cuda").manual_seed(8)
+    sizes = [2048 * 40, 128 * 1001 + 64, 4098, 2048 * 7]
+
+    def make():
+        ts = []
+        for n in sizes:
+            ts.append(dict(n=n, p=torch.randn(n, device="cuda", generator=gen) * 0.02,
+                           g=torch.randn(n, device="cuda", generator=gen) * 1e-3,
+                           mc=torch.zeros((n + 1) // 2, dtype=torch.uint8, device="cuda"),
+                           vc=torch.zeros((n + 1) // 2, dtype=torch.uint8, device="cuda"),
+                           ms=torch.zeros((n + 127) // 128, device="cuda"),
+                           vs=torch.zeros((n + 127) // 128, device="cuda")))
+        return ts
+
+    captured = make()
+    eager = [{k: (v.clone() if torch.is_tensor(v) else v) for k, v in t.items()} for t in captured]
+
+    def table(ts):
+        return np.array([(t["p"].data_ptr(), t["g"].data_ptr(), t["mc"].data_ptr(), t["vc"].data_ptr(),
+                          t["ms"].data_ptr(), t["vs"].data_ptr(), t["n"], 3.0, 0.0) for t in ts],
+                        dtype=nat.ADAMW4BIT_TENSOR)
+
+    def enqueue(ts):
+        tb = table(ts)
+        st = lib.lpmm_adamw4bit_step_multi(tb.ctypes.data, len(ts), dqm.data_ptr(), dqv.data_ptr(), HYPER["beta1"],
+                                           HYPER["beta2"], HYPER["lr"], HYPER["wd"], HYPER["eps"],
+                                           torch.cuda.current_stream().cuda_stream)
+        assert st == 0, lib.lpmm_status_string(st)
+
+    side = torch.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            enqueue(captured)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    # capture records, it does not run: the buffers are untouched so far
+    assert all(torch.equal(c["p"], e["p"]) and int(c["mc"].max()) == 0 for c, e in zip(captured, eager))
+    for replay in range(3):
+        graph.replay()
+        enqueue(eager)
+        scratch = torch.randn(1 << 16, device="cuda", generator=gen).sum()  # unrelated eager work between replays
+        torch.cuda.synchronize()
+        assert torch.isfinite(scratch)
+        for c, e in zip(captured, eager):
+            for k in ("p", "mc", "vc", "ms", "vs"):
+                assert torch.equal(c[k], e[k]), f"{k} of the {c['n']}-element tensor differs on replay {replay}"
+        for c in captured:  # new gradients for the next replay, written into the captured buffers
+            c["g"].copy_(torch.randn(c["n"], device="cuda", generator=gen) * 1e-3)
+        for c, e in zip(captured, eager):
+            e["g"].copy_(c["g"])
