@@ -257,3 +257,38 @@ def test_utils_metrics_and_bookkeeping():
     assert utils.get_metric_fn("min")(1, 2) and utils.get_metric_fn("max")(2, 1)
     with pytest.raises(NotImplementedError):
         utils.get_metric_fn("median")
+
+
+def test_every_shipped_configuration_merges_to_the_reference_settings():
+    """The 13 files under lpmm/configs carry the reference's names; merged over the defaults each
+    must give the settings of the reference's file of that name (lpmm/configs/*.yml there):
+    (m enabled, m bits, m block size, v bits, v scale type)."""
+    import lpmm
+    from lpmm.config import get_config
+
+    want = {
+        "default.yml": (True, 4, 128, 4, "rank1"),
+        "default_5b.yml": (True, 5, 128, 5, "rank1"),
+        "default_6b.yml": (True, 6, 128, 6, "rank1"),
+        "default_7b.yml": (True, 7, 128, 7, "rank1"),
+        "default_8b.yml": (True, 8, 128, 8, "rank1"),
+        "1st_moment_group_256.yml": (True, 4, 256, 4, "rank1"),
+        "1st_moment_group_512.yml": (True, 4, 512, 4, "rank1"),
+        "1st_moment_group_1024.yml": (True, 4, 1024, 4, "rank1"),
+        "1st_moment_group_2048.yml": (True, 4, 2048, 4, "rank1"),
+        "1st_moment_group_4096.yml": (True, 4, 4096, 4, "rank1"),
+        "2nd_moment_group_128.yml": (True, 4, 128, 4, "group"),
+        "2nd_moment_only_default.yml": (False, 4, 128, 4, "rank1"),
+        "2nd_moment_only_group_128.yml": (False, 4, 128, 4, "group"),
+    }
+    cfg_dir = os.path.join(os.path.dirname(lpmm.config.__file__), "configs")
+    assert sorted(os.listdir(cfg_dir)) == sorted(want)
+    for name, (m_on, m_bits, m_gp, v_bits, v_scale) in want.items():
+        q = get_config(os.path.join(cfg_dir, name)).QUANT
+        got = (q.M.ENABLE, q.M.BITS, q.M.GROUP_SIZE, q.SQM.BITS, q.SQM.SCALE_TYPE.DEFAULT)
+        assert got == (m_on, m_bits, m_gp, v_bits, v_scale), name
+        # everything else stays at the defaults the two files share
+        assert q.SQM.ENABLE is True and q.SQM.GROUP_SIZE == 128 and q.M.SCALE_TYPE.DEFAULT == "group"
+        assert q.M.QUANT_TYPE.DEFAULT == "nonlinear" and q.SQM.QUANT_TYPE.DEFAULT == "power-1"
+        assert q.M.ROUND_TYPE == "real-nearest" and q.SQM.ROUND_TYPE == "real-nearest"
+        assert q.M.SIGNED is True and q.SQM.SIGNED is False and q.M.THRESHOLD == 4096
