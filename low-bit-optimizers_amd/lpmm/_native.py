@@ -9,6 +9,8 @@ import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "liblpmm_hip.so")
+MULTI_MAX = 48  # tensors per launch of the fused step (LPMM_MULTI_MAX in include/lpmm_hip.h)
+RANK1_MULTI_MAX = 32  # tensors per launch of the two-pass rank-1 step (kR1Max in csrc/nonfused_rank1.hip)
 ABI_VERSION = 1
 
 _vp = ctypes.c_void_p

@@ -151,6 +151,16 @@ class AdamW(LowBitOptimizer):
         md_v = self.get_qmetadata_by_state_name("exp_avg_sq")
         quant, plain = {}, {}  # device -> list of records
         factored_work = []
+        lib = _native.lib()
+
+        def launch_quant(key, records):
+            dev, qm_ptr, qv_ptr = key
+            table = np.array(records, dtype=_native.ADAMW4BIT_TENSOR)
+            with torch.cuda.device(dev):
+                st = lib.lpmm_adamw4bit_step_multi(table.ctypes.data, len(records), qm_ptr, qv_ptr, beta1, beta2,
+                                                   lr, wd, eps, _native.current_stream(dev))
+            _native.check(st, "fused 4-bit AdamW step")
+
         for p, grad, state, factored in work:
             state["step"] += 1
             step = state["step"].item()
@@ -192,9 +202,15 @@ class AdamW(LowBitOptimizer):
                     oh_v["max1"] = torch.zeros((blocks,), dtype=torch.float32, device=p.device)
                 key = (p.device, state["exp_avg_qstate"]["qmap"].data_ptr(),
                        state["exp_avg_sq_qstate"]["qmap"].data_ptr())
-                quant.setdefault(key, []).append(
+                pending = quant.setdefault(key, [])
+                pending.append(
                     (p.data_ptr(), grad.data_ptr(), state["exp_avg"].data_ptr(), state["exp_avg_sq"].data_ptr(),
                      oh_m["max1"].data_ptr(), oh_v["max1"].data_ptr(), n, step, 0.0))
+                if len(pending) == _native.MULTI_MAX:
+                    # one launch's worth: enqueue it now, so that the GPU works while the host
+                    # walks the remaining tensors
+                    launch_quant(key, pending)
+                    pending.clear()
             else:
                 if _is_placeholder(state["exp_avg"]):
                     state["exp_avg"] = torch.zeros_like(p, memory_format=torch.preserve_format)
@@ -205,13 +221,9 @@ class AdamW(LowBitOptimizer):
                      p.numel(), step, 0.0))
 
         self._factored_steps(group, factored_work)
-        lib = _native.lib()
-        for (dev, qm_ptr, qv_ptr), records in quant.items():
-            table = np.array(records, dtype=_native.ADAMW4BIT_TENSOR)
-            with torch.cuda.device(dev):
-                st = lib.lpmm_adamw4bit_step_multi(table.ctypes.data, len(records), qm_ptr, qv_ptr, beta1, beta2,
-                                                   lr, wd, eps, _native.current_stream(dev))
-            _native.check(st, "fused 4-bit AdamW step")
+        for key, records in quant.items():
+            if records:
+                launch_quant(key, records)
         for dev, records in plain.items():
             table = np.array(records, dtype=_native.ADAMW_FP32_TENSOR)
             with torch.cuda.device(dev):
@@ -247,6 +259,24 @@ class AdamW(LowBitOptimizer):
         v_rank1 = fits(md_v) and md_v["scale_type"] == "rank1"
         batched, batched_rank1, plain = {}, {}, {}
         factored_work = []
+
+        def launch_group(key, records):
+            dev, qm_ptr, qv_ptr = key
+            table = np.array(records, dtype=_native.ADAMW4BIT_TENSOR)
+            with torch.cuda.device(dev):
+                st = lib.lpmm_nonfused_adamw4bit_step_multi(table.ctypes.data, len(records), qm_ptr, qv_ptr, beta1,
+                                                            beta2, lr, wd, eps, _native.current_stream(dev))
+            _native.check(st, "non-fused 4-bit AdamW step")
+
+        def launch_rank1(key, records):
+            dev, qm_ptr, qv_ptr = key
+            table = np.array(records, dtype=_native.NONFUSED_RANK1_TENSOR)
+            with torch.cuda.device(dev):
+                st = lib.lpmm_nonfused_adamw4bit_rank1_step_multi(table.ctypes.data, len(records), qm_ptr, qv_ptr,
+                                                                  beta1, beta2, lr, wd, eps,
+                                                                  _native.current_stream(dev))
+            _native.check(st, "non-fused 4-bit AdamW step (rank-1 second moment)")
+
         for p, grad, state, factored in work:
             state["step"] += 1
             step = state["step"].item()
@@ -259,10 +289,18 @@ class AdamW(LowBitOptimizer):
                 key = (p.device, state["exp_avg_qstate"]["qmap"].data_ptr(),
                        state["exp_avg_sq_qstate"]["qmap"].data_ptr())
                 if v_group128:
-                    batched.setdefault(key, []).append(self._nonfused_record(p, grad, state, step))
+                    pending = batched.setdefault(key, [])
+                    pending.append(self._nonfused_record(p, grad, state, step))
+                    if len(pending) == _native.MULTI_MAX:  # one launch's worth: enqueue it now
+                        launch_group(key, pending)
+                        pending.clear()
                     continue
                 if v_rank1 and p.dim() == 2 and p.shape[1] % 128 == 0:
-                    batched_rank1.setdefault(key, []).append(self._nonfused_rank1_record(p, grad, state, step))
+                    pending = batched_rank1.setdefault(key, [])
+                    pending.append(self._nonfused_rank1_record(p, grad, state, step))
+                    if len(pending) == _native.RANK1_MULTI_MAX:
+                        launch_rank1(key, pending)
+                        pending.clear()
                     continue
             m = self._materialise(p, state, "exp_avg", en_m, md_m)
             v = self._materialise(p, state, "exp_avg_sq", en_v, md_v)
@@ -286,19 +324,12 @@ class AdamW(LowBitOptimizer):
                 st = lib.lpmm_nonfused_update_multi(table.ctypes.data, len(records), beta1, beta2, lr, wd, eps,
                                                     _native.current_stream(dev))
             _native.check(st, "non-fused AdamW update")
-        for (dev, qm_ptr, qv_ptr), records in batched.items():
-            table = np.array(records, dtype=_native.ADAMW4BIT_TENSOR)
-            with torch.cuda.device(dev):
-                st = lib.lpmm_nonfused_adamw4bit_step_multi(table.ctypes.data, len(records), qm_ptr, qv_ptr, beta1,
-                                                            beta2, lr, wd, eps, _native.current_stream(dev))
-            _native.check(st, "non-fused 4-bit AdamW step")
-        for (dev, qm_ptr, qv_ptr), records in batched_rank1.items():
-            table = np.array(records, dtype=_native.NONFUSED_RANK1_TENSOR)
-            with torch.cuda.device(dev):
-                st = lib.lpmm_nonfused_adamw4bit_rank1_step_multi(table.ctypes.data, len(records), qm_ptr, qv_ptr,
-                                                                  beta1, beta2, lr, wd, eps,
-                                                                  _native.current_stream(dev))
-            _native.check(st, "non-fused 4-bit AdamW step (rank-1 second moment)")
+        for key, records in batched.items():
+            if records:
+                launch_group(key, records)
+        for key, records in batched_rank1.items():
+            if records:
+                launch_rank1(key, records)
 
     def _nonfused_record(self, p, grad, state, step):
         """The tensor's record for the one-pass non-fused step; creates the quantised states

@@ -38,6 +38,8 @@ def test_record_layouts_match_header():
     assert _native.ADAMW4BIT_TENSOR.itemsize == 64 and _native.ADAMW_FP32_TENSOR.itemsize == 48
     assert _native.ADAMW4BIT_TENSOR.fields["n"][1] == 48 and _native.ADAMW4BIT_TENSOR.fields["step"][1] == 56
     assert _native.ADAMW_FP32_TENSOR.fields["n"][1] == 32 and _native.ADAMW_FP32_TENSOR.fields["step"][1] == 40
+    header = open(os.path.join(ROOT, "include", "lpmm_hip.h")).read()
+    assert int(re.search(r"#define LPMM_MULTI_MAX (\d+)", header).group(1)) == _native.MULTI_MAX
 
 
 def test_argument_errors_without_gpu():
