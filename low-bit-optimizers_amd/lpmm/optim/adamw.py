@@ -97,20 +97,39 @@ class AdamW(LowBitOptimizer):
 
     # ---- state ---------------------------------------------------------------------------
     def _state_of(self, group, p):
-        """Create the parameter's state on first use (lpmm/optim/adamw.py:114-129)."""
+        """The parameter's state, created on first use (lpmm/optim/adamw.py:114-129), and whether its
+        second moment is factored (decided once, when the state is created: the keys tell)."""
         state = self.state[p]
+        if len(state) != 0:
+            return state, "exp_avg_sq_row" in state
         factored, _ = self._get_options(group, p.shape)
-        if len(state) == 0:
-            state["step"] = torch.tensor(0.0)  # on the host: reading it never syncs the GPU
-            state["exp_avg"] = torch.zeros((), dtype=torch.float, device=p.device)
-            self.init_qstate(p, "exp_avg")
-            if factored:
-                state["exp_avg_sq_row"] = torch.zeros(p.shape[:-1], device=p.device)
-                state["exp_avg_sq_col"] = torch.zeros(p.shape[:-2] + p.shape[-1:], device=p.device)
-            else:
-                state["exp_avg_sq"] = torch.zeros((), dtype=torch.float, device=p.device)
-            self.init_qstate(p, "exp_avg_sq")
+        state["step"] = torch.tensor(0.0)  # on the host: reading it never syncs the GPU
+        state["exp_avg"] = torch.zeros((), dtype=torch.float, device=p.device)
+        self.init_qstate(p, "exp_avg")
+        if factored:
+            state["exp_avg_sq_row"] = torch.zeros(p.shape[:-1], device=p.device)
+            state["exp_avg_sq_col"] = torch.zeros(p.shape[:-2] + p.shape[-1:], device=p.device)
+        else:
+            state["exp_avg_sq"] = torch.zeros((), dtype=torch.float, device=p.device)
+        self.init_qstate(p, "exp_avg_sq")
         return state, factored
+
+    def _next_step(self, state):
+        """state["step"] += 1 and its value as a Python float.  The count is a 0-dim float32 tensor
+        on the host, as in the reference (lpmm/optim/adamw.py:119); it is advanced through a numpy
+        view of the same memory, which costs a fraction of a tensor operation, and the view is
+        rebuilt whenever the tensor has been replaced (load_state_dict)."""
+        t = state["step"]
+        views = self.__dict__.setdefault("_step_views", {})
+        hit = views.get(id(state))
+        if hit is None or hit[0] is not t:
+            if t.device.type != "cpu" or t.dtype != torch.float32 or t.dim() != 0:
+                t += 1
+                return t.item()
+            hit = views[id(state)] = (t, t.numpy())
+        view = hit[1]
+        view += 1.0
+        return float(view)
 
     def _enabled(self, p, state, name):
         if id(p) in self.override_q_enable:
@@ -162,8 +181,7 @@ class AdamW(LowBitOptimizer):
             _native.check(st, "fused 4-bit AdamW step")
 
         for p, grad, state, factored in work:
-            state["step"] += 1
-            step = state["step"].item()
+            step = self._next_step(state)
             if factored:
                 # the fused kernel does not cover the factored case (adamw.py:472-495)
                 factored_work.append((p, grad, state, step))
@@ -233,6 +251,9 @@ class AdamW(LowBitOptimizer):
 
     @staticmethod
     def _check_fp32_cuda(p, grad):
+        if (p.dtype is torch.float32 and grad.dtype is torch.float32 and p.is_cuda and grad.is_cuda
+                and p.is_contiguous() and grad.is_contiguous()):
+            return
         for t, name in ((p, "p"), (grad, "g")):
             if not t.is_cuda:
                 raise RuntimeError(f"{name} must be a CUDA tensor!")
@@ -278,8 +299,7 @@ class AdamW(LowBitOptimizer):
             _native.check(st, "non-fused 4-bit AdamW step (rank-1 second moment)")
 
         for p, grad, state, factored in work:
-            state["step"] += 1
-            step = state["step"].item()
+            step = self._next_step(state)
             if factored:
                 factored_work.append((p, grad, state, step))
                 continue
