@@ -265,6 +265,18 @@ int64_t lpmm_factored_workspace_bytes(int64_t rows, int64_t cols);
 int lpmm_factored_stats(const float *g, int64_t rows, int64_t cols, float *row, float *col,
                         float *row_mean_all, double beta2, void *workspace, void *stream);
 
+/* lpmm_factored_stats without the workspace argument, for callers that cannot allocate device
+ * memory (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).
+ * No counterpart in the reference.  The partial sums go to an array of
+ * LPMM_FACTORED_STATIC_BYTES that the library's code object holds on every GPU it runs on until
+ * the process ends; the call allocates and frees nothing.  Shapes whose
+ * lpmm_factored_workspace_bytes(rows, cols) exceeds that size return LPMM_ERR_SIZE.  All calls
+ * on one GPU share the array: calls that overlap on one GPU (different streams) race.  Same
+ * results as lpmm_factored_stats. */
+#define LPMM_FACTORED_STATIC_BYTES (32u << 20)
+int lpmm_factored_stats_static(const float *g, int64_t rows, int64_t cols, float *row, float *col,
+                               float *row_mean_all, double beta2, void *stream);
+
 /* Pass 2: p *= 1-lr*wd; m = dequant(m_codes); m.lerp_(g, 1-beta1);
  * v = row/row_mean_all * col; p += -lr/bc1 * m / (sqrt(v)/sqrt(bc2) + eps); m re-quantised
  * with 'group' scaling, gp_sz 128, into the non-fused packed layout (adamw.py:596-625).

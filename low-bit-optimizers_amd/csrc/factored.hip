@@ -10,6 +10,8 @@
 // Row/column means of g*g are summed in double in a fixed order and rounded once.
 #include "lpmm_update.hpp"
 
+#include <mutex>
+
 namespace lpmm {
 
 constexpr int kFThreads = 256;
@@ -607,8 +609,9 @@ extern "C" int64_t lpmm_factored_workspace_bytes(int64_t rows, int64_t cols)
     return (ty * cols + tx * rows + row_blocks + 1) * (int64_t)sizeof(double);
 }
 
-extern "C" int lpmm_factored_stats(const float *g, int64_t rows, int64_t cols, float *row, float *col,
-                                   float *row_mean_all, double beta2, void *workspace, void *stream)
+// argument checks shared by the two forms of the statistics pass
+static int factored_stats_check(const float *g, int64_t rows, int64_t cols, const float *row, const float *col,
+                                const float *row_mean_all)
 {
     if (rows <= 0 || cols <= 0)
         return LPMM_ERR_SIZE;
@@ -616,22 +619,29 @@ extern "C" int lpmm_factored_stats(const float *g, int64_t rows, int64_t cols, f
     LPMM_REQUIRE_PTR(row);
     LPMM_REQUIRE_PTR(col);
     LPMM_REQUIRE_PTR(row_mean_all);
-    LPMM_REQUIRE_PTR(workspace);
     LPMM_REQUIRE_ALIGN(g, 4);
     LPMM_REQUIRE_ALIGN(row, 4);
     LPMM_REQUIRE_ALIGN(col, 4);
     LPMM_REQUIRE_ALIGN(row_mean_all, 4);
-    LPMM_REQUIRE_ALIGN(workspace, 8);
     const int64_t ty = (rows + kSRows - 1) / kSRows, tx = (cols + kSCols - 1) / kSCols;
-    if (ty > 65535 || tx > 0x7fffffffLL)
+    const int64_t row_blocks = (rows + kFThreads - 1) / kFThreads;
+    const int64_t col_blocks = (cols + 63) / 64;
+    if (ty > 65535 || tx > 0x7fffffffLL || row_blocks + col_blocks > 0x7fffffffLL)
         return LPMM_ERR_SIZE;
+    return LPMM_OK;
+}
+
+// the three launches of the statistics pass; `workspace` is a device address of at least
+// lpmm_factored_workspace_bytes(rows, cols) bytes, 8-byte aligned
+static int factored_stats_launch(const float *g, int64_t rows, int64_t cols, float *row, float *col,
+                                 float *row_mean_all, double beta2, void *workspace, void *stream)
+{
+    const int64_t ty = (rows + kSRows - 1) / kSRows, tx = (cols + kSCols - 1) / kSCols;
     double *colpart = static_cast<double *>(workspace);
     double *rowpart = colpart + ty * cols;
     double *rowblock = rowpart + tx * rows;
     const int64_t row_blocks = (rows + kFThreads - 1) / kFThreads;
     const int64_t col_blocks = (cols + 63) / 64;
-    if (row_blocks + col_blocks > 0x7fffffffLL)
-        return LPMM_ERR_SIZE;
     const bool vec = aligned_to(g, 16) && (cols % 4) == 0;
     hipLaunchKernelGGL(factored_partial_kernel, dim3((uint32_t)tx, (uint32_t)ty), dim3(kFThreads), 0,
                        (hipStream_t)stream, g, rows, cols, colpart, rowpart, vec);
@@ -647,6 +657,57 @@ extern "C" int lpmm_factored_stats(const float *g, int64_t rows, int64_t cols, f
     hipLaunchKernelGGL(factored_mean_kernel, dim3(1), dim3(kWave), 0, (hipStream_t)stream, rowblock,
                        (int)row_blocks, rows, row_mean_all);
     return launch_status();
+}
+
+extern "C" int lpmm_factored_stats(const float *g, int64_t rows, int64_t cols, float *row, float *col,
+                                   float *row_mean_all, double beta2, void *workspace, void *stream)
+{
+    const int st = factored_stats_check(g, rows, cols, row, col, row_mean_all);
+    if (st != LPMM_OK)
+        return st;
+    LPMM_REQUIRE_PTR(workspace);
+    LPMM_REQUIRE_ALIGN(workspace, 8);
+    return factored_stats_launch(g, rows, cols, row, col, row_mean_all, beta2, workspace, stream);
+}
+
+// The workspace of lpmm_factored_stats_static: one array per GPU, held by the library's code
+// object until the process ends.  In host code the name below is only a handle for
+// hipGetSymbolAddress; kernels receive the device address that call returns.
+static __device__ __align__(256) unsigned char scratch[LPMM_FACTORED_STATIC_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_lock;
+void *g_scratch_ptr[kMaxDevices];  // the current device's copy of `scratch`, looked up once per device
+}  // namespace
+
+extern "C" int lpmm_factored_stats_static(const float *g, int64_t rows, int64_t cols, float *row, float *col,
+                                          float *row_mean_all, double beta2, void *stream)
+{
+    const int st = factored_stats_check(g, rows, cols, row, col, row_mean_all);
+    if (st != LPMM_OK)
+        return st;
+    if (lpmm_factored_workspace_bytes(rows, cols) > (int64_t)LPMM_FACTORED_STATIC_BYTES)
+        return LPMM_ERR_SIZE;
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices)
+        return LPMM_ERR_LAUNCH;
+    void *ws = nullptr;
+    {
+        std::lock_guard<std::mutex> hold(g_scratch_lock);
+        if (g_scratch_ptr[dev] == nullptr) {
+            void *ptr = nullptr;
+            if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || ptr == nullptr) {
+                (void)hipGetLastError();
+                return LPMM_ERR_LAUNCH;
+            }
+            g_scratch_ptr[dev] = ptr;
+        }
+        ws = g_scratch_ptr[dev];
+    }
+    // every partial the finalize kernels read is written by the partial kernel of the same call:
+    // nothing in the array has to start at zero
+    return factored_stats_launch(g, rows, cols, row, col, row_mean_all, beta2, ws, stream);
 }
 
 extern "C" int lpmm_factored_update(float *p, const float *g, uint8_t *m_codes, float *m_max1,

@@ -47,6 +47,7 @@ PROTOTYPES = {
     "lpmm_nonfused_adamw4bit_rank1_step_multi": (_int, [_vp, _i64, _vp, _vp] + [_d] * 5 + [_vp]),
     "lpmm_factored_workspace_bytes": (_i64, [_i64, _i64]),
     "lpmm_factored_stats": (_int, [_vp, _i64, _i64, _vp, _vp, _vp, _d, _vp, _vp]),
+    "lpmm_factored_stats_static": (_int, [_vp, _i64, _i64, _vp, _vp, _vp, _d, _vp]),
     "lpmm_factored_update": (_int, [_vp] * 8 + [_i64, _i64] + [_d] * 6 + [_int, _vp]),
     "lpmm_factored_step_multi": (_int, [_vp, _i64, _vp] + [_d] * 5 + [_vp]),
     "lpmm_factored_update_fp32m": (_int, [_vp] * 6 + [_i64, _i64] + [_d] * 6 + [_vp]),
