@@ -32,10 +32,29 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 BYTES_PER_PARAM_4BIT = 14.125  # p r/w 8 + g 4 + m codes 1 + v codes 1 + scales 16/128
 BYTES_PER_PARAM_FP32 = 28.0    # p, m, v r/w + g r
 MULTI_MAX = 48                 # tensors per launch record (LPMM_MULTI_MAX)
-# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
-# script (each counter scaled by what it reads for a plain 1 GiB copy, --copy-probe; the summary is
-# kept under profiles/).  Algorithmic bytes per launch for that workload: 19.035e9.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"llama7b": 19.127e9}
+# HBM bytes per launch of the dominant kernel are not measured by this script: they come from
+# rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this same command (each counter scaled by what it
+# reads for a plain 1 GiB copy, --copy-probe), whose summary is kept in this file; the line
+# "traffic_bytes_per_launch: <number>" in it is what the JSON reports, with the file named as
+# "traffic_source".
+TRAFFIC_PROFILE = {"llama7b": "profiles/fused_adamw4bit_llama7b_pmc.md"}
+
+
+def recorded_traffic(workload):
+    """(bytes per launch, source) from the committed counter summary, or (None, None)."""
+    rel = TRAFFIC_PROFILE.get(workload)
+    if rel is None:
+        return None, None
+    try:
+        with open(os.path.join(ROOT, rel)) as fh:
+            for line in fh:
+                if line.startswith("traffic_bytes_per_launch:"):
+                    return float(line.split(":", 1)[1]), (
+                        rel + " (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of an earlier run of this command; "
+                        "not measured in this run)")
+    except OSError:
+        pass
+    return None, None
 
 
 def llama7b_shapes():
@@ -133,6 +152,73 @@ def cpu_baseline(torch, steps=10):
                   f"median of {steps} steps after 1 warm-up",
         "fused_step_c_restatement_params_per_s": n / sorted(fused_times[1:])[1],
     }
+
+
+def verify_one_more_step(torch, opt, params):
+    """Are the timed launches doing the work?  Takes the states the timed steps left for three
+    sampled tensors (a quantised one from the middle of a launch group, the last quantised one,
+    an fp32-state one), runs ONE more optimizer step over the whole set, and compares what that
+    step wrote for them with the CPU oracle's step from the same states: codes and scales bit
+    for bit, parameters within 1e-6 relative.  Outside the timed region; the oracle is only the
+    checker.  Returns (ok, description)."""
+    import numpy as np
+
+    from oracle import oracle as O
+
+    quant = [i for i, p in enumerate(params) if p.numel() > 4096]
+    plain = [i for i, p in enumerate(params) if p.numel() <= 4096]
+    picks = []
+    if quant:
+        small = [i for i in quant if params[i].numel() <= (1 << 26)] or quant
+        picks.append(small[len(small) // 2])
+        if quant[-1] not in picks and params[quant[-1]].numel() <= (1 << 28):
+            picks.append(quant[-1])
+    if plain:
+        picks.append(plain[len(plain) // 2])
+    group = opt.param_groups[0]
+    hyper = (group["betas"][0], group["betas"][1], group["lr"], group["weight_decay"], group["eps"])
+    qm, qv = O.qmap_m(), O.qmap_v()
+
+    def host(t):
+        return t.detach().cpu().numpy().reshape(-1).copy()
+
+    before = {}
+    for i in picks:
+        st = opt.state[params[i]]
+        snap = {"p": host(params[i]), "g": host(params[i].grad)}
+        if params[i].numel() > 4096:
+            snap.update(mc=host(st["exp_avg"]).view(np.uint8), vc=host(st["exp_avg_sq"]).view(np.uint8),
+                        ms=host(st["exp_avg_qstate"]["overhead"]["max1"]),
+                        vs=host(st["exp_avg_sq_qstate"]["overhead"]["max1"]))
+        else:
+            snap.update(m=host(st["exp_avg"]), v=host(st["exp_avg_sq"]))
+        before[i] = snap
+    opt.step()
+    torch.cuda.synchronize()
+    problems = []
+    for i in picks:
+        st, b = opt.state[params[i]], before[i]
+        step = float(st["step"])
+        p_old = b["p"].copy()
+        if "mc" in b:
+            O.adamw4bit_step(b["p"], b["g"], b["mc"], b["vc"], b["ms"], b["vs"], qm, qv, *hyper, step)
+            same = (np.array_equal(host(st["exp_avg"]).view(np.uint8), b["mc"])
+                    and np.array_equal(host(st["exp_avg_sq"]).view(np.uint8), b["vc"])
+                    and np.array_equal(host(st["exp_avg_qstate"]["overhead"]["max1"]), b["ms"])
+                    and np.array_equal(host(st["exp_avg_sq_qstate"]["overhead"]["max1"]), b["vs"]))
+        else:
+            O.adamw_fp32_step(b["p"], b["g"], b["m"], b["v"], *hyper, step)
+            same = np.array_equal(host(st["exp_avg"]), b["m"]) and np.array_equal(host(st["exp_avg_sq"]), b["v"])
+        got = host(params[i]).astype(np.float64)
+        yard = np.maximum(np.maximum(np.abs(b["p"]), np.abs(p_old)), np.finfo(np.float32).tiny)
+        p_ok = bool(np.all(np.abs(got - b["p"]) <= 1e-6 * yard))
+        if not (same and p_ok):
+            problems.append(f"tensor {i} {tuple(params[i].shape)}: states {'equal' if same else 'DIFFER'}, "
+                            f"parameters {'within 1e-6' if p_ok else 'DIFFER'}")
+    what = ", ".join(f"#{i} {tuple(params[i].shape)}" for i in picks)
+    if problems:
+        return False, "; ".join(problems)
+    return True, f"step {int(step)} of tensors {what}: codes, scales and fp32 states bit-exact, parameters within 1e-6"
 
 
 @contextlib.contextmanager
@@ -363,6 +449,9 @@ def main():
     recording["on"] = False
     per_step_ms = sorted(marks[i].elapsed_time(marks[i + 1]) for i in range(args.steps))
 
+    verified, verified_on = verify_one_more_step(torch, opt, params)
+    traffic, traffic_source = recorded_traffic(args.workload)
+
     ms_per_step = elapsed * 1e3 / args.steps
     value = n_total / (elapsed / args.steps)
     kernel_ms_per_step = sum(e0.elapsed_time(e1) for e0, e1 in events) / args.steps
@@ -386,6 +475,9 @@ def main():
         "vs_baseline": None,
         "dtype": "f32",
         "data": "synthetic",
+        # one more step after the timed region, checked against the CPU oracle on sampled tensors
+        "verified": verified,
+        "verified_on": verified_on,
         "config": {"workload": desc, "tensors": len(params), "params": n_total, "quantized_params": n_quant,
                    "launches_per_step": launches_per_step + 1},
         "effective_gbs": (n_quant * BYTES_PER_PARAM_4BIT + (n_total - n_quant) * BYTES_PER_PARAM_FP32)
@@ -400,7 +492,8 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBS,
-            "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(args.workload),
+            "traffic": traffic,
+            "traffic_source": traffic_source,
             "bytes_per_launch": bytes_per_launch,
             "avg_launch_ms": launch_ms,
         },
@@ -408,6 +501,8 @@ def main():
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(torch)
     print(json.dumps(out))
+    if not verified:
+        sys.exit("bench.py: the step after the timed region does not match the CPU oracle: " + verified_on)
 
 
 if __name__ == "__main__":

@@ -337,6 +337,21 @@ int lpmm_factored_update_fp32m(float *p, const float *g, float *m, const float *
 int lpmm_selftest_arithmetic(unsigned long long *counts, uint32_t sqrt_stride, uint64_t pairs,
                              uint32_t seed, void *stream);
 
+/* Diagnostic (no counterpart in the reference): runs the code assignment exactly as the kernels
+ * run it (LDS tables, saturating byte conversion, byte permute, median-of-three clamp) against
+ * the plain count of midpoints below x -- the reference search of
+ * lpmm/cpp_extension/fused_adamw_kernel.cu:27-49 -- on the device.  counts: 10 zero-initialised
+ * device uint64:
+ *   [0] values tried with the standard first-moment map: all 2^32 bit patterns, NaNs included
+ *   (they must give code 15), [1] wrong codes; [2], [3] the same with the standard
+ *   second-moment map; [4] values <= 1 tried with the bare closed form of the second-moment
+ *   code, [5] wrong codes; [6] values tried through the division by the group maximum with the
+ *   first-moment map (256 maxima: both ends of the range that divides by the corrected
+ *   reciprocal with their neighbours, zero, subnormal, huge, infinite, random; numerators
+ *   within 128 floats of every midpoint * maximum and random), [7] wrong codes; [8], [9] the
+ *   same with the second-moment map.  Every odd entry must stay 0. */
+int lpmm_selftest_encoders(unsigned long long *counts, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -13,7 +13,7 @@ import os
 
 import yaml
 
-__all__ = ["Node", "get_config", "CONFIG_DIR"]
+__all__ = ["Node", "get_config", "config_from_mapping", "to_plain", "CONFIG_DIR"]
 
 CONFIG_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "configs")
 
@@ -55,6 +55,26 @@ def _to_plain(value):
     if isinstance(value, dict):
         return {k: _to_plain(v) for k, v in value.items()}
     return value
+
+
+def to_plain(config):
+    """The config as nested builtin dicts (what a checkpoint stores)."""
+    return _to_plain(config)
+
+
+def config_from_mapping(mapping):
+    """A config node from any nested mapping that carries the optimizer's keys (a plain dict
+    from a checkpoint, a Node, a yacs CfgNode).  Raises if QUANT.M / QUANT.SQM are missing."""
+    if not isinstance(mapping, dict):
+        raise TypeError(f"qconfig of a checkpoint must be a mapping, not {type(mapping).__name__}")
+    node = _to_node(_to_plain(mapping))
+    for state in ("M", "SQM"):
+        sub = node.get("QUANT", {}).get(state)
+        missing = [k for k in ("ENABLE", "THRESHOLD", "BITS", "SCALE_TYPE", "QUANT_TYPE", "ROUND_TYPE", "GROUP_SIZE",
+                               "SIGNED") if sub is None or k not in sub]
+        if missing:
+            raise ValueError(f"qconfig of the checkpoint lacks QUANT.{state} keys {missing}")
+    return node
 
 
 def _state_node(bits, scale_type, quant_type, round_type, group_size, signed, enable=True):

@@ -15,6 +15,7 @@ handful of multi-tensor launches instead of one launch per tensor, and each quan
 dequantise / update of the non-fused path is one HIP kernel instead of a chain of
 PyTorch passes.
 """
+import weakref
 from typing import Optional
 
 import numpy as np
@@ -38,13 +39,16 @@ _ZERO_BYTE = {}
 
 def _zero_byte(qmap):
     """int8 value of a packed byte whose two codes both select the map entry nearest 0.0
-    (what quantising a zero tensor stores); looked up once per map."""
+    (what quantising a zero tensor stores); looked up once per map tensor.  The cache entry
+    remembers which tensor object it was made for: an address the allocator hands to another
+    map later does not hit it."""
     key = (qmap.device, qmap.data_ptr(), qmap._version)
-    if key not in _ZERO_BYTE:
+    hit = _ZERO_BYTE.get(key)
+    if hit is None or hit[0]() is not qmap:
         code = int(torch.argmin(qmap.abs()).item())
         byte = code | (code << 4)
-        _ZERO_BYTE[key] = byte - 256 if byte > 127 else byte
-    return _ZERO_BYTE[key]
+        hit = _ZERO_BYTE[key] = (weakref.ref(qmap), byte - 256 if byte > 127 else byte)
+    return hit[1]
 
 
 class AdamW(LowBitOptimizer):

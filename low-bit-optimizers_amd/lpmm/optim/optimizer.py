@@ -7,7 +7,7 @@ from itertools import chain
 
 import torch
 
-from ..config import get_config
+from ..config import config_from_mapping, get_config, to_plain
 from ..functional import create_general_qmap
 
 __all__ = ["LowBitOptimizer"]
@@ -72,15 +72,21 @@ class LowBitOptimizer(torch.optim.Optimizer):
 
     # ---- checkpointing -----------------------------------------------------------------
     def state_dict(self):
+        """torch's state dict plus 'qconfig' (lpmm/optim/optimizer.py:68-71).  The config is
+        stored as a plain nested dict with the reference's keys, so that the checkpoint holds
+        builtin types and tensors only and loads with `torch.load(..., weights_only=True)`;
+        the reference stores its yacs CfgNode object, which needs yacs to unpickle."""
         out = super().state_dict()
-        out["qconfig"] = self.qconfig
+        out["qconfig"] = to_plain(self.qconfig)
         return out
 
     def load_state_dict(self, state_dict):
         """Restore a state_dict().  Tensors move to their parameter's device; floating-point
         state follows the parameter's dtype, except `step` and the packed int8 code tensors,
         which are kept as they are (lpmm/optim/optimizer.py:73-136)."""
-        self.qconfig = state_dict["qconfig"]
+        # any mapping with the reference's keys: the plain dict written by state_dict() above, a
+        # config node of this package, or a yacs CfgNode (a dict subclass) from a reference checkpoint
+        self.qconfig = config_from_mapping(state_dict["qconfig"])
         state_dict = deepcopy(state_dict)
         groups, saved_groups = self.param_groups, state_dict["param_groups"]
         if len(groups) != len(saved_groups):
@@ -115,6 +121,39 @@ class LowBitOptimizer(torch.optim.Optimizer):
             s["params"] = g["params"]
             new_groups.append(s)
         self.__setstate__({"state": state, "param_groups": new_groups})
+        self._intern_qmaps()
+
+    def _intern_qmaps(self):
+        """After a load every state holds its own copy of its quantisation map.  States whose
+        map has the same contents share one tensor again (the optimizer's cached map where it
+        is the same), as they do after init_qstate: the multi-tensor launches group tensors by
+        their maps, and hundreds of 64-byte device tensors would be wasted otherwise."""
+        pool = {}
+        for key, qmap in self.qmaps.items():
+            if isinstance(qmap, torch.Tensor):
+                pool[(qmap.device, qmap.dtype, tuple(qmap.tolist()))] = qmap
+        for state in self.state.values():
+            if not isinstance(state, dict):
+                continue
+            for name, qstate in state.items():
+                if not (isinstance(name, str) and name.endswith("_qstate") and isinstance(qstate, dict)):
+                    continue
+                qmap = qstate.get("qmap")
+                if not isinstance(qmap, torch.Tensor):
+                    continue
+                key = (qmap.device, qmap.dtype, tuple(qmap.tolist()))
+                qstate["qmap"] = shared = pool.setdefault(key, qmap)
+                # states created after the load (init_qstate) should pick up the same tensor
+                try:
+                    md = self.get_qmetadata_by_state_name(name[: -len("_qstate")])
+                except (ValueError, NotImplementedError):
+                    continue
+                ckey = (md["quant_type"], md["b"], md["signed"])
+                if ckey not in self.qmaps:
+                    self.qmaps[ckey] = create_general_qmap(*ckey)
+                cached = self.qmaps[ckey]
+                if cached is not shared and tuple(cached.tolist()) == key[2] and cached.dtype == shared.dtype:
+                    self.qmaps[ckey] = shared
 
     # ---- to be provided by subclasses --------------------------------------------------
     @torch.no_grad()

@@ -241,6 +241,30 @@ def test_near_exact_arithmetic_selftest():
     assert c[9] == 0x5d800000 - 0x21800000 + 1 and c[10] == 0   # its reciprocal: exact on the whole range
 
 
+def test_device_encoders_exhaustive():
+    """The code assignment as the kernels run it on the device (LDS encode table + median-of-three
+    clamp for m; fma + ceil + saturating byte conversion + byte permute for v; the division by
+    the group maximum in front of both) against the count of midpoints below x, i.e. the
+    reference search (lpmm/cpp_extension/fused_adamw_kernel.cu:27-49): all 2^32 bit patterns
+    through both maps, NaN -> 15 included, and 256 group maxima around and outside the range
+    that divides by the corrected reciprocal."""
+    lib = _native().lib()
+    counts = torch.zeros(10, dtype=torch.int64, device="cuda")
+    st = lib.lpmm_selftest_encoders(counts.data_ptr(), torch.cuda.current_stream().cuda_stream)
+    assert st == 0
+    torch.cuda.synchronize()
+    c = counts.cpu().tolist()
+    print("m: %d tried, %d wrong; v: %d tried, %d wrong; bare v form: %d tried, %d wrong; "
+          "scaled m: %d tried, %d wrong; scaled v: %d tried, %d wrong" % tuple(c))
+    assert c[0] == 1 << 32 and c[2] == 1 << 32
+    # the bare form is tried on whole groups of 8 consecutive patterns that are all <= 1.0: the
+    # finite negative values and [+0, 1.0) (1.0 and -inf share their groups with values above 1.0
+    # and NaNs; they go through the guarded form above)
+    assert c[4] == (0xff800000 - 0x80000000) + 0x3f800000
+    assert c[6] == 256 * (1 << 16) * 8 and c[8] == c[6]
+    assert c[1] == 0 and c[3] == 0 and c[5] == 0 and c[7] == 0 and c[9] == 0
+
+
 def test_fused_multi_step_under_graph_capture(qmaps):
     """The library only enqueues kernels on the stream it is given (no allocation, no memset, no
     synchronisation), so a multi-tensor step can be recorded into a HIP graph.  Each of three
