@@ -9,6 +9,10 @@ sequence on the host cores, bounded sample).
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload llama7b|gpt2xl|tiny]
 
+After the timed region the default run also measures, on the same box, what plain streaming
+kernels with the fused step's access pattern reach (`roofline.calibration`; `--workload calibrate`
+prints the full table alone).
+
 Two further workloads measure the other kernels of the path with the same JSON shape:
 `--workload quant64m` (stand-alone quantise/dequantise round trip on 2^26 values) and
 `--workload factored` (factored second moment on LLaMA-7B MLP/attention shapes) and
@@ -87,12 +91,14 @@ WORKLOADS = {
 }
 
 
-def make_params(torch, shapes, dev, heavy_tailed):
-    params = []
+def make_params(torch, shapes, dev, heavy_tailed, interleaved=False):
+    """Synthetic parameters and gradients.  All parameters are allocated first and all gradients
+    after them, the order in which a model and its first backward pass allocate them;
+    `interleaved` puts each gradient right behind its parameter instead (for square tensors the
+    two streams are then an exact power of two apart, which costs 1-2 % on this memory system)."""
     gen = torch.Generator(device=dev)
-    for i, shape in enumerate(shapes):
-        gen.manual_seed(10000 + i)
-        p = torch.nn.Parameter(torch.randn(shape, device=dev, generator=gen) * 0.02)
+
+    def grad_for(i, shape):
         gen.manual_seed(20000 + i)
         z = torch.randn(shape, device=dev, generator=gen)
         if heavy_tailed:  # Student-t, 3 degrees of freedom: z / sqrt((a^2+b^2+c^2)/3)
@@ -102,8 +108,18 @@ def make_params(torch, shapes, dev, heavy_tailed):
                 s.addcmul_(a, a)
             z.div_(s.div_(3.0).sqrt_())
             del s, a
-        p.grad = z.mul_(1e-3)
+        return z.mul_(1e-3)
+
+    params = []
+    for i, shape in enumerate(shapes):
+        gen.manual_seed(10000 + i)
+        p = torch.nn.Parameter(torch.randn(shape, device=dev, generator=gen) * 0.02)
+        if interleaved:
+            p.grad = grad_for(i, shape)
         params.append(p)
+    if not interleaved:
+        for i, p in enumerate(params):
+            p.grad = grad_for(i, p.shape)
     return params
 
 
@@ -152,6 +168,62 @@ def cpu_baseline(torch, steps=10):
                   f"median of {steps} steps after 1 warm-up",
         "fused_step_c_restatement_params_per_s": n / sorted(fused_times[1:])[1],
     }
+
+
+PROBE_KINDS = {"read": (0, 4.0), "write": (1, 4.0), "copy": (2, 8.0), "update_2r1w": (3, 12.0),
+               "fused_mix": (4, BYTES_PER_PARAM_4BIT)}
+# dynamic LDS per workgroup -> workgroups resident per CU (160 KB of LDS per CU)
+PROBE_RESIDENCY = {8: 0, 6: 26 * 1024, 5: 30 * 1024, 4: 40 * 1024, 3: 53 * 1024, 2: 80 * 1024}
+
+
+def calibrate(torch, lib, n=1 << 29, iters=5, full=False):
+    """What the memory system of this box gives to plain streaming kernels with the fused step's
+    access pattern (lpmm_stream_probe: same workgroup shape, tile, lane layout and nontemporal
+    accesses, no arithmetic): read, write, copy, the in-place 2-reads-1-write update, and the seven
+    streams of the fused step at several residencies.  GB/s over `iters` back-to-back launches on
+    2^29 elements of random data (events on the launch stream), after 2 warm-up launches."""
+    from lpmm import _native
+
+    dev = torch.device("cuda:0")
+    gen = torch.Generator(device=dev).manual_seed(7)
+    a = torch.randn(n, device=dev, generator=gen) * 0.02
+    b = torch.randn(n, device=dev, generator=gen) * 1e-3
+    c0 = torch.randint(0, 256, (n // 2,), dtype=torch.uint8, device=dev, generator=gen)
+    c1 = torch.randint(0, 256, (n // 2,), dtype=torch.uint8, device=dev, generator=gen)
+    s0 = torch.ones(n // 128, device=dev)
+    s1 = torch.ones(n // 128, device=dev)
+    stream = _native.current_stream(dev)
+
+    def rate(kind, lds):
+        code, bytes_per_elt = PROBE_KINDS[kind]
+
+        def launch():
+            st = lib.lpmm_stream_probe(code, a.data_ptr(), b.data_ptr(), c0.data_ptr(), c1.data_ptr(), s0.data_ptr(),
+                                       s1.data_ptr(), n, lds, stream)
+            _native.check(st, "stream probe")
+
+        launch()
+        launch()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(iters):
+            launch()
+        e1.record()
+        torch.cuda.synchronize()
+        return n * bytes_per_elt * iters / (e0.elapsed_time(e1) * 1e-3) / 1e9
+
+    out = {"elements": n, "unit": "GB/s", "data": "random"}
+    res_list = sorted(PROBE_RESIDENCY, reverse=True)
+    for kind in ("read", "write", "copy", "update_2r1w"):
+        if full:
+            out[kind] = {str(r): round(rate(kind, PROBE_RESIDENCY[r]), 1) for r in res_list}
+        else:
+            out[kind] = round(max(rate(kind, PROBE_RESIDENCY[r]) for r in (8, 4)), 1)
+    mix = {str(r): round(rate("fused_mix", PROBE_RESIDENCY[r]), 1) for r in res_list}
+    out["fused_mix_by_workgroups_per_cu"] = mix
+    out["fused_mix_best"] = max(mix.values())
+    del a, b, c0, c1, s0, s1
+    return out
 
 
 def verify_one_more_step(torch, opt, params):
@@ -370,8 +442,12 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=2)
-    ap.add_argument("--workload", default="llama7b", choices=sorted(WORKLOADS) + ["quant64m", "factored", "nonfused_group", "nonfused_rank1"])
+    ap.add_argument("--workload", default="llama7b", choices=sorted(WORKLOADS) + ["quant64m", "factored", "nonfused_group", "nonfused_rank1", "calibrate"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--interleaved-grads", action="store_true",
+                    help="allocate each gradient right behind its parameter instead of all parameters first")
+    ap.add_argument("--no-calibration", action="store_true",
+                    help="skip the streaming-rate calibration that follows the timed region")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run three plain 1 GiB device copies first (calibration dispatches for "
                          "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs)")
@@ -399,6 +475,19 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
+    if args.workload == "calibrate":
+        cal = calibrate(torch, lib, iters=max(args.steps, 3), full=True)
+        best = cal["fused_mix_best"]
+        print(json.dumps({
+            "metric": "streaming-rate calibration: the fused step's seven-stream access pattern without arithmetic",
+            "value": best, "unit": "GB/s", "n_gpus": 1, "steps": max(args.steps, 3), "warmup": 2,
+            "ms_per_step": cal["elements"] * BYTES_PER_PARAM_4BIT / best / 1e6, "higher_is_better": True,
+            "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+            "config": {"workload": "lpmm_stream_probe on 2^29 elements, all kinds and residencies"},
+            "roofline": {"bound": "hbm", "kernel": "lpmm::probe_fused_mix_kernel", "achieved": best,
+                         "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": best / HBM_PEAK_GBS, "traffic": None},
+            "calibration": cal}))
+        return
     if args.workload == "quant64m":
         return run_quant_roundtrip(torch, args)
     if args.workload == "factored":
@@ -408,7 +497,8 @@ def main():
 
     desc, shape_fn = WORKLOADS[args.workload]
     shapes = shape_fn()
-    params = make_params(torch, shapes, dev, heavy_tailed=(args.workload == "llama7b"))
+    params = make_params(torch, shapes, dev, heavy_tailed=(args.workload == "llama7b"),
+                         interleaved=args.interleaved_grads)
     opt = lpmm.optim.AdamW(params, lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01, fused=True)
 
     n_total = sum(p.numel() for p in params)
@@ -498,6 +588,11 @@ def main():
             "avg_launch_ms": launch_ms,
         },
     }
+    if not args.no_calibration:
+        # the same box, the same run: what plain streaming kernels with this access pattern reach
+        cal = calibrate(torch, lib)
+        out["roofline"]["calibration"] = cal
+        out["roofline"]["frac_of_fused_mix_best"] = achieved / cal["fused_mix_best"]
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(torch)
     print(json.dumps(out))

@@ -352,6 +352,24 @@ int lpmm_selftest_arithmetic(unsigned long long *counts, uint32_t sqrt_stride, u
  *   same with the second-moment map.  Every odd entry must stay 0. */
 int lpmm_selftest_encoders(unsigned long long *counts, void *stream);
 
+/* Diagnostic (no counterpart in the reference): streaming-rate calibration.  Kernels that move
+ * bytes the way the fused 4-bit step moves them (256-thread workgroups, 2048-element tiles, the
+ * same lane-to-address layout, nontemporal accesses, one-shot grid) with no arithmetic to speak
+ * of, so that their rate is what the memory system gives to the access pattern itself:
+ *   LPMM_PROBE_READ       a read                                   4 B/element
+ *   LPMM_PROBE_WRITE      a written                                4 B/element
+ *   LPMM_PROBE_COPY       a = b                                    8 B/element
+ *   LPMM_PROBE_UPDATE     a += b in place (2 reads : 1 write)     12 B/element
+ *   LPMM_PROBE_FUSED_MIX  the seven streams of lpmm_adamw4bit_step: a, b read, a written,
+ *                         codes0/1 (n/2 bytes each) and scale0/1 (n/128 floats each) read and
+ *                         written                                 14.125 B/element
+ * n: a multiple of 2048; a, b: fp32[n], 16-byte aligned.  lds_bytes (0..163840) of dynamic LDS
+ * that the kernels never touch cap the workgroups resident per CU at floor(160 KB / lds_bytes)
+ * (0: the hardware's own limit of 8).  Buffers a kind does not use may be NULL. */
+enum { LPMM_PROBE_READ = 0, LPMM_PROBE_WRITE = 1, LPMM_PROBE_COPY = 2, LPMM_PROBE_UPDATE = 3, LPMM_PROBE_FUSED_MIX = 4 };
+int lpmm_stream_probe(int kind, float *a, const float *b, uint8_t *codes0, uint8_t *codes1, float *scale0,
+                      float *scale1, int64_t n, int64_t lds_bytes, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -10,11 +10,11 @@
 // every 16-byte load of a row covers 256 contiguous bytes and the group maxima are 7
 // in-register max + 4 DPP steps: no LDS traffic and no atomics for the reduction.  A
 // 256-thread workgroup covers a tile of 2048 elements = 16 groups.  LDS holds the two
-// 16-entry maps (decode) and the 2 KB first-moment encode table.
+// 16-entry maps (decode) and the 4 KB first-moment encode table (one entry per bucket byte).
 //
 // When the maps passed in are the standard ones (dynamic-exponent signed map for m,
 // (k+1)/16 for v; checked on the device, no host round trip), the codes are assigned by
-// lpmm_encode.hpp (table for m, closed form for v) and the divisions by the group maximum
+// lpmm_encode.hpp and lpmm_codec.hpp (bucket table for m, closed form for v) and the divisions by the group maximum
 // use the correctly rounded reciprocal plus one fma correction step; both give the same
 // results as the generic search and the plain division, which remain as the fallback for
 // any other map.
@@ -28,15 +28,37 @@ constexpr int kThreads = 256;
 constexpr int kEltsPerLane = 8;
 constexpr int kTile = kThreads * kEltsPerLane;  // 2048 elements = 16 groups
 
-// LDS per workgroup.  The tables need kLdsBytes; the allocation is larger on purpose, so that
-// at most 5 workgroups (20 waves) are resident on a CU (160 KB of LDS).  With the 7 that the
-// registers would allow, the waves that are not computing all sit in the memory queues, and
-// the HBM system of MI355X sustains less with deeper queues: the bare access pattern of this
-// kernel runs at 5.9 TB/s with 8 resident workgroups per CU and at 6.2-6.4 TB/s with 3-5; the
-// kernel itself gains 3 % with 5 and loses with 4 (too few waves to cover the arithmetic).
-constexpr uint32_t kFusedLdsBytes = 30 * 1024;
-static_assert(160 * 1024 / kFusedLdsBytes == 5, "residency cap");
-static_assert(kFusedLdsBytes >= kLdsBytes, "tables do not fit");
+// LDS per workgroup.  The tables need kLdsBytes; the allocation is larger on purpose: it caps
+// the workgroups resident on a CU (160 KB of LDS).  With the 7 that the registers would allow,
+// the waves that are not computing all sit in the memory queues, and the HBM system of MI355X
+// sustains less with deeper queues: streaming kernels with this kernel's access pattern and no
+// arithmetic (lpmm_stream_probe) peak at 4-5 resident workgroups per CU and lose 3 % at 8.
+// Measured optimum of the kernel itself: 4 per CU (40 KB) where every tensor of the launch is a
+// whole number of tiles (the straight-line variant; LLaMA-7B-shaped set 15.80 ms per step with 5,
+// 15.43 with 4, and only 5.05 TB/s with 3: too few waves to cover the arithmetic), 5 per CU
+// (30 KB) for the guarded variant (GPT-2-XL-shaped set 3.74 ms per step with 5, 3.81 with 4).
+#ifndef LPMM_FUSED_LDS_KB_WHOLE
+#define LPMM_FUSED_LDS_KB_WHOLE 40
+#endif
+#ifndef LPMM_FUSED_LDS_KB_RAGGED
+#define LPMM_FUSED_LDS_KB_RAGGED 30
+#endif
+template <bool ALLFULL>
+constexpr uint32_t fused_lds_bytes()
+{
+    return (ALLFULL ? LPMM_FUSED_LDS_KB_WHOLE : LPMM_FUSED_LDS_KB_RAGGED) * 1024u;
+}
+static_assert(fused_lds_bytes<true>() >= kLdsBytes && fused_lds_bytes<false>() >= kLdsBytes, "tables do not fit");
+static_assert(kThreads == kEncEntries, "lds_fill_load / lds_fill_store: one encode-table entry per thread");
+// Waves of the straight-line variant of the fused arithmetic pause this many units of 64 cycles before their first load.
+// The memory system has an optimum number of requests in flight that lies between what 4 and 5
+// resident workgroups per CU keep there; the pause trims the 4.  Measured on the LLaMA-7B-shaped
+// launches: 0 -> 6.36 TB/s, 4 -> 6.40, 6 -> 6.41, 8 -> 6.41, 10 -> 6.37, 20 -> 6.13; pauses that differ
+// between neighbouring workgroups lose 3-5 % (tiles next to each other should be in flight together).
+#ifndef LPMM_FUSED_START_DELAY
+#define LPMM_FUSED_START_DELAY 6
+#endif
+constexpr int kStartDelay = LPMM_FUSED_START_DELAY;
 
 
 struct Tensor4 {
@@ -226,8 +248,7 @@ __device__ __forceinline__ void group_step(const Tensor4 &t, const TileView &w, 
         }
     }
     // every lane of the row takes part, also those past the end of the tensor
-    amax_m = row16_max(amax_m);
-    amax_v = row16_max(amax_v);
+    row16_max2(amax_m, amax_v);
     if (!any)
         return;
 
@@ -281,7 +302,10 @@ __global__ __launch_bounds__(kThreads) void adamw4bit_kernel(const Multi4 args,
                                                              const float *__restrict__ qmap_m,
                                                              const float *__restrict__ qmap_v)
 {
-    __shared__ __align__(16) uint32_t lds[kFusedLdsBytes / 4];
+    __shared__ __align__(16) uint32_t lds[fused_lds_bytes<ALLFULL>() / 4];
+    // a short pause before the first load: see kStartDelay
+    if (ALLFULL && !Arith::kPadded && kStartDelay > 0)
+        __builtin_amdgcn_s_sleep(kStartDelay);
     // the small loads first: maps and encode table for LDS
     const LdsFill fill = lds_fill_load(qmap_m, qmap_v);
 

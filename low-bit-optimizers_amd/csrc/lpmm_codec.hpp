@@ -123,25 +123,35 @@ __device__ __forceinline__ T lds_read(const uint32_t *lds, uint32_t byte_off)
     return *reinterpret_cast<const T *>(reinterpret_cast<const char *>(lds) + byte_off);
 }
 
-// Threads [0,16) copy map 0, [16,32) map 1 (if given), [0, 2*kEncBuckets) the encode table.
-// The caller synchronises the workgroup afterwards.
+// The encode-table entry of bucket idx (0..255), from the stored table: 80 entries of global
+// memory serve all 256 buckets, so a workgroup's table costs 10 cache lines, not 32.
+__device__ __forceinline__ uint4 enc_entry(uint32_t idx)
+{
+    uint4 e = *reinterpret_cast<const uint4 *>(kEncTableM[enc_m_stored_index(idx)]);
+    if (idx == kEncNanBucket)
+        e.y = e.z = 15u;
+    return e;
+}
+
+// Threads [0,16) copy map 0, [16,32) map 1 (if given), all threads the encode table (one
+// 16-byte entry each, in rounds of the workgroup's size).  The caller synchronises the
+// workgroup afterwards.
 __device__ __forceinline__ void lds_fill(uint32_t *lds, const float *__restrict__ q0, const float *__restrict__ q1)
 {
     if (threadIdx.x < 16)
         lds[kLdsQ0 / 4 + threadIdx.x] = __float_as_uint(q0[threadIdx.x]);
     else if (threadIdx.x < 32 && q1 != nullptr)
         lds[kLdsQ1 / 4 + threadIdx.x - 16] = __float_as_uint(q1[threadIdx.x - 16]);
-    if (threadIdx.x < 2 * kEncBuckets) {
-        const uint4 e = *reinterpret_cast<const uint4 *>(kEncTableM[threadIdx.x]);
-        *reinterpret_cast<uint4 *>(reinterpret_cast<char *>(lds) + e.w) = e;  // e.w: the entry's LDS offset
-    }
+    for (uint32_t i = threadIdx.x; i < (uint32_t)kEncEntries; i += blockDim.x)
+        *reinterpret_cast<uint4 *>(reinterpret_cast<char *>(lds) + kEncLdsBegin + 16 * i) = enc_entry(i);
 }
 
-// The same in two halves, so that a kernel can issue these small loads first, start its
-// streaming loads, and write LDS once the small ones have arrived (loads return in order).
-// Every thread loads and every thread stores (threads past the tables repeat an entry, so some
-// addresses are written several times with the same value): no branch surrounds either half,
-// and the wait before the stores counts exactly the loads issued in between.
+// The same in two halves for workgroups of exactly kEncEntries threads, so that a kernel can
+// issue these small loads first, start its streaming loads, and write LDS once the small ones
+// have arrived (loads return in order).  Every thread loads and every thread stores (threads
+// past the maps repeat a map entry, so some addresses are written several times with the same
+// value): no branch surrounds either half, and the wait before the stores counts exactly the
+// loads issued in between.
 struct LdsFill {
     uint32_t q;
     uint4 e;
@@ -153,26 +163,34 @@ __device__ __forceinline__ LdsFill lds_fill_load(const float *__restrict__ q0, c
     const uint32_t t = threadIdx.x;
     const float *qp = ((t & 16) == 0) ? q0 + (t & 15) : q1 + (t & 15);
     f.q = __float_as_uint(*qp);
-    const uint32_t te = t < 2 * kEncBuckets ? t : 2 * kEncBuckets - 1;
-    f.e = *reinterpret_cast<const uint4 *>(kEncTableM[te]);
+    f.e = enc_entry(t);
     return f;
 }
 
 __device__ __forceinline__ void lds_fill_store(uint32_t *lds, const LdsFill &f)
 {
     lds[threadIdx.x & 31] = f.q;  // kLdsQ0 = 0, kLdsQ1 = 64: the two maps are adjacent
-    *reinterpret_cast<uint4 *>(reinterpret_cast<char *>(lds) + f.e.w) = f.e;
+    *reinterpret_cast<uint4 *>(reinterpret_cast<char *>(lds) + kEncLdsBegin + 16 * threadIdx.x) = f.e;
 }
 static_assert(kLdsQ0 == 0 && kLdsQ1 == 64, "lds_fill_store writes the maps back to back");
 
-// Codes of 8 already divided values with the standard first-moment map: nibble k = code of x[k].
+// Codes of 8 values with the standard first-moment map: nibble k = code of x[k].  The bucket of
+// a value is its conversion to an 8-bit float (two values per instruction, the four bytes of a
+// word are the buckets of four values); the bucket's table entry {thr, code_le, code_gt} decides
+// with one compare.  Any float is a legal input; a NaN gives 15.
 __device__ __forceinline__ uint32_t encode8_std_m(const uint32_t *lds, const float (&x)[8])
 {
     uint32_t w = 0;
 #pragma unroll
-    for (int k = 0; k < 8; ++k) {
-        const uint4 e = lds_read<uint4>(lds, enc_m_lds_offset(x[k]));
-        w |= enc_m_pick(x[k], e.x, e.y, e.z) << (4 * k);
+    for (int h = 0; h < 2; ++h) {
+        int b = __builtin_amdgcn_cvt_pk_bf8_f32(x[4 * h], x[4 * h + 1], 0, false);
+        b = __builtin_amdgcn_cvt_pk_bf8_f32(x[4 * h + 2], x[4 * h + 3], b, true);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const uint32_t off = (((uint32_t)b >> (8 * k)) & 0xffu) << 4;
+            const uint4 e = lds_read<uint4>(lds, kEncLdsBegin + off);
+            w |= enc_m_pick(x[4 * h + k], e.x, e.y, e.z) << (4 * (4 * h + k));
+        }
     }
     return w;
 }

@@ -43,13 +43,29 @@ __device__ __forceinline__ float dpp_f32(float v)
     return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, false));
 }
 
+// One step: v = max(v, v of the lane the DPP control names).  The exchange is an operand
+// modifier of the max itself (one instruction per step).  A DPP operand may be read two wait
+// states after the instruction that wrote it at the earliest; inline assembly is outside the
+// compiler's hazard handling, so the s_nop in front supplies them.
+#define LPMM_DPP_MAX(ctrl) "s_nop 1\n\tv_max_f32_dpp %0, %0, %0 " ctrl " row_mask:0xf bank_mask:0xf\n\t"
+#define LPMM_DPP_MAX2(ctrl)                                              \
+    "s_nop 0\n\tv_max_f32_dpp %0, %0, %0 " ctrl " row_mask:0xf bank_mask:0xf\n\t" \
+    "v_max_f32_dpp %1, %1, %1 " ctrl " row_mask:0xf bank_mask:0xf\n\t"
+
 __device__ __forceinline__ float row16_max(float v)
 {
-    v = fmaxf(v, dpp_f32<0xB1>(v));   // quad_perm [1,0,3,2]
-    v = fmaxf(v, dpp_f32<0x4E>(v));   // quad_perm [2,3,0,1]
-    v = fmaxf(v, dpp_f32<0x141>(v));  // row_half_mirror
-    v = fmaxf(v, dpp_f32<0x140>(v));  // row_mirror
+    asm(LPMM_DPP_MAX("quad_perm:[1,0,3,2]") LPMM_DPP_MAX("quad_perm:[2,3,0,1]")
+            LPMM_DPP_MAX("row_half_mirror") LPMM_DPP_MAX("row_mirror")
+        : "+v"(v));
     return v;
+}
+
+// Two row maxima at once: the second value's instruction fills one of the wait states of the first.
+__device__ __forceinline__ void row16_max2(float &a, float &b)
+{
+    asm("s_nop 1\n\t" LPMM_DPP_MAX2("quad_perm:[1,0,3,2]") LPMM_DPP_MAX2("quad_perm:[2,3,0,1]")
+            LPMM_DPP_MAX2("row_half_mirror") LPMM_DPP_MAX2("row_mirror")
+        : "+v"(a), "+v"(b));
 }
 
 // Row layout: the 16 lanes of a DPP row own one 128-element group, lane l the elements

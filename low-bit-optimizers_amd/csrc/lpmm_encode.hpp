@@ -22,13 +22,20 @@ namespace lpmm {
 
 #include "std_tables.inc"
 
-// The first-moment encode table lives in LDS at byte (bucket index * 16) for x >= 0 and
-// kEncSignStride bytes further for x < 0; bucket indices run from kEncLo to kEncHi, so the
-// bytes below kEncLo*16 are free for other use.
-static constexpr uint32_t kEncLdsBegin = (uint32_t)kEncLo * 16;
-static constexpr uint32_t kEncLdsEnd = (uint32_t)(kEncHi + 1) * 16 + kEncSignStride;
-static_assert((uint32_t)(kEncHi + 1) * 16 <= kEncSignStride, "sign bit collides with the bucket offset");
-static_assert(kEncMantBits == 2, "shifts below assume 21 dropped mantissa bits");
+// The first-moment encode table lives in LDS at kEncLdsBegin + 16 * (bucket byte); the bytes
+// between the two maps and the table are free for other use.
+static constexpr uint32_t kEncLdsBegin = 4224;
+static constexpr uint32_t kEncLdsEnd = kEncLdsBegin + (uint32_t)kEncEntries * 16;
+
+// Where bucket `idx` (0..255) sits in the stored table, and whether it is the NaN bucket,
+// whose entry is patched to code 15 on both sides.
+LPMM_HD uint32_t enc_m_stored_index(uint32_t idx)
+{
+    uint32_t m = idx & 127u;
+    m = m < kEncCompactLo ? kEncCompactLo : (m > kEncCompactHi ? kEncCompactHi : m);
+    return (idx >> 7) * kEncCompactPerSign + m - kEncCompactLo;
+}
+static constexpr uint32_t kEncNanBucket = 0xfeu;
 
 LPMM_HD uint32_t f32_bits(float x)
 {
@@ -52,18 +59,28 @@ LPMM_HD float bits_f32(uint32_t u)
 #endif
 }
 
-// LDS byte offset of x's table entry {thr, code_le, code_gt}.
-LPMM_HD uint32_t enc_m_lds_offset(float x)
+// The bucket byte of x: x converted to an 8-bit float with 5 exponent and 2 mantissa bits, round
+// to nearest even, overflow to infinity (0x7c), every NaN to 0xfe.  On the device this is one
+// v_cvt_pk_bf8_f32 for two values (encode8_std_m in lpmm_codec.hpp); this host twin restates the
+// conversion for the exhaustive check of the table.
+#if !defined(__HIP_DEVICE_COMPILE__)
+static inline uint32_t enc_m_bucket_host(float x)
 {
-    const float lo = bits_f32(kEncClampLoBits), hi = bits_f32(kEncClampHiBits);
-#if defined(__HIP_DEVICE_COMPILE__)
-    const float a = __builtin_amdgcn_fmed3f(__builtin_fabsf(x), lo, hi);
-#else
-    const float a = std::fmin(std::fmax(std::fabs(x), lo), hi);
-#endif
-    // (bits(a) >> 21) * 16, plus kEncSignStride when the sign bit of x is set
-    return ((f32_bits(a) >> 17) & 0x3FF0u) | ((f32_bits(x) >> 18) & kEncSignStride);
+    const uint32_t b = f32_bits(x), sign = (b >> 31) << 7, mag = b & 0x7fffffffu;
+    if (mag > 0x7f800000u)
+        return 0xfeu;
+    if ((mag >> 23) >= 113u) {
+        const uint32_t r = (mag + 0xfffffu + ((mag >> 21) & 1u)) >> 21;
+        return sign | (r - 448u < 0x7cu ? r - 448u : 0x7cu);
+    }
+    const double q = (double)bits_f32(mag) * 65536.0;  // multiples of 2^-16 below 2^-14
+    uint32_t n = (uint32_t)q;
+    const double frac = q - (double)n;
+    if (frac > 0.5 || (frac == 0.5 && (n & 1u)))
+        ++n;
+    return sign | n;
 }
+#endif
 
 // thr is compared as a float: magnitudes order like their bit patterns, and the "no
 // midpoint in this bucket" pattern 0xffffffff is a NaN, which never compares below.

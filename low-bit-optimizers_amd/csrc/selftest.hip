@@ -90,10 +90,8 @@ __device__ __forceinline__ void selftest_lds_setup(uint32_t *lds)
         lds[kLdsQ0 / 4 + i] = kStdQmapMBits[i];
         lds[kLdsQ1 / 4 + i] = kStdQmapVBits[i];
     }
-    for (uint32_t i = threadIdx.x; i < 2 * kEncBuckets; i += blockDim.x) {
-        const uint4 e = *reinterpret_cast<const uint4 *>(kEncTableM[i]);
-        *reinterpret_cast<uint4 *>(reinterpret_cast<char *>(lds) + e.w) = e;
-    }
+    for (uint32_t i = threadIdx.x; i < (uint32_t)kEncEntries; i += blockDim.x)
+        *reinterpret_cast<uint4 *>(reinterpret_cast<char *>(lds) + kEncLdsBegin + 16 * i) = enc_entry(i);
     __syncthreads();
 }
 

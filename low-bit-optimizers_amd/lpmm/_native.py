@@ -51,6 +51,7 @@ PROTOTYPES = {
     "lpmm_factored_update": (_int, [_vp] * 8 + [_i64, _i64] + [_d] * 6 + [_int, _vp]),
     "lpmm_factored_step_multi": (_int, [_vp, _i64, _vp] + [_d] * 5 + [_vp]),
     "lpmm_factored_update_fp32m": (_int, [_vp] * 6 + [_i64, _i64] + [_d] * 6 + [_vp]),
+    "lpmm_stream_probe": (_int, [_int] + [_vp] * 6 + [_i64, _i64, _vp]),
     "lpmm_selftest_encoders": (_int, [_vp, _vp]),
     "lpmm_selftest_arithmetic": (_int, [_vp, ctypes.c_uint32, ctypes.c_uint64, ctypes.c_uint32, _vp]),
 }

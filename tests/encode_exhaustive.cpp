@@ -35,12 +35,10 @@ int main()
         if ((xb & 0x7fffffffu) > 0x7f800000u) continue;  // NaN
         float x;
         memcpy(&x, &xb, 4);
-        // the LDS layout of the table: bucket*16 bytes, negative half kEncSignStride further
-        const uint32_t off = enc_m_lds_offset(x);
-        const uint32_t sign = off >= kEncLdsBegin + kEncSignStride ? 1u : 0u;
-        const uint32_t bucket = (off - sign * kEncSignStride) / 16 - (uint32_t)kEncLo;
-        if (off < kEncLdsBegin || off + 16 > kEncLdsEnd || bucket >= (uint32_t)kEncBuckets) { ++bad_m; continue; }
-        const uint32_t *e = kEncTableM[sign * kEncBuckets + bucket];
+        // the table is indexed by the bucket byte (the 8-bit float conversion, restated on the host)
+        const uint32_t bucket = enc_m_bucket_host(x);
+        if (bucket >= (uint32_t)kEncEntries) { ++bad_m; continue; }
+        const uint32_t *e = kEncTableM[enc_m_stored_index(bucket)];
         if ((int)enc_m_pick(x, e[0], e[1], e[2]) != ref_search(qm, x)) ++bad_m;
         if ((int)enc_v_linear(x) != ref_search(qv, x)) ++bad_v;
         ++checked;
