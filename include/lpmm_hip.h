@@ -289,8 +289,7 @@ int lpmm_factored_update(float *p, const float *g, uint8_t *m_codes, float *m_ma
 
 /* Both passes for a list of row-major R x C tensors whose column count is a multiple of 128
  * and whose first moment is quantised (4-bit, 'group', gp_sz 128): statistics and update of
- * all tensors in four launches per batch (up to 24 tensors and about 384 MB of gradients, so
- * that the second read of a batch's gradients is served largely from the memory-side cache)
+ * all tensors in four launches per group of up to 24 tensors
  * instead of four per tensor.  Same results as
  * lpmm_factored_stats followed by lpmm_factored_update.  workspace: device scratch of
  * lpmm_factored_workspace_bytes(rows, cols) bytes per tensor, 8-byte aligned, not shared

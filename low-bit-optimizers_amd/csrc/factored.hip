@@ -51,110 +51,69 @@ __global__ __launch_bounds__(kFThreads) void nonfused_update_kernel(float *__res
 // Factored statistics, pass A: partial row/column sums of g*g over tiles of
 // kSRows x kSCols, accumulated in double.  Partials go to the workspace:
 //   colpart[ty][c]  (ty = row-tile index)   rowpart[tx][r]  (tx = column-tile index)
+// One-shot: a wave takes 16 rows x 256 columns of the tile (a lane: 4 columns of each row) and
+// issues all 16 loads at once; there is no loop, so the grid's many small workgroups keep the
+// memory system as busy as a plain streaming read does.  The wave owns its rows (their sums go
+// straight to rowpart); the column sums of the four waves meet in LDS in a fixed order.
 // ---------------------------------------------------------------------------------------
 constexpr int kSRows = 64;
-constexpr int kSCols = 1024;  // 256 threads x 4 columns
-constexpr int kSUnroll = 8;   // rows in flight per lane (wave_sum8_f64 reduces 8 rows at once)
+constexpr int kSCols = 256;   // 64 lanes x 4 columns
+constexpr int kSWaveRows = kSRows / (kFThreads / kWave);  // 16
+static_assert(kSWaveRows == 16, "two wave_sum8_f64 reductions per wave");
 
 __device__ __forceinline__ void partial_body(const float *__restrict__ g, int64_t R, int64_t C,
                                              double *__restrict__ colpart, double *__restrict__ rowpart, bool vec,
                                              uint32_t bx, uint32_t by)
 {
-    const int64_t c0 = (int64_t)bx * kSCols + (int64_t)threadIdx.x * 4;
-    const int64_t r0 = (int64_t)by * kSRows;
-    const int64_t r1 = (r0 + kSRows < R) ? r0 + kSRows : R;
-    const bool lane_vec = vec && c0 + 4 <= C;
-    __shared__ double s_part[kFThreads / kWave][kSRows];  // row sums of the tile, per wave
-    double *rp = rowpart + (int64_t)bx * R;  // one row partial per workgroup
-    double cs[4] = {0.0, 0.0, 0.0, 0.0};
-    const int lane = threadIdx.x & (kWave - 1);
-    if (vec && r0 + kSRows <= R && (int64_t)(bx + 1) * kSCols <= C) {
-        // whole tile (uniform over the workgroup, so no load sits behind a branch): two register
-        // buffers of 8 rows; the loads of a batch are in flight while the batch before it is summed
-        float4 a[kSUnroll], b[kSUnroll];
-        // uniform row addresses plus a 32-bit lane offset: no 64-bit address per row in registers
-        const float *tile = g + r0 * C + (int64_t)bx * kSCols;
-        const uint32_t lane_off = threadIdx.x * 4u;
-        auto fetch = [&](float4(&t)[kSUnroll], int i) {
+    __shared__ double s_col[kFThreads / kWave][kSCols];
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6;
+    const int64_t c0 = (int64_t)bx * kSCols + lane * 4;
+    const int64_t r0 = (int64_t)by * kSRows + wave * kSWaveRows;
+    float4 t[kSWaveRows];
+    if (vec && c0 + 4 <= C && r0 + kSWaveRows <= R) {
+        const float *base = g + r0 * C + c0;
 #pragma unroll
-            for (int j = 0; j < kSUnroll; ++j) {
-                const float *row = tile + (int64_t)(i * kSUnroll + j) * C;
-                t[j] = load4_keep(row + lane_off);  // kept in the caches: the update pass reads g again
-            }
-        };
-        auto sum = [&](const float4(&t)[kSUnroll], int i) {
-            double rs[kSUnroll];
-#pragma unroll
-            for (int j = 0; j < kSUnroll; ++j) {
-                const float u[4] = {t[j].x * t[j].x, t[j].y * t[j].y, t[j].z * t[j].z, t[j].w * t[j].w};
-                rs[j] = ((double)u[0] + (double)u[1]) + ((double)u[2] + (double)u[3]);
-#pragma unroll
-                for (int k = 0; k < 4; ++k)
-                    cs[k] += (double)u[k];
-            }
-            const double tot = wave_sum8_f64(rs, lane);
-            if ((lane & 7) == 0)
-                s_part[threadIdx.x >> 6][i * kSUnroll + (lane >> 3)] = tot;
-        };
-        constexpr int kBatches = kSRows / kSUnroll;
-        static_assert(kBatches % 2 == 0 && kBatches >= 4, "two batches per iteration, the last pair peeled");
-        fetch(a, 0);
-#pragma unroll 1
-        for (int i = 0; i < kBatches - 2; i += 2) {
-            fetch(b, i + 1);
-            sum(a, i);
-            fetch(a, i + 2);
-            sum(b, i + 1);
-        }
-        fetch(b, kBatches - 1);
-        sum(a, kBatches - 2);
-        sum(b, kBatches - 1);
+        for (int u = 0; u < kSWaveRows; ++u)
+            t[u] = load4(base + (int64_t)u * C);
     } else {
-        for (int64_t rb = r0; rb < r1; rb += kSUnroll) {
-            float u[kSUnroll][4];
-            if (lane_vec && rb + kSUnroll <= r1) {
-                // straight-line: all loads of the batch are in flight before the first use
-                float4 t[kSUnroll];
 #pragma unroll
-                for (int j = 0; j < kSUnroll; ++j)
-                    t[j] = load4_keep(g + (rb + j) * C + c0);
+        for (int u = 0; u < kSWaveRows; ++u) {
+            const int64_t r = r0 + u;
+            float e[4];
 #pragma unroll
-                for (int j = 0; j < kSUnroll; ++j) {
-                    u[j][0] = t[j].x * t[j].x; u[j][1] = t[j].y * t[j].y; u[j][2] = t[j].z * t[j].z; u[j][3] = t[j].w * t[j].w;
-                }
-            } else {
-#pragma unroll
-                for (int j = 0; j < kSUnroll; ++j) {
-                    const int64_t r = rb + j;
-#pragma unroll
-                    for (int k = 0; k < 4; ++k) {
-                        const float t = (r < r1 && c0 + k < C) ? g[r * C + c0 + k] : 0.0f;
-                        u[j][k] = t * t;
-                    }
-                }
-            }
-            double rs[kSUnroll];
-#pragma unroll
-            for (int j = 0; j < kSUnroll; ++j) {
-                rs[j] = ((double)u[j][0] + (double)u[j][1]) + ((double)u[j][2] + (double)u[j][3]);
-#pragma unroll
-                for (int k = 0; k < 4; ++k)
-                    cs[k] += (double)u[j][k];
-            }
-            // the wave's 8 row sums at once: lane 8j ends up with the sum of row j
-            const double tot = wave_sum8_f64(rs, lane);
-            if ((lane & 7) == 0)
-                s_part[threadIdx.x >> 6][(int)(rb - r0) + (lane >> 3)] = tot;
+            for (int k = 0; k < 4; ++k)
+                e[k] = (r < R && c0 + k < C) ? g[r * C + c0 + k] : 0.0f;
+            t[u] = make_float4(e[0], e[1], e[2], e[3]);
         }
     }
-    __syncthreads();
-    if (threadIdx.x < kSRows && r0 + threadIdx.x < r1)
-        rp[r0 + threadIdx.x] = (s_part[0][threadIdx.x] + s_part[1][threadIdx.x]) +
-                               (s_part[2][threadIdx.x] + s_part[3][threadIdx.x]);
+    double cs[4] = {0.0, 0.0, 0.0, 0.0};
+    double *rp = rowpart + (int64_t)bx * R;
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+        double rs[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const float4 &x = t[half * 8 + j];
+            const float u[4] = {x.x * x.x, x.y * x.y, x.z * x.z, x.w * x.w};
+            rs[j] = ((double)u[0] + (double)u[1]) + ((double)u[2] + (double)u[3]);
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+                cs[k] += (double)u[k];
+        }
+        // the wave's 8 row sums at once: lane 8j ends up with the sum of row j of this half
+        const double tot = wave_sum8_f64(rs, lane);
+        const int64_t r = r0 + half * 8 + (lane >> 3);
+        if ((lane & 7) == 0 && r < R)
+            rp[r] = tot;
+    }
 #pragma unroll
     for (int k = 0; k < 4; ++k)
-        if (c0 + k < C)
-            colpart[(int64_t)by * C + c0 + k] = cs[k];
+        s_col[wave][lane * 4 + k] = cs[k];
+    __syncthreads();
+    const int64_t c = (int64_t)bx * kSCols + threadIdx.x;
+    if (threadIdx.x < kSCols && c < C)
+        colpart[(int64_t)by * C + c] = (s_col[0][threadIdx.x] + s_col[1][threadIdx.x]) +
+                                       (s_col[2][threadIdx.x] + s_col[3][threadIdx.x]);
 }
 
 __global__ __launch_bounds__(kFThreads) void factored_partial_kernel(const float *__restrict__ g, int64_t R,
@@ -350,24 +309,44 @@ __global__ __launch_bounds__(kFThreads) void factored_update_kernel(
 }
 
 // The same pass when the column count is a multiple of 128: every 128-element group of the
-// flattened tensor is a 128-column piece of one row, the grid is (column chunks, rows), the
-// 16 lanes of a DPP row own one group in the row layout of the fused step (lane l: columns
-// [4l, 4l+4) and [64+4l, 64+4l+4) of the piece; whole cache lines per store), and no index
-// division is needed.  Workgroup (0,0) also writes the pad codes past the tensor.
+// flattened tensor is a 128-column piece of one row.  A workgroup takes 16 consecutive groups of
+// the flattened tensor (2048 contiguous elements, whatever the row length), the 16 lanes of a
+// DPP row own one group in the row layout of the fused step (lane l: columns [4l, 4l+4) and
+// [64+4l, 64+4l+4) of the piece; whole cache lines per store).  The tile's first (row, column
+// group) comes from one division per workgroup; a group past the end of a row moves to the next
+// row (rows shorter than a tile divide once more per lane).  Tile 0 also writes the pad codes
+// past the tensor.
+#ifndef LPMM_FA_UPD_LDS_KB
+#define LPMM_FA_UPD_LDS_KB 0
+#endif
+constexpr uint32_t kFaUpdLds = LPMM_FA_UPD_LDS_KB * 1024u > kLdsBytes ? LPMM_FA_UPD_LDS_KB * 1024u : kLdsBytes;
+
 __device__ __forceinline__ void update_rows128_body(
     float *__restrict__ p, const float *__restrict__ g, uint8_t *__restrict__ m_codes,
     float *__restrict__ m_max1, const float *__restrict__ qmap_m, const float *__restrict__ row,
     const float *__restrict__ col, const float *__restrict__ row_mean_all, int64_t R, int64_t C,
-    int64_t n_padded, const NfHyper &h, bool first_step, uint32_t bx, int64_t by)
+    int64_t n_padded, const NfHyper &h, bool first_step, uint32_t tile)
 {
-    __shared__ __align__(16) uint32_t lds[kLdsBytes / 4];
+    __shared__ __align__(16) uint32_t lds[kFaUpdLds / 4];
     const int64_t n = R * C;
     const int lane16 = threadIdx.x & 15;
-    const int64_t r = by;
-    const int64_t c0 = (int64_t)bx * kFTile + (int64_t)(threadIdx.x >> 4) * kGroup;  // first column of the group
-    const bool live = c0 < C;  // uniform over the 16 lanes of the group
-    const int64_t gbase = r * C + c0;
-    const int64_t grp = gbase / kGroup;
+    const uint32_t col_blocks = (uint32_t)(C / kGroup);
+    const int64_t g0 = (int64_t)tile * (kFTile / kGroup);   // first group of the tile (uniform)
+    const int64_t r0 = g0 / col_blocks;
+    uint32_t cb = (uint32_t)(g0 - r0 * col_blocks) + (threadIdx.x >> 4);
+    int64_t r = r0;
+    if (col_blocks >= kFTile / kGroup) {  // uniform: a tile spans at most two rows
+        if (cb >= col_blocks) {
+            cb -= col_blocks;
+            ++r;
+        }
+    } else {
+        r += cb / col_blocks;
+        cb = cb % col_blocks;
+    }
+    const int64_t grp = g0 + (threadIdx.x >> 4);
+    const bool live = grp * kGroup < n;  // uniform over the 16 lanes of the group
+    const int64_t gbase = grp * kGroup;
     float *pp = p + gbase + lane16 * 4;
     uint16_t *mcp = reinterpret_cast<uint16_t *>(m_codes + (gbase >> 1)) + lane16;
     // the group's loads first, the LDS tables afterwards
@@ -376,7 +355,7 @@ __device__ __forceinline__ void update_rows128_body(
     float sm = 0.0f, row_r = 0.0f, mean_all = 1.0f;
     if (live) {
         const float *gp = g + gbase + lane16 * 4;
-        const float *cp = col + c0 + lane16 * 4;
+        const float *cp = col + (int64_t)cb * kGroup + lane16 * 4;
         a0 = load4(pp);
         a1 = load4(pp + 64);
         b0 = load4(gp);
@@ -394,7 +373,7 @@ __device__ __forceinline__ void update_rows128_body(
     lds_fill(lds, qmap_m, nullptr);
     const int kind = classify_map(qmap_m);
     lds_barrier();
-    if (bx == 0 && by == 0) {
+    if (tile == 0) {
         const float z[kFElts] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
         const uint32_t wz = kind == kMapStdM ? encode8_std_m(lds, z)
                                              : encode8_generic(make_mids(reinterpret_cast<const float *>(lds) + kLdsQ0 / 4), z);
@@ -440,7 +419,7 @@ __global__ __launch_bounds__(kFThreads) void factored_update_rows128_kernel(
     int64_t n_padded, NfHyper h, bool first_step)
 {
     update_rows128_body(p, g, m_codes, m_max1, qmap_m, row, col, row_mean_all, R, C, n_padded, h, first_step,
-                        blockIdx.x, blockIdx.y);
+                        blockIdx.x);
 }
 
 // The same update with an fp32 first moment (tensors at or under the quantisation threshold,
@@ -485,17 +464,16 @@ struct TensorFa {
     int64_t n_padded;
     uint32_t tiles_x, tiles_y;  // statistics tiles
     uint32_t row_blocks;        // finalize: workgroups that take rows; the rest take 64 columns each
-    uint32_t upd_x;             // update: 2048-column chunks per row
+    uint32_t upd_x;             // update: 2048-element tiles of the tensor
     uint32_t first_step;
     float neg_step_size, bc2_sqrt, rbc2_sqrt;
 };
 
-// Gradient bytes per launch batch.  The update pass re-reads the gradient that the
-// statistics pass of the same batch has just read, and walks it back to front, so the part
-// that the 256 MB memory-side cache still holds is not fetched from HBM a second time.
-// Smaller batches hit more often but pay four launches each: 384 MB measured best on
-// LLaMA-7B MLP shapes (2 % faster than batches bounded by the tensor count alone).
-constexpr int64_t kFaBatchBytes = (int64_t)384 << 20;
+// Launch groups are bounded by the tensor count alone.  Both passes stream the gradient from HBM
+// (nontemporal loads): batches small enough for the statistics pass to leave the gradient in the
+// 256 MB memory-side cache for the update were measured too (384 MB per batch: 10.6 ms per step on
+// LLaMA-7B MLP shapes against 10.4 with groups bounded by the tensor count alone and streaming
+// loads in the statistics pass).
 
 struct MultiFa {
     TensorFa t[kFaMax];
@@ -546,13 +524,10 @@ __global__ void factored_mean_multi_kernel(const MultiFa args)
 __global__ __launch_bounds__(kFThreads) void factored_update_multi_kernel(const MultiFa args,
                                                                           const float *__restrict__ qmap_m)
 {
-    // last tile first: the statistics pass has just read g front to back, so its tail is what
-    // the memory-side cache still holds when the batch is larger than that cache
-    const uint32_t block = gridDim.x - 1u - blockIdx.x;
+    const uint32_t block = blockIdx.x;
     const int i = find_slot(args.start_upd, block);
     const TensorFa &t = args.t[i];
     const uint32_t local = block - args.start_upd[i];
-    const uint32_t by = local / t.upd_x, bx = local - by * t.upd_x;
     NfHyper h;
     h.decay = args.decay;
     h.w1 = args.w1;
@@ -563,7 +538,7 @@ __global__ __launch_bounds__(kFThreads) void factored_update_multi_kernel(const 
     h.bc2_sqrt = t.bc2_sqrt;
     h.rbc2_sqrt = t.rbc2_sqrt;
     update_rows128_body(t.p, t.g, t.mc, t.ms, qmap_m, t.row, t.col, t.mean, t.R, t.C, t.n_padded, h,
-                        t.first_step != 0, bx, by);
+                        t.first_step != 0, local);
 }
 
 inline int64_t round_up(int64_t a, int64_t b) { return (a + b - 1) / b * b; }
@@ -742,9 +717,8 @@ extern "C" int lpmm_factored_update(float *p, const float *g, uint8_t *m_codes, 
         return LPMM_ERR_SIZE;
     const bool vec = aligned_to(p, 16) && aligned_to(g, 16);
     const NfHyper h = make_nf_hyper(beta1, beta2, lr, weight_decay, eps, step);
-    if ((cols % kGroup) == 0 && rows <= 65535 && vec && aligned_to(col, 16) && aligned_to(m_codes, 4)) {
-        const uint32_t gx = (uint32_t)((cols + kFTile - 1) / kFTile);
-        hipLaunchKernelGGL(factored_update_rows128_kernel, dim3(gx, (uint32_t)rows), dim3(kFThreads), 0,
+    if ((cols % kGroup) == 0 && vec && aligned_to(col, 16) && aligned_to(m_codes, 4)) {
+        hipLaunchKernelGGL(factored_update_rows128_kernel, dim3((uint32_t)tiles), dim3(kFThreads), 0,
                            (hipStream_t)stream, p, g, m_codes, m_max1, qmap_m, row, col, row_mean_all, rows, cols,
                            n_padded, h, first_step != 0);
     } else if ((cols % 8) == 0 && aligned_to(col, 16))
@@ -834,20 +808,15 @@ extern "C" int lpmm_factored_step_multi(const lpmm_factored_tensor *tensors, int
     while (i < count) {
         int k = 0;
         uint64_t n_stats = 0, n_fin = 0, n_upd = 0;
-        int64_t g_bytes = 0;
         args.start_stats[0] = args.start_fin[0] = args.start_upd[0] = 0;
         while (i < count && k < kFaMax) {
             const lpmm_factored_tensor &t = tensors[i];
-            const int64_t t_bytes = t.rows * t.cols * 4;  // the grid limits above keep rows * cols below 2^43
-            if (k > 0 && g_bytes + t_bytes > kFaBatchBytes)
-                break;
-            g_bytes += t_bytes;
             const uint64_t ty = (uint64_t)((t.rows + kSRows - 1) / kSRows), tx = (uint64_t)((t.cols + kSCols - 1) / kSCols);
             const uint64_t row_blocks = (uint64_t)((t.rows + kFThreads - 1) / kFThreads);
             const uint64_t fin = row_blocks + (uint64_t)((t.cols + 63) / 64);
-            const uint64_t ux = (uint64_t)((t.cols + kFTile - 1) / kFTile);
+            const uint64_t ux = (uint64_t)(round_up(t.rows * t.cols, kFTile) / kFTile);  // update tiles of the tensor
             if (n_stats + tx * ty > 0x7fffffffULL || n_fin + fin > 0x7fffffffULL ||
-                n_upd + ux * (uint64_t)t.rows > 0x7fffffffULL) {
+                n_upd + ux > 0x7fffffffULL) {
                 if (k == 0)
                     return LPMM_ERR_SIZE;  // cannot happen after the checks above
                 break;
@@ -877,7 +846,7 @@ extern "C" int lpmm_factored_step_multi(const lpmm_factored_tensor *tensors, int
             d.rbc2_sqrt = h.rbc2_sqrt;
             n_stats += tx * ty;
             n_fin += fin;
-            n_upd += ux * (uint64_t)t.rows;
+            n_upd += ux;
             ++k;
             args.start_stats[k] = (uint32_t)n_stats;
             args.start_fin[k] = (uint32_t)n_fin;

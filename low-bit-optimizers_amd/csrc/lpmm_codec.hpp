@@ -20,9 +20,6 @@ __device__ __forceinline__ float4 load4(const float *p)
     const v4f t = __builtin_nontemporal_load(reinterpret_cast<const v4f *>(p));
     return make_float4(t.x, t.y, t.z, t.w);
 }
-// A load that leaves its line in the caches: for an operand that a later pass of the same
-// step reads again (the gradient in the statistics pass of a two-pass step).
-__device__ __forceinline__ float4 load4_keep(const float *p) { return *reinterpret_cast<const float4 *>(p); }
 __device__ __forceinline__ void store4(float *p, float4 v)
 {
     const v4f t = {v.x, v.y, v.z, v.w};

@@ -29,7 +29,10 @@ namespace lpmm {
 constexpr int kThreads = 256;
 constexpr int kEltsPerLane = 8;
 constexpr int kDppRows = kThreads / 16;  // 128-column groups a workgroup handles per pass
-constexpr int kTileRows = 16;            // tensor rows per workgroup
+#ifndef LPMM_R1_ROWS
+#define LPMM_R1_ROWS 16
+#endif
+constexpr int kTileRows = LPMM_R1_ROWS;  // tensor rows per workgroup (more where one pass of a narrow tile covers more)
 constexpr int kR1Max = 32;               // tensors per launch
 constexpr int kMaxLgWide = 3;
 constexpr int kMaxWide = 1 << kMaxLgWide;
@@ -62,6 +65,7 @@ struct TensorR1 {
     // rows of (1 << lg_wide) adjacent groups each
     uint32_t lg_wide;
     uint32_t col_tiles;  // ceil(col_blocks / (1 << lg_wide))
+    uint32_t tile_rows;  // max(kTileRows, rows of one pass)
 };
 
 struct MultiR1 {
@@ -103,9 +107,9 @@ __device__ __forceinline__ Geometry geometry(const TensorR1 &t, uint32_t tile, i
     q.col_tile = tile - rb * t.col_tiles;
     q.wide = 1 << t.lg_wide;
     q.cg = q.col_tile * q.wide + (drow & (q.wide - 1));
-    q.row0 = (int64_t)rb * kTileRows + (drow >> t.lg_wide);
+    q.row0 = (int64_t)rb * t.tile_rows + (drow >> t.lg_wide);
     q.step = kDppRows >> t.lg_wide;
-    q.passes = kTileRows / q.step;
+    q.passes = (int)t.tile_rows / q.step;
     return q;
 }
 
@@ -131,11 +135,21 @@ __global__ __launch_bounds__(kThreads) void rank1_clear_kernel(const MultiR1 arg
     }
 }
 
+#ifndef LPMM_R1_PREFETCH
+#define LPMM_R1_PREFETCH 0
+#endif
+#ifndef LPMM_R1_WAVES
+#define LPMM_R1_WAVES 6
+#endif
 // 6 waves per SIMD: at most 80 registers
-__global__ __launch_bounds__(kThreads, 6) void rank1_update_kernel(const MultiR1 args, const float *__restrict__ qmap_m,
+__global__ __launch_bounds__(kThreads, LPMM_R1_WAVES) void rank1_update_kernel(const MultiR1 args, const float *__restrict__ qmap_m,
                                                                 const float *__restrict__ qmap_v)
 {
-    __shared__ __align__(16) uint32_t lds[(kColExtra + kMaxWide * kRedSlotWords * 4) / 4];
+#ifndef LPMM_R1_LDS_KB
+#define LPMM_R1_LDS_KB 0
+#endif
+    constexpr uint32_t kNeed = kColExtra + kMaxWide * kRedSlotWords * 4;
+    __shared__ __align__(16) uint32_t lds[(LPMM_R1_LDS_KB * 1024 > kNeed ? LPMM_R1_LDS_KB * 1024 : kNeed) / 4];
     uint32_t *colred = lds + kColExtra / 4;
     lds_fill(lds, qmap_m, qmap_v);
     for (int j = threadIdx.x; j < kMaxWide * (int)kRedSlotWords; j += kThreads)
@@ -172,26 +186,41 @@ __global__ __launch_bounds__(kThreads, 6) void rank1_update_kernel(const MultiR1
     if (q.cg < t.col_blocks) {  // the whole DPP row
         const uint32_t co_off = kColOld + (slot * kGroup + lane16 * 4) * 4;
         uint32_t *red = colred + slot * kRedSlotWords + lane16;
-#pragma unroll 1
-        for (int it = 0; it < q.passes; ++it) {
-            const int64_t r = q.row0 + it * q.step;
-            if (r >= t.rows)
-                break;
+        // operands of one pass, as loaded
+        struct PassRegs {
+            float4 a0, a1, b0, b1;
+            uint32_t m0, m1, v0, v1;
+            float sm, ro;
+        };
+        auto fetch = [&](int64_t r, PassRegs &x) {
+            const int64_t grp = r * t.col_blocks + q.cg;
+            const int64_t gbase = grp * kGroup;
+            const float *pp = t.p + gbase + lane16 * 4;
+            const float *gp = t.g + gbase + lane16 * 4;
+            x.a0 = load4(pp);
+            x.a1 = load4(pp + 64);
+            x.b0 = load4(gp);
+            x.b1 = load4(gp + 64);
+            const uint16_t *mcp = reinterpret_cast<const uint16_t *>(t.mc + (gbase >> 1)) + lane16;
+            const uint16_t *vcp = reinterpret_cast<const uint16_t *>(t.vc + (gbase >> 1)) + lane16;
+            x.m0 = load_u16(mcp);
+            x.m1 = load_u16(mcp + 16);
+            x.v0 = load_u16(vcp);
+            x.v1 = load_u16(vcp + 16);
+            x.sm = t.ms[grp];
+            x.ro = t.row_old[r];
+        };
+        auto work = [&](int64_t r, const PassRegs &x) {
             const int64_t grp = r * t.col_blocks + q.cg;
             const int64_t gbase = grp * kGroup;
             float *pp = t.p + gbase + lane16 * 4;
-            const float *gp = t.g + gbase + lane16 * 4;
-            const float4 a0 = load4(pp), a1 = load4(pp + 64);
-            const float4 b0 = load4(gp), b1 = load4(gp + 64);
             uint16_t *mcp = reinterpret_cast<uint16_t *>(t.mc + (gbase >> 1)) + lane16;
-            const uint16_t *vcp = reinterpret_cast<const uint16_t *>(t.vc + (gbase >> 1)) + lane16;
-            const uint32_t wm = load_u16(mcp) | (load_u16(mcp + 16) << 16);
-            const uint32_t wv = load_u16(vcp) | (load_u16(vcp + 16) << 16);
-            const float sm = t.ms[grp];
-            const float ro = t.row_old[r];
+            const uint32_t wm = x.m0 | (x.m1 << 16);
+            const uint32_t wv = x.v0 | (x.v1 << 16);
+            const float sm = x.sm, ro = x.ro;
             float pv[kEltsPerLane], gv[kEltsPerLane], m[kEltsPerLane], v[kEltsPerLane], co[kEltsPerLane];
-            unpack8(a0, a1, pv);
-            unpack8(b0, b1, gv);
+            unpack8(x.a0, x.a1, pv);
+            unpack8(x.b0, x.b1, gv);
             unpack8(lds_read<float4>(lds, co_off), lds_read<float4>(lds, co_off + 256), co);
 
             const Nibbles nm = split_nibbles(wm), nv = split_nibbles(wv);
@@ -205,8 +234,7 @@ __global__ __launch_bounds__(kThreads, 6) void rank1_update_kernel(const MultiR1
                 vmax = fmaxf(vmax, v[k]);
                 atomicMax(red + k * 16, __float_as_uint(v[k]));
             }
-            amax_m = row16_max(amax_m);
-            vmax = row16_max(vmax);
+            row16_max2(amax_m, vmax);
             const uint32_t cm = encode8_scaled(lds, kLdsQ0, kind_m, m, amax_m);
 
             store4(pp, make_float4(pv[0], pv[1], pv[2], pv[3]));
@@ -217,15 +245,46 @@ __global__ __launch_bounds__(kThreads, 6) void rank1_update_kernel(const MultiR1
                 t.ms[grp] = amax_m;
                 atomic_max_nonneg(t.row_new + r, vmax);
             }
+        };
+#if LPMM_R1_PREFETCH
+        // two passes per iteration: the loads of the second are in flight while the first computes,
+        // and those of the next iteration's first while the second computes
+        PassRegs xa, xb;
+        const int64_t last = t.rows - 1;
+        fetch(q.row0 < t.rows ? q.row0 : last, xa);
+#pragma unroll 1
+        for (int it = 0; it < q.passes; it += 2) {
+            const int64_t r0 = q.row0 + it * q.step, r1 = r0 + q.step, r2 = r1 + q.step;
+            if (r0 >= t.rows)
+                break;
+            fetch(r1 < t.rows ? r1 : last, xb);  // unconditional: a row past the end re-reads the last one
+            work(r0, xa);
+            if (it + 1 >= q.passes || r1 >= t.rows)
+                break;
+            fetch(r2 < t.rows ? r2 : last, xa);
+            work(r1, xb);
         }
+#else
+#pragma unroll 1
+        for (int it = 0; it < q.passes; ++it) {
+            const int64_t r = q.row0 + it * q.step;
+            if (r >= t.rows)
+                break;
+            PassRegs x;
+            fetch(r, x);
+            work(r, x);
+        }
+#endif
     }
     __syncthreads();
     // column j of the tile = element k of lane l of slot s
     for (int j = threadIdx.x; j < q.wide * kGroup; j += kThreads) {
         const int w = j & (kGroup - 1);
         const int k = ((w >> 6) << 2) | (w & 3), l = (w >> 2) & 15;
-        if (tile_c0 + j < cols)
-            atomic_max_nonneg(t.col_new + tile_c0 + j, __uint_as_float(colred[(j >> 7) * kRedSlotWords + k * 16 + l]));
+        if (tile_c0 + j < cols) {
+            const float mine = __uint_as_float(colred[(j >> 7) * kRedSlotWords + k * 16 + l]);
+            atomic_max_nonneg(t.col_new + tile_c0 + j, mine);
+        }
     }
 }
 
@@ -318,6 +377,9 @@ using namespace lpmm;
 // tensor's tiles without a column group; otherwise the width that wastes least.
 static uint32_t choose_lg_wide(uint32_t col_blocks)
 {
+#ifdef LPMM_R1_FORCE_LG
+    return LPMM_R1_FORCE_LG;
+#endif
     uint32_t best = 0;
     double best_use = 0.0;
     for (int lg = kMaxLgWide; lg >= 0; --lg) {
@@ -354,7 +416,7 @@ extern "C" int lpmm_nonfused_adamw4bit_rank1_step_multi(const lpmm_nonfused_rank
         if (t.rows == 0 || t.cols == 0)
             continue;
         const int64_t col_blocks = t.cols / kGroup;
-        const int64_t row_blocks = (t.rows + kTileRows - 1) / kTileRows;
+        const int64_t row_blocks = (t.rows + kTileRows - 1) / kTileRows;  // an upper bound
         if (col_blocks > 0x7fffffffLL / 2 || row_blocks > 0x7fffffffLL / col_blocks ||
             t.rows > INT64_MAX / t.cols)
             return LPMM_ERR_SIZE;
@@ -402,7 +464,9 @@ extern "C" int lpmm_nonfused_adamw4bit_rank1_step_multi(const lpmm_nonfused_rank
             const uint32_t col_blocks = (uint32_t)(t.cols / kGroup);
             const uint32_t lg_wide = choose_lg_wide(col_blocks);
             const uint32_t col_tiles = (col_blocks + (1u << lg_wide) - 1) >> lg_wide;
-            const uint64_t nt = (uint64_t)((t.rows + kTileRows - 1) / kTileRows) * col_tiles;
+            const uint32_t pass_rows = (uint32_t)kDppRows >> lg_wide;
+            const uint32_t tile_rows = pass_rows > (uint32_t)kTileRows ? pass_rows : (uint32_t)kTileRows;
+            const uint64_t nt = (uint64_t)((t.rows + tile_rows - 1) / tile_rows) * col_tiles;
             if (tiles + nt > 0x7fffffffULL)
                 break;
             TensorR1 &d = args.t[k];
@@ -419,6 +483,7 @@ extern "C" int lpmm_nonfused_adamw4bit_rank1_step_multi(const lpmm_nonfused_rank
             d.col_blocks = col_blocks;
             d.lg_wide = lg_wide;
             d.col_tiles = col_tiles;
+            d.tile_rows = tile_rows;
             const NfHyper h = make_nf_hyper(beta1, beta2, lr, weight_decay, eps, t.step);
             d.neg_step_size = h.neg_step_size;
             d.bc2_sqrt = h.bc2_sqrt;

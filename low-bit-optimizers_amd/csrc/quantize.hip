@@ -354,6 +354,60 @@ __global__ __launch_bounds__(kQThreads) void rank1_stats_kernel(const float *__r
             atomic_max_nonneg(colmax + c0 + k, cm[k]);
 }
 
+// The same statistics, one-shot: a workgroup takes a tile of 32 rows x 256 columns, a wave 8 of
+// those rows (a lane: 4 columns of each), and issues all its loads at once -- no loop, so the
+// grid's many small workgroups keep the memory system busy the way a plain streaming read does.
+// Column maxima of the four waves meet in LDS: one atomic per column and tile.  Requires whole
+// tiles' worth of vector access: 16-byte aligned x, columns a multiple of 4.
+constexpr int kStat2Rows = 32, kStat2Cols = 256;
+#ifndef LPMM_STAT2_LDS_KB
+#define LPMM_STAT2_LDS_KB 4
+#endif
+
+__global__ __launch_bounds__(kQThreads) void rank1_stats_tile_kernel(const float *__restrict__ x, int64_t R, int64_t C,
+                                                                     uint32_t tiles_x, float *__restrict__ rowmax,
+                                                                     float *__restrict__ colmax)
+{
+    __shared__ float s_col[LPMM_STAT2_LDS_KB * 256];  // [4 waves][256 columns] used; the rest caps residency
+    const uint32_t ty = blockIdx.x / tiles_x, tx = blockIdx.x - ty * tiles_x;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t c0 = (int64_t)tx * kStat2Cols + lane * 4;
+    const int64_t r0 = (int64_t)ty * kStat2Rows + wave * 8;
+    const bool cols_in = c0 + 4 <= C;
+    float4 t[8];
+    if (cols_in && r0 + 8 <= R) {
+        const float *base = x + r0 * C + c0;
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            t[u] = load4(base + (int64_t)u * C);
+    } else {
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            t[u] = (cols_in && r0 + u < R) ? load4(x + (r0 + u) * C + c0) : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    }
+    float rm[8], cm[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+        const float a0 = fabsf(t[u].x), a1 = fabsf(t[u].y), a2 = fabsf(t[u].z), a3 = fabsf(t[u].w);
+        rm[u] = fmaxf(fmaxf(a0, a1), fmaxf(a2, a3));
+        cm[0] = fmaxf(cm[0], a0);
+        cm[1] = fmaxf(cm[1], a1);
+        cm[2] = fmaxf(cm[2], a2);
+        cm[3] = fmaxf(cm[3], a3);
+    }
+    const float m = wave_max8(rm, lane);  // lane 8u: maximum of row r0 + u over the wave's 256 columns
+    if ((lane & 7) == 0 && r0 + (lane >> 3) < R)
+        atomic_max_nonneg(rowmax + r0 + (lane >> 3), m);
+    *reinterpret_cast<float4 *>(s_col + wave * kStat2Cols + lane * 4) = make_float4(cm[0], cm[1], cm[2], cm[3]);
+    __syncthreads();
+    const int64_t c = (int64_t)tx * kStat2Cols + threadIdx.x;
+    if (c < C) {
+        const float v = fmaxf(fmaxf(s_col[threadIdx.x], s_col[kStat2Cols + threadIdx.x]),
+                              fmaxf(s_col[2 * kStat2Cols + threadIdx.x], s_col[3 * kStat2Cols + threadIdx.x]));
+        atomic_max_nonneg(colmax + c, v);
+    }
+}
+
 // Normalise by min(rowmax[r], colmax[c]), search, pack.  Flattened indexing: a lane's 8
 // values may straddle rows (any C).
 __global__ __launch_bounds__(kQThreads) void quant_rank1_kernel(const float *__restrict__ x, int64_t n,
@@ -730,8 +784,13 @@ extern "C" int lpmm_rank1_stats(const float *x, int64_t rows, int64_t cols, floa
     hipLaunchKernelGGL(fill_zero_kernel, dim3((uint32_t)((mx + 255) / 256)), dim3(256), 0,
                        (hipStream_t)stream, rowmax, rows, colmax, cols);
     const bool vec = aligned_to(x, 16) && (cols % 4) == 0;
-    hipLaunchKernelGGL(rank1_stats_kernel, dim3((uint32_t)gx, (uint32_t)gy), dim3(kQThreads), 0,
-                       (hipStream_t)stream, x, rows, cols, rowmax, colmax, vec);
+    const int64_t tx = (cols + kStat2Cols - 1) / kStat2Cols, ty = (rows + kStat2Rows - 1) / kStat2Rows;
+    if (vec && tx * ty <= 0x7fffffffLL)
+        hipLaunchKernelGGL(rank1_stats_tile_kernel, dim3((uint32_t)(tx * ty)), dim3(kQThreads), 0, (hipStream_t)stream,
+                           x, rows, cols, (uint32_t)tx, rowmax, colmax);
+    else
+        hipLaunchKernelGGL(rank1_stats_kernel, dim3((uint32_t)gx, (uint32_t)gy), dim3(kQThreads), 0,
+                           (hipStream_t)stream, x, rows, cols, rowmax, colmax, vec);
     return launch_status();
 }
 
