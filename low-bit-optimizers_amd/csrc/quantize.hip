@@ -241,6 +241,11 @@ __global__ __launch_bounds__(kQThreads) void dequant_group_kernel(const uint8_t 
 // Row layout (as in the fused step): 16 lanes own one 128-value group, lane l owns values
 // [4l, 4l+4) and [64+4l, 64+4l+4), so that every 16-byte store of a row covers whole cache
 // lines.  Handles the groups that lie fully inside the tensor; n must be >= 128.
+#ifndef LPMM_DQ_LDS_KB
+#define LPMM_DQ_LDS_KB 0
+#endif
+// the map needs 16 words (32 allocated); more caps the workgroups resident per CU
+constexpr int kDequantLdsWords = LPMM_DQ_LDS_KB > 0 ? LPMM_DQ_LDS_KB * 256 : 32;
 template <int T>
 __global__ __launch_bounds__(kQThreads) void dequant_group_rows_kernel(const uint8_t *__restrict__ codes,
                                                                        const float *__restrict__ max1,
@@ -248,7 +253,7 @@ __global__ __launch_bounds__(kQThreads) void dequant_group_rows_kernel(const uin
                                                                        int64_t full_groups, int rows_per_group,
                                                                        float *__restrict__ out)
 {
-    __shared__ __align__(16) uint32_t lds[32];
+    __shared__ __align__(16) uint32_t lds[kDequantLdsWords];
     const int lane16 = threadIdx.x & 15;
     // T passes of 16 rows each; the loads of all passes first, the map afterwards
     const int64_t row0 = (int64_t)blockIdx.x * T * (kQThreads / 16) + (threadIdx.x >> 4);
@@ -446,12 +451,58 @@ __global__ __launch_bounds__(kQThreads) void quant_rank1_kernel(const float *__r
     store_u32(reinterpret_cast<uint32_t *>(codes + (base >> 1)), encode8_plain(lds, kLdsQ0, kind, xs));
 }
 
+// Codes of v[k] / min(cmx[k], rm) for a lane's 8 values of one row.  The column maxima stay the
+// same for every row a lane handles, so their correctly rounded reciprocals are formed once
+// (col_rcp); with the row's reciprocal that turns every division into one multiply and two fmas
+// that give the correctly rounded quotient (|v| <= scale by construction).  Scales outside the
+// range in which the reciprocal is exact, and maps other than the two standard ones, take the
+// plain division and the generic search.
+struct ColRcp {
+    float rc[kQElts];
+    bool safe;
+};
+
+__device__ __forceinline__ ColRcp col_rcp(const float (&cmx)[kQElts])
+{
+    ColRcp c;
+    c.safe = true;
+#pragma unroll
+    for (int k = 0; k < kQElts; ++k) {
+        c.rc[k] = rcp_exact(cmx[k]);
+        c.safe = c.safe && rc_safe(cmx[k]);
+    }
+    return c;
+}
+
+__device__ __forceinline__ uint32_t encode8_rank1(const uint32_t *lds, int kind, const float (&v)[kQElts],
+                                                  const float (&cmx)[kQElts], const ColRcp &cr, float rm)
+{
+    float xs[kQElts];
+    if (kind != kMapGeneric && __all(cr.safe && rc_safe(rm))) {
+        const float rr = rcp_exact(rm);
+#pragma unroll
+        for (int k = 0; k < kQElts; ++k) {
+            const bool by_col = cmx[k] < rm;
+            xs[k] = div_by_rc(v[k], by_col ? cmx[k] : rm, by_col ? cr.rc[k] : rr);
+        }
+        // the closed form of the second-moment code needs 0 <= x <= 1; values below 0 are legal here
+        return kind == kMapStdM ? encode8_std_m(lds, xs) : encode8_plain(lds, kLdsQ0, kind, xs);
+    }
+#pragma unroll
+    for (int k = 0; k < kQElts; ++k)
+        xs[k] = v[k] / ((cmx[k] < rm) ? cmx[k] : rm);
+    return encode8_plain(lds, kLdsQ0, kind, xs);
+}
+
 // The same when C is a multiple of 8: a lane's 8 values lie in one row, the grid is
 // (column chunks, rows) and no index division is needed.  Workgroup (0,0) also writes the
 // pad codes past the tensor.
 constexpr int kR1Cols = kQThreads * kQElts;  // columns per workgroup
 
-constexpr int kR1RowsPerWg = 4;  // rows of one column chunk per workgroup: the column maxima are loaded once
+#ifndef LPMM_R1_ROWS_PER_WG
+#define LPMM_R1_ROWS_PER_WG 4
+#endif
+constexpr int kR1RowsPerWg = LPMM_R1_ROWS_PER_WG;  // rows of one column chunk per workgroup: the column maxima are loaded once
 
 __global__ __launch_bounds__(kQThreads) void quant_rank1_rows_kernel(const float *__restrict__ x, int64_t R,
                                                                      int64_t C, const float *__restrict__ rowmax,
@@ -495,19 +546,73 @@ __global__ __launch_bounds__(kQThreads) void quant_rank1_rows_kernel(const float
     if (!live)
         return;
     const float cmx[kQElts] = {ca.x, ca.y, ca.z, ca.w, cb.x, cb.y, cb.z, cb.w};
+    const ColRcp cr = col_rcp(cmx);
 #pragma unroll
     for (int t = 0; t < T; ++t) {
         if (r0 + t >= R)
             break;
         const float v[kQElts] = {a[t].x, a[t].y, a[t].z, a[t].w, b[t].x, b[t].y, b[t].z, b[t].w};
-        float xs[kQElts];
-#pragma unroll
-        for (int k = 0; k < kQElts; ++k) {
-            const float st = (cmx[k] < rm[t]) ? cmx[k] : rm[t];
-            xs[k] = v[k] / st;
-        }
         store_u32(reinterpret_cast<uint32_t *>(codes + (((r0 + t) * C + c) >> 1)),
-                  encode8_plain(lds, kLdsQ0, kind, xs));
+                  encode8_rank1(lds, kind, v, cmx, cr, rm[t]));
+    }
+}
+
+// The same in the row layout of the fused step for column counts that are a multiple of 128:
+// 16 lanes own 128 consecutive columns of one row, lane l the columns [4l, 4l+4) and
+// [64+4l, 64+4l+4), so that every 16-byte load covers whole cache lines.
+__global__ __launch_bounds__(kQThreads) void quant_rank1_rows128_kernel(const float *__restrict__ x, int64_t R,
+                                                                        int64_t C, const float *__restrict__ rowmax,
+                                                                        const float *__restrict__ colmax,
+                                                                        const float *__restrict__ qmap,
+                                                                        uint8_t *__restrict__ codes, int64_t n_padded)
+{
+    constexpr int T = kR1RowsPerWg;
+    __shared__ __align__(16) uint32_t lds[kLdsBytes / 4];
+    const int64_t n = R * C;
+    const int lane16 = threadIdx.x & 15;
+    const int64_t r0 = (int64_t)blockIdx.y * T;
+    const int64_t c0 = (int64_t)blockIdx.x * kR1Cols + (int64_t)(threadIdx.x >> 4) * kGroup;
+    const bool live = c0 < C;  // uniform over the 16 lanes of a group
+    float4 a[T], b[T], ca, cb;
+    float rm[T];
+    if (live) {
+        const float *cmp = colmax + c0 + lane16 * 4;
+        ca = *reinterpret_cast<const float4 *>(cmp);
+        cb = *reinterpret_cast<const float4 *>(cmp + 64);
+#pragma unroll
+        for (int t = 0; t < T; ++t) {
+            if (r0 + t < R) {
+                const float *p = x + (r0 + t) * C + c0 + lane16 * 4;
+                a[t] = load4(p);
+                b[t] = load4(p + 64);
+                rm[t] = rowmax[r0 + t];
+            }
+        }
+    }
+    lds_fill(lds, qmap, nullptr);
+    const int kind = classify_map(qmap);
+    lds_barrier();
+    if (blockIdx.x == 0 && blockIdx.y == 0) {
+        const float z[kQElts] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+        const uint32_t wz = encode8_plain(lds, kLdsQ0, kind, z);
+        for (int64_t i = n + (int64_t)threadIdx.x * kQElts; i < n_padded; i += kR1Cols)
+            *reinterpret_cast<uint32_t *>(codes + (i >> 1)) = wz;
+        if (threadIdx.x == 0)
+            codes[n_padded / 2] = 0;
+    }
+    if (!live)
+        return;
+    const float cmx[kQElts] = {ca.x, ca.y, ca.z, ca.w, cb.x, cb.y, cb.z, cb.w};
+    const ColRcp cr = col_rcp(cmx);
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+        if (r0 + t >= R)
+            break;
+        const float v[kQElts] = {a[t].x, a[t].y, a[t].z, a[t].w, b[t].x, b[t].y, b[t].z, b[t].w};
+        const uint32_t w = encode8_rank1(lds, kind, v, cmx, cr, rm[t]);
+        uint16_t *cp = reinterpret_cast<uint16_t *>(codes + (((r0 + t) * C + c0) >> 1)) + lane16;
+        store_u16(cp, w & 0xFFFFu);
+        store_u16(cp + 16, w >> 16);
     }
 }
 
@@ -602,7 +707,7 @@ __global__ __launch_bounds__(kQThreads) void dequant_rank1_rows128_kernel(const 
                                                                           int64_t C, float *__restrict__ out)
 {
     constexpr int T = kR1RowsPerWg;
-    __shared__ __align__(16) uint32_t lds[32];
+    __shared__ __align__(16) uint32_t lds[kDequantLdsWords];
     const int lane16 = threadIdx.x & 15;
     const int64_t r0 = (int64_t)blockIdx.y * T;
     const int64_t c0 = (int64_t)blockIdx.x * kR1Cols + (int64_t)(threadIdx.x >> 4) * kGroup;
@@ -720,7 +825,10 @@ extern "C" int lpmm_quant_group(const float *x, int64_t n, int64_t gp_sz, const 
     if (!tiles_ok(n_groups * gp_sz, kQTile, &tiles))
         return LPMM_ERR_SIZE;
     const int64_t n_padded = (int64_t)tiles * kQTile;
-    constexpr int kT = 4;  // tiles per workgroup
+#ifndef LPMM_QG_T
+#define LPMM_QG_T 2
+#endif
+    constexpr int kT = LPMM_QG_T;  // tiles per workgroup
     if (gp_sz > kQTile)
         hipLaunchKernelGGL((quant_group_kernel<2 * kQThreads, 1>), dim3((tiles + 1) / 2), dim3(2 * kQThreads), 0,
                            (hipStream_t)stream, x, n, (int)(gp_sz / kGroup), qmap, codes, max1, n_groups, n_padded,
@@ -751,7 +859,10 @@ extern "C" int lpmm_dequant_group(const uint8_t *codes, const float *max1, const
     const int64_t full_groups = n / kGroup;
     if (vec && full_groups > 0 && full_groups <= 0x7fffffffLL * 16) {
         // whole 128-value rows in the row layout, the ragged tail (< 128 values) element-wise
-        constexpr int kT = 4;  // passes of 16 rows per workgroup
+#ifndef LPMM_DQ_T
+#define LPMM_DQ_T 2
+#endif
+        constexpr int kT = LPMM_DQ_T;  // passes of 16 rows per workgroup
         hipLaunchKernelGGL(dequant_group_rows_kernel<kT>, dim3((uint32_t)((full_groups + 16 * kT - 1) / (16 * kT))),
                            dim3(kQThreads), 0, (hipStream_t)stream, codes, max1, qmap, full_groups,
                            (int)(gp_sz / kGroup), out);
@@ -823,8 +934,12 @@ extern "C" int lpmm_quant_rank1(const float *x, int64_t rows, int64_t cols, cons
     if (rank1_rows_ok(x, colmax, codes, rows, cols)) {
         const uint32_t gx = (uint32_t)((cols + kR1Cols - 1) / kR1Cols);
         const uint32_t gy = (uint32_t)((rows + kR1RowsPerWg - 1) / kR1RowsPerWg);
-        hipLaunchKernelGGL(quant_rank1_rows_kernel, dim3(gx, gy), dim3(kQThreads), 0,
-                           (hipStream_t)stream, x, rows, cols, rowmax, colmax, qmap, codes, n_padded);
+        if ((cols % kGroup) == 0)
+            hipLaunchKernelGGL(quant_rank1_rows128_kernel, dim3(gx, gy), dim3(kQThreads), 0,
+                               (hipStream_t)stream, x, rows, cols, rowmax, colmax, qmap, codes, n_padded);
+        else
+            hipLaunchKernelGGL(quant_rank1_rows_kernel, dim3(gx, gy), dim3(kQThreads), 0,
+                               (hipStream_t)stream, x, rows, cols, rowmax, colmax, qmap, codes, n_padded);
     } else {
         hipLaunchKernelGGL(quant_rank1_kernel, dim3(tiles), dim3(kQThreads), 0, (hipStream_t)stream, x, n, cols,
                            rowmax, colmax, qmap, codes, n_padded, aligned_to(x, 16));

@@ -28,27 +28,44 @@ __device__ __forceinline__ void fill_map(float *lds_map, const float *__restrict
         lds_map[j] = qmap[j];
 }
 
-// quantize_bsearch<false> (quantization_kernel.cu:397-427) as the stored code: the reference
-// casts the int to uint8_t (one code per byte) or masks it (packed), so NaN (-1) becomes 255
-// or the all-ones code.
+// quantize_bsearch<false> (quantization_kernel.cu:397-427) as the stored code, without a data
+// dependent branch.  The reference returns 0 for x <= q[0] and N-1 for q[N-1] <= x; otherwise it
+// finds lo = the first entry above x (upper bound) and answers lo or lo-1 by the midpoint test
+// mid = (q[lo-1] + q[lo]) * 0.5f < x.  Here the upper bound of the non-decreasing map (repeated
+// entries included) is built from its bits, one compare per step, every lane the same `bits`
+// steps; the two ends and NaN are selects afterwards.  For NaN the reference's search ends at
+// lo = 0 and returns -1, which it casts to uint8_t (one code per byte: 255) or masks (packed:
+// the all-ones code).
 __device__ __forceinline__ uint32_t search_code(const float *lds_map, int bits, float x)
 {
-    int lo = 0, hi = 1 << bits;
-    if (x <= lds_map[0])
-        return 0u;
-    if (lds_map[hi - 1] <= x)
-        return (uint32_t)(hi - 1);
-    while (lo < hi) {
-        const int mi = (lo + hi) >> 1;
-        if (lds_map[mi] <= x)
-            lo = mi + 1;
-        else
-            hi = mi;
+    const uint32_t n = 1u << bits;
+    // pos = number of entries among the first n-1 that are <= x: all entries before pos are <= x.
+    // The first three levels of the search look at the same seven entries in every lane (every
+    // eighth of the map): those compares run on registers (the entries are read once per kernel:
+    // the loads below do not depend on x and are hoisted), only the levels below them go to LDS
+    // with a per-lane address.
+    uint32_t pos = 0;
+    uint32_t step = n >> 1;
+    if (bits >= 3) {
+        const uint32_t eighth = n >> 3;
+        uint32_t cnt = 0;
+#pragma unroll
+        for (uint32_t j = 1; j < 8; ++j)
+            cnt += (lds_map[j * eighth - 1] <= x) ? 1u : 0u;
+        pos = cnt * eighth;
+        step = eighth >> 1;
     }
-    if (lo == 0)  // only NaN gets here; the reference's read of qmap[-1] does not change its result
-        return codes_per_byte(bits) == 1 ? 255u : (1u << bits) - 1u;
-    const float mid = (lds_map[lo - 1] + lds_map[lo]) * 0.5f;
-    return (uint32_t)((mid < x) ? lo : lo - 1);
+    for (; step > 0; step >>= 1)
+        pos += (lds_map[pos + step - 1] <= x) ? step : 0u;
+    // pos <= n-1.  Inside the map's range the upper bound is pos (q[n-1] > x there), at least 1
+    const uint32_t lo = pos > 0 ? pos : 1u;
+    const float below = lds_map[lo - 1], above = lds_map[lo];
+    const float mid = (below + above) * 0.5f;
+    uint32_t code = (mid < x) ? lo : lo - 1u;
+    code = (lds_map[n - 1] <= x) ? n - 1u : code;
+    code = (x <= lds_map[0]) ? 0u : code;
+    const uint32_t nan_code = codes_per_byte(bits) == 1 ? 255u : n - 1u;
+    return (x != x) ? nan_code : code;
 }
 
 // codes of the lane's 8 values (base = index of the first, a multiple of 8) into the array
@@ -315,9 +332,23 @@ __global__ __launch_bounds__(THREADS) void quant_group_bits_kernel(const float *
     if (grp < n_groups) {
         if ((base % gp_sz) == 0)
             max1[grp] = amax;
+        // |v| <= amax: with the correctly rounded reciprocal one multiply and two fmas give the
+        // correctly rounded quotient; group maxima outside the reciprocal's exact range (0 included:
+        // 0/0 must give NaN) take the plain division
+        float xs[kBElts];
+        if (__all(rc_safe(amax))) {
+            const float rc = rcp_exact(amax);
+#pragma unroll
+            for (int k = 0; k < kBElts; ++k)
+                xs[k] = div_by_rc(v[k], amax, rc);
+        } else {
+#pragma unroll
+            for (int k = 0; k < kBElts; ++k)
+                xs[k] = v[k] / amax;
+        }
 #pragma unroll
         for (int k = 0; k < kBElts; ++k)
-            c[k] = search_code(lds_map, bits, v[k] / amax);
+            c[k] = search_code(lds_map, bits, xs[k]);
     } else {
         // padding added by the re-grouping to 2048: plain zeros, not divided by anything
         const uint32_t z = search_code(lds_map, bits, 0.0f);
