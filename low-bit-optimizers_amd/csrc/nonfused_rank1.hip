@@ -135,26 +135,43 @@ __global__ __launch_bounds__(kThreads) void rank1_clear_kernel(const MultiR1 arg
     }
 }
 
-#ifndef LPMM_R1_PREFETCH
-#define LPMM_R1_PREFETCH 0
-#endif
+// operands of one pass of a DPP row, as loaded
+struct PassRegs {
+    float4 a0, a1, b0, b1;
+    uint32_t m0, m1, v0, v1;
+    float sm, ro;
+};
+
+__device__ __forceinline__ void pass_fetch(const TensorR1 &t, uint32_t cg, int lane16, int64_t r, PassRegs &x)
+{
+    const int64_t grp = r * t.col_blocks + cg;
+    const int64_t gbase = grp * kGroup;
+    const float *pp = t.p + gbase + lane16 * 4;
+    const float *gp = t.g + gbase + lane16 * 4;
+    x.a0 = load4(pp);
+    x.a1 = load4(pp + 64);
+    x.b0 = load4(gp);
+    x.b1 = load4(gp + 64);
+    const uint16_t *mcp = reinterpret_cast<const uint16_t *>(t.mc + (gbase >> 1)) + lane16;
+    const uint16_t *vcp = reinterpret_cast<const uint16_t *>(t.vc + (gbase >> 1)) + lane16;
+    x.m0 = load_u16(mcp);
+    x.m1 = load_u16(mcp + 16);
+    x.v0 = load_u16(vcp);
+    x.v1 = load_u16(vcp + 16);
+    x.sm = t.ms[grp];
+    x.ro = t.row_old[r];
+}
+
 #ifndef LPMM_R1_WAVES
-#define LPMM_R1_WAVES 6
+#define LPMM_R1_WAVES 4
 #endif
-// 6 waves per SIMD: at most 80 registers
+// 4 waves per SIMD, up to 128 registers: the first pass's operands stay live across the prologue and
+// the lane's column statistics across the passes (with 5 or 6 the compiler spills or re-reads)
 __global__ __launch_bounds__(kThreads, LPMM_R1_WAVES) void rank1_update_kernel(const MultiR1 args, const float *__restrict__ qmap_m,
                                                                 const float *__restrict__ qmap_v)
 {
-#ifndef LPMM_R1_LDS_KB
-#define LPMM_R1_LDS_KB 0
-#endif
-    constexpr uint32_t kNeed = kColExtra + kMaxWide * kRedSlotWords * 4;
-    __shared__ __align__(16) uint32_t lds[(LPMM_R1_LDS_KB * 1024 > kNeed ? LPMM_R1_LDS_KB * 1024 : kNeed) / 4];
+    __shared__ __align__(16) uint32_t lds[(kColExtra + kMaxWide * kRedSlotWords * 4) / 4];
     uint32_t *colred = lds + kColExtra / 4;
-    lds_fill(lds, qmap_m, qmap_v);
-    for (int j = threadIdx.x; j < kMaxWide * (int)kRedSlotWords; j += kThreads)
-        colred[j] = 0u;
-    const int kind_m = classify_map(qmap_m);
     const int lo = find_tensor(args);
     const TensorR1 &t = args.t[lo];
     const uint32_t tl = blockIdx.x - args.tile_start[lo];
@@ -162,8 +179,30 @@ __global__ __launch_bounds__(kThreads, LPMM_R1_WAVES) void rank1_update_kernel(c
     const Geometry q = geometry(t, tl, drow);
     const int64_t cols = (int64_t)t.col_blocks * kGroup;
     const int64_t tile_c0 = (int64_t)q.col_tile * q.wide * kGroup;
-    for (int j = threadIdx.x; j < q.wide * kGroup; j += kThreads)
-        lds[kColOld / 4 + j] = (tile_c0 + j < cols) ? __float_as_uint(t.col_old[tile_c0 + j]) : 0u;
+
+    // Order of the prologue: the small loads that feed LDS (maps, encode table, the tile's current
+    // column statistics), then the streaming loads of the first pass, then the LDS writes (the
+    // small loads were issued first and return first) and a barrier that orders LDS only -- the
+    // first pass's operands are on their way while the tables are set up.
+    const LdsFill fill = lds_fill_load(qmap_m, qmap_v);
+    constexpr int kColPerThread = kMaxWide * kGroup / kThreads;
+    uint32_t co_in[kColPerThread];
+#pragma unroll
+    for (int i = 0; i < kColPerThread; ++i) {
+        const int j = threadIdx.x + i * kThreads;
+        co_in[i] = (j < q.wide * kGroup && tile_c0 + j < cols) ? __float_as_uint(t.col_old[tile_c0 + j]) : 0u;
+    }
+    const bool row_live = q.cg < t.col_blocks;  // the whole DPP row
+    PassRegs x;
+    if (row_live && q.row0 < t.rows)
+        pass_fetch(t, q.cg, lane16, q.row0, x);
+    lds_fill_store(lds, fill);
+    for (int j = threadIdx.x; j < kMaxWide * (int)kRedSlotWords; j += kThreads)
+        colred[j] = 0u;
+#pragma unroll
+    for (int i = 0; i < kColPerThread; ++i)
+        lds[kColOld / 4 + threadIdx.x + i * kThreads] = co_in[i];
+    const int kind_m = classify_map(qmap_m);
     NfHyper h;
     h.decay = args.decay;
     h.w1 = args.w1;
@@ -173,7 +212,7 @@ __global__ __launch_bounds__(kThreads, LPMM_R1_WAVES) void rank1_update_kernel(c
     h.neg_step_size = t.neg_step_size;
     h.bc2_sqrt = t.bc2_sqrt;
     h.rbc2_sqrt = t.rbc2_sqrt;
-    __syncthreads();
+    lds_barrier();
 
     if (tl == 0) {
         const float z[kEltsPerLane] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
@@ -183,34 +222,19 @@ __global__ __launch_bounds__(kThreads, LPMM_R1_WAVES) void rank1_update_kernel(c
     }
 
     const int slot = drow & (q.wide - 1);
-    if (q.cg < t.col_blocks) {  // the whole DPP row
+    if (row_live) {
         const uint32_t co_off = kColOld + (slot * kGroup + lane16 * 4) * 4;
         uint32_t *red = colred + slot * kRedSlotWords + lane16;
-        // operands of one pass, as loaded
-        struct PassRegs {
-            float4 a0, a1, b0, b1;
-            uint32_t m0, m1, v0, v1;
-            float sm, ro;
-        };
-        auto fetch = [&](int64_t r, PassRegs &x) {
-            const int64_t grp = r * t.col_blocks + q.cg;
-            const int64_t gbase = grp * kGroup;
-            const float *pp = t.p + gbase + lane16 * 4;
-            const float *gp = t.g + gbase + lane16 * 4;
-            x.a0 = load4(pp);
-            x.a1 = load4(pp + 64);
-            x.b0 = load4(gp);
-            x.b1 = load4(gp + 64);
-            const uint16_t *mcp = reinterpret_cast<const uint16_t *>(t.mc + (gbase >> 1)) + lane16;
-            const uint16_t *vcp = reinterpret_cast<const uint16_t *>(t.vc + (gbase >> 1)) + lane16;
-            x.m0 = load_u16(mcp);
-            x.m1 = load_u16(mcp + 16);
-            x.v0 = load_u16(vcp);
-            x.v1 = load_u16(vcp + 16);
-            x.sm = t.ms[grp];
-            x.ro = t.row_old[r];
-        };
-        auto work = [&](int64_t r, const PassRegs &x) {
+        // a lane keeps its eight columns through all passes: their statistics come out of LDS once
+        float co[kEltsPerLane];
+        unpack8(lds_read<float4>(lds, co_off), lds_read<float4>(lds, co_off + 256), co);
+#pragma unroll 1
+        for (int it = 0; it < q.passes; ++it) {
+            const int64_t r = q.row0 + it * q.step;
+            if (r >= t.rows)
+                break;
+            if (it > 0)
+                pass_fetch(t, q.cg, lane16, r, x);
             const int64_t grp = r * t.col_blocks + q.cg;
             const int64_t gbase = grp * kGroup;
             float *pp = t.p + gbase + lane16 * 4;
@@ -218,10 +242,9 @@ __global__ __launch_bounds__(kThreads, LPMM_R1_WAVES) void rank1_update_kernel(c
             const uint32_t wm = x.m0 | (x.m1 << 16);
             const uint32_t wv = x.v0 | (x.v1 << 16);
             const float sm = x.sm, ro = x.ro;
-            float pv[kEltsPerLane], gv[kEltsPerLane], m[kEltsPerLane], v[kEltsPerLane], co[kEltsPerLane];
+            float pv[kEltsPerLane], gv[kEltsPerLane], m[kEltsPerLane], v[kEltsPerLane];
             unpack8(x.a0, x.a1, pv);
             unpack8(x.b0, x.b1, gv);
-            unpack8(lds_read<float4>(lds, co_off), lds_read<float4>(lds, co_off + 256), co);
 
             const Nibbles nm = split_nibbles(wm), nv = split_nibbles(wv);
             float amax_m = 0.0f, vmax = 0.0f;
@@ -245,46 +268,15 @@ __global__ __launch_bounds__(kThreads, LPMM_R1_WAVES) void rank1_update_kernel(c
                 t.ms[grp] = amax_m;
                 atomic_max_nonneg(t.row_new + r, vmax);
             }
-        };
-#if LPMM_R1_PREFETCH
-        // two passes per iteration: the loads of the second are in flight while the first computes,
-        // and those of the next iteration's first while the second computes
-        PassRegs xa, xb;
-        const int64_t last = t.rows - 1;
-        fetch(q.row0 < t.rows ? q.row0 : last, xa);
-#pragma unroll 1
-        for (int it = 0; it < q.passes; it += 2) {
-            const int64_t r0 = q.row0 + it * q.step, r1 = r0 + q.step, r2 = r1 + q.step;
-            if (r0 >= t.rows)
-                break;
-            fetch(r1 < t.rows ? r1 : last, xb);  // unconditional: a row past the end re-reads the last one
-            work(r0, xa);
-            if (it + 1 >= q.passes || r1 >= t.rows)
-                break;
-            fetch(r2 < t.rows ? r2 : last, xa);
-            work(r1, xb);
         }
-#else
-#pragma unroll 1
-        for (int it = 0; it < q.passes; ++it) {
-            const int64_t r = q.row0 + it * q.step;
-            if (r >= t.rows)
-                break;
-            PassRegs x;
-            fetch(r, x);
-            work(r, x);
-        }
-#endif
     }
     __syncthreads();
     // column j of the tile = element k of lane l of slot s
     for (int j = threadIdx.x; j < q.wide * kGroup; j += kThreads) {
         const int w = j & (kGroup - 1);
         const int k = ((w >> 6) << 2) | (w & 3), l = (w >> 2) & 15;
-        if (tile_c0 + j < cols) {
-            const float mine = __uint_as_float(colred[(j >> 7) * kRedSlotWords + k * 16 + l]);
-            atomic_max_nonneg(t.col_new + tile_c0 + j, mine);
-        }
+        if (tile_c0 + j < cols)
+            atomic_max_nonneg(t.col_new + tile_c0 + j, __uint_as_float(colred[(j >> 7) * kRedSlotWords + k * 16 + l]));
     }
 }
 
@@ -322,7 +314,17 @@ __global__ __launch_bounds__(kThreads) void rank1_requant_kernel(const MultiR1 a
     if (q.cg >= t.col_blocks)
         return;
 
+    // a lane keeps its eight columns through all passes: their old and new statistics and the
+    // reciprocals of the new ones come out of LDS once
     const uint32_t col_off = ((drow & (q.wide - 1)) * kGroup + lane16 * 4) * 4;
+    float co[kEltsPerLane], cn[kEltsPerLane], rcn[kEltsPerLane];
+    unpack8(lds_read<float4>(lds, kColOld + col_off), lds_read<float4>(lds, kColOld + col_off + 256), co);
+    unpack8(lds_read<float4>(lds, kColNew + col_off), lds_read<float4>(lds, kColNew + col_off + 256), cn);
+    unpack8(lds_read<float4>(lds, kColRcp + col_off), lds_read<float4>(lds, kColRcp + col_off + 256), rcn);
+    bool cols_safe = true;
+#pragma unroll
+    for (int k = 0; k < kEltsPerLane; ++k)
+        cols_safe = cols_safe && rc_safe(cn[k]);
 #pragma unroll 1
     for (int it = 0; it < q.passes; ++it) {
         const int64_t r = q.row0 + it * q.step;
@@ -334,34 +336,31 @@ __global__ __launch_bounds__(kThreads) void rank1_requant_kernel(const MultiR1 a
         uint16_t *vcp = reinterpret_cast<uint16_t *>(t.vc + (gbase >> 1)) + lane16;
         const uint32_t wv = load_u16(vcp) | (load_u16(vcp + 16) << 16);
         const float ro = t.row_old[r], rn = t.row_new[r];
-        float gv[kEltsPerLane], v[kEltsPerLane], s[kEltsPerLane], x[kEltsPerLane], co[kEltsPerLane], cn[kEltsPerLane];
+        float gv[kEltsPerLane], v[kEltsPerLane], x[kEltsPerLane];
         unpack8(b0, b1, gv);
-        unpack8(lds_read<float4>(lds, kColOld + col_off), lds_read<float4>(lds, kColOld + col_off + 256), co);
-        unpack8(lds_read<float4>(lds, kColNew + col_off), lds_read<float4>(lds, kColNew + col_off + 256), cn);
         const Nibbles nv = split_nibbles(wv);
-        bool safe = true;
 #pragma unroll
         for (int k = 0; k < kEltsPerLane; ++k) {
             v[k] = decode_nibble(lds, kLdsQ0, nv, k) * ((co[k] < ro) ? co[k] : ro);
             nonfused_second_moment(v[k], gv[k], h);
-            s[k] = (cn[k] < rn) ? cn[k] : rn;
-            safe = safe && rc_safe(s[k]);
         }
         uint32_t w;
-        if (kind == kMapStdV && __all(safe)) {
+        // every scale the wave divides by is a column or the row statistic: all in the range in
+        // which the reciprocal is exact?
+        if (kind == kMapStdV && __all(cols_safe && rc_safe(rn))) {
             // the correctly rounded reciprocal of whichever statistic is the scale, then one
             // multiply and two fmas: the correctly rounded quotient (v <= scale by construction)
-            const float rcr = rcp_exact(rn);  // used only where rn is the scale and in range
-            float rcn[kEltsPerLane];
-            unpack8(lds_read<float4>(lds, kColRcp + col_off), lds_read<float4>(lds, kColRcp + col_off + 256), rcn);
+            const float rcr = rcp_exact(rn);
 #pragma unroll
-            for (int k = 0; k < kEltsPerLane; ++k)
-                x[k] = div_by_rc(v[k], s[k], (cn[k] < rn) ? rcn[k] : rcr);
+            for (int k = 0; k < kEltsPerLane; ++k) {
+                const bool by_col = cn[k] < rn;
+                x[k] = div_by_rc(v[k], by_col ? cn[k] : rn, by_col ? rcn[k] : rcr);
+            }
             w = encode8_std_v(x);
         } else {
 #pragma unroll
             for (int k = 0; k < kEltsPerLane; ++k)
-                x[k] = v[k] / s[k];
+                x[k] = v[k] / ((cn[k] < rn) ? cn[k] : rn);
             w = encode8_plain(lds, kLdsQ0, kind, x);
         }
         store_u16(vcp, w & 0xFFFFu);
@@ -377,9 +376,6 @@ using namespace lpmm;
 // tensor's tiles without a column group; otherwise the width that wastes least.
 static uint32_t choose_lg_wide(uint32_t col_blocks)
 {
-#ifdef LPMM_R1_FORCE_LG
-    return LPMM_R1_FORCE_LG;
-#endif
     uint32_t best = 0;
     double best_use = 0.0;
     for (int lg = kMaxLgWide; lg >= 0; --lg) {
