@@ -106,6 +106,16 @@ int lpmm_adamw_fp32_step_multi(const lpmm_adamw_fp32_tensor *tensors, int64_t co
                                float beta1, float beta2, float lr, float weight_decay,
                                float eps, void *stream);
 
+/* The same step for IEEE half-precision tensors: the p, g, m and v of every record point to
+ * fp16[n] (2-byte aligned); all arithmetic is float.  Replaces fused_adamw.adamw_single_tensor
+ * for at::Half tensors (the kernel template instantiated by AT_DISPATCH_FLOATING_TYPES_AND_HALF,
+ * lpmm/cpp_extension/fused_adamw_kernel.cu:52-78, :188): every element read converts to float,
+ * every write rounds to half, and the parameter update reads the moments back after their
+ * rounding.  (The 4-bit operator cannot run half tensors in the reference either: its float32
+ * scales are read through the parameters' type, :229-230.) */
+int lpmm_adamw_fp16_step_multi(const lpmm_adamw_fp32_tensor *tensors, int64_t count, float beta1,
+                               float beta2, float lr, float weight_decay, float eps, void *stream);
+
 /* ---------------------------------------------------------------------------------------
  * (b) Stand-alone quantise / dequantise in the non-fused packed layout
  *     (NG*1024 + 1 bytes, NG = ceil(numel_scaled/2048); lpmm/functional.py:359-369,

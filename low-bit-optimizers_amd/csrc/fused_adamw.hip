@@ -20,6 +20,7 @@
 // any other map.
 #include "lpmm_update.hpp"
 
+#include <hip/hip_fp16.h>
 #include <math.h>
 
 namespace lpmm {
@@ -426,6 +427,43 @@ __global__ __launch_bounds__(kThreads) void adamw_fp32_kernel(const MultiF args)
     }
 }
 
+// The fp32-state step on half-precision tensors: p, g, m and v are stored as IEEE half, every
+// operation runs in float.  The reference's kernel is instantiated for at::Half by its dispatch
+// macro (fused_adamw_kernel.cu:52-78, :188); there every read of a tensor element converts it to
+// float and every write rounds the float result to half, so the parameter update sees the moments
+// *after* their rounding to half (it reads exp_avg and exp_avg_sq back from memory).
+__global__ __launch_bounds__(kThreads) void adamw_fp16_kernel(const MultiF args)
+{
+    int lo = 0, hi = args.count;
+    while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (args.tile_start[mid] <= blockIdx.x)
+            lo = mid;
+        else
+            hi = mid;
+    }
+    const TensorF &t = args.t[lo];
+    const FusedArith a(args, t);
+    const Hyper &h = a.h;
+    __half *p = reinterpret_cast<__half *>(t.p), *m = reinterpret_cast<__half *>(t.m), *v = reinterpret_cast<__half *>(t.v);
+    const __half *g = reinterpret_cast<const __half *>(t.g);
+    const int64_t tile0 = (int64_t)(blockIdx.x - args.tile_start[lo]) * kTileF;
+#pragma unroll
+    for (int k = 0; k < kTileF / kThreads; ++k) {
+        const int64_t i = tile0 + k * kThreads + threadIdx.x;
+        if (i < t.n) {
+            const float gf = __half2float(g[i]), pf = __half2float(p[i]);
+            const __half mh = __float2half_rn(h.beta1 * __half2float(m[i]) + h.omb1 * gf);
+            const __half vh = __float2half_rn(h.beta2 * __half2float(v[i]) + h.omb2 * gf * gf);
+            m[i] = mh;
+            v[i] = vh;
+            const float denom = (div_by_rc(sqrt_fast(__half2float(vh)), h.c2s, h.rc2s) + h.eps) * h.c1;
+            const float update = div_fast(__half2float(mh), denom) + (h.wd * pf);
+            p[i] = __float2half_rn(pf - (h.lr * update));
+        }
+    }
+}
+
 }  // namespace lpmm
 
 using namespace lpmm;
@@ -575,10 +613,11 @@ extern "C" int lpmm_adamw4bit_step(float *p, const float *g, uint8_t *m_codes, u
     return lpmm_adamw4bit_step_multi(&t, 1, qmap_m, qmap_v, beta1, beta2, lr, weight_decay, eps, stream);
 }
 
-template <class Arith, class PerTensor>
+template <class Arith, bool HALF = false, class PerTensor>
 static int step_multi_fp32(const lpmm_adamw_fp32_tensor *tensors, int64_t count, const float (&scalars)[7],
                            PerTensor per_tensor, void *stream)
 {
+    constexpr uintptr_t kEltAlign = HALF ? 2 : 4;
     if (count < 0)
         return LPMM_ERR_SIZE;
     if (count == 0)
@@ -594,10 +633,10 @@ static int step_multi_fp32(const lpmm_adamw_fp32_tensor *tensors, int64_t count,
         LPMM_REQUIRE_PTR(t.g);
         LPMM_REQUIRE_PTR(t.m);
         LPMM_REQUIRE_PTR(t.v);
-        LPMM_REQUIRE_ALIGN(t.p, 4);
-        LPMM_REQUIRE_ALIGN(t.g, 4);
-        LPMM_REQUIRE_ALIGN(t.m, 4);
-        LPMM_REQUIRE_ALIGN(t.v, 4);
+        LPMM_REQUIRE_ALIGN(t.p, kEltAlign);
+        LPMM_REQUIRE_ALIGN(t.g, kEltAlign);
+        LPMM_REQUIRE_ALIGN(t.m, kEltAlign);
+        LPMM_REQUIRE_ALIGN(t.v, kEltAlign);
     }
     MultiF args;
     for (int j = 0; j < 7; ++j)
@@ -633,8 +672,11 @@ static int step_multi_fp32(const lpmm_adamw_fp32_tensor *tensors, int64_t count,
         args.count = k;
         for (int j = k + 1; j <= kMultiFMax; ++j)
             args.tile_start[j] = (uint32_t)tiles;
-        hipLaunchKernelGGL(adamw_fp32_kernel<Arith>, dim3((uint32_t)tiles), dim3(kThreads), 0,
-                           (hipStream_t)stream, args);
+        if (HALF)
+            hipLaunchKernelGGL(adamw_fp16_kernel, dim3((uint32_t)tiles), dim3(kThreads), 0, (hipStream_t)stream, args);
+        else
+            hipLaunchKernelGGL(adamw_fp32_kernel<Arith>, dim3((uint32_t)tiles), dim3(kThreads), 0,
+                               (hipStream_t)stream, args);
         const int st = launch_status();
         if (st != LPMM_OK)
             return st;
@@ -653,6 +695,18 @@ extern "C" int lpmm_adamw_fp32_step_multi(const lpmm_adamw_fp32_tensor *tensors,
                                            *rc2s = 1.0f / *c2s;
                                        },
                                        stream);
+}
+
+extern "C" int lpmm_adamw_fp16_step_multi(const lpmm_adamw_fp32_tensor *tensors, int64_t count, float beta1,
+                                          float beta2, float lr, float weight_decay, float eps, void *stream)
+{
+    const float scalars[7] = {beta1, beta2, 1 - beta1, 1 - beta2, lr, weight_decay, eps};
+    return step_multi_fp32<FusedArith, true>(tensors, count, scalars,
+                                             [=](float step, float *c1, float *c2s, float *rc2s) {
+                                                 bias_corrections(beta1, beta2, step, c1, c2s);
+                                                 *rc2s = 1.0f / *c2s;
+                                             },
+                                             stream);
 }
 
 extern "C" int lpmm_nonfused_update_multi(const lpmm_adamw_fp32_tensor *tensors, int64_t count, double beta1,

@@ -27,6 +27,7 @@ PROTOTYPES = {
     "lpmm_adamw4bit_step_multi": (_int, [_vp, _i64, _vp, _vp] + [_f] * 5 + [_vp]),
     "lpmm_adamw_fp32_step": (_int, [_vp] * 4 + [_i64] + [_f] * 6 + [_vp]),
     "lpmm_adamw_fp32_step_multi": (_int, [_vp, _i64] + [_f] * 5 + [_vp]),
+    "lpmm_adamw_fp16_step_multi": (_int, [_vp, _i64] + [_f] * 5 + [_vp]),
     "lpmm_pack_nonlinear_4bit": (_int, [_vp, _vp, _i64, _vp, _vp]),
     "lpmm_unpack_nonlinear_4bit": (_int, [_vp, _vp, _i64, _vp, _vp]),
     "lpmm_quant_group": (_int, [_vp, _i64, _i64, _vp, _vp, _vp, _vp]),

@@ -12,7 +12,9 @@ def check_cuda_tensor_float(t, name, *, fp32_only=True):
     if t.dtype not in (torch.float32, torch.float16):
         raise RuntimeError(f"The type of {name} is not kFloat32 or kFloat16!")
     if fp32_only and t.dtype != torch.float32:
-        raise RuntimeError(f"The type of {name} is kFloat16: this build implements the fp32 path only")
+        raise RuntimeError(f"The type of {name} is kFloat16: this operator is implemented for float32 only "
+                           "(half tensors are accepted by adamw_single_tensor alone, the one operator "
+                           "the reference can run them through)")
 
 
 def check_cuda_tensor_dim_float(t, name, n_dim):

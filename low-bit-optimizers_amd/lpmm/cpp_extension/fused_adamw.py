@@ -2,6 +2,7 @@
 module (lpmm/cpp_extension/fused_adamw.cc:82-83), same positional signatures, in-place on the
 caller's tensors, returning None.  Work is enqueued on torch's current stream of the
 tensors' device."""
+import numpy as np
 import torch
 
 from .. import _native
@@ -11,11 +12,13 @@ __all__ = ["adamw_single_tensor", "adamw4bit_single_tensor"]
 
 
 def adamw_single_tensor(p, g, exp_avg, exp_avg_sq, beta1, beta2, lr, weight_decay, eps, step):
-    """fp32-state fused AdamW step (lpmm/cpp_extension/fused_adamw.cc:15-41)."""
-    check_cuda_tensor_float(p, "p")
-    check_cuda_tensor_float(exp_avg, "exp_avg")
-    check_cuda_tensor_float(exp_avg_sq, "exp_avg_sq")
-    check_cuda_tensor_float(g, "g")
+    """Fused AdamW step on states of the parameters' type (lpmm/cpp_extension/fused_adamw.cc:15-41):
+    float32, or float16 as the reference's dispatch also instantiates
+    (lpmm/cpp_extension/fused_adamw_kernel.cu:188); all four tensors must have the same type."""
+    for t, name in ((p, "p"), (exp_avg, "exp_avg"), (exp_avg_sq, "exp_avg_sq"), (g, "g")):
+        check_cuda_tensor_float(t, name, fp32_only=False)
+        if t.dtype != p.dtype:
+            raise RuntimeError(f"expected scalar type {p.dtype} but found {t.dtype} for {name}")
     n = p.numel()
     if exp_avg.numel() != n:
         raise RuntimeError("number of elements in exp_avg and p tensors should be equal")
@@ -25,9 +28,15 @@ def adamw_single_tensor(p, g, exp_avg, exp_avg_sq, beta1, beta2, lr, weight_deca
         raise RuntimeError("number of elements in g and p tensors should be equal")
     dev = same_device(p, g, exp_avg, exp_avg_sq)
     with torch.cuda.device(dev):
-        st = _native.lib().lpmm_adamw_fp32_step(
-            p.data_ptr(), g.data_ptr(), exp_avg.data_ptr(), exp_avg_sq.data_ptr(), n,
-            beta1, beta2, lr, weight_decay, eps, step, _native.current_stream(dev))
+        if p.dtype is torch.float16:
+            table = np.array([(p.data_ptr(), g.data_ptr(), exp_avg.data_ptr(), exp_avg_sq.data_ptr(), n, step, 0.0)],
+                             dtype=_native.ADAMW_FP32_TENSOR)
+            st = _native.lib().lpmm_adamw_fp16_step_multi(table.ctypes.data, 1, beta1, beta2, lr, weight_decay, eps,
+                                                          _native.current_stream(dev))
+        else:
+            st = _native.lib().lpmm_adamw_fp32_step(
+                p.data_ptr(), g.data_ptr(), exp_avg.data_ptr(), exp_avg_sq.data_ptr(), n,
+                beta1, beta2, lr, weight_decay, eps, step, _native.current_stream(dev))
     _native.check(st, "adamw_single_tensor")
 
 

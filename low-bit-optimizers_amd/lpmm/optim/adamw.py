@@ -172,7 +172,7 @@ class AdamW(LowBitOptimizer):
         lr, wd, eps = group["lr"], group["weight_decay"], group["eps"]
         md_m = self.get_qmetadata_by_state_name("exp_avg")
         md_v = self.get_qmetadata_by_state_name("exp_avg_sq")
-        quant, plain = {}, {}  # device -> list of records
+        quant, plain, plain16 = {}, {}, {}  # device -> list of records
         factored_work = []
         lib = _native.lib()
 
@@ -194,8 +194,10 @@ class AdamW(LowBitOptimizer):
             if en_m != en_v:
                 raise ValueError("For same tensor, exp_avg and exp_avg_sq should be both quantized or "
                                  f"unquantized simultaneously, but get ({en_m} {en_v})")
-            self._check_fp32_cuda(p, grad)
             if en_m:
+                self._check_fp32_cuda(p, grad, "the 4-bit fused operator reads its float32 scales through the "
+                                      "parameters' type, in the reference as well "
+                                      "(lpmm/cpp_extension/fused_adamw_kernel.cu:229-230)")
                 if md_m["b"] != 4 or md_v["b"] != 4:
                     # the reference's fused kernel reads and writes 4-bit codes whatever the
                     # configuration says (fused_adamw_kernel.cu:113, :157); refuse instead
@@ -234,11 +236,21 @@ class AdamW(LowBitOptimizer):
                     launch_quant(key, pending)
                     pending.clear()
             else:
+                # fp32 states in the parameters' type: float32, or float16 as the reference's operator
+                # also accepts (lpmm/cpp_extension/fused_adamw_kernel.cu:188, common.h:15-27)
+                half = p.dtype is torch.float16
+                if not half:
+                    self._check_fp32_cuda(p, grad)
+                elif not (grad.dtype is torch.float16 and p.is_cuda and grad.is_cuda and p.is_contiguous()
+                          and grad.is_contiguous()):
+                    raise RuntimeError("p and g must be contiguous CUDA tensors of the same type (float16)")
                 if _is_placeholder(state["exp_avg"]):
                     state["exp_avg"] = torch.zeros_like(p, memory_format=torch.preserve_format)
                 if _is_placeholder(state["exp_avg_sq"]):
                     state["exp_avg_sq"] = torch.zeros_like(p, memory_format=torch.preserve_format)
-                plain.setdefault(p.device, []).append(
+                if state["exp_avg"].dtype is not p.dtype or state["exp_avg_sq"].dtype is not p.dtype:
+                    raise RuntimeError("exp_avg and exp_avg_sq must have the parameter's type")
+                (plain16 if half else plain).setdefault(p.device, []).append(
                     (p.data_ptr(), grad.data_ptr(), state["exp_avg"].data_ptr(), state["exp_avg_sq"].data_ptr(),
                      p.numel(), step, 0.0))
 
@@ -252,9 +264,15 @@ class AdamW(LowBitOptimizer):
                 st = lib.lpmm_adamw_fp32_step_multi(table.ctypes.data, len(records), beta1, beta2, lr, wd, eps,
                                                     _native.current_stream(dev))
             _native.check(st, "fused fp32 AdamW step")
+        for dev, records in plain16.items():
+            table = np.array(records, dtype=_native.ADAMW_FP32_TENSOR)
+            with torch.cuda.device(dev):
+                st = lib.lpmm_adamw_fp16_step_multi(table.ctypes.data, len(records), beta1, beta2, lr, wd, eps,
+                                                    _native.current_stream(dev))
+            _native.check(st, "fused fp16 AdamW step")
 
     @staticmethod
-    def _check_fp32_cuda(p, grad):
+    def _check_fp32_cuda(p, grad, why="quantised states and the non-fused path are implemented for float32 only"):
         if (p.dtype is torch.float32 and grad.dtype is torch.float32 and p.is_cuda and grad.is_cuda
                 and p.is_contiguous() and grad.is_contiguous()):
             return
@@ -264,7 +282,7 @@ class AdamW(LowBitOptimizer):
             if not t.is_contiguous():
                 raise RuntimeError(f"{name} must be contiguous!")
             if t.dtype != torch.float32:
-                raise RuntimeError(f"The type of {name} is {t.dtype}: this build implements the fp32 path only")
+                raise RuntimeError(f"The type of {name} is {t.dtype}, float32 is required here: {why}")
 
     # ---- non-fused path (lpmm/optim/adamw.py:332-436) -----------------------------------
     def _step_single(self, group, work):

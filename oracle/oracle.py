@@ -303,6 +303,38 @@ def adamw_fp32_step(p, g, m, v, beta1, beta2, lr, wd, eps, step):
     _adamw_fp32(p, g, m, v, p.size, beta1, beta2, lr, wd, eps, step)
 
 
+_libm = ctypes.CDLL("libm.so.6")
+_libm.powf.restype = ctypes.c_float
+_libm.powf.argtypes = [ctypes.c_float, ctypes.c_float]
+
+
+def _powf(a, b):
+    return np.float32(_libm.powf(float(a), float(b)))
+
+
+def adamw_fp16_step(p, g, m, v, beta1, beta2, lr, wd, eps, step):
+    """adamw_cuda_kernel<at::Half> (lpmm/cpp_extension/fused_adamw_kernel.cu:52-78, instantiated by
+    the dispatch at :188) on float16 arrays, in place.  c10::Half converts to float for every
+    arithmetic operator and rounds to nearest even on assignment, so: the moments are formed in
+    float and stored as half (:66-67); the update reads them back *after* that rounding (:72-73),
+    runs in float with the float scalars of the fp32 step, and the parameter is rounded to half on
+    its store (:74).  numpy float32 arithmetic rounds every operation once, like the kernel built
+    without contraction."""
+    f = np.float32
+    assert p.dtype == g.dtype == m.dtype == v.dtype == np.float16
+    b1, b2, lr_, wd_, eps_, st = f(beta1), f(beta2), f(lr), f(wd), f(eps), f(step)
+    omb1, omb2 = f(1) - b1, f(1) - b2
+    gf, pf = g.astype(f), p.astype(f)
+    m[...] = (b1 * m.astype(f) + omb1 * gf).astype(np.float16)
+    v[...] = (b2 * v.astype(f) + (omb2 * gf) * gf).astype(np.float16)
+    c1 = f(1) - _powf(b1, st)  # the C library's powf, as in the C restatement of the fp32 step
+    c2s = np.sqrt(f(1) - _powf(b2, st), dtype=f)
+    denom = (np.sqrt(v.astype(f), dtype=f) / c2s + eps_) * c1
+    with np.errstate(divide="ignore", invalid="ignore", over="ignore"):
+        update = m.astype(f) / denom + wd_ * pf
+        p[...] = (pf - lr_ * update).astype(np.float16)
+
+
 def adamw4bit_step(p, g, m_codes, v_codes, m_scale, v_scale, qm, qv, beta1, beta2, lr, wd, eps,
                    step):
     n = p.size

@@ -123,6 +123,38 @@ def test_fp32_step_matches_oracle(oracle):
             np.testing.assert_array_equal(to_np(v), v_ref)
 
 
+def test_fp16_step_matches_oracle(oracle):
+    """lpmm_adamw_fp16_step_multi (p, g, m, v stored as half, arithmetic in float, the update
+    reading the moments after their rounding to half) against the float16 restatement of
+    adamw_cuda_kernel<at::Half>: several tensors per call, each with its own step, five steps."""
+    nat = _native()
+    lib = nat.lib()
+    rng = np.random.default_rng(31)
+    sizes = [1, 7, 1600, 4096, 1025] + [int(k) for k in rng.integers(1, 4097, 70)]
+    host, dev = [], []
+    for n in sizes:
+        arrs = [(rng.standard_normal(n) * 0.02).astype(np.float16), None,
+                np.zeros(n, np.float16), np.zeros(n, np.float16)]
+        host.append(arrs)
+        dev.append([to_dev(a) if a is not None else None for a in arrs])
+    for s in range(1, 6):
+        steps = [float(s + i % 3) for i in range(len(sizes))]
+        for h, d, n in zip(host, dev, sizes):
+            h[1] = (rng.standard_normal(n) * 1e-2).astype(np.float16)
+            d[1] = to_dev(h[1])
+        table = np.array([(d[0].data_ptr(), d[1].data_ptr(), d[2].data_ptr(), d[3].data_ptr(), n, st, 0.0)
+                          for d, n, st in zip(dev, sizes, steps)], dtype=nat.ADAMW_FP32_TENSOR)
+        st = lib.lpmm_adamw_fp16_step_multi(table.ctypes.data, len(sizes), 0.9, 0.999, 1e-3, 0.01, 1e-8,
+                                            torch.cuda.current_stream().cuda_stream)
+        assert st == 0
+        torch.cuda.synchronize()
+        for (p, g, m, v), d, step in zip(host, dev, steps):
+            oracle.adamw_fp16_step(p, g, m, v, 0.9, 0.999, 1e-3, 0.01, 1e-8, step)
+            np.testing.assert_array_equal(to_np(d[2]), m)
+            np.testing.assert_array_equal(to_np(d[3]), v)
+            np.testing.assert_array_equal(to_np(d[0]), p)
+
+
 def test_multi_tensor_matches_single(oracle, qmaps):
     """lpmm_adamw4bit_step_multi over many tensors (more than one launch record) gives the
     same bytes as the oracle run tensor by tensor, each tensor with its own step."""

@@ -485,3 +485,53 @@ def test_param_groups_missing_grads_and_closure(oracle, qmaps, fused):
         else:
             np.testing.assert_array_equal(to_np(st["exp_avg"]).view(np.uint8), r["m"][0])
             np.testing.assert_array_equal(to_np(st["exp_avg_sq"]).view(np.uint8), r["v"][0])
+
+
+def test_half_parameters_on_the_fused_path(oracle):
+    """float16 parameters: tensors at or under the threshold keep half states and go through the
+    half instantiation of the fp32-state operator, as in the reference
+    (lpmm/optim/adamw.py:543-561, lpmm/cpp_extension/fused_adamw_kernel.cu:188); a tensor whose
+    states would be quantised is refused, as the reference's 4-bit operator fails on it
+    (float32 scales read through the parameters' type, :229-230); the non-fused path is float32
+    only here."""
+    import lpmm
+    from lpmm.cpp_extension import fused_adamw
+
+    rng = np.random.default_rng(17)
+    shapes = [(1600,), (64, 64), (3, 5, 7)]
+    host = [(rng.standard_normal(s) * 0.02).astype(np.float16) for s in shapes]
+    params = [torch.nn.Parameter(to_dev(h)) for h in host]
+    opt = lpmm.optim.AdamW(params, fused=True, **H)
+    ms = [np.zeros(h.size, np.float16) for h in host]
+    vs = [np.zeros(h.size, np.float16) for h in host]
+    for step in range(1, 5):
+        grads = [(rng.standard_normal(s) * 1e-2).astype(np.float16) for s in shapes]
+        for p, g in zip(params, grads):
+            p.grad = to_dev(g)
+        opt.step()
+        torch.cuda.synchronize()
+        for p, h, g, m, v in zip(params, host, grads, ms, vs):
+            oracle.adamw_fp16_step(h.reshape(-1), g.reshape(-1), m, v, H["betas"][0], H["betas"][1], H["lr"],
+                                   H["weight_decay"], H["eps"], float(step))
+            st = opt.state[p]
+            assert st["exp_avg"].dtype == torch.float16 and st["exp_avg"].shape == p.shape
+            np.testing.assert_array_equal(to_np(st["exp_avg"]).reshape(-1), m)
+            np.testing.assert_array_equal(to_np(st["exp_avg_sq"]).reshape(-1), v)
+            np.testing.assert_array_equal(to_np(p.detach()), h)
+    # the reference-named operator accepts half as well
+    p = to_dev(host[0].copy()); g = to_dev((rng.standard_normal(shapes[0]) * 1e-2).astype(np.float16))
+    m = torch.zeros_like(p); v = torch.zeros_like(p)
+    want_p, want_m, want_v = host[0].copy(), np.zeros(1600, np.float16), np.zeros(1600, np.float16)
+    fused_adamw.adamw_single_tensor(p, g, m, v, 0.9, 0.999, 1e-3, 0.01, 1e-8, 1.0)
+    oracle.adamw_fp16_step(want_p, to_np(g), want_m, want_v, 0.9, 0.999, 1e-3, 0.01, 1e-8, 1.0)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(to_np(p), want_p)
+    with pytest.raises(RuntimeError, match="expected scalar type"):
+        fused_adamw.adamw_single_tensor(p, g.float(), m, v, 0.9, 0.999, 1e-3, 0.01, 1e-8, 1.0)
+    # quantised states with half parameters: refused, with the reason
+    big = torch.nn.Parameter(torch.zeros(128, 64, dtype=torch.float16, device="cuda"))
+    big.grad = torch.zeros_like(big)
+    with pytest.raises(RuntimeError, match="float32 is required"):
+        lpmm.optim.AdamW([big], fused=True).step()
+    with pytest.raises(RuntimeError, match="float32 is required"):
+        lpmm.optim.AdamW([big], fused=False).step()

@@ -74,7 +74,8 @@ def test_argument_errors_without_gpu():
     assert lib.lpmm_factored_stats(ptr, 8, 8, ptr, ptr, ptr, 0.999, None, None) == NULL
     assert lib.lpmm_factored_update(ptr, ptr, ptr, ptr, ptr, ptr, ptr, ptr, 0, 8, 0.9, 0.999, 1e-3, 0.01, 1e-8, 1.0,
                                     0, None) == SIZE
-    assert lib.lpmm_factored_workspace_bytes(4096, 11008) == (64 * 11008 + 11 * 4096 + 16 + 1) * 8  # 64-row tiles
+    # 64 x 256 tiles: 64 row tiles of column partials, 43 column tiles of row partials, 16 row-block sums, the mean
+    assert lib.lpmm_factored_workspace_bytes(4096, 11008) == (64 * 11008 + 43 * 4096 + 16 + 1) * 8
     assert lib.lpmm_status_string(NULL).decode().startswith("a required pointer")
     with pytest.raises(RuntimeError, match="status 3"):
         _native.check(SIZE, "probe")

@@ -313,3 +313,56 @@ def test_golden_nonfused_fixture(oracle, qmaps, kind):
             for j, a in enumerate(st.v[1:]):
                 np.testing.assert_array_equal(a, gold[f"vs{j}_{k}"])
     np.testing.assert_array_equal(p, gold[f"p_{kind}3"])
+
+
+def test_fp16_step_pinned_by_the_fp32_step(oracle):
+    """The float16 restatement of adamw_cuda_kernel<at::Half> against the C restatement of the
+    float kernel, where the two must agree: with beta1 = beta2 = 0.5 and dyadic moments and
+    gradients the new moments are exactly representable in half, so rounding them changes
+    nothing and the half step's parameter is the float step's parameter rounded to half once.
+    A wrong rounding point, operand order or bias correction in the half restatement fails it."""
+    rng = np.random.default_rng(0)
+    n = 8192
+    m = (rng.integers(-64, 64, n) / 64).astype(np.float16)
+    g = (rng.integers(-32, 32, n) / 32).astype(np.float16)
+    v = (rng.integers(1, 64, n) / 64).astype(np.float16)
+    p = rng.standard_normal(n).astype(np.float16)
+    for step in (1.0, 3.0, 40.0):
+        p32, g32, m32, v32 = (a.astype(np.float32) for a in (p, g, m, v))
+        oracle.adamw_fp32_step(p32, g32, m32, v32, 0.5, 0.5, 1e-2, 0.01, 1e-8, step)
+        ph, mh, vh = p.copy(), m.copy(), v.copy()
+        oracle.adamw_fp16_step(ph, g, mh, vh, 0.5, 0.5, 1e-2, 0.01, 1e-8, step)
+        np.testing.assert_array_equal(mh.astype(np.float32), m32)
+        np.testing.assert_array_equal(vh.astype(np.float32), v32)
+        np.testing.assert_array_equal(ph, p32.astype(np.float16))
+        assert np.any(ph != p)
+
+
+def test_fp16_step_reads_the_rounded_moments(oracle):
+    """With ordinary hyper-parameters the new moments are not representable in half.  They must
+    equal the float step's moments rounded to half once, and the parameter must come from those
+    rounded moments (lpmm/cpp_extension/fused_adamw_kernel.cu:66-73 reads exp_avg and exp_avg_sq
+    back from memory): an update formed from the unrounded moments differs somewhere."""
+    rng = np.random.default_rng(1)
+    n = 4096
+    p = (rng.standard_normal(n) * 0.02).astype(np.float16)
+    g = (rng.standard_normal(n) * 1e-2).astype(np.float16)
+    m = (rng.standard_normal(n) * 1e-2).astype(np.float16)
+    v = (rng.standard_normal(n) ** 2 * 1e-4).astype(np.float16)
+    ph, mh, vh = p.copy(), m.copy(), v.copy()
+    oracle.adamw_fp16_step(ph, g, mh, vh, 0.9, 0.999, 1e-3, 0.01, 1e-8, 5.0)
+    p32, g32, m32, v32 = (a.astype(np.float32) for a in (p, g, m, v))
+    oracle.adamw_fp32_step(p32, g32, m32, v32, 0.9, 0.999, 1e-3, 0.01, 1e-8, 5.0)
+    np.testing.assert_array_equal(mh, m32.astype(np.float16))
+    np.testing.assert_array_equal(vh, v32.astype(np.float16))
+    f = np.float32
+    c1 = f(1) - f(0.9) ** f(5)
+    c2s = np.sqrt(f(1) - f(0.999) ** f(5))
+
+    def update(mm, vv):
+        pf = p.astype(f)
+        return (pf - f(1e-3) * (mm / ((np.sqrt(vv) / c2s + f(1e-8)) * c1) + f(0.01) * pf)).astype(np.float16)
+
+    from_rounded = update(mh.astype(f), vh.astype(f))
+    assert np.mean(from_rounded == ph) > 0.999  # the C library's powf and ** may differ in the last place
+    assert np.any(update(m32, v32) != from_rounded)
