@@ -162,8 +162,26 @@ int lpmm_quant_rank1(const float *x, int64_t rows, int64_t cols, const float *ro
 int lpmm_dequant_rank1(const uint8_t *codes, const float *rowmax, const float *colmax,
                        const float *qmap, int64_t rows, int64_t cols, float *out, void *stream);
 
+/* Rank-1 statistics of a contiguous tensor of 1..LPMM_RANK1_ND_MAX dimensions:
+ * stats[i][j] = max |x| over the elements whose i-th index is j (stats[i] holds shape[i] floats).
+ * Replaces get_sm3_statistics (lpmm/functional.py:512-531) for tensors the 2-D entry point
+ * above does not cover; the statistics are cleared by the call itself.  `shape` and `stats` are
+ * host arrays of ndim entries.  `work` is NULL or device memory for numel / shape[ndim-1] floats:
+ * with it, a last dimension of 32 or more goes through the 2-D kernel (x is still read once). */
+#define LPMM_RANK1_ND_MAX 8
+int lpmm_rank1_stats_nd(const float *x, int ndim, const int64_t *shape, float *const *stats, float *work,
+                        void *stream);
+
+/* row_scale[r] = min over the leading dimensions i < ndim-1 of stats[i][index_i(r)], r running
+ * over the rows of the (numel / shape[ndim-1]) x shape[ndim-1] view; NaN if any of them is
+ * (torch.min).  With row_scale as `rowmax` and stats[ndim-1] as `colmax`, lpmm_quant_rank1 /
+ * lpmm_dequant_rank1 (and their _bits forms) on that 2-D view apply the reference's scale
+ * min_i stats[i] (lpmm/functional.py:503-509) to the N-D tensor.  stats[ndim-1] is not read. */
+int lpmm_rank1_row_scale_nd(const float *const *stats, int ndim, const int64_t *shape, float *row_scale,
+                            void *stream);
+
 /* ---------------------------------------------------------------------------------------
- * The same six operations for any code width 1..8 (lpmm/configs/default_{5,6,7,8}b.yml use
+ * The same six operations for any code width 1..8(lpmm/configs/default_{5,6,7,8}b.yml use
  * 5..8).  Storage follows lpmm/cpp_extension/quantization_kernel.cu:592-601, :695-705:
  * widths 1, 2, 4 pack 8/bits codes per byte (code j of a byte at bit j*bits), every other
  * width stores one code per byte; arrays hold n_padded*storage_bits/8 + 1 bytes and must be

@@ -35,6 +35,8 @@ PROTOTYPES = {
     "lpmm_rank1_stats": (_int, [_vp, _i64, _i64, _vp, _vp, _vp]),
     "lpmm_quant_rank1": (_int, [_vp, _i64, _i64, _vp, _vp, _vp, _vp, _vp]),
     "lpmm_dequant_rank1": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _vp, _vp]),
+    "lpmm_rank1_stats_nd": (_int, [_vp, _int, _vp, _vp, _vp, _vp]),
+    "lpmm_rank1_row_scale_nd": (_int, [_vp, _int, _vp, _vp, _vp]),
     "lpmm_pack_nonlinear": (_int, [_vp, _vp, _int, _i64, _vp, _vp]),
     "lpmm_pack_nonlinear_sr": (_int, [_vp, _vp, _int, _i64, ctypes.c_uint64, ctypes.c_uint64, _vp, _vp]),
     "lpmm_unpack_nonlinear": (_int, [_vp, _vp, _int, _i64, _vp, _vp]),

@@ -11,8 +11,10 @@ for widths that do not divide 8 one code per byte; `max1` of shape (G, 1) for 'g
 
 Where the reference chains abs / max / div / cat / pack (and unpack / mul) as separate
 passes, each call here is one HIP kernel (two for rank-1 quantisation: statistics, then
-normalise + search + pack).
+normalise + search + pack; tensors of 3..8 dimensions add a kernel that folds the leading
+dimensions' statistics into one scale per row of the (numel / last, last) view).
 """
+import ctypes
 import math
 
 import torch
@@ -21,6 +23,7 @@ from . import _native
 from .cpp_extension import quantization as ext_quantization
 
 PACK_GROUP = 2048
+RANK1_ND_MAX = 8  # dimensions the rank-1 kernels take (LPMM_RANK1_ND_MAX)
 
 _NONLINEAR_TYPES = ("nonlinear", "power-1", "power-2", "power-3", "float-point", "nonlinear-nozero")
 
@@ -119,10 +122,19 @@ def _max_reduce_except_dim(tensor, dim):
     return result
 
 
+def _ptr_array(tensors):
+    return (ctypes.c_void_p * len(tensors))(*[t.data_ptr() for t in tensors])
+
+
+def _shape_array(shape):
+    return (ctypes.c_int64 * len(shape))(*shape)
+
+
 def get_sm3_statistics(x, **kwargs):
-    """max|x| over all dimensions but one, for each dimension (keepdim shapes).  2-D float32
-    CUDA tensors take one HIP kernel that reads x once."""
-    if x.dim() == 2 and x.is_cuda and x.dtype == torch.float32:
+    """max|x| over all dimensions but one, for each dimension (keepdim shapes).  float32 CUDA
+    tensors of 2..8 dimensions take HIP kernels that read x once."""
+    on_hip = x.is_cuda and x.dtype == torch.float32 and x.numel() > 0
+    if x.dim() == 2 and on_hip:
         xc = x.contiguous()
         rows, cols = xc.shape
         rowmax = torch.empty((rows, 1), dtype=torch.float32, device=x.device)
@@ -132,8 +144,47 @@ def get_sm3_statistics(x, **kwargs):
                                                 _native.current_stream(x.device))
         _native.check(st, "rank1_stats")
         return [rowmax, colmax]
+    if 2 < x.dim() <= RANK1_ND_MAX and on_hip:
+        xc = x.contiguous()
+        shape = tuple(xc.shape)
+        stats = []
+        for i, d in enumerate(shape):
+            keep = [1] * len(shape)
+            keep[i] = d
+            stats.append(torch.empty(keep, dtype=torch.float32, device=x.device))
+        work = None
+        if shape[-1] >= 32:  # long last dimension: the 2-D kernel plus a fold of its row maxima
+            work = torch.empty((xc.numel() // shape[-1],), dtype=torch.float32, device=x.device)
+        with torch.cuda.device(x.device):
+            st = _native.lib().lpmm_rank1_stats_nd(xc.data_ptr(), len(shape), _shape_array(shape), _ptr_array(stats),
+                                                   work.data_ptr() if work is not None else None,
+                                                   _native.current_stream(x.device))
+        _native.check(st, "rank1_stats_nd")
+        return stats
     qx = x.abs()
     return [_max_reduce_except_dim(qx, i) for i in range(x.dim())]
+
+
+def _row_scale_nd(max_dims, shape):
+    """For a tensor of more than two dimensions: per row of its (numel / shape[-1], shape[-1])
+    view the smallest statistic of the leading dimensions.  With the last dimension's
+    statistics as column maxima the 2-D kernels then scale by min over all dimensions, which
+    is _compute_sm3_scale_tensor (lpmm/functional.py:503-509)."""
+    if len(shape) > RANK1_ND_MAX:
+        raise NotImplementedError(f"rank-1 scaling of a {len(shape)}-D tensor: the kernels take up to "
+                                  f"{RANK1_ND_MAX} dimensions")
+    dev = max_dims[0].device
+    stats = [m.to(torch.float32).contiguous() for m in max_dims]
+    for m, d in zip(stats, shape):
+        if m.numel() != d:
+            raise ValueError(f"max_dims do not belong to a tensor of shape {tuple(shape)}")
+    rows = math.prod(shape[:-1])
+    row_scale = torch.empty((rows,), dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        st = _native.lib().lpmm_rank1_row_scale_nd(_ptr_array(stats), len(shape), _shape_array(tuple(shape)),
+                                                   row_scale.data_ptr(), _native.current_stream(dev))
+    _native.check(st, "rank1_row_scale_nd")
+    return row_scale, stats[-1]
 
 
 def _compute_sm3_scale_tensor(max_dims):
@@ -222,20 +273,26 @@ def quant_group_(x, qmap, gp_sz, codes=None, max1=None, b=4):
 
 
 def quant_rank1_(x, qmap, codes=None, b=4):
-    """'rank1' scaling of a contiguous 2-D float32 CUDA tensor: statistics kernel, then
-    normalise + search + pack kernel."""
-    rows, cols = x.shape
+    """'rank1' scaling of a contiguous float32 CUDA tensor of two or more dimensions:
+    statistics kernel(s), then normalise + search + pack kernel (more than two dimensions: on
+    the (numel / shape[-1], shape[-1]) view with the leading dimensions' minima as row scale)."""
     max_dims = get_sm3_statistics(x)
+    if x.dim() == 2:
+        rows, cols = x.shape
+        rowmax, colmax = max_dims
+    else:
+        rows, cols = x.numel() // x.shape[-1], x.shape[-1]
+        rowmax, colmax = _row_scale_nd(max_dims, x.shape)
     if codes is None:
         codes = torch.empty((packed_nbytes(rows * cols, b),), dtype=torch.int8, device=x.device)
     lib = _native.lib()
     with torch.cuda.device(x.device):
         stream = _native.current_stream(x.device)
         if b == 4:
-            st = lib.lpmm_quant_rank1(x.data_ptr(), rows, cols, max_dims[0].data_ptr(), max_dims[1].data_ptr(),
+            st = lib.lpmm_quant_rank1(x.data_ptr(), rows, cols, rowmax.data_ptr(), colmax.data_ptr(),
                                       qmap.data_ptr(), codes.data_ptr(), stream)
         else:
-            st = lib.lpmm_quant_rank1_bits(x.data_ptr(), rows, cols, max_dims[0].data_ptr(), max_dims[1].data_ptr(),
+            st = lib.lpmm_quant_rank1_bits(x.data_ptr(), rows, cols, rowmax.data_ptr(), colmax.data_ptr(),
                                            qmap.data_ptr(), b, codes.data_ptr(), stream)
     _native.check(st, "quant_rank1")
     return codes, max_dims
@@ -270,10 +327,10 @@ def vectorwise_quant(x, **kwargs):
         md["max1"] = max1
         md["scaled_shape"] = torch.Size((max1.shape[0], gp_sz))
     elif scale_type == "rank1":
-        if nearest and src.dim() == 2:
+        if nearest and 2 <= src.dim() <= RANK1_ND_MAX and src.numel() > 0:
             codes, max_dims = quant_rank1_(src, qmap, b=b)
         else:
-            max_dims = get_sm3_statistics(src.abs())
+            max_dims = get_sm3_statistics(src)
             codes = nonlinear_quant(src.div(_compute_sm3_scale_tensor(max_dims)), qmap, b,
                                     round_type=kwargs["round_type"])
         md["max_dims"] = max_dims
@@ -285,8 +342,8 @@ def vectorwise_quant(x, **kwargs):
 
 
 def vectorwise_dequant(qx, denormalized=True, **kwargs):
-    """Dequantise packed codes to a tensor of kwargs['shape'] (the parameter's shape).
-    lpmm/functional.py:62-151."""
+    """Dequantise packed codes to a tensor of kwargs['shape'] (the parameter's shape) with the
+    strides kwargs['stride'] records (None: contiguous).  lpmm/functional.py:62-151."""
     _require_supported(kwargs, qx)
     qmap = _select_qmap(kwargs)
     dtype, stride = kwargs["dtype"], kwargs["stride"]
@@ -319,18 +376,22 @@ def vectorwise_dequant(qx, denormalized=True, **kwargs):
             x = recon_grouped_tensor(x.mul(kwargs["max1"]), shape)
     elif scale_type == "rank1":
         max_dims = kwargs["max_dims"]
-        if len(scaled_shape) == 2:
-            rows, cols = scaled_shape
+        if 2 <= len(scaled_shape) <= RANK1_ND_MAX and numel(scaled_shape) > 0:
+            if len(scaled_shape) == 2:
+                rows, cols = scaled_shape
+                rowmax, colmax = max_dims
+            else:
+                rows, cols = numel(scaled_shape[:-1]), scaled_shape[-1]
+                rowmax, colmax = _row_scale_nd(max_dims, scaled_shape)
             x = torch.empty(scaled_shape, dtype=torch.float32, device=dev)
             with torch.cuda.device(dev):
                 stream = _native.current_stream(dev)
                 if b == 4:
-                    st = lib.lpmm_dequant_rank1(codes.data_ptr(), max_dims[0].data_ptr(), max_dims[1].data_ptr(),
+                    st = lib.lpmm_dequant_rank1(codes.data_ptr(), rowmax.data_ptr(), colmax.data_ptr(),
                                                 qmap.data_ptr(), rows, cols, x.data_ptr(), stream)
                 else:
-                    st = lib.lpmm_dequant_rank1_bits(codes.data_ptr(), max_dims[0].data_ptr(),
-                                                     max_dims[1].data_ptr(), qmap.data_ptr(), b, rows, cols,
-                                                     x.data_ptr(), stream)
+                    st = lib.lpmm_dequant_rank1_bits(codes.data_ptr(), rowmax.data_ptr(), colmax.data_ptr(),
+                                                     qmap.data_ptr(), b, rows, cols, x.data_ptr(), stream)
             _native.check(st, "dequant_rank1")
         else:
             x = nonlinear_dequant(codes, qmap, b, shape=scaled_shape, round_type=kwargs["round_type"])
@@ -338,7 +399,7 @@ def vectorwise_dequant(qx, denormalized=True, **kwargs):
     else:
         raise NotImplementedError(f"scale_type {scale_type!r}: this build implements 'group' and 'rank1'")
 
-    if x.stride() != stride:
+    if stride is not None and x.stride() != stride:
         recon = torch.empty_strided(x.shape, stride, dtype=dtype, layout=torch.strided, device=dev)
         recon.copy_(x)
         return recon

@@ -272,17 +272,50 @@ class AdamW(LowBitOptimizer):
             _native.check(st, "fused fp16 AdamW step")
 
     @staticmethod
-    def _check_fp32_cuda(p, grad, why="quantised states and the non-fused path are implemented for float32 only"):
+    def _check_fp32_cuda(p, grad, why="quantised states and the non-fused path are implemented for float32 only",
+                         strided_ok=False):
         if (p.dtype is torch.float32 and grad.dtype is torch.float32 and p.is_cuda and grad.is_cuda
-                and p.is_contiguous() and grad.is_contiguous()):
+                and (strided_ok or (p.is_contiguous() and grad.is_contiguous()))):
             return
         for t, name in ((p, "p"), (grad, "g")):
             if not t.is_cuda:
                 raise RuntimeError(f"{name} must be a CUDA tensor!")
-            if not t.is_contiguous():
+            if not strided_ok and not t.is_contiguous():
                 raise RuntimeError(f"{name} must be contiguous!")
             if t.dtype != torch.float32:
                 raise RuntimeError(f"The type of {name} is {t.dtype}, float32 is required here: {why}")
+
+    @classmethod
+    def _dense_operands(cls, p, grad, held):
+        """The parameter and its gradient as the non-fused kernels take them: contiguous float32.
+        The reference's non-fused step is a chain of PyTorch ops and accepts any strides
+        (lpmm/optim/adamw.py:394-422; its quantiser flattens in index order, functional.py:404-422).
+        A strided operand is copied to a contiguous tensor in index order, which leaves every
+        value and every quantisation group as they are there.  `held` keeps the copies alive until
+        the step's kernels are enqueued (launches are deferred and take raw pointers); the updated
+        copy of a strided parameter is written back then (_write_back)."""
+        cls._check_fp32_cuda(p, grad, strided_ok=True)
+        if p.is_contiguous() and grad.is_contiguous():
+            return p, grad
+        dense = p if p.is_contiguous() else p.detach().contiguous()
+        grad = grad.contiguous()
+        held.append((p if dense is not p else None, dense, grad))
+        return dense, grad
+
+    @staticmethod
+    def _write_back(held):
+        for p, dense, _ in held:
+            if p is not None:
+                p.copy_(dense)
+        held.clear()
+
+    @staticmethod
+    def _state_stride(p):
+        """Strides the reference records for a state of p: those of
+        zeros_like(p, memory_format=preserve_format) (lpmm/optim/adamw.py:395, functional.py:32)."""
+        if p.is_contiguous():
+            return p.stride()
+        return torch.empty_like(p, device="meta", memory_format=torch.preserve_format).stride()
 
     # ---- non-fused path (lpmm/optim/adamw.py:332-436) -----------------------------------
     def _step_single(self, group, work):
@@ -302,6 +335,7 @@ class AdamW(LowBitOptimizer):
         v_rank1 = fits(md_v) and md_v["scale_type"] == "rank1"
         batched, batched_rank1, plain = {}, {}, {}
         factored_work = []
+        held = []  # contiguous copies of strided operands
 
         def launch_group(key, records):
             dev, qm_ptr, qv_ptr = key
@@ -325,34 +359,34 @@ class AdamW(LowBitOptimizer):
             if factored:
                 factored_work.append((p, grad, state, step))
                 continue
-            self._check_fp32_cuda(p, grad)
+            dense, grad = self._dense_operands(p, grad, held)
             en_m, en_v = self._enabled(p, state, "exp_avg"), self._enabled(p, state, "exp_avg_sq")
             if m_group128 and en_m and en_v:
                 key = (p.device, state["exp_avg_qstate"]["qmap"].data_ptr(),
                        state["exp_avg_sq_qstate"]["qmap"].data_ptr())
                 if v_group128:
                     pending = batched.setdefault(key, [])
-                    pending.append(self._nonfused_record(p, grad, state, step))
+                    pending.append(self._nonfused_record(p, dense, grad, state, step))
                     if len(pending) == _native.MULTI_MAX:  # one launch's worth: enqueue it now
                         launch_group(key, pending)
                         pending.clear()
                     continue
                 if v_rank1 and p.dim() == 2 and p.shape[1] % 128 == 0:
                     pending = batched_rank1.setdefault(key, [])
-                    pending.append(self._nonfused_rank1_record(p, grad, state, step))
+                    pending.append(self._nonfused_rank1_record(p, dense, grad, state, step))
                     if len(pending) == _native.RANK1_MULTI_MAX:
                         launch_rank1(key, pending)
                         pending.clear()
                     continue
             m = self._materialise(p, state, "exp_avg", en_m, md_m)
             v = self._materialise(p, state, "exp_avg_sq", en_v, md_v)
-            if not en_m and not en_v and p.is_contiguous() and m.is_contiguous() and v.is_contiguous():
+            if not en_m and not en_v and m.is_contiguous() and v.is_contiguous():
                 # fp32 states (small tensors): all of them in one launch
                 plain.setdefault(p.device, []).append(
-                    (p.data_ptr(), grad.data_ptr(), m.data_ptr(), v.data_ptr(), p.numel(), step, 0.0))
+                    (dense.data_ptr(), grad.data_ptr(), m.data_ptr(), v.data_ptr(), p.numel(), step, 0.0))
                 continue
             with torch.cuda.device(p.device):
-                st = lib.lpmm_nonfused_update(p.data_ptr(), grad.data_ptr(), m.data_ptr(), v.data_ptr(), p.numel(),
+                st = lib.lpmm_nonfused_update(dense.data_ptr(), grad.data_ptr(), m.data_ptr(), v.data_ptr(), p.numel(),
                                               beta1, beta2, lr, wd, eps, step, _native.current_stream(p.device))
             _native.check(st, "non-fused AdamW update")
             if en_m:
@@ -372,8 +406,9 @@ class AdamW(LowBitOptimizer):
         for key, records in batched_rank1.items():
             if records:
                 launch_rank1(key, records)
+        self._write_back(held)
 
-    def _nonfused_record(self, p, grad, state, step):
+    def _nonfused_record(self, p, dense, grad, state, step):
         """The tensor's record for the one-pass non-fused step; creates the quantised states
         on first use: all-zero moments in the layout and with the metadata vectorwise_quant
         gives them (lpmm/optim/adamw.py:425-434)."""
@@ -387,13 +422,13 @@ class AdamW(LowBitOptimizer):
                                          dtype=torch.int8, device=p.device)
                 oh = qstate["overhead"]
                 oh.clear()
-                oh.update({"dtype": p.dtype, "stride": p.stride(),
+                oh.update({"dtype": p.dtype, "stride": self._state_stride(p),
                            "max1": torch.zeros((groups, 1), dtype=torch.float32, device=p.device),
                            "scaled_shape": torch.Size((groups, 128))})
             ptrs.append((state[name].data_ptr(), qstate["overhead"]["max1"].data_ptr()))
-        return (p.data_ptr(), grad.data_ptr(), ptrs[0][0], ptrs[1][0], ptrs[0][1], ptrs[1][1], n, step, 0.0)
+        return (dense.data_ptr(), grad.data_ptr(), ptrs[0][0], ptrs[1][0], ptrs[0][1], ptrs[1][1], n, step, 0.0)
 
-    def _nonfused_rank1_record(self, p, grad, state, step):
+    def _nonfused_rank1_record(self, p, dense, grad, state, step):
         """The tensor's record for the two-pass step with a rank-1 second moment.  The kernels
         leave the statistics of the new second moment in a second pair of buffers; the pairs
         trade places here, so that the state's `max_dims` always are the statistics its codes
@@ -406,14 +441,14 @@ class AdamW(LowBitOptimizer):
         if _is_placeholder(state["exp_avg"]):
             state["exp_avg"] = torch.full((packed_nbytes(n),), _zero_byte(qs_m["qmap"]), dtype=torch.int8, device=dev)
             qs_m["overhead"].clear()
-            qs_m["overhead"].update({"dtype": p.dtype, "stride": p.stride(),
+            qs_m["overhead"].update({"dtype": p.dtype, "stride": self._state_stride(p),
                                      "max1": torch.zeros((groups, 1), dtype=torch.float32, device=dev),
                                      "scaled_shape": torch.Size((groups, 128))})
         if _is_placeholder(state["exp_avg_sq"]):
             state["exp_avg_sq"] = torch.full((packed_nbytes(n),), _zero_byte(qs_v["qmap"]), dtype=torch.int8,
                                              device=dev)
             qs_v["overhead"].clear()
-            qs_v["overhead"].update({"dtype": p.dtype, "stride": p.stride(), "dim": 2, "max1": None,
+            qs_v["overhead"].update({"dtype": p.dtype, "stride": self._state_stride(p), "dim": 2, "max1": None,
                                      "max_dims": [torch.zeros((rows, 1), dtype=torch.float32, device=dev),
                                                   torch.zeros((1, cols), dtype=torch.float32, device=dev)],
                                      "scaled_shape": p.shape})
@@ -424,7 +459,7 @@ class AdamW(LowBitOptimizer):
             nxt = [torch.empty_like(cur[0]), torch.empty_like(cur[1])]
         self._spare_stats[p] = cur
         oh["max_dims"] = nxt
-        return (p.data_ptr(), grad.data_ptr(), state["exp_avg"].data_ptr(), qs_m["overhead"]["max1"].data_ptr(),
+        return (dense.data_ptr(), grad.data_ptr(), state["exp_avg"].data_ptr(), qs_m["overhead"]["max1"].data_ptr(),
                 state["exp_avg_sq"].data_ptr(), cur[0].data_ptr(), cur[1].data_ptr(), nxt[0].data_ptr(),
                 nxt[1].data_ptr(), rows, cols, step, 0.0)
 
@@ -438,8 +473,10 @@ class AdamW(LowBitOptimizer):
         return d
 
     def _materialise(self, p, state, name, enabled, md):
-        """fp32 view of a state for the update: zeros at the first step, the dequantised
-        tensor when quantised, the state itself otherwise (adamw.py:394-409)."""
+        """Contiguous fp32 tensor of a state for the update, in the parameter's index order:
+        zeros at the first step, the dequantised tensor when quantised, the state itself
+        otherwise (adamw.py:394-409).  The reference gives the tensor the strides its metadata
+        records; the kernels here work on the contiguous form of the same values."""
         t = state[name]
         if _is_placeholder(t):
             state[name] = t = torch.zeros_like(p, memory_format=torch.contiguous_format)
@@ -448,13 +485,16 @@ class AdamW(LowBitOptimizer):
             qstate = state[f"{name}_qstate"]
             kw = dict(qstate["overhead"])
             kw.update(md)
-            out = vectorwise_dequant(t, qmap=qstate["qmap"], shape=p.shape, **kw)
-            return out.contiguous()
+            kw["stride"] = None  # no re-striding of the temporary
+            return vectorwise_dequant(t, qmap=qstate["qmap"], shape=p.shape, **kw)
+        if not t.is_contiguous():  # e.g. loaded from a checkpoint of a strided parameter
+            state[name] = t = t.contiguous()
         return t
 
     def _requantise(self, p, state, name, x, md):
         qstate = state[f"{name}_qstate"]
         qx, gen = vectorwise_quant(x, qmap=qstate["qmap"], shape=p.shape, **md)
+        gen["stride"] = self._state_stride(p)
         state[name] = qx
         qstate["overhead"].clear()
         qstate["overhead"].update(gen)
@@ -473,11 +513,12 @@ class AdamW(LowBitOptimizer):
                   and md_m["round_type"] == "real-nearest")
         lib = _native.lib()
         batched = {}
+        held = []  # contiguous copies of strided operands
         for p, grad, state, step in items:
+            dense, grad = self._dense_operands(p, grad, held)
             if not (m_fits and p.dim() == 2 and p.shape[1] % 128 == 0 and self._enabled(p, state, "exp_avg")):
-                self._factored_step(group, p, grad, state, step)
+                self._factored_step(group, p, dense, grad, state, step)
                 continue
-            self._check_fp32_cuda(p, grad)
             rows, cols = p.shape
             qstate = state["exp_avg_qstate"]
             first = _is_placeholder(state["exp_avg"])
@@ -485,13 +526,13 @@ class AdamW(LowBitOptimizer):
                 groups = p.numel() // 128
                 state["exp_avg"] = torch.empty((packed_nbytes(p.numel()),), dtype=torch.int8, device=p.device)
                 qstate["overhead"].clear()
-                qstate["overhead"].update({"dtype": p.dtype, "stride": p.stride(),
+                qstate["overhead"].update({"dtype": p.dtype, "stride": self._state_stride(p),
                                            "max1": torch.empty((groups, 1), dtype=torch.float32, device=p.device),
                                            "scaled_shape": torch.Size((groups, 128))})
             key = (p.device, qstate["qmap"].data_ptr())
             ws = (lib.lpmm_factored_workspace_bytes(rows, cols) + 255) // 256 * 256
             batched.setdefault(key, []).append(
-                [p.data_ptr(), grad.data_ptr(), state["exp_avg"].data_ptr(), qstate["overhead"]["max1"].data_ptr(),
+                [dense.data_ptr(), grad.data_ptr(), state["exp_avg"].data_ptr(), qstate["overhead"]["max1"].data_ptr(),
                  state["exp_avg_sq_row"].data_ptr(), state["exp_avg_sq_col"].data_ptr(), ws, rows, cols, step,
                  1 if first else 0])
         for (dev, qm_ptr), records in batched.items():
@@ -504,11 +545,12 @@ class AdamW(LowBitOptimizer):
                 st = lib.lpmm_factored_step_multi(table.ctypes.data, len(records), qm_ptr, beta1, beta2, lr, wd, eps,
                                                   _native.current_stream(dev))
             _native.check(st, "factored step")
+        self._write_back(held)
 
-    def _factored_step(self, group, p, grad, state, step):
+    def _factored_step(self, group, p, dense, grad, state, step):
+        """One factored tensor outside the multi-tensor launch; `dense` is p or its contiguous copy."""
         beta1, beta2 = group["betas"]
         lr, wd, eps = group["lr"], group["weight_decay"], group["eps"]
-        self._check_fp32_cuda(p, grad)
         lib = _native.lib()
         dev = p.device
         rows, cols = p.shape[-2], p.shape[-1]
@@ -536,19 +578,19 @@ class AdamW(LowBitOptimizer):
                     max1 = torch.empty((groups, 1), dtype=torch.float32, device=dev)
                 else:
                     max1 = qstate["overhead"]["max1"]
-                st = lib.lpmm_factored_update(p.data_ptr(), grad.data_ptr(), state["exp_avg"].data_ptr(),
+                st = lib.lpmm_factored_update(dense.data_ptr(), grad.data_ptr(), state["exp_avg"].data_ptr(),
                                               max1.data_ptr(), qstate["qmap"].data_ptr(), row.data_ptr(),
                                               col.data_ptr(), mean_all.data_ptr(), rows, cols, beta1, beta2, lr, wd,
                                               eps, step, 1 if first else 0, stream)
                 _native.check(st, "factored update")
                 qstate["overhead"].clear()
-                qstate["overhead"].update({"dtype": p.dtype, "stride": p.stride(), "max1": max1,
+                qstate["overhead"].update({"dtype": p.dtype, "stride": self._state_stride(p), "max1": max1,
                                            "scaled_shape": torch.Size((groups, 128))})
                 return
             m = self._materialise(p, state, "exp_avg", en_m, md_m)
             for b in range(batch):
                 off = 4 * b * rows * cols
-                st = lib.lpmm_factored_update_fp32m(p.data_ptr() + off, grad.data_ptr() + off, m.data_ptr() + off,
+                st = lib.lpmm_factored_update_fp32m(dense.data_ptr() + off, grad.data_ptr() + off, m.data_ptr() + off,
                                                     row.data_ptr() + 4 * b * rows, col.data_ptr() + 4 * b * cols,
                                                     mean_all.data_ptr() + 4 * b, rows, cols, beta1, beta2, lr, wd,
                                                     eps, step, stream)

@@ -299,6 +299,39 @@ def dequant_rank1_bits(codes, rowmax, colmax, qmap, bits, r, c):
     return (unpack_nonlinear(codes, qmap, bits, r * c).reshape(r, c) * st).astype(np.float32)
 
 
+def rank1_stats_nd(x):
+    """get_sm3_statistics (lpmm/functional.py:512-531) for any number of dimensions: for each
+    dimension the maximum of |x| over all the others, as 1-D arrays."""
+    a = np.abs(_c(x, np.float32))
+    return [a.max(axis=tuple(j for j in range(a.ndim) if j != i)).astype(np.float32) for i in range(a.ndim)]
+
+
+def rank1_scale_nd(stats, shape):
+    """_compute_sm3_scale_tensor (lpmm/functional.py:503-509): the statistics broadcast to the
+    tensor's shape and folded with an elementwise minimum, dimension 0 first."""
+    scale = None
+    for i, st in enumerate(stats):
+        keep = [1] * len(shape)
+        keep[i] = shape[i]
+        other = np.broadcast_to(_c(st, np.float32).reshape(keep), shape)
+        scale = other if scale is None else np.where(other < scale, other, scale)
+    return np.ascontiguousarray(scale, dtype=np.float32)
+
+
+def quant_rank1_nd_bits(x, stats, qmap, bits):
+    """lpmm/functional.py:190-203 + :359-369 for a tensor of any number of dimensions."""
+    x = _c(x, np.float32)
+    with np.errstate(invalid="ignore", divide="ignore"):
+        normed = (x / rank1_scale_nd(stats, x.shape)).astype(np.float32).reshape(-1)
+    return pack_nonlinear(_pad_to(normed, PACK_GROUP), qmap, bits)
+
+
+def dequant_rank1_nd_bits(codes, stats, qmap, bits, shape):
+    """lpmm/functional.py:97-106 for a tensor of any number of dimensions."""
+    n = int(np.prod(shape))
+    return (unpack_nonlinear(codes, qmap, bits, n).reshape(shape) * rank1_scale_nd(stats, shape)).astype(np.float32)
+
+
 def adamw_fp32_step(p, g, m, v, beta1, beta2, lr, wd, eps, step):
     _adamw_fp32(p, g, m, v, p.size, beta1, beta2, lr, wd, eps, step)
 
@@ -418,7 +451,8 @@ def factored_update(p, g, m, row, col, row_mean_all, beta1, beta2, lr, wd, eps, 
 class NonFusedState:
     """Optimizer state of one tensor in the non-fused layout (adamw.py:119-129,
     functional.py:32-34, :240): packed codes of NG*1024+1 bytes plus max1 (G,) for 'group'
-    scaling or (rowmax, colmax) for 'rank1' on a 2-D tensor."""
+    scaling, (rowmax, colmax) for 'rank1' on a 2-D tensor, (codes, [stat_0, ...]) for 'rank1' on
+    a tensor of more dimensions."""
 
     def __init__(self, shape, v_scale_type="group", factored=False, bits=4):
         self.bits = bits  # code width of both moments (lpmm/configs/default_{5,6,7,8}b.yml)
@@ -459,6 +493,8 @@ def nonfused_step(p, g, state, qm, qv, lr, beta1, beta2, eps, wd):
     m = np.zeros(n, np.float32) if state.m is None else deq_g(state.m, qm)
     if state.v is None:
         v = np.zeros(n, np.float32)
+    elif _v_is_rank1(state) and len(state.shape) > 2:
+        v = dequant_rank1_nd_bits(state.v[0], state.v[1], qv, b, state.shape).reshape(-1)
     elif _v_is_rank1(state):
         r, c = state.shape
         v = np.ascontiguousarray(deq_r(state.v, qv, r, c)).reshape(-1)
@@ -466,7 +502,11 @@ def nonfused_step(p, g, state, qm, qv, lr, beta1, beta2, eps, wd):
         v = deq_g(state.v, qv)
     nonfused_update(pf, gf, m, v, beta1, beta2, lr, wd, eps, float(state.step))
     state.m = q_g(m, qm)
-    if _v_is_rank1(state):
+    if _v_is_rank1(state) and len(state.shape) > 2:
+        vn = v.reshape(state.shape)
+        stats = rank1_stats_nd(vn)
+        state.v = (quant_rank1_nd_bits(vn, stats, qv, b), stats)
+    elif _v_is_rank1(state):
         r, c = state.shape
         v2 = v.reshape(r, c)
         rowmax, colmax = rank1_stats(v2)

@@ -138,6 +138,129 @@ def test_nonfused_optimizer_matches_oracle(oracle, qmaps, v_scale):
     assert_rel(to_np(params[2]), host[2], 'p small', scale=host[2])
 
 
+def test_nonfused_rank1_on_tensors_of_more_than_two_dimensions(oracle, qmaps):
+    """Default configuration (rank-1 second moment) on 3-D and 4-D parameters: statistics,
+    quantiser and dequantiser run in HIP (N-D statistics kernels plus the 2-D kernels on the
+    flattened view) and leave the oracle's codes and statistics."""
+    import lpmm
+
+    qm, qv = qmaps
+    rng = np.random.default_rng(21)
+    shapes = [(6, 40, 64), (32, 16, 3, 3), (4, 24, 130)]
+    host, params = _params(shapes, rng)
+    cfg = os.path.join(os.path.dirname(lpmm.config.__file__), "configs", "default.yml")
+    opt = lpmm.optim.AdamW(params, fused=False, qconfig=cfg, **H)
+    states = [oracle.NonFusedState(s, v_scale_type="rank1") for s in shapes]
+    for step in range(1, 4):
+        grads = [(rng.standard_normal(s) * 1e-3).astype(np.float32) for s in shapes]
+        for p, g in zip(params, grads):
+            p.grad = to_dev(g)
+        opt.step()
+        before = [h.copy() for h in host]
+        for h, g, st in zip(host, grads, states):
+            oracle.nonfused_step(h, g, st, qm, qv, H["lr"], 0.9, 0.999, H["eps"], H["weight_decay"])
+        torch.cuda.synchronize()
+        for i, (p, h, st, b) in enumerate(zip(params, host, states, before)):
+            what = f"tensor {i} {shapes[i]} step {step}"
+            s = opt.state[p]
+            n = h.size
+            oh = s["exp_avg_sq_qstate"]["overhead"]
+            assert oh["dim"] == len(shapes[i]) and oh["scaled_shape"] == torch.Size(shapes[i]) and oh["max1"] is None
+            for d, (got, want) in enumerate(zip(oh["max_dims"], st.v[1])):
+                keep = [1] * len(shapes[i])
+                keep[d] = shapes[i][d]
+                assert tuple(got.shape) == tuple(keep)
+                np.testing.assert_array_equal(to_np(got).reshape(-1), want, err_msg=f"statistics {d} of {what}")
+            np.testing.assert_array_equal(to_np(s["exp_avg"]).view(np.uint8)[: (n + 1) // 2], st.m[0][: (n + 1) // 2])
+            np.testing.assert_array_equal(to_np(s["exp_avg_sq"]).view(np.uint8)[: (n + 1) // 2], st.v[0][: (n + 1) // 2])
+            assert_rel(to_np(p.detach()), h, "p of " + what, scale=b)
+
+
+STRIDED_MODES = {
+    "rank1": dict(fused=False, qconfig="default.yml"),
+    "group": dict(fused=False, qconfig="2nd_moment_group_128.yml"),
+    "factored": dict(fused=False, factor_second_moment=True),
+    "factored_on_fused": dict(fused=True, factor_second_moment=True),
+}
+
+
+@pytest.mark.parametrize("mode", sorted(STRIDED_MODES))
+def test_strided_parameters_equal_their_contiguous_twins(mode):
+    """Non-contiguous parameters and gradients on the non-fused paths (the reference's PyTorch
+    ops take any strides, lpmm/optim/adamw.py:394-422, and its quantiser flattens in index
+    order): the same values in a contiguous tensor must give the same bytes, the strided
+    parameter is updated in its own storage, and the states record the strides the reference
+    records (those of zeros_like(p, preserve_format))."""
+    import lpmm
+
+    kw = dict(STRIDED_MODES[mode])
+    if "qconfig" in kw:
+        kw["qconfig"] = os.path.join(os.path.dirname(lpmm.config.__file__), "configs", kw["qconfig"])
+    rng = np.random.default_rng(8)
+    dev = "cuda"
+    # a transposed matrix (dense, permuted strides), every other column of a wider matrix (gaps),
+    # a permuted 3-D tensor, a strided small vector with fp32 states, a transposed ragged matrix
+    bases = [to_dev((rng.standard_normal((256, 96)) * 0.02).astype(np.float32)),
+             to_dev((rng.standard_normal((64, 512)) * 0.02).astype(np.float32)),
+             to_dev((rng.standard_normal((40, 6, 64)) * 0.02).astype(np.float32)),
+             to_dev((rng.standard_normal((4000,)) * 0.02).astype(np.float32)),
+             to_dev((rng.standard_normal((130, 70)) * 0.02).astype(np.float32))]
+    views = [lambda t: t.t(), lambda t: t[:, ::2], lambda t: t.permute(1, 0, 2), lambda t: t[::2], lambda t: t.t()]
+    if mode == "factored":
+        bases, views = bases[:2] + bases[3:], views[:2] + views[3:]
+    elif mode == "factored_on_fused":
+        # tensors that are not factored go to the fused operator there, which demands contiguous
+        # operands in the reference as well (lpmm/cpp_extension/common.h:4)
+        bases, views = bases[:2] + bases[4:], views[:2] + views[4:]
+    strided = [torch.nn.Parameter(v(b)) for v, b in zip(views, bases)]
+    assert not any(p.is_contiguous() for p in strided)
+    twins = [torch.nn.Parameter(p.detach().contiguous().clone()) for p in strided]
+    opt_s = lpmm.optim.AdamW(strided, **H, **kw)
+    opt_t = lpmm.optim.AdamW(twins, **H, **kw)
+    for step in range(3):
+        for i, (p, t) in enumerate(zip(strided, twins)):
+            g = to_dev((rng.standard_normal(tuple(p.shape)) * 1e-3).astype(np.float32))
+            t.grad = g
+            if i % 2 == 0:  # a gradient with the parameter's strides, else a contiguous one
+                gs = torch.empty_strided(p.shape, p.stride(), device=dev)
+                gs.copy_(g)
+                p.grad = gs
+            else:
+                p.grad = g.clone()
+        opt_s.step()
+        opt_t.step()
+    torch.cuda.synchronize()
+    for i, (p, t, v, b) in enumerate(zip(strided, twins, views, bases)):
+        assert not p.is_contiguous() and p.data_ptr() == b.data_ptr()
+        assert torch.equal(p.detach(), t.detach()), f"parameter {i} differs from its contiguous twin"
+        assert torch.equal(v(b), t.detach()), f"parameter {i}: the strided storage was not updated"
+        ss, st = opt_s.state[p], opt_t.state[t]
+        assert ss.keys() == st.keys()
+        for name in ("exp_avg", "exp_avg_sq", "exp_avg_sq_row", "exp_avg_sq_col"):
+            if name in ss:
+                assert ss[name].shape == st[name].shape
+                n = ss[name].numel() - (1 if ss[name].dtype == torch.int8 else 0)  # the byte past the codes
+                assert torch.equal(ss[name].reshape(-1)[:n], st[name].reshape(-1)[:n]), f"{name} of parameter {i}"
+        for name in ("exp_avg", "exp_avg_sq"):
+            oh_s, oh_t = ss[f"{name}_qstate"]["overhead"], st.get(f"{name}_qstate", {}).get("overhead", {})
+            for key in ("max1", "max_dims"):
+                if oh_s.get(key) is not None:
+                    a = oh_s[key] if isinstance(oh_s[key], list) else [oh_s[key]]
+                    c = oh_t[key] if isinstance(oh_t[key], list) else [oh_t[key]]
+                    assert all(torch.equal(x, y) for x, y in zip(a, c)), f"{key} of {name} of parameter {i}"
+            if "stride" in oh_s:
+                want = torch.empty_like(p, device="meta", memory_format=torch.preserve_format).stride()
+                assert tuple(oh_s["stride"]) == tuple(want)
+    # dequantising through the public function restores the recorded strides
+    import lpmm.functional as F
+
+    s0 = opt_s.state[strided[0]]
+    md = opt_s.get_qmetadata_by_state_name("exp_avg")
+    m = F.vectorwise_dequant(s0["exp_avg"], qmap=s0["exp_avg_qstate"]["qmap"], shape=strided[0].shape,
+                             **{**s0["exp_avg_qstate"]["overhead"], **md})
+    assert m.stride() == strided[0].stride() and m.shape == strided[0].shape
+
+
 @pytest.mark.parametrize("fused", [False, True])
 def test_factored_optimizer_matches_oracle(oracle, qmaps, fused):
     import lpmm

@@ -108,6 +108,82 @@ def test_rank1(oracle, qmaps, shape):
         np.testing.assert_array_equal(to_np(out), oracle.dequant_rank1(want_codes, want_row, want_col, qmap, r, c))
 
 
+ND_SHAPES = [(6, 50, 40), (64, 64, 3, 3), (5, 7, 2049), (3, 4, 5, 6, 7), (2, 1, 3000, 2), (2, 2, 2, 2, 2, 2, 2, 33),
+             (3, 1, 1, 5000), (4, 512, 1024), (7, 4100)]
+
+
+@pytest.mark.parametrize("with_work", [False, True])
+@pytest.mark.parametrize("shape", ND_SHAPES)
+def test_rank1_nd(oracle, qmaps, shape, with_work):
+    """Rank-1 statistics of tensors of up to 8 dimensions (one-pass kernel, and the 2-D kernel
+    plus a fold of its row maxima when a workspace is passed), the row scale derived from them
+    and the 2-D quantise / dequantise kernels on the flattened view, against the N-D oracle."""
+    import ctypes
+
+    lib = _lib()
+    rng = np.random.default_rng(sum(shape) + len(shape))
+    n = int(np.prod(shape))
+    nd = len(shape)
+    shape_arr = (ctypes.c_int64 * nd)(*shape)
+    for qmap, bits, x in ((qmaps[1], 4, _unsigned(rng, n).reshape(shape)), (qmaps[0], 4, _signed(rng, n).reshape(shape)),
+                          (oracle.create_pow_map(5, False, 1), 5, _unsigned(rng, n).reshape(shape))):
+        x[(0,) * nd] = 0.0
+        x[(slice(None),) * (nd - 1) + (shape[-1] - 1,)] = 0.0  # an all-zero slice of the last dimension: scale 0
+        want_stats = oracle.rank1_stats_nd(x)
+        dx, dq = to_dev(x), to_dev(qmap)
+        stats = [torch.full((d,), -1.0, dtype=torch.float32, device="cuda") for d in shape]
+        ptrs = (ctypes.c_void_p * nd)(*[t.data_ptr() for t in stats])
+        work = torch.full((n // shape[-1],), -1.0, dtype=torch.float32, device="cuda") if with_work else None
+        st = lib.lpmm_rank1_stats_nd(dx.data_ptr(), nd, shape_arr, ptrs, work.data_ptr() if with_work else None,
+                                     _stream())
+        assert st == 0
+        torch.cuda.synchronize()
+        for i, (got, want) in enumerate(zip(stats, want_stats)):
+            np.testing.assert_array_equal(to_np(got), want, err_msg=f"statistics of dimension {i}")
+        rows, cols = n // shape[-1], shape[-1]
+        row_scale = torch.full((rows,), -1.0, dtype=torch.float32, device="cuda")
+        assert lib.lpmm_rank1_row_scale_nd(ptrs, nd, shape_arr, row_scale.data_ptr(), _stream()) == 0
+        torch.cuda.synchronize()
+        lead = oracle.rank1_scale_nd(want_stats[:-1], shape[:-1]) if nd > 1 else None
+        np.testing.assert_array_equal(to_np(row_scale), lead.reshape(-1))
+        want_codes = oracle.quant_rank1_nd_bits(x, want_stats, qmap, bits)
+        codes = torch.full((want_codes.size,), 0x55, dtype=torch.uint8, device="cuda")
+        out = torch.empty(shape, dtype=torch.float32, device="cuda")
+        if bits == 4:
+            assert lib.lpmm_quant_rank1(dx.data_ptr(), rows, cols, row_scale.data_ptr(), stats[-1].data_ptr(),
+                                        dq.data_ptr(), codes.data_ptr(), _stream()) == 0
+            assert lib.lpmm_dequant_rank1(codes.data_ptr(), row_scale.data_ptr(), stats[-1].data_ptr(), dq.data_ptr(),
+                                          rows, cols, out.data_ptr(), _stream()) == 0
+        else:
+            assert lib.lpmm_quant_rank1_bits(dx.data_ptr(), rows, cols, row_scale.data_ptr(), stats[-1].data_ptr(),
+                                             dq.data_ptr(), bits, codes.data_ptr(), _stream()) == 0
+            assert lib.lpmm_dequant_rank1_bits(codes.data_ptr(), row_scale.data_ptr(), stats[-1].data_ptr(),
+                                               dq.data_ptr(), bits, rows, cols, out.data_ptr(), _stream()) == 0
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(to_np(codes), want_codes)
+        np.testing.assert_array_equal(to_np(out), oracle.dequant_rank1_nd_bits(want_codes, want_stats, qmap, bits, shape))
+
+
+def test_rank1_nd_rejects_bad_arguments():
+    import ctypes
+
+    lib = _lib()
+    x = torch.zeros(64, device="cuda")
+    stats = [torch.zeros(4, device="cuda") for _ in range(3)]
+    ptrs = (ctypes.c_void_p * 3)(*[t.data_ptr() for t in stats])
+    shape = (ctypes.c_int64 * 3)(4, 4, 4)
+    assert lib.lpmm_rank1_stats_nd(x.data_ptr(), 0, shape, ptrs, None, _stream()) == 5
+    assert lib.lpmm_rank1_stats_nd(x.data_ptr(), 9, shape, ptrs, None, _stream()) == 5
+    assert lib.lpmm_rank1_stats_nd(None, 3, shape, ptrs, None, _stream()) == 1
+    assert lib.lpmm_rank1_stats_nd(x.data_ptr(), 3, (ctypes.c_int64 * 3)(4, 0, 4), ptrs, None, _stream()) == 3
+    assert lib.lpmm_rank1_stats_nd(x.data_ptr(), 3, (ctypes.c_int64 * 3)(2 ** 31, 2 ** 31, 4), ptrs, None, _stream()) == 3
+    assert lib.lpmm_rank1_stats_nd(x.data_ptr(), 3, shape, (ctypes.c_void_p * 3)(stats[0].data_ptr(), None, None), None,
+                                   _stream()) == 1
+    assert lib.lpmm_rank1_row_scale_nd(ptrs, 1, shape, x.data_ptr(), _stream()) == 5
+    assert lib.lpmm_rank1_row_scale_nd(ptrs, 3, shape, None, _stream()) == 1
+    torch.cuda.synchronize()
+
+
 def test_functional_round_trip_metadata(oracle, qmaps):
     """vectorwise_quant / vectorwise_dequant: layout, metadata and values as the reference
     defines them (lpmm/functional.py:26-151)."""
@@ -150,7 +226,7 @@ def test_functional_round_trip_metadata(oracle, qmaps):
     back = F.vectorwise_dequant(qb, qmap=qv, shape=db.shape, **{**gen, **md_v})
     np.testing.assert_array_equal(to_np(back), oracle.dequant_group(to_np(qb).view(np.uint8), to_np(gen["max1"]), qmaps[1], b.size))
 
-    # 3-D rank1 (statistics through PyTorch reductions, search + pack in HIP)
+    # 3-D rank1: N-D statistics kernels, then the 2-D kernels on the (6*50, 40) view
     w = _unsigned(rng, 6 * 50 * 40).reshape(6, 50, 40)
     dw = to_dev(w)
     qw, gen = F.vectorwise_quant(dw, qmap=qv, shape=dw.shape, **md_v)
@@ -163,6 +239,9 @@ def test_functional_round_trip_metadata(oracle, qmaps):
     back = F.vectorwise_dequant(qw, qmap=qv, shape=dw.shape, **{**gen, **md_v})
     want = oracle.unpack_nonlinear_4bit(to_np(qw).view(np.uint8), qmaps[1], w.size).reshape(w.shape) * st
     np.testing.assert_array_equal(to_np(back), want.astype(np.float32))
+    assert gen["dim"] == 3 and [tuple(m.shape) for m in gen["max_dims"]] == [(6, 1, 1), (1, 50, 1), (1, 1, 40)]
+    for m, want_st in zip(gen["max_dims"], oracle.rank1_stats_nd(w)):
+        np.testing.assert_array_equal(to_np(m).reshape(-1), want_st)
 
 
 def test_shim_pack_unpack_signatures(oracle, qmaps):

@@ -205,6 +205,70 @@ def test_rank1_equals_numpy_and_special_cases(oracle, qmaps):
     assert nibbles(oracle.quant_rank1(y, row, col, qv), y.size).reshape(20, 30)[3, 7] == 15
 
 
+def test_rank1_nd_reduces_to_2d_and_to_library_ops(oracle, qmaps):
+    """The N-D restatement of rank-1 scaling: on a 2-D tensor it is the (pinned) 2-D C
+    functions bit for bit; on 3-D and 4-D tensors its statistics and scale are what the
+    reference's op sequence gives when PyTorch's CPU kernels run it (max over every other
+    dimension with keepdim, then a chain of torch.min: lpmm/functional.py:503-531), and what a
+    loop over all indices gives; a separable tensor a_i b_j c_k has the factors as statistics."""
+    qv = qmaps[1]
+    rng = np.random.default_rng(11)
+    x2 = (rng.standard_normal((37, 53)) ** 2).astype(f32)
+    x2[4, :] = 0.0
+    stats = oracle.rank1_stats_nd(x2)
+    row, col = oracle.rank1_stats(x2)
+    assert np.array_equal(stats[0], row) and np.array_equal(stats[1], col)
+    codes = oracle.quant_rank1_nd_bits(x2, stats, qv, 4)
+    assert np.array_equal(codes, oracle.quant_rank1(x2, row, col, qv))
+    assert np.array_equal(oracle.dequant_rank1_nd_bits(codes, stats, qv, 4, x2.shape),
+                          oracle.dequant_rank1(codes, row, col, qv, 37, 53))
+    for shape in [(3, 5, 7), (2, 3, 4, 5), (6, 1, 9)]:
+        x = (rng.standard_normal(shape) ** 2).astype(f32)
+        x[(0,) * len(shape)] = 0.0
+        stats = oracle.rank1_stats_nd(x)
+        scale = oracle.rank1_scale_nd(stats, shape)
+        # the reference's op sequence on PyTorch CPU kernels
+        t = torch.from_numpy(x).abs()
+        max_dims = []
+        for i in range(t.dim()):
+            red = t
+            for d in range(t.dim()):
+                if d != i:
+                    red = red.max(dim=d, keepdim=True).values
+            max_dims.append(red)
+        ts = max_dims[0].clone()
+        for other in max_dims[1:]:
+            ts = torch.min(ts, other)
+        for st, md in zip(stats, max_dims):
+            assert np.array_equal(st, md.numpy().reshape(-1))
+        assert np.array_equal(scale, ts.numpy())
+        # a loop over all indices
+        want = [np.zeros(d, f32) for d in shape]
+        for idx in np.ndindex(*shape):
+            for i, j in enumerate(idx):
+                want[i][j] = max(want[i][j], abs(x[idx]))
+        for st, w in zip(stats, want):
+            assert np.array_equal(st, w)
+        for idx in np.ndindex(*shape):
+            assert scale[idx] == min(want[i][j] for i, j in enumerate(idx))
+        # codes: the map search on x / scale, zero padding to the pack group
+        codes = oracle.quant_rank1_nd_bits(x, stats, qv, 4)
+        normed = np.zeros(2048, f32)
+        with np.errstate(invalid="ignore"):
+            normed[: x.size] = (x / scale).reshape(-1)
+        assert np.array_equal(nibbles(codes, 2048), oracle.qmapping(qv, normed))
+        back = oracle.dequant_rank1_nd_bits(codes, stats, qv, 4, shape)
+        assert np.array_equal(back, (qv[nibbles(codes, x.size)].reshape(shape) * scale).astype(f32))
+    a, b, c = rng.random(6).astype(f32), rng.random(5).astype(f32), rng.random(4).astype(f32)
+    a[2] = b[0] = c[3] = 1.0
+    # powers of two keep the products exact
+    a, b, c = (np.exp2(np.floor(np.log2(v))).astype(f32) for v in (a, b, c))
+    y = (a[:, None, None] * b[None, :, None] * c[None, None, :]).astype(f32)
+    stats = oracle.rank1_stats_nd(y)
+    assert np.array_equal(stats[0], a) and np.array_equal(stats[1], b) and np.array_equal(stats[2], c)
+    assert nibbles(oracle.quant_rank1_nd_bits(y, stats, qv, 4), y.size).reshape(y.shape)[2, 0, 3] == 15
+
+
 def test_nonfused_c_update_follows_torch_cpu_ops(oracle, qmaps):
     """The C restatement of the non-fused step against the same op sequence run by PyTorch's
     CPU kernels (library ops), on a 2-D tensor, group-128 m and rank-1 v, 4 steps."""
