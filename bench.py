@@ -171,7 +171,7 @@ def cpu_baseline(torch, steps=10):
 
 
 PROBE_KINDS = {"read": (0, 4.0), "write": (1, 4.0), "copy": (2, 8.0), "update_2r1w": (3, 12.0),
-               "fused_mix": (4, BYTES_PER_PARAM_4BIT)}
+               "fused_mix": (4, BYTES_PER_PARAM_4BIT), "fused_mix_dword_codes": (5, BYTES_PER_PARAM_4BIT)}
 # dynamic LDS per workgroup -> workgroups resident per CU (160 KB of LDS per CU)
 PROBE_RESIDENCY = {8: 0, 6: 26 * 1024, 5: 30 * 1024, 4: 40 * 1024, 3: 53 * 1024, 2: 80 * 1024}
 
@@ -222,6 +222,9 @@ def calibrate(torch, lib, n=1 << 29, iters=5, full=False):
     mix = {str(r): round(rate("fused_mix", PROBE_RESIDENCY[r]), 1) for r in res_list}
     out["fused_mix_by_workgroups_per_cu"] = mix
     out["fused_mix_best"] = max(mix.values())
+    if full:  # the same streams with one 4-byte code access per lane and state instead of two 2-byte ones
+        out["fused_mix_dword_codes_by_workgroups_per_cu"] = {
+            str(r): round(rate("fused_mix_dword_codes", PROBE_RESIDENCY[r]), 1) for r in res_list}
     del a, b, c0, c1, s0, s1
     return out
 
@@ -320,10 +323,14 @@ def _time_events(torch, fn, iters):
 
 
 def run_quant_roundtrip(torch, args):
-    """Stand-alone quantise + dequantise round trip on 2^26 fp32 values (4-bit packed output):
-    group-128 with the signed dynamic-exponent map (N(0,1) with 0.1 % outliers x50), group-128
-    with the unsigned linear map (|N|^2), rank-1 on the unsigned data viewed 8192 x 8192."""
+    """Stand-alone quantise + dequantise round trip on 2^26 fp32 values (--bits wide codes, 4 by
+    default: packed two per byte; 3 and 5..8 take a byte each): group-128 with the signed
+    dynamic-exponent map (N(0,1) with 0.1 % outliers x50), group-128 with the unsigned linear
+    map (|N|^2), rank-1 on the unsigned data viewed 8192 x 8192 and 64 x 1024 x 1024."""
     import lpmm.functional as F
+
+    b = args.bits
+    code_bytes = F.storage_bits(b) / 8.0
 
     dev = torch.device("cuda:0")
     n = 1 << 26
@@ -335,16 +342,21 @@ def run_quant_roundtrip(torch, args):
     signed[idx] *= 50.0
     g.manual_seed(3)
     unsigned = torch.randn(n, device=dev, generator=g) ** 2
-    qm = F.create_general_qmap("nonlinear", 4, True).to(dev)
-    qv = F.create_general_qmap("power-1", 4, False).to(dev)
-    md_m = dict(b=4, scale_type="group", quant_type="nonlinear", round_type="real-nearest", gp_sz=128, signed=True)
-    md_vg = dict(b=4, scale_type="group", quant_type="power-1", round_type="real-nearest", gp_sz=128, signed=False)
+    qm = F.create_general_qmap("nonlinear", b, True).to(dev)
+    qv = F.create_general_qmap("power-1", b, False).to(dev)
+    md_m = dict(b=b, scale_type="group", quant_type="nonlinear", round_type="real-nearest", gp_sz=128, signed=True)
+    md_vg = dict(b=b, scale_type="group", quant_type="power-1", round_type="real-nearest", gp_sz=128, signed=False)
     md_vr = dict(md_vg, scale_type="rank1")
     variants = []
+    # bytes per value: 4 read or written as fp32, the code, a scale per 128 values; the rank-1
+    # quantiser reads the values twice (statistics, then normalise + search + pack)
+    one_pass, two_pass = 4 + code_bytes + 4 / 128, 8 + code_bytes
     for name, x, qmap, md, bytes_q, bytes_dq in (
-            ("group-128 signed DE map", signed, qm, md_m, 4.53125, 4.53125),
-            ("group-128 unsigned linear map", unsigned, qv, md_vg, 4.53125, 4.53125),
-            ("rank-1 8192x8192 unsigned linear map", unsigned.view(8192, 8192), qv, md_vr, 8.5, 4.5)):
+            ("group-128 signed DE map", signed, qm, md_m, one_pass, one_pass),
+            ("group-128 unsigned linear map", unsigned, qv, md_vg, one_pass, one_pass),
+            ("rank-1 8192x8192 unsigned linear map", unsigned.view(8192, 8192), qv, md_vr, two_pass, 4 + code_bytes),
+            ("rank-1 64x1024x1024 unsigned linear map", unsigned.view(64, 1024, 1024), qv, md_vr, two_pass,
+             4 + code_bytes)):
         qx, gen = F.vectorwise_quant(x, qmap=qmap, shape=x.shape, **md)
         kw = {**gen, **md}
         back = F.vectorwise_dequant(qx, qmap=qmap, shape=x.shape, **kw)
@@ -355,12 +367,13 @@ def run_quant_roundtrip(torch, args):
                          "quant_gbs": n * bytes_q / t_q / 1e6, "dequant_gbs": n * bytes_dq / t_dq / 1e6, "relerr": relerr})
     v0 = variants[0]
     print(json.dumps({
-        "metric": "4-bit quantize+dequantize round trip (group-128, signed map): values/sec, 1 MI355X",
+        "metric": f"{b}-bit quantize+dequantize round trip (group-128, signed map): values/sec, 1 MI355X",
         "value": v0["roundtrip_values_per_s"], "unit": "values/s", "n_gpus": 1, "steps": args.steps, "warmup": 2,
         "ms_per_step": v0["quant_ms"] + v0["dequant_ms"], "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "quantize+dequantize round trip on 2^26 fp32 values, 4-bit packed output"},
-        "roofline": {"bound": "hbm", "kernel": "lpmm::quant_group_kernel", "achieved": v0["quant_gbs"],
+        "config": {"workload": f"quantize+dequantize round trip on 2^26 fp32 values, {b}-bit codes"},
+        "roofline": {"bound": "hbm", "kernel": "lpmm::quant_group_kernel" if b == 4 else "lpmm::quant_group_bits_kernel",
+                     "achieved": v0["quant_gbs"],
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": v0["quant_gbs"] / HBM_PEAK_GBS, "traffic": None},
         "variants": variants}))
 
@@ -443,6 +456,7 @@ def main():
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--workload", default="llama7b", choices=sorted(WORKLOADS) + ["quant64m", "factored", "nonfused_group", "nonfused_rank1", "calibrate"])
+    ap.add_argument("--bits", type=int, default=4, choices=range(1, 9), help="code width of --workload quant64m")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--interleaved-grads", action="store_true",
                     help="allocate each gradient right behind its parameter instead of all parameters first")

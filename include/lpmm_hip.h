@@ -390,10 +390,15 @@ int lpmm_selftest_encoders(unsigned long long *counts, void *stream);
  *   LPMM_PROBE_FUSED_MIX  the seven streams of lpmm_adamw4bit_step: a, b read, a written,
  *                         codes0/1 (n/2 bytes each) and scale0/1 (n/128 floats each) read and
  *                         written                                 14.125 B/element
- * n: a multiple of 2048; a, b: fp32[n], 16-byte aligned.  lds_bytes (0..163840) of dynamic LDS
+ *   LPMM_PROBE_FUSED_MIX_DWORD  the same with one 4-byte code access per lane and state
+ *                         instead of two 2-byte ones              14.125 B/element
+ * n: a multiple of 2048; a, b: fp32[n], 16-byte aligned; code arrays 4-byte aligned.  lds_bytes (0..163840) of dynamic LDS
  * that the kernels never touch cap the workgroups resident per CU at floor(160 KB / lds_bytes)
  * (0: the hardware's own limit of 8).  Buffers a kind does not use may be NULL. */
-enum { LPMM_PROBE_READ = 0, LPMM_PROBE_WRITE = 1, LPMM_PROBE_COPY = 2, LPMM_PROBE_UPDATE = 3, LPMM_PROBE_FUSED_MIX = 4 };
+enum {
+    LPMM_PROBE_READ = 0, LPMM_PROBE_WRITE = 1, LPMM_PROBE_COPY = 2, LPMM_PROBE_UPDATE = 3, LPMM_PROBE_FUSED_MIX = 4,
+    LPMM_PROBE_FUSED_MIX_DWORD = 5
+};
 int lpmm_stream_probe(int kind, float *a, const float *b, uint8_t *codes0, uint8_t *codes1, float *scale0,
                       float *scale1, int64_t n, int64_t lds_bytes, void *stream);
 

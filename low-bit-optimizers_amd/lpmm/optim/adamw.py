@@ -272,7 +272,10 @@ class AdamW(LowBitOptimizer):
             _native.check(st, "fused fp16 AdamW step")
 
     @staticmethod
-    def _check_fp32_cuda(p, grad, why="quantised states and the non-fused path are implemented for float32 only",
+    def _check_fp32_cuda(p, grad, why="quantised states and the non-fused path compute in float32 only (the "
+                         "reference runs other types there through PyTorch's kernels of that type, one rounding "
+                         "per op: lpmm/optim/adamw.py:394-434, lpmm/functional.py:184-203); keep float32 master "
+                         "weights, or use fused=True for float16 tensors whose states are not quantised",
                          strided_ok=False):
         if (p.dtype is torch.float32 and grad.dtype is torch.float32 and p.is_cuda and grad.is_cuda
                 and (strided_ok or (p.is_contiguous() and grad.is_contiguous()))):
