@@ -6,11 +6,12 @@
 // (:476, :550), written as 0 here.
 //
 // The 4-bit kernels of quantize.hip stay the fast path for the width the optimizers use by
-// default; these kernels serve the other widths (lpmm/configs/default_{5,6,7,8}b.yml) with the
-// same flattened work layout: a lane owns 8 consecutive values, a 256-thread workgroup one
-// 2048-value pack group.  The map (2^bits entries) sits in LDS and the code is found by the
-// reference's own search (upper bound, then the midpoint test, :397-427), so maps with
-// repeated entries behave as there.
+// default; these kernels serve the other widths (lpmm/configs/default_{5,6,7,8}b.yml).  The
+// flat kernels let a lane own 8 consecutive values, a 256-thread workgroup one 2048-value pack
+// group; the widths with one code per byte also have kernels in the row layout of the 4-bit
+// path (further down) for whole tiles.  The map (2^bits entries) sits in LDS and the code is
+// found by the reference's own search (upper bound, then the midpoint test, :397-427), so maps
+// with repeated entries behave as there.
 #include "lpmm_codec.hpp"
 
 namespace lpmm {
@@ -19,7 +20,7 @@ constexpr int kBThreads = 256;
 constexpr int kBElts = 8;
 constexpr int kBTile = kBThreads * kBElts;  // 2048
 
-__device__ __forceinline__ int codes_per_byte(int bits) { return (bits == 1 || bits == 2 || bits == 4) ? 8 / bits : 1; }
+__host__ __device__ __forceinline__ int codes_per_byte(int bits) { return (bits == 1 || bits == 2 || bits == 4) ? 8 / bits : 1; }
 
 // the map, 2^bits floats, into LDS; the caller synchronises
 __device__ __forceinline__ void fill_map(float *lds_map, const float *__restrict__ qmap, int bits)
@@ -31,41 +32,101 @@ __device__ __forceinline__ void fill_map(float *lds_map, const float *__restrict
 // quantize_bsearch<false> (quantization_kernel.cu:397-427) as the stored code, without a data
 // dependent branch.  The reference returns 0 for x <= q[0] and N-1 for q[N-1] <= x; otherwise it
 // finds lo = the first entry above x (upper bound) and answers lo or lo-1 by the midpoint test
-// mid = (q[lo-1] + q[lo]) * 0.5f < x.  Here the upper bound of the non-decreasing map (repeated
-// entries included) is built from its bits, one compare per step, every lane the same `bits`
-// steps; the two ends and NaN are selects afterwards.  For NaN the reference's search ends at
-// lo = 0 and returns -1, which it casts to uint8_t (one code per byte: 255) or masks (packed:
-// the all-ones code).
-__device__ __forceinline__ uint32_t search_code(const float *lds_map, int bits, float x)
+// mid = (q[lo-1] + q[lo]) * 0.5f < x.  For NaN its search ends at lo = 0 and returns -1, which it
+// casts to uint8_t (one code per byte: 255) or masks (packed: the all-ones code).
+//
+// Here the upper bound among the first N-1 entries of the non-decreasing map (repeated entries
+// included) comes from a descent through the entries in breadth-first order: node i of the
+// perfect tree over q[0..N-2] holds its in-order entry, i = 2i + (node <= x) for `bits` levels,
+// and i - N is the number of entries <= x.  A binary search over the sorted array would read, at
+// every level, entries that are a power of two apart -- all in the same LDS bank; in
+// breadth-first order the nodes of a level are neighbours, so up to 32 of them sit in 32
+// different banks (and lanes that read the same node share one access).  The midpoints are
+// formed once per workgroup with the reference's expression.
+struct SearchLds {
+    float tree[256];  // [1, N): breadth-first; [0]: q[0]
+    float mid[256];   // [1, N): (q[lo-1] + q[lo]) * 0.5f; [0]: q[N-1]
+};
+
+// the caller synchronises
+__device__ __forceinline__ void fill_search(SearchLds &t, const float *__restrict__ qmap, int bits)
 {
     const uint32_t n = 1u << bits;
-    // pos = number of entries among the first n-1 that are <= x: all entries before pos are <= x.
-    // The first three levels of the search look at the same seven entries in every lane (every
-    // eighth of the map): those compares run on registers (the entries are read once per kernel:
-    // the loads below do not depend on x and are hoisted), only the levels below them go to LDS
-    // with a per-lane address.
-    uint32_t pos = 0;
-    uint32_t step = n >> 1;
-    if (bits >= 3) {
-        const uint32_t eighth = n >> 3;
-        uint32_t cnt = 0;
-#pragma unroll
-        for (uint32_t j = 1; j < 8; ++j)
-            cnt += (lds_map[j * eighth - 1] <= x) ? 1u : 0u;
-        pos = cnt * eighth;
-        step = eighth >> 1;
+    for (uint32_t j = threadIdx.x; j < n; j += blockDim.x) {
+        if (j == 0) {
+            t.tree[0] = qmap[0];
+            t.mid[0] = qmap[n - 1];
+        } else {
+            const uint32_t level = 31u - (uint32_t)__clz((int)j);
+            const uint32_t k = j - (1u << level);
+            t.tree[j] = qmap[(((2u * k + 1u) << (bits - 1 - level))) - 1u];
+            t.mid[j] = (qmap[j - 1] + qmap[j]) * 0.5f;
+        }
     }
-    for (; step > 0; step >>= 1)
-        pos += (lds_map[pos + step - 1] <= x) ? step : 0u;
-    // pos <= n-1.  Inside the map's range the upper bound is pos (q[n-1] > x there), at least 1
+}
+
+__device__ __forceinline__ uint32_t search_code(const SearchLds &t, int bits, float x)
+{
+    const uint32_t n = 1u << bits;
+    uint32_t i = 1;
+    for (int l = 0; l < bits; ++l)
+        i = 2u * i + ((t.tree[i] <= x) ? 1u : 0u);
+    const uint32_t pos = i - n;  // entries among the first n-1 that are <= x
+    // Inside the map's range the upper bound is pos (q[n-1] > x there), at least 1
     const uint32_t lo = pos > 0 ? pos : 1u;
-    const float below = lds_map[lo - 1], above = lds_map[lo];
-    const float mid = (below + above) * 0.5f;
-    uint32_t code = (mid < x) ? lo : lo - 1u;
-    code = (lds_map[n - 1] <= x) ? n - 1u : code;
-    code = (x <= lds_map[0]) ? 0u : code;
+    uint32_t code = (t.mid[lo] < x) ? lo : lo - 1u;
+    code = (t.mid[0] <= x) ? n - 1u : code;
+    code = (x <= t.tree[0]) ? 0u : code;
     const uint32_t nan_code = codes_per_byte(bits) == 1 ? 255u : n - 1u;
     return (x != x) ? nan_code : code;
+}
+
+// The same for a lane's 8 values at once: the levels are the outer loop, so that the 8 reads of
+// a level are in flight together instead of 8 x `bits` dependent ones in a row.
+__device__ __forceinline__ void search_codes8(const SearchLds &t, int bits, const float (&x)[8], uint32_t (&code)[8])
+{
+    const uint32_t n = 1u << bits;
+    // a = byte offset of the node (4 i): one shift-or per level, no separate address computation
+    uint32_t a[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k)
+        a[k] = 4;
+    const char *tree = reinterpret_cast<const char *>(t.tree);
+    for (int l = 0; l < bits; ++l) {
+        // The eight compares write eight different scalar register pairs and the eight selects
+        // follow them: a select may read a mask two wait states after the compare that wrote it
+        // at the earliest, which the seven instructions in between supply (the compiler's own
+        // code goes through VCC and pays a pause per value and level).
+        float node[8];
+        uint64_t le[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k)
+            node[k] = *reinterpret_cast<const float *>(tree + a[k]);
+#pragma unroll
+        for (int k = 0; k < 8; ++k)
+            asm volatile("v_cmp_le_f32_e64 %0, %1, %2" : "=s"(le[k]) : "v"(node[k]), "v"(x[k]));
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            uint32_t step;
+            asm volatile("v_cndmask_b32_e64 %0, 0, 4, %1" : "=v"(step) : "s"(le[k]));
+            a[k] = (a[k] << 1) | step;
+        }
+    }
+    uint32_t i[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k)
+        i[k] = a[k] >> 2;
+    const float first = t.tree[0], last = t.mid[0];
+    const uint32_t nan_code = codes_per_byte(bits) == 1 ? 255u : n - 1u;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        const uint32_t pos = i[k] - n;
+        const uint32_t lo = pos > 0 ? pos : 1u;
+        uint32_t c = (t.mid[lo] < x[k]) ? lo : lo - 1u;
+        c = (last <= x[k]) ? n - 1u : c;
+        c = (x[k] <= first) ? 0u : c;
+        code[k] = (x[k] != x[k]) ? nan_code : c;
+    }
 }
 
 // codes of the lane's 8 values (base = index of the first, a multiple of 8) into the array
@@ -155,8 +216,8 @@ __global__ __launch_bounds__(kBThreads) void pack_bits_kernel(const float *__res
                                                               const float *__restrict__ qmap, int bits,
                                                               int64_t n_padded, uint8_t *__restrict__ out, bool vec)
 {
-    __shared__ float lds_map[256];
-    fill_map(lds_map, qmap, bits);
+    __shared__ SearchLds lds_map;
+    fill_search(lds_map, qmap, bits);
     __syncthreads();
     const int64_t base = ((int64_t)blockIdx.x * kBThreads + threadIdx.x) * kBElts;
     if (base == 0)
@@ -166,9 +227,7 @@ __global__ __launch_bounds__(kBThreads) void pack_bits_kernel(const float *__res
     float v[kBElts];
     load_values(x, base, n_padded, vec, v);
     uint32_t c[kBElts];
-#pragma unroll
-    for (int k = 0; k < kBElts; ++k)
-        c[k] = search_code(lds_map, bits, v[k]);
+    search_codes8(lds_map, bits, v, c);
     store_codes(out, base, bits, c);
 }
 
@@ -302,9 +361,9 @@ __global__ __launch_bounds__(THREADS) void quant_group_bits_kernel(const float *
                                                                    float *__restrict__ max1, int64_t n_groups,
                                                                    int64_t n_padded, bool vec)
 {
-    __shared__ float lds_map[256];
+    __shared__ SearchLds lds_map;
     __shared__ float s_row[THREADS / 16];
-    fill_map(lds_map, qmap, bits);
+    fill_search(lds_map, qmap, bits);
     const int64_t base = ((int64_t)blockIdx.x * THREADS + threadIdx.x) * kBElts;
     if (base == 0)
         codes[last_byte(n_padded, bits)] = 0;
@@ -346,9 +405,7 @@ __global__ __launch_bounds__(THREADS) void quant_group_bits_kernel(const float *
             for (int k = 0; k < kBElts; ++k)
                 xs[k] = v[k] / amax;
         }
-#pragma unroll
-        for (int k = 0; k < kBElts; ++k)
-            c[k] = search_code(lds_map, bits, xs[k]);
+        search_codes8(lds_map, bits, xs, c);
     } else {
         // padding added by the re-grouping to 2048: plain zeros, not divided by anything
         const uint32_t z = search_code(lds_map, bits, 0.0f);
@@ -389,8 +446,8 @@ __global__ __launch_bounds__(kBThreads) void quant_rank1_bits_kernel(const float
                                                                      uint8_t *__restrict__ codes, int64_t n_padded,
                                                                      bool vec)
 {
-    __shared__ float lds_map[256];
-    fill_map(lds_map, qmap, bits);
+    __shared__ SearchLds lds_map;
+    fill_search(lds_map, qmap, bits);
     __syncthreads();
     const int64_t base = ((int64_t)blockIdx.x * kBThreads + threadIdx.x) * kBElts;
     if (base == 0)
@@ -403,20 +460,21 @@ __global__ __launch_bounds__(kBThreads) void quant_rank1_bits_kernel(const float
     int64_t c = base - r * C;
     float rm = (base < n) ? rowmax[r] : 0.0f;
     uint32_t code[kBElts];
+    float xs[kBElts];
 #pragma unroll
     for (int k = 0; k < kBElts; ++k) {
-        float xs = 0.0f;  // padding added by the re-grouping to 2048
+        xs[k] = 0.0f;  // padding added by the re-grouping to 2048
         if (base + k < n) {
             const float cmx = colmax[c];
-            xs = v[k] / ((cmx < rm) ? cmx : rm);
+            xs[k] = v[k] / ((cmx < rm) ? cmx : rm);
             if (++c == C) {
                 c = 0;
                 ++r;
                 rm = (base + k + 1 < n) ? rowmax[r] : 0.0f;
             }
         }
-        code[k] = search_code(lds_map, bits, xs);
     }
+    search_codes8(lds_map, bits, xs, code);
     store_codes(codes, base, bits, code);
 }
 
@@ -451,6 +509,292 @@ __global__ __launch_bounds__(kBThreads) void dequant_rank1_bits_kernel(const uin
         }
     }
     store_values(out, base, n, vec, v);
+}
+
+// ---------------------------------------------------------------------------------------
+// Row layout for the widths that store one code per byte (3, 5, 6, 7, 8 bits): as in the 4-bit
+// kernels of quantize.hip, 16 lanes (one DPP row) own 128 consecutive values, lane l the values
+// [4l, 4l+4) and [64+4l, 64+4l+4), so that every 16-byte access of a row covers whole cache
+// lines and a lane's codes are two aligned 4-byte words.  These kernels take the part of a
+// tensor that consists of whole 2048-value tiles (whole 128-value groups for the dequantiser);
+// the flat kernels above take the rest and every packed width.
+// ---------------------------------------------------------------------------------------
+constexpr int kBRowsT = 2;       // tiles (passes of 16 groups) per workgroup: loads first, map afterwards
+constexpr int kBRank1Rows = 4;   // rows of one 2048-column chunk per workgroup of the rank-1 kernels
+
+__device__ __forceinline__ uint32_t bytes4(uint32_t a, uint32_t b, uint32_t c, uint32_t d)
+{
+    return a | (b << 8) | (c << 16) | (d << 24);
+}
+
+__device__ __forceinline__ void unpack8(const float4 &a, const float4 &b, float (&o)[kBElts])
+{
+    o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w;
+    o[4] = b.x; o[5] = b.y; o[6] = b.z; o[7] = b.w;
+}
+
+__device__ __forceinline__ void decode_bytes(uint32_t w0, uint32_t w1, uint32_t mask, const float *lds_map,
+                                             float (&v)[kBElts])
+{
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        v[k] = lds_map[((w0 >> (8 * k)) & 0xFFu) & mask];
+        v[4 + k] = lds_map[((w1 >> (8 * k)) & 0xFFu) & mask];
+    }
+}
+
+template <int T>
+__global__ __launch_bounds__(kBThreads) void quant_group_bits_rows_kernel(const float *__restrict__ x,
+                                                                          int64_t full_tiles, int rows_per_group,
+                                                                          const float *__restrict__ qmap, int bits,
+                                                                          uint8_t *__restrict__ codes,
+                                                                          float *__restrict__ max1, int64_t trailing)
+{
+    __shared__ SearchLds lds_map;
+    __shared__ float s_row[T][kBThreads / 16];
+    const int lane16 = threadIdx.x & 15, wrow = threadIdx.x >> 4;
+    const int64_t tile0 = (int64_t)blockIdx.x * T;
+    float v[T][kBElts];
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+        float4 a = make_float4(0.0f, 0.0f, 0.0f, 0.0f), b = a;
+        if (tile0 + t < full_tiles) {  // uniform over the workgroup
+            const float *p = x + (tile0 + t) * kBTile + wrow * kGroup + lane16 * 4;
+            a = load4(p);
+            b = load4(p + 64);
+        }
+        unpack8(a, b, v[t]);
+    }
+    fill_search(lds_map, qmap, bits);
+    if (blockIdx.x == 0 && threadIdx.x == 0)
+        codes[trailing] = 0;
+    float amax[T];
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+        float m = 0.0f;
+#pragma unroll
+        for (int k = 0; k < kBElts; ++k)
+            m = fmaxf(m, fabsf(v[t][k]));
+        amax[t] = row16_max(m);
+        if (lane16 == 0)
+            s_row[t][wrow] = amax[t];
+    }
+    lds_barrier();
+    const int first = wrow & ~(rows_per_group - 1);
+    const int64_t gp_sz = (int64_t)rows_per_group * kGroup;
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+        if (tile0 + t >= full_tiles)
+            break;
+        if (rows_per_group > 1) {
+            amax[t] = s_row[t][first];
+            for (int r = 1; r < rows_per_group; ++r)
+                amax[t] = fmaxf(amax[t], s_row[t][first + r]);
+        }
+        const int64_t base = (tile0 + t) * kBTile + wrow * kGroup;
+        if ((base % gp_sz) == 0 && lane16 == 0)
+            max1[base / gp_sz] = amax[t];
+        float xs[kBElts];
+        if (__all(rc_safe(amax[t]))) {
+            const float rc = rcp_exact(amax[t]);
+#pragma unroll
+            for (int k = 0; k < kBElts; ++k)
+                xs[k] = div_by_rc(v[t][k], amax[t], rc);
+        } else {
+#pragma unroll
+            for (int k = 0; k < kBElts; ++k)
+                xs[k] = v[t][k] / amax[t];
+        }
+        uint32_t c[kBElts];
+        search_codes8(lds_map, bits, xs, c);
+        uint32_t *cp = reinterpret_cast<uint32_t *>(codes + base) + lane16;
+        store_u32(cp, bytes4(c[0], c[1], c[2], c[3]));
+        store_u32(cp + 16, bytes4(c[4], c[5], c[6], c[7]));
+    }
+}
+
+template <int T>
+__global__ __launch_bounds__(kBThreads) void dequant_group_bits_rows_kernel(const uint8_t *__restrict__ codes,
+                                                                            const float *__restrict__ max1,
+                                                                            const float *__restrict__ qmap, int bits,
+                                                                            int64_t full_groups, int64_t rows_per_group,
+                                                                            float *__restrict__ out)
+{
+    __shared__ float lds_map[256];
+    const int lane16 = threadIdx.x & 15;
+    const int64_t row0 = (int64_t)blockIdx.x * T * (kBThreads / 16) + (threadIdx.x >> 4);
+    uint32_t w0[T], w1[T];
+    float s[T];
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+        const int64_t row = row0 + t * (kBThreads / 16);
+        w0[t] = w1[t] = 0;
+        s[t] = 0.0f;
+        if (row < full_groups) {
+            const uint32_t *cp = reinterpret_cast<const uint32_t *>(codes + row * kGroup) + lane16;
+            w0[t] = load_u32(cp);
+            w1[t] = load_u32(cp + 16);
+            s[t] = max1[row / rows_per_group];
+        }
+    }
+    fill_map(lds_map, qmap, bits);
+    lds_barrier();
+    const uint32_t mask = (1u << bits) - 1u;
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+        const int64_t row = row0 + t * (kBThreads / 16);
+        if (row >= full_groups)
+            continue;
+        float v[kBElts];
+        decode_bytes(w0[t], w1[t], mask, lds_map, v);
+        float *o = out + row * kGroup + lane16 * 4;
+        store4(o, make_float4(v[0] * s[t], v[1] * s[t], v[2] * s[t], v[3] * s[t]));
+        store4(o + 64, make_float4(v[4] * s[t], v[5] * s[t], v[6] * s[t], v[7] * s[t]));
+    }
+}
+
+// 'rank1' scaling, columns a multiple of 128: grid (2048-column chunks, groups of kBRank1Rows
+// rows).  A lane keeps the maxima of its 8 columns, and their correctly rounded reciprocals,
+// over the rows of its workgroup; x / min(rowmax, colmax) is then one multiply and two fmas that
+// give the correctly rounded quotient (|x| <= scale by construction) wherever all the scales of
+// the wave lie in the range in which the reciprocal is exact, and the plain division otherwise.
+__global__ __launch_bounds__(kBThreads) void quant_rank1_bits_rows128_kernel(const float *__restrict__ x, int64_t R,
+                                                                             int64_t C,
+                                                                             const float *__restrict__ rowmax,
+                                                                             const float *__restrict__ colmax,
+                                                                             const float *__restrict__ qmap, int bits,
+                                                                             uint8_t *__restrict__ codes,
+                                                                             int64_t n_padded)
+{
+    constexpr int T = kBRank1Rows;
+    __shared__ SearchLds lds_map;
+    const int64_t n = R * C;
+    const int lane16 = threadIdx.x & 15;
+    const int64_t r0 = (int64_t)blockIdx.y * T;
+    const int64_t c0 = (int64_t)blockIdx.x * kBTile + (int64_t)(threadIdx.x >> 4) * kGroup;
+    const bool live = c0 < C;  // uniform over the 16 lanes of a group
+    float4 a[T], b[T], ca, cb;
+    float rm[T];
+    if (live) {
+        const float *cmp = colmax + c0 + lane16 * 4;
+        ca = *reinterpret_cast<const float4 *>(cmp);
+        cb = *reinterpret_cast<const float4 *>(cmp + 64);
+#pragma unroll
+        for (int t = 0; t < T; ++t) {
+            if (r0 + t < R) {
+                const float *p = x + (r0 + t) * C + c0 + lane16 * 4;
+                a[t] = load4(p);
+                b[t] = load4(p + 64);
+                rm[t] = rowmax[r0 + t];
+            }
+        }
+    }
+    fill_search(lds_map, qmap, bits);
+    lds_barrier();
+    if (blockIdx.x == 0 && blockIdx.y == 0) {
+        // the padding added by the re-grouping to 2048: plain zeros, not divided by anything
+        const uint32_t z = search_code(lds_map, bits, 0.0f);
+        const uint32_t wz = bytes4(z, z, z, z);
+        for (int64_t i = n + (int64_t)threadIdx.x * 4; i < n_padded; i += kBThreads * 4)
+            *reinterpret_cast<uint32_t *>(codes + i) = wz;
+        if (threadIdx.x == 0)
+            codes[n_padded] = 0;
+    }
+    if (!live)
+        return;
+    float cmx[kBElts], crc[kBElts];
+    unpack8(ca, cb, cmx);
+    bool cols_safe = true;
+#pragma unroll
+    for (int k = 0; k < kBElts; ++k) {
+        crc[k] = rcp_exact(cmx[k]);
+        cols_safe = cols_safe && rc_safe(cmx[k]);
+    }
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+        if (r0 + t >= R)
+            break;
+        float v[kBElts], xs[kBElts];
+        unpack8(a[t], b[t], v);
+        if (__all(cols_safe && rc_safe(rm[t]))) {
+            const float rr = rcp_exact(rm[t]);
+#pragma unroll
+            for (int k = 0; k < kBElts; ++k) {
+                const bool by_col = cmx[k] < rm[t];
+                xs[k] = div_by_rc(v[k], by_col ? cmx[k] : rm[t], by_col ? crc[k] : rr);
+            }
+        } else {
+#pragma unroll
+            for (int k = 0; k < kBElts; ++k)
+                xs[k] = v[k] / ((cmx[k] < rm[t]) ? cmx[k] : rm[t]);
+        }
+        uint32_t c[kBElts];
+        search_codes8(lds_map, bits, xs, c);
+        uint32_t *cp = reinterpret_cast<uint32_t *>(codes + (r0 + t) * C + c0) + lane16;
+        store_u32(cp, bytes4(c[0], c[1], c[2], c[3]));
+        store_u32(cp + 16, bytes4(c[4], c[5], c[6], c[7]));
+    }
+}
+
+__global__ __launch_bounds__(kBThreads) void dequant_rank1_bits_rows128_kernel(const uint8_t *__restrict__ codes,
+                                                                               const float *__restrict__ rowmax,
+                                                                               const float *__restrict__ colmax,
+                                                                               const float *__restrict__ qmap, int bits,
+                                                                               int64_t R, int64_t C,
+                                                                               float *__restrict__ out)
+{
+    constexpr int T = kBRank1Rows;
+    __shared__ float lds_map[256];
+    const int lane16 = threadIdx.x & 15;
+    const int64_t r0 = (int64_t)blockIdx.y * T;
+    const int64_t c0 = (int64_t)blockIdx.x * kBTile + (int64_t)(threadIdx.x >> 4) * kGroup;
+    const bool live = c0 < C;
+    uint32_t w0[T], w1[T];
+    float rm[T];
+    float4 ca, cb;
+    if (live) {
+        const float *cmp = colmax + c0 + lane16 * 4;
+        ca = *reinterpret_cast<const float4 *>(cmp);
+        cb = *reinterpret_cast<const float4 *>(cmp + 64);
+#pragma unroll
+        for (int t = 0; t < T; ++t) {
+            if (r0 + t < R) {
+                const uint32_t *cp = reinterpret_cast<const uint32_t *>(codes + (r0 + t) * C + c0) + lane16;
+                w0[t] = load_u32(cp);
+                w1[t] = load_u32(cp + 16);
+                rm[t] = rowmax[r0 + t];
+            }
+        }
+    }
+    fill_map(lds_map, qmap, bits);
+    lds_barrier();
+    if (!live)
+        return;
+    float cmx[kBElts];
+    unpack8(ca, cb, cmx);
+    const uint32_t mask = (1u << bits) - 1u;
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+        if (r0 + t >= R)
+            break;
+        float v[kBElts];
+        decode_bytes(w0[t], w1[t], mask, lds_map, v);
+#pragma unroll
+        for (int k = 0; k < kBElts; ++k)
+            v[k] *= (cmx[k] < rm[t]) ? cmx[k] : rm[t];
+        float *o = out + (r0 + t) * C + c0 + lane16 * 4;
+        store4(o, make_float4(v[0], v[1], v[2], v[3]));
+        store4(o + 64, make_float4(v[4], v[5], v[6], v[7]));
+    }
+}
+
+// rank-1 row kernels: one code per byte, columns a multiple of 128, aligned operands, rows fit grid.y
+inline bool rank1_bits_rows_ok(int bits, const void *x, const void *colmax, const void *codes, int64_t rows,
+                               int64_t cols)
+{
+    return codes_per_byte(bits) == 1 && (cols % kGroup) == 0 && rows <= 65535LL * kBRank1Rows &&
+           (cols + kBTile - 1) / kBTile <= 0x7fffffffLL && aligned_to(x, 16) && aligned_to(colmax, 16) &&
+           aligned_to(codes, 4);
 }
 
 inline bool bits_ok(int bits) { return bits >= 1 && bits <= 8; }
@@ -546,6 +890,20 @@ extern "C" int lpmm_quant_group_bits(const float *x, int64_t n, int64_t gp_sz, c
     if (!tiles_for(n_groups * gp_sz, &tiles))
         return LPMM_ERR_SIZE;
     const int64_t n_padded = (int64_t)tiles * kBTile;
+    hipStream_t s = (hipStream_t)stream;
+    const int64_t full_tiles = n / kBTile;
+    if (codes_per_byte(bits) == 1 && gp_sz <= kBTile && full_tiles > 0 && aligned_to(x, 16)) {
+        // whole tiles in the row layout, the ragged end and the padding by the flat kernel
+        const uint32_t wgs = (uint32_t)((full_tiles + kBRowsT - 1) / kBRowsT);
+        hipLaunchKernelGGL(quant_group_bits_rows_kernel<kBRowsT>, dim3(wgs), dim3(kBThreads), 0, s, x, full_tiles,
+                           (int)(gp_sz / kGroup), qmap, bits, codes, max1, n_padded);
+        const int64_t done = full_tiles * kBTile;
+        if (done < n_padded)
+            hipLaunchKernelGGL(quant_group_bits_kernel<kBThreads>, dim3((uint32_t)((n_padded - done) / kBTile)),
+                               dim3(kBThreads), 0, s, x + done, n - done, (int)(gp_sz / kGroup), qmap, bits,
+                               codes + done, max1 + done / gp_sz, n_groups - done / gp_sz, n_padded - done, true);
+        return launch_status();
+    }
     if (gp_sz > kBTile)
         hipLaunchKernelGGL(quant_group_bits_kernel<2 * kBThreads>, dim3((tiles + 1) / 2), dim3(2 * kBThreads), 0,
                            (hipStream_t)stream, x, n, (int)(gp_sz / kGroup), qmap, bits, codes, max1, n_groups,
@@ -573,6 +931,18 @@ extern "C" int lpmm_dequant_group_bits(const uint8_t *codes, const float *max1, 
     uint32_t tiles;
     if (!tiles_for(n, &tiles))
         return LPMM_ERR_SIZE;
+    const int64_t full_groups = n / kGroup;
+    if (codes_per_byte(bits) == 1 && full_groups > 0 && aligned_to(out, 16)) {
+        constexpr int64_t per_wg = (int64_t)kBRowsT * (kBThreads / 16);
+        hipLaunchKernelGGL(dequant_group_bits_rows_kernel<kBRowsT>, dim3((uint32_t)((full_groups + per_wg - 1) / per_wg)),
+                           dim3(kBThreads), 0, (hipStream_t)stream, codes, max1, qmap, bits, full_groups,
+                           gp_sz / kGroup, out);
+        const int64_t done = full_groups * kGroup;
+        if (done < n)  // fewer than 128 values, all in the group of value `done`
+            hipLaunchKernelGGL(dequant_group_bits_kernel, dim3(1), dim3(kBThreads), 0, (hipStream_t)stream,
+                               codes + done, max1 + done / gp_sz, qmap, bits, n - done, gp_sz, out + done, false);
+        return launch_status();
+    }
     hipLaunchKernelGGL(dequant_group_bits_kernel, dim3(tiles), dim3(kBThreads), 0, (hipStream_t)stream, codes, max1,
                        qmap, bits, n, gp_sz, out, aligned_to(out, 16));
     return launch_status();
@@ -598,6 +968,12 @@ extern "C" int lpmm_quant_rank1_bits(const float *x, int64_t rows, int64_t cols,
     uint32_t tiles;
     if (!tiles_for(n, &tiles))
         return LPMM_ERR_SIZE;
+    if (rank1_bits_rows_ok(bits, x, colmax, codes, rows, cols)) {
+        const dim3 grid((uint32_t)((cols + kBTile - 1) / kBTile), (uint32_t)((rows + kBRank1Rows - 1) / kBRank1Rows));
+        hipLaunchKernelGGL(quant_rank1_bits_rows128_kernel, grid, dim3(kBThreads), 0, (hipStream_t)stream, x, rows, cols,
+                           rowmax, colmax, qmap, bits, codes, (int64_t)tiles * kBTile);
+        return launch_status();
+    }
     hipLaunchKernelGGL(quant_rank1_bits_kernel, dim3(tiles), dim3(kBThreads), 0, (hipStream_t)stream, x, n, cols,
                        rowmax, colmax, qmap, bits, codes, (int64_t)tiles * kBTile, aligned_to(x, 16));
     return launch_status();
@@ -623,6 +999,12 @@ extern "C" int lpmm_dequant_rank1_bits(const uint8_t *codes, const float *rowmax
     uint32_t tiles;
     if (!tiles_for(n, &tiles))
         return LPMM_ERR_SIZE;
+    if (rank1_bits_rows_ok(bits, out, colmax, codes, rows, cols)) {
+        const dim3 grid((uint32_t)((cols + kBTile - 1) / kBTile), (uint32_t)((rows + kBRank1Rows - 1) / kBRank1Rows));
+        hipLaunchKernelGGL(dequant_rank1_bits_rows128_kernel, grid, dim3(kBThreads), 0, (hipStream_t)stream, codes,
+                           rowmax, colmax, qmap, bits, rows, cols, out);
+        return launch_status();
+    }
     hipLaunchKernelGGL(dequant_rank1_bits_kernel, dim3(tiles), dim3(kBThreads), 0, (hipStream_t)stream, codes, rowmax,
                        colmax, qmap, bits, n, cols, out, aligned_to(out, 16));
     return launch_status();

@@ -51,7 +51,8 @@ def test_pack_unpack_bits(oracle, bits):
 
 
 @pytest.mark.parametrize("bits", BITS)
-@pytest.mark.parametrize("n,gp_sz", [(4097, 128), (2048 * 5 + 3, 512), (50000, 2048), (4096 * 3 + 17, 4096), (100, 128)])
+@pytest.mark.parametrize("n,gp_sz", [(4097, 128), (2048 * 5 + 3, 512), (50000, 2048), (4096 * 3 + 17, 4096), (100, 128),
+                                     (2048 * 4, 128), (2048 * 3 + 128 * 5, 256), (2048 * 7 + 130, 1024)])
 def test_quant_dequant_group_bits(oracle, bits, n, gp_sz):
     lib = _lib()
     rng = np.random.default_rng(n + bits)
@@ -100,7 +101,7 @@ def test_width_4_generic_kernels_equal_the_fast_path(oracle, qmaps):
 
 
 @pytest.mark.parametrize("bits", [2, 3, 5, 8])
-@pytest.mark.parametrize("shape", [(64, 80), (33, 1000), (257, 1029)])
+@pytest.mark.parametrize("shape", [(64, 80), (33, 1000), (257, 1029), (70, 256), (5, 2176), (130, 128)])
 def test_rank1_bits(oracle, bits, shape):
     lib = _lib()
     r, c = shape
@@ -110,6 +111,7 @@ def test_rank1_bits(oracle, bits, shape):
          ).astype(np.float32)
     x[3, :] = 0.0
     x[:, 7] = 0.0
+    x[4, :] *= 1e-25  # a row whose scales lie below the range of the reciprocal-based division
     rowmax, colmax = oracle.rank1_stats(x)
     want = oracle.quant_rank1_bits(x, rowmax, colmax, qmap, bits)
     dx, dq, dr, dc = to_dev(x), to_dev(qmap), to_dev(rowmax), to_dev(colmax)
