@@ -231,6 +231,27 @@ def test_state_dict_round_trip_keeps_packed_int8():
     with pytest.raises(ValueError):
         lpmm.optim.AdamW([torch.nn.Parameter(torch.zeros(2)), torch.nn.Parameter(torch.zeros(2))]).load_state_dict(sd)
 
+    # the reference stores its yacs CfgNode under 'qconfig' (lpmm/optim/optimizer.py:68-71): a dict subclass with
+    # attribute access, nested in itself.  Any such mapping is accepted and becomes this package's own node type.
+    class CfgNodeLike(dict):
+        def __getattr__(self, name):
+            if name in self:
+                return self[name]
+            raise AttributeError(name)
+
+    def wrap(value):
+        return CfgNodeLike({k: wrap(v) for k, v in value.items()}) if isinstance(value, dict) else value
+
+    sd3 = dict(sd, qconfig=wrap(sd["qconfig"]))
+    sd3["qconfig"]["QUANT"]["SQM"]["SCALE_TYPE"]["DEFAULT"] = "rank1"
+    opt3 = lpmm.optim.AdamW([torch.nn.Parameter(torch.zeros(64, 65, dtype=torch.float64))], fused=True)
+    opt3.load_state_dict(sd3)
+    assert type(opt3.qconfig) is lpmm.config.Node and type(opt3.qconfig.QUANT.SQM) is lpmm.config.Node
+    assert opt3.qconfig.QUANT.SQM.SCALE_TYPE.DEFAULT == "rank1"
+    assert type(opt3.state_dict()["qconfig"]) is dict
+    with pytest.raises(ValueError, match="lacks QUANT.M"):
+        opt3.load_state_dict(dict(sd, qconfig={"QUANT": {"SQM": sd["qconfig"]["QUANT"]["SQM"]}}))
+
 
 def test_oracle_under_sanitizers(tmp_path):
     """The oracle's C code under AddressSanitizer + UBSan on ragged sizes (host only)."""
