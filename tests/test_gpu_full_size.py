@@ -235,3 +235,26 @@ def test_indexing_beyond_two_to_the_31_elements(qmaps):
     # and the round trip is what quantisation promises: every value within its group's scale
     err = (out_a[: 1 << 20] - g[: 1 << 20]).abs().max()
     assert float(err) <= float(max_a[: 1 << 13].max())
+
+
+@pytest.mark.parametrize("shape", [(64, 1024, 1024), (512, 512, 3, 3), (16, 8, 128, 4096)])
+def test_rank1_nd_statistics_at_size(oracle, qmaps, shape):
+    """Rank-1 statistics, quantise and dequantise of 3-D and 4-D tensors of 2.4e6 .. 6.7e7 values through
+    lpmm.functional against the N-D oracle (the stacked-matrix shapes take the 2-D kernel plus the fold of its row
+    maxima, the convolution-shaped one the one-pass kernel on the tensor itself)."""
+    import lpmm.functional as F
+
+    rng = np.random.default_rng(len(shape) * 100 + shape[0])
+    x = (rng.standard_normal(shape, dtype=np.float32) ** 2).astype(np.float32)
+    x *= np.exp(rng.standard_normal((shape[0],) + (1,) * (len(shape) - 1))).astype(np.float32)
+    dx = to_dev(x)
+    md = dict(b=4, scale_type="rank1", quant_type="power-1", round_type="real-nearest", gp_sz=128, signed=False)
+    dq = to_dev(qmaps[1])
+    codes, gen = F.vectorwise_quant(dx, qmap=dq, shape=dx.shape, **md)
+    want_stats = oracle.rank1_stats_nd(x)
+    for i, (got, want) in enumerate(zip(gen["max_dims"], want_stats)):
+        np.testing.assert_array_equal(to_np(got).reshape(-1), want, err_msg=f"statistics of dimension {i}")
+    want_codes = oracle.quant_rank1_nd_bits(x, want_stats, qmaps[1], 4)
+    np.testing.assert_array_equal(to_np(codes).view(np.uint8), want_codes)
+    back = F.vectorwise_dequant(codes, qmap=dq, shape=dx.shape, **{**gen, **md})
+    np.testing.assert_array_equal(to_np(back), oracle.dequant_rank1_nd_bits(want_codes, want_stats, qmaps[1], 4, shape))
