@@ -5,6 +5,14 @@ cpu_baseline leg of bench.py as the checker.  The shipped package never imports 
 
 All arrays are C-contiguous numpy arrays; "in place" functions mutate their arguments
 exactly like the reference's kernels mutate the tensors they are given.
+
+Functions restated here in numpy rather than in C, and what pins them (tests/test_oracle_*.py):
+  adamw_fp16_step     the float step of the C oracle on inputs exactly representable in half, and a
+                      float16 round trip of it operation by operation (moments re-read after rounding).
+  rank1_*_nd          on a 2-D tensor the 2-D C functions bit for bit; on 3-D/4-D tensors the
+                      reference's op sequence run by PyTorch's CPU kernels and a loop over all indices.
+  map construction    the bit patterns the reference's recipe gives when PyTorch's ops run it
+                      (tests/golden/qmaps.json).
 """
 import ctypes
 import os
