@@ -123,7 +123,7 @@ def make_params(torch, shapes, dev, heavy_tailed, interleaved=False):
     return params
 
 
-def cpu_baseline(torch, steps=10):
+def cpu_baseline(torch, steps=100):
     """The reference's non-fused PyTorch path (op sequence of _single_tensor_adamw4bit) on the
     host cores: one 4096x4096 fp32 parameter, m group-128 / v rank-1, all threads."""
     from oracle.nonfused_torch import TorchNonFusedAdamW
