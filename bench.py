@@ -7,7 +7,7 @@ with the step throughput (params/s), the HBM roofline of the dominant kernel mea
 with events on the launch stream, and a CPU baseline (the reference's non-fused PyTorch op
 sequence on the host cores, bounded sample).
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload llama7b|gpt2xl|tiny]    (defaults: 50 steps, 5 warm-up)
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload llama7b|gpt2xl|tiny]    (defaults: 100 steps, 10 warm-up)
 
 After the timed region the default run also measures, on the same box, what plain streaming
 kernels with the fused step's access pattern reach (`roofline.calibration`; `--workload calibrate`
@@ -453,8 +453,8 @@ def run_nonfused(torch, args, v_scale):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="llama7b", choices=sorted(WORKLOADS) + ["quant64m", "factored", "nonfused_group", "nonfused_rank1", "calibrate"])
     ap.add_argument("--bits", type=int, default=4, choices=range(1, 9), help="code width of --workload quant64m")
     ap.add_argument("--no-cpu-baseline", action="store_true")
