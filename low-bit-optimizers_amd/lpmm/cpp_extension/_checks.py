@@ -12,19 +12,18 @@ def check_cuda_tensor_float(t, name, *, fp32_only=True):
     if t.dtype not in (torch.float32, torch.float16):
         raise RuntimeError(f"The type of {name} is not kFloat32 or kFloat16!")
     if fp32_only and t.dtype != torch.float32:
-        raise RuntimeError(f"The type of {name} is kFloat16: this operator is implemented for float32 only "
-                           "(half tensors are accepted by adamw_single_tensor alone, the one operator "
-                           "the reference can run them through)")
+        raise RuntimeError(f"The type of {name} is kFloat16: float32 is required here (half tensors are accepted "
+                           "where the reference can run them: adamw_single_tensor and the data of pack_nonlinear)")
 
 
-def check_cuda_tensor_dim_float(t, name, n_dim):
+def check_cuda_tensor_dim_float(t, name, n_dim, *, fp32_only=True):
     if not t.is_cuda:
         raise RuntimeError(f"{name} must be a CUDA tensor!")
     if not t.is_contiguous():
         raise RuntimeError(f"{name} must be contiguous!")
     if t.dim() != n_dim:
         raise RuntimeError(f"The dimension of {name} is not correct!")
-    check_cuda_tensor_float(t, name)
+    check_cuda_tensor_float(t, name, fp32_only=fp32_only)
 
 
 def check_cuda_tensor_dim_type(t, name, n_dim, dtype):

@@ -26,7 +26,7 @@ def _storage_bits(bits):
 
 
 def pack_nonlinear(data, qmap, bits, stochastic):
-    """data: float32 (num_groups, group_size), already normalised.  Returns int8 of
+    """data: float32 or float16 (num_groups, group_size), already normalised.  Returns int8 of
     storage_bits*numel/8 + 1 bytes (lpmm/cpp_extension/quantization_kernel.cu:475-477, :549-550; storage_bits
     is `bits` for 1, 2 and 4 and 8 otherwise); the final byte,
     left uninitialised by the reference, is 0.
@@ -35,9 +35,16 @@ def pack_nonlinear(data, qmap, bits, stochastic):
     (lpmm/cpp_extension/quantization_kernel.cu:480-487): a (seed, offset) pair from torch's default
     generator of the device, whose offset advances by group_size * work_per_thread rounded up
     to a multiple of 4.  With stochastic=False the generator is left alone (the reference
-    advances it there too, although its kernel ignores the numbers)."""
-    check_cuda_tensor_dim_float(data, "data", 2)
+    advances it there too, although its kernel ignores the numbers).
+
+    Half data: the reference's kernel is instantiated for at::Half as well and widens every value to
+    float before the search (lpmm/cpp_extension/quantization_kernel.cu:489-507, :450); the widening is
+    exact, so the codes are those of data.float(), which is what runs here.  The map must be float32
+    there too (qmap.data_ptr<float>())."""
+    check_cuda_tensor_dim_float(data, "data", 2, fp32_only=False)
     check_cuda_tensor_dim_float(qmap, "qmap", 1)
+    if data.dtype is torch.float16:
+        data = data.float()
     _check_bits(bits, qmap)
     if data.size(1) % (4 * (8 // _storage_bits(bits))) != 0 or data.numel() % 8 != 0:
         raise RuntimeError("Expected group_size % work_per_thread == 0 to be true, but got false.")

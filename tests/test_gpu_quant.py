@@ -257,6 +257,14 @@ def test_shim_pack_unpack_signatures(oracle, qmaps):
     np.testing.assert_array_equal(to_np(packed).view(np.uint8), oracle.pack_nonlinear_4bit(x, qmaps[1]))
     un = ext.unpack_nonlinear(packed, dq, 4, 3, 2048)
     assert un.shape == (3, 2048) and un.dtype == torch.float32
+    # half data is widened to float before the search, as in the reference's at::Half instantiation
+    xh = to_dev(x).half()
+    for bits, qmap in ((4, qmaps[1]), (5, oracle.create_pow_map(5, False, 1))):
+        got = ext.pack_nonlinear(xh, to_dev(qmap), bits, False)
+        want = oracle.pack_nonlinear(to_np(xh).astype(np.float32).reshape(-1), qmap, bits)
+        np.testing.assert_array_equal(to_np(got).view(np.uint8), want)
+    with pytest.raises(RuntimeError, match="kFloat16"):
+        ext.pack_nonlinear(to_dev(x), dq.half(), 4, False)  # the map must be float32 there as well
     with pytest.raises(RuntimeError):
         ext.pack_nonlinear(torch.from_numpy(x), dq, 4, False)  # CPU tensor
     with pytest.raises(RuntimeError):
