@@ -305,8 +305,12 @@ def vectorwise_quant(x, **kwargs):
     qmap = _select_qmap(kwargs)
     md = {"dtype": x.dtype, "stride": x.stride()}
     src = x.detach()
-    if src.dtype != torch.float32:
-        raise NotImplementedError(f"{src.dtype} states: this build implements the fp32 path only")
+    if src.dtype not in (torch.float32, torch.float16):
+        raise NotImplementedError(f"{src.dtype} states: the quantisers take float32 and float16")
+    # float16 states (half parameters on the non-fused path): the scaling runs as PyTorch device ops
+    # of that type, one rounding per op, exactly the reference's chain (lpmm/functional.py:184-203);
+    # the search and the packing widen each value to float, as the reference's half kernel does
+    fp32 = src.dtype is torch.float32
     src = src.contiguous()
     scale_type = kwargs["scale_type"]
     b = kwargs["b"]
@@ -315,7 +319,7 @@ def vectorwise_quant(x, **kwargs):
         md["dim"] = src.dim()
     # stochastic rounding: scaling by PyTorch device ops as in the reference
     # (lpmm/functional.py:184-203), the search and packing by the HIP operator
-    nearest = kwargs["round_type"] == "real-nearest"
+    nearest = kwargs["round_type"] == "real-nearest" and fp32
     if as_group:
         gp_sz = kwargs["gp_sz"] if scale_type == "group" else 128
         if nearest and _group_gp_sz_ok(gp_sz):
@@ -360,7 +364,7 @@ def vectorwise_dequant(qx, denormalized=True, **kwargs):
         shape = kwargs["shape"]
         gp_sz = scaled_shape[1]
         n = shape.numel()
-        if gp_sz % 128 == 0:
+        if gp_sz % 128 == 0 and kwargs["max1"].dtype is torch.float32:
             x = torch.empty(shape, dtype=torch.float32, device=dev)
             with torch.cuda.device(dev):
                 stream = _native.current_stream(dev)
@@ -376,7 +380,8 @@ def vectorwise_dequant(qx, denormalized=True, **kwargs):
             x = recon_grouped_tensor(x.mul(kwargs["max1"]), shape)
     elif scale_type == "rank1":
         max_dims = kwargs["max_dims"]
-        if 2 <= len(scaled_shape) <= RANK1_ND_MAX and numel(scaled_shape) > 0:
+        if (2 <= len(scaled_shape) <= RANK1_ND_MAX and numel(scaled_shape) > 0
+                and all(m.dtype is torch.float32 for m in max_dims)):
             if len(scaled_shape) == 2:
                 rows, cols = scaled_shape
                 rowmax, colmax = max_dims

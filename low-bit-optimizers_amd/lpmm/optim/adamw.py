@@ -15,6 +15,7 @@ handful of multi-tensor launches instead of one launch per tensor, and each quan
 dequantise / update of the non-fused path is one HIP kernel instead of a chain of
 PyTorch passes.
 """
+import math
 import weakref
 from typing import Optional
 
@@ -272,10 +273,9 @@ class AdamW(LowBitOptimizer):
             _native.check(st, "fused fp16 AdamW step")
 
     @staticmethod
-    def _check_fp32_cuda(p, grad, why="quantised states and the non-fused path compute in float32 only (the "
-                         "reference runs other types there through PyTorch's kernels of that type, one rounding "
-                         "per op: lpmm/optim/adamw.py:394-434, lpmm/functional.py:184-203); keep float32 master "
-                         "weights, or use fused=True for float16 tensors whose states are not quantised",
+    def _check_fp32_cuda(p, grad, why="the HIP kernels of this path compute in float32 (float16 parameters take "
+                         "the reference's own chain of PyTorch ops on the non-fused path, and the fp32-state "
+                         "operator under fused=True; the factored second moment and bfloat16 are float32 only)",
                          strided_ok=False):
         if (p.dtype is torch.float32 and grad.dtype is torch.float32 and p.is_cuda and grad.is_cuda
                 and (strided_ok or (p.is_contiguous() and grad.is_contiguous()))):
@@ -362,6 +362,9 @@ class AdamW(LowBitOptimizer):
             if factored:
                 factored_work.append((p, grad, state, step))
                 continue
+            if p.dtype is torch.float16:
+                self._half_step(group, p, grad, state, step, md_m, md_v)
+                continue
             dense, grad = self._dense_operands(p, grad, held)
             en_m, en_v = self._enabled(p, state, "exp_avg"), self._enabled(p, state, "exp_avg_sq")
             if m_group128 and en_m and en_v:
@@ -410,6 +413,48 @@ class AdamW(LowBitOptimizer):
             if records:
                 launch_rank1(key, records)
         self._write_back(held)
+
+    def _half_step(self, group, p, grad, state, step, md_m, md_v):
+        """float16 parameters on the non-fused path.  The reference runs them through PyTorch's
+        float16 kernels, every op rounding to half once (lpmm/optim/adamw.py:367-369, :394-434), with
+        half states, half statistics and a scaling in half (lpmm/functional.py:184-203, :97-118).  The
+        same chain of PyTorch device ops runs here, so every rounding falls where it falls there;
+        the code search, packing and unpacking are the HIP operators."""
+        if not (p.is_cuda and grad.is_cuda):
+            raise RuntimeError("p and g must be CUDA tensors!")
+        if grad.dtype is not torch.float16:
+            raise RuntimeError(f"The type of g is {grad.dtype}: half parameters need half gradients "
+                               "(the reference's lerp_ raises for mixed types as well)")
+        beta1, beta2 = group["betas"]
+        lr, wd, eps = group["lr"], group["weight_decay"], group["eps"]
+        p.mul_(1 - lr * wd)
+        moments = []
+        for name, md in (("exp_avg", md_m), ("exp_avg_sq", md_v)):
+            t = state[name]
+            if _is_placeholder(t):
+                t = torch.zeros_like(p, memory_format=torch.preserve_format)
+            elif self._enabled(p, state, name):
+                qstate = state[f"{name}_qstate"]
+                kw = dict(qstate["overhead"])
+                kw.update(md)
+                t = vectorwise_dequant(t, qmap=qstate["qmap"], shape=p.shape, **kw)
+            moments.append(t)
+        m, v = moments
+        m.lerp_(grad, 1 - beta1)
+        v.mul_(beta2).addcmul_(grad, grad, value=1 - beta2)
+        bias_correction1 = 1 - beta1 ** step
+        bias_correction2 = 1 - beta2 ** step
+        denom = (v.sqrt() / math.sqrt(bias_correction2)).add_(eps)
+        p.addcdiv_(m, denom, value=-(lr / bias_correction1))
+        for name, t, md in (("exp_avg", m, md_m), ("exp_avg_sq", v, md_v)):
+            if self._enabled(p, state, name):
+                qstate = state[f"{name}_qstate"]
+                qx, gen = vectorwise_quant(t, qmap=qstate["qmap"], shape=p.shape, **md)
+                state[name] = qx
+                qstate["overhead"].clear()
+                qstate["overhead"].update(gen)
+            else:
+                state[name] = t
 
     def _nonfused_record(self, p, dense, grad, state, step):
         """The tensor's record for the one-pass non-fused step; creates the quantised states

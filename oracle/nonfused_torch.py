@@ -30,7 +30,8 @@ def _group(x, gp_sz):
 def _pack(normed, qmap):
     """functional.py:361-363: re-group to 2048 and pack two 4-bit codes per byte."""
     grouped = _group(normed, O.PACK_GROUP)
-    return torch.from_numpy(O.pack_nonlinear_4bit(grouped.numpy(), qmap))
+    # half data is widened to float by the reference's kernel (quantization_kernel.cu:450)
+    return torch.from_numpy(O.pack_nonlinear_4bit(grouped.float().numpy(), qmap))
 
 
 def _unpack(codes, qmap, numel):
@@ -49,8 +50,10 @@ def quant_group(x, qmap, gp_sz=128):
 def dequant_group(codes, max1, qmap, shape, gp_sz=128):
     """functional.py:393-400, :115-118."""
     g = max1.shape[0]
+    # the unpacked values are float32; times half statistics they stay float32 (type promotion), and
+    # the result takes the state's type at the end (functional.py:150)
     x = _unpack(codes, qmap, g * gp_sz).view(g, gp_sz).mul(max1)
-    return x.flatten()[: math.prod(shape)].view(shape)
+    return x.flatten()[: math.prod(shape)].view(shape).to(max1.dtype)
 
 
 def quant_rank1(x, qmap):
@@ -74,7 +77,7 @@ def dequant_rank1(codes, max_dims, qmap, shape):
     st = max_dims[0].clone()
     for md in max_dims[1:]:
         st = torch.min(st, md)
-    return _unpack(codes, qmap, math.prod(shape)).view(shape).mul(st)
+    return _unpack(codes, qmap, math.prod(shape)).view(shape).mul(st).to(st.dtype)
 
 
 class TorchNonFusedAdamW:

@@ -656,5 +656,65 @@ def test_half_parameters_on_the_fused_path(oracle):
     big.grad = torch.zeros_like(big)
     with pytest.raises(RuntimeError, match="float32 is required"):
         lpmm.optim.AdamW([big], fused=True).step()
+    # ... and so is the factored second moment with half parameters
     with pytest.raises(RuntimeError, match="float32 is required"):
-        lpmm.optim.AdamW([big], fused=False).step()
+        lpmm.optim.AdamW([big], fused=False, factor_second_moment=True).step()
+    bf = torch.nn.Parameter(torch.zeros(128, 64, dtype=torch.bfloat16, device="cuda"))
+    bf.grad = torch.zeros_like(bf)
+    with pytest.raises(RuntimeError, match="float32 is required"):
+        lpmm.optim.AdamW([bf], fused=False).step()
+
+
+@pytest.mark.parametrize("v_scale", ["rank1", "group"])
+def test_half_parameters_on_the_nonfused_path(v_scale):
+    """float16 parameters with fused=False: the reference's own chain of float16 PyTorch ops
+    (lpmm/optim/adamw.py:394-434, lpmm/functional.py:184-203, :97-118), here on the device with the HIP
+    pack / unpack operators, against the same chain run by PyTorch's CPU kernels with the C oracle's
+    pack / unpack.  Both round to half after every op; a float-level last-bit difference between the two
+    libraries' kernels can cross a half rounding boundary now and then, so values are compared to one
+    half ulp, codes to a small budget, and every step starts from the device's own state."""
+    import lpmm
+    from oracle.nonfused_torch import TorchNonFusedAdamW
+
+    torch.manual_seed(5)
+    shapes = [(96, 160), (11008,), (2000,)]  # quantised 2-D, quantised 1-D, fp16 states
+    hyper = dict(lr=1e-2, betas=(0.9, 0.999), eps=1e-3, weight_decay=0.01)
+    host = [(torch.randn(s) * 0.5).half() for s in shapes]
+    params = [torch.nn.Parameter(h.cuda()) for h in host]
+    cfg = os.path.join(os.path.dirname(lpmm.config.__file__), "configs",
+                       "default.yml" if v_scale == "rank1" else "2nd_moment_group_128.yml")
+    opt = lpmm.optim.AdamW(params, fused=False, qconfig=cfg, **hyper)
+    ref = TorchNonFusedAdamW([h.clone() for h in host[:2]], v_scale_type=v_scale, **hyper)
+    ulp = 2.0 ** -10
+    for step in range(1, 4):
+        grads = [(torch.randn(s) * 0.3).half() for s in shapes]
+        for p, g in zip(params, grads):
+            p.grad = g.cuda()
+        opt.step()
+        ref.step(grads[:2])
+        torch.cuda.synchronize()
+        for i in range(2):
+            st, rs = opt.state[params[i]], ref.state[i]
+            n = host[i].numel()
+            assert params[i].dtype == torch.float16 and st["exp_avg"].dtype == torch.int8
+            got_p, want_p = params[i].detach().cpu().float(), ref.params[i].float()
+            assert torch.all((got_p - want_p).abs() <= 2 * ulp * want_p.abs().clamp_min(2.0 ** -14)), f"p {i} step {step}"
+            oh_m, oh_v = st["exp_avg_qstate"]["overhead"], st["exp_avg_sq_qstate"]["overhead"]
+            assert oh_m["max1"].dtype == torch.float16 and oh_m["dtype"] == torch.float16
+            gm1, wm1 = oh_m["max1"].cpu().float().reshape(-1), rs["m"][1].float().reshape(-1)
+            assert torch.all((gm1 - wm1).abs() <= 2 * ulp * wm1.abs()), f"m scales {i} step {step}"
+            dm = np.mean(nibbles(to_np(st["exp_avg"]), n) != nibbles(rs["m"][0].numpy(), n))
+            dv = np.mean(nibbles(to_np(st["exp_avg_sq"]), n) != nibbles(rs["v"][0].numpy(), n))
+            assert dm < 2e-3 and dv < 2e-3, (i, step, dm, dv)
+            if v_scale == "rank1" and i == 0:
+                assert oh_v["dim"] == 2 and oh_v["max_dims"][0].dtype == torch.float16
+            # continue from the device's state
+            ref.params[i].copy_(params[i].detach().cpu())
+            rs["m"] = (st["exp_avg"].cpu().clone(), oh_m["max1"].cpu().clone())
+            if v_scale == "rank1" and i == 0:
+                rs["v"] = (st["exp_avg_sq"].cpu().clone(), [m.cpu().clone() for m in oh_v["max_dims"]])
+            else:
+                rs["v"] = (st["exp_avg_sq"].cpu().clone(), oh_v["max1"].cpu().clone())
+        small = opt.state[params[2]]
+        assert small["exp_avg"].dtype == torch.float16 and small["exp_avg_sq"].dtype == torch.float16
+    assert all(torch.isfinite(p).all() for p in params)
