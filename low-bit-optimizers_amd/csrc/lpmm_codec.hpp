@@ -263,6 +263,26 @@ __device__ __forceinline__ uint32_t encode8_plain(const uint32_t *lds, uint32_t 
     return w;
 }
 
+// Packed codes of a 128-value group in the row layout: lane l of the DPP row works on the 16-bit
+// halves l (elements 4l .. 4l+3) and 16 + l (elements 64+4l .. 64+4l+3) of the group's 64 bytes, as
+// the word  half l | half (16 + l) << 16.  In memory the group is 16 dwords, dword d = halves 2d, 2d+1.
+// Lane 2i accesses dword i (the first halves of lanes 2i and 2i+1), lane 2i+1 dword 8 + i (their second
+// halves); one exchange between the two lanes turns the memory form into the lane form and back
+// (it is its own inverse): even lane {own.lo, neighbour.lo}, odd lane {neighbour.hi, own.hi}.
+__device__ __forceinline__ uint32_t code_dword_of_lane(int lane16)
+{
+    return (lane16 & 1) ? 8u + ((uint32_t)lane16 >> 1) : (uint32_t)lane16 >> 1;
+}
+__device__ __forceinline__ uint32_t code_swap_selector(int lane16)
+{
+    return (lane16 & 1) ? 0x03020706u : 0x05040100u;  // v_perm_b32 byte selectors, {neighbour, own}
+}
+__device__ __forceinline__ uint32_t swap_code_halves(uint32_t w, uint32_t selector)
+{
+    const uint32_t nb = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)w, 0xB1 /* quad_perm:[1,0,3,2] */, 0xF, 0xF, false);
+    return __builtin_amdgcn_perm(nb, w, selector);
+}
+
 // Decode offsets: byte j of `even` / `odd` holds 4 * nibble (2j) / (2j+1) of the code word.
 struct Nibbles {
     uint32_t even, odd;

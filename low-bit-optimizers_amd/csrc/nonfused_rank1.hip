@@ -16,12 +16,21 @@
 //
 // 18.5 bytes per parameter cross HBM instead of 50.  The column count must be a multiple of
 // 128, so that the 128-value groups of m never straddle rows: 16 lanes (one DPP row) own 128
-// consecutive columns of one tensor row.  A 256-thread workgroup covers 16 rows by
+// consecutive columns of one tensor row.  A 256-thread workgroup covers tile_rows rows by
 // 128 << lg_wide columns, per pass (16 >> lg_wide) rows of (1 << lg_wide) adjacent groups, so
-// that its accesses to a row are contiguous runs of 512 << lg_wide bytes.  16 rows by 1024
-// columns measured best on the LLaMA-7B shapes: smaller tiles pay for the column atomics and
-// the per-workgroup set-up, larger ones leave too few workgroups to balance the last wave of
-// them over the chip.  lg_wide is chosen per tensor on the host.
+// that its accesses to a row are contiguous runs of 512 << lg_wide bytes.
+//
+// Both kernels run at the rate the memory system gives to their access structure, not at that
+// of their arithmetic (with the arithmetic taken out they take the same time).  Measured on the
+// LLaMA-7B shapes: a workgroup that walks through many passes is slower than the same accesses
+// made by short-lived workgroups in dispatch order (tiles of 1 or 2 passes run at the rate of
+// the one-shot fused step, 8 passes over 16 rows by 1024 columns 13 % below it), but short
+// tiles mean more column atomics and more tile set-up.  Tiles of 64 rows by 256 columns
+// (8 passes of 8 rows) are the best compromise for both kernels.  The row blocks that are
+// resident together interleave their passes (block k of a group of `comb` blocks takes the rows
+// of pass i at (i * comb + k) * pass_rows), so that at any time a group works on one contiguous
+// band of the tensor instead of on `comb` bands a tile apart.  Together 2130 -> 1990 us (first
+// pass) and 770 -> 705 us (second pass) per launch of 8.4e8 elements.
 #include "lpmm_update.hpp"
 
 namespace lpmm {
@@ -29,13 +38,23 @@ namespace lpmm {
 constexpr int kThreads = 256;
 constexpr int kEltsPerLane = 8;
 constexpr int kDppRows = kThreads / 16;  // 128-column groups a workgroup handles per pass
-#ifndef LPMM_R1_ROWS
-#define LPMM_R1_ROWS 16
-#endif
-constexpr int kTileRows = LPMM_R1_ROWS;  // tensor rows per workgroup (more where one pass of a narrow tile covers more)
 constexpr int kR1Max = 32;               // tensors per launch
 constexpr int kMaxLgWide = 3;
 constexpr int kMaxWide = 1 << kMaxLgWide;
+// Tile policy: widest tile (lg of 128-column groups), tensor rows per workgroup (more where one pass
+// of a narrow tile covers more), workgroups taken to be resident together.
+#ifndef LPMM_R1_LG
+#define LPMM_R1_LG 1
+#endif
+#ifndef LPMM_R1_ROWS
+#define LPMM_R1_ROWS 64
+#endif
+#ifndef LPMM_R1_RESIDENT
+#define LPMM_R1_RESIDENT 256
+#endif
+constexpr int kPolicyLgWide = LPMM_R1_LG;
+constexpr uint32_t kPolicyRows = LPMM_R1_ROWS, kPolicyResident = LPMM_R1_RESIDENT;
+static_assert(LPMM_R1_LG <= kMaxLgWide, "the LDS column arrays hold 128 << 3 columns");
 // Per-column data of a tile lives in LDS, not in registers (occupancy): the current column
 // statistics in the unused bytes between the maps and the encode table, further arrays after
 // the table.
@@ -47,6 +66,14 @@ constexpr uint32_t kColExtra = (kLdsBytes + 15) / 16 * 16;  // first byte after 
 // of a wave hit different banks) per column group: word k * 16 + lane16 of a slot is element k
 // of lane lane16.
 constexpr uint32_t kRedSlotWords = kGroup + 16;
+
+// A workgroup covers tile_rows rows x (128 << lg_wide) columns: per pass, (16 >> lg_wide) rows of
+// (1 << lg_wide) adjacent groups each.
+struct TileShape {
+    uint32_t lg_wide : 8;
+    uint32_t tile_rows : 24;  // max(the policy's rows, rows of one pass)
+    uint32_t comb;            // row blocks whose passes interleave
+};
 
 struct TensorR1 {
     float *p;
@@ -61,11 +88,7 @@ struct TensorR1 {
     int64_t rows;
     uint32_t col_blocks;  // columns / 128
     float neg_step_size, bc2_sqrt, rbc2_sqrt;
-    // a workgroup covers kTileRows rows x (128 << lg_wide) columns: per pass, (16 >> lg_wide)
-    // rows of (1 << lg_wide) adjacent groups each
-    uint32_t lg_wide;
-    uint32_t col_tiles;  // ceil(col_blocks / (1 << lg_wide))
-    uint32_t tile_rows;  // max(kTileRows, rows of one pass)
+    TileShape tile;
 };
 
 struct MultiR1 {
@@ -103,13 +126,18 @@ struct Geometry {
 __device__ __forceinline__ Geometry geometry(const TensorR1 &t, uint32_t tile, int drow)
 {
     Geometry q;
-    const uint32_t rb = tile / t.col_tiles;
-    q.col_tile = tile - rb * t.col_tiles;
-    q.wide = 1 << t.lg_wide;
+    const TileShape &ts = t.tile;
+    q.wide = 1 << ts.lg_wide;
+    const uint32_t col_tiles = (t.col_blocks + q.wide - 1) >> ts.lg_wide;
+    const uint32_t rb = tile / col_tiles;
+    q.col_tile = tile - rb * col_tiles;
     q.cg = q.col_tile * q.wide + (drow & (q.wide - 1));
-    q.row0 = (int64_t)rb * t.tile_rows + (drow >> t.lg_wide);
-    q.step = kDppRows >> t.lg_wide;
-    q.passes = (int)t.tile_rows / q.step;
+    const int pass_rows = kDppRows >> ts.lg_wide;
+    q.passes = (int)ts.tile_rows / pass_rows;
+    // block k of group grp: pass i covers the rows from (grp * passes * comb + i * comb + k) * pass_rows on
+    const uint32_t grp = rb / ts.comb, k = rb - grp * ts.comb;
+    q.row0 = (int64_t)grp * ts.tile_rows * ts.comb + (int64_t)k * pass_rows + (drow >> ts.lg_wide);
+    q.step = pass_rows * (int)ts.comb;
     return q;
 }
 
@@ -270,7 +298,8 @@ __global__ __launch_bounds__(kThreads, LPMM_R1_WAVES) void rank1_update_kernel(c
             }
         }
     }
-    __syncthreads();
+    // the column maxima meet in LDS: nothing below depends on the global stores still in flight
+    lds_barrier();
     // column j of the tile = element k of lane l of slot s
     for (int j = threadIdx.x; j < q.wide * kGroup; j += kThreads) {
         const int w = j & (kGroup - 1);
@@ -325,6 +354,9 @@ __global__ __launch_bounds__(kThreads) void rank1_requant_kernel(const MultiR1 a
 #pragma unroll
     for (int k = 0; k < kEltsPerLane; ++k)
         cols_safe = cols_safe && rc_safe(cn[k]);
+    // the group's 64 code bytes move as one dword per lane (whole lines per access; with the
+    // arithmetic taken out this pass is 11 % faster than with two 16-bit accesses per lane)
+    const uint32_t code_dword = code_dword_of_lane(lane16), code_sel = code_swap_selector(lane16);
 #pragma unroll 1
     for (int it = 0; it < q.passes; ++it) {
         const int64_t r = q.row0 + it * q.step;
@@ -333,8 +365,8 @@ __global__ __launch_bounds__(kThreads) void rank1_requant_kernel(const MultiR1 a
         const int64_t gbase = (r * t.col_blocks + q.cg) * kGroup;
         const float *gp = t.g + gbase + lane16 * 4;
         const float4 b0 = load4(gp), b1 = load4(gp + 64);
-        uint16_t *vcp = reinterpret_cast<uint16_t *>(t.vc + (gbase >> 1)) + lane16;
-        const uint32_t wv = load_u16(vcp) | (load_u16(vcp + 16) << 16);
+        uint32_t *vcp = reinterpret_cast<uint32_t *>(t.vc + (gbase >> 1)) + code_dword;
+        const uint32_t wv = swap_code_halves(load_u32(vcp), code_sel);
         const float ro = t.row_old[r], rn = t.row_new[r];
         float gv[kEltsPerLane], v[kEltsPerLane], x[kEltsPerLane];
         unpack8(b0, b1, gv);
@@ -363,8 +395,7 @@ __global__ __launch_bounds__(kThreads) void rank1_requant_kernel(const MultiR1 a
                 x[k] = v[k] / ((cn[k] < rn) ? cn[k] : rn);
             w = encode8_plain(lds, kLdsQ0, kind, x);
         }
-        store_u16(vcp, w & 0xFFFFu);
-        store_u16(vcp + 16, w >> 16);
+        store_u32(vcp, swap_code_halves(w, code_sel));
     }
 }
 
@@ -372,13 +403,13 @@ __global__ __launch_bounds__(kThreads) void rank1_requant_kernel(const MultiR1 a
 
 using namespace lpmm;
 
-// The widest tile (longest contiguous runs) that leaves at most 5 % of the DPP rows of a
-// tensor's tiles without a column group; otherwise the width that wastes least.
+// The widest tile the policy allows (longest contiguous runs) that leaves at most 5 % of the DPP
+// rows of a tensor's tiles without a column group; otherwise the width that wastes least.
 static uint32_t choose_lg_wide(uint32_t col_blocks)
 {
     uint32_t best = 0;
     double best_use = 0.0;
-    for (int lg = kMaxLgWide; lg >= 0; --lg) {
+    for (int lg = kPolicyLgWide; lg >= 0; --lg) {
         const uint32_t wide = 1u << lg;
         const double use = (double)col_blocks / (double)((col_blocks + wide - 1) / wide * wide);
         if (use >= 0.95)
@@ -389,6 +420,23 @@ static uint32_t choose_lg_wide(uint32_t col_blocks)
         }
     }
     return best;
+}
+
+// Tile shape of a rows x (128 * col_blocks) tensor, and its tile count.
+static uint64_t shape_tiles(int64_t rows, uint32_t col_blocks, TileShape &ts)
+{
+    const uint32_t lg_wide = choose_lg_wide(col_blocks);
+    const uint32_t col_tiles = (col_blocks + (1u << lg_wide) - 1) >> lg_wide;
+    const uint32_t pass_rows = (uint32_t)kDppRows >> lg_wide;
+    const uint32_t tile_rows = pass_rows > kPolicyRows ? pass_rows : kPolicyRows;
+    const uint64_t row_blocks = (uint64_t)((rows + tile_rows - 1) / tile_rows);
+    uint64_t comb = kPolicyResident / col_tiles;
+    comb = comb < 1 ? 1 : comb;
+    comb = comb > row_blocks ? row_blocks : comb;
+    ts.lg_wide = lg_wide;
+    ts.tile_rows = tile_rows;
+    ts.comb = (uint32_t)comb;
+    return (row_blocks + comb - 1) / comb * comb * col_tiles;  // whole groups: the last may hold empty blocks
 }
 
 extern "C" int lpmm_nonfused_adamw4bit_rank1_step_multi(const lpmm_nonfused_rank1_tensor *tensors, int64_t count,
@@ -412,7 +460,8 @@ extern "C" int lpmm_nonfused_adamw4bit_rank1_step_multi(const lpmm_nonfused_rank
         if (t.rows == 0 || t.cols == 0)
             continue;
         const int64_t col_blocks = t.cols / kGroup;
-        const int64_t row_blocks = (t.rows + kTileRows - 1) / kTileRows;  // an upper bound
+        // an upper bound: tiles hold at least 16 rows, the last group adds fewer than `resident` blocks
+        const int64_t row_blocks = (t.rows + kDppRows - 1) / kDppRows + kPolicyResident;
         if (col_blocks > 0x7fffffffLL / 2 || row_blocks > 0x7fffffffLL / col_blocks ||
             t.rows > INT64_MAX / t.cols)
             return LPMM_ERR_SIZE;
@@ -458,14 +507,10 @@ extern "C" int lpmm_nonfused_adamw4bit_rank1_step_multi(const lpmm_nonfused_rank
                 continue;
             }
             const uint32_t col_blocks = (uint32_t)(t.cols / kGroup);
-            const uint32_t lg_wide = choose_lg_wide(col_blocks);
-            const uint32_t col_tiles = (col_blocks + (1u << lg_wide) - 1) >> lg_wide;
-            const uint32_t pass_rows = (uint32_t)kDppRows >> lg_wide;
-            const uint32_t tile_rows = pass_rows > (uint32_t)kTileRows ? pass_rows : (uint32_t)kTileRows;
-            const uint64_t nt = (uint64_t)((t.rows + tile_rows - 1) / tile_rows) * col_tiles;
+            TensorR1 &d = args.t[k];
+            const uint64_t nt = shape_tiles(t.rows, col_blocks, d.tile);
             if (tiles + nt > 0x7fffffffULL)
                 break;
-            TensorR1 &d = args.t[k];
             d.p = t.p;
             d.g = t.g;
             d.mc = t.m_codes;
@@ -477,9 +522,6 @@ extern "C" int lpmm_nonfused_adamw4bit_rank1_step_multi(const lpmm_nonfused_rank
             d.col_new = t.v_colmax_next;
             d.rows = t.rows;
             d.col_blocks = col_blocks;
-            d.lg_wide = lg_wide;
-            d.col_tiles = col_tiles;
-            d.tile_rows = tile_rows;
             const NfHyper h = make_nf_hyper(beta1, beta2, lr, weight_decay, eps, t.step);
             d.neg_step_size = h.neg_step_size;
             d.bc2_sqrt = h.bc2_sqrt;
@@ -489,8 +531,11 @@ extern "C" int lpmm_nonfused_adamw4bit_rank1_step_multi(const lpmm_nonfused_rank
             args.tile_start[++k] = (uint32_t)tiles;
             ++i;
         }
-        if (k == 0)
+        if (k == 0) {
+            if (i < count)
+                return LPMM_ERR_SIZE;  // a single tensor with more tiles than a grid holds
             continue;
+        }
         args.count = k;
         for (int j = k + 1; j <= kR1Max; ++j)
             args.tile_start[j] = (uint32_t)tiles;
