@@ -309,16 +309,22 @@ __global__ __launch_bounds__(kFThreads) void factored_update_kernel(
 }
 
 // The same pass when the column count is a multiple of 128: every 128-element group of the
-// flattened tensor is a 128-column piece of one row.  A workgroup takes 16 consecutive groups of
-// the flattened tensor (2048 contiguous elements, whatever the row length), the 16 lanes of a
-// DPP row own one group in the row layout of the fused step (lane l: columns [4l, 4l+4) and
-// [64+4l, 64+4l+4) of the piece; whole cache lines per store).  The tile's first (row, column
-// group) comes from one division per workgroup; a group past the end of a row moves to the next
-// row (rows shorter than a tile divide once more per lane).  Tile 0 also writes the pad codes
-// past the tensor.
+// flattened tensor is a 128-column piece of one row.  A workgroup takes a tile of 8 rows by 2
+// adjacent groups (2048 elements in runs of 1 KB), the 16 lanes of a DPP row own one group in
+// the row layout of the fused step (lane l: columns [4l, 4l+4) and [64+4l, 64+4l+4) of the
+// piece; whole cache lines per store).  The 8 rows of a tile read the same column statistics,
+// which a tile of 16 consecutive groups of one row does not: 1970 -> 1880 us per launch of
+// 8.6e8 elements on the LLaMA-7B MLP shapes (4 rows by 4 groups 1905 us, 16 rows by 1 group
+// 2060 us: its 512-byte runs cost more than the shared statistics save).  Tile 0 also writes
+// the pad codes past the tensor.
 #ifndef LPMM_FA_UPD_LDS_KB
 #define LPMM_FA_UPD_LDS_KB 0
 #endif
+#ifndef LPMM_FA_TILE_ROWS
+#define LPMM_FA_TILE_ROWS 8
+#endif
+constexpr uint32_t kFaTileRows = LPMM_FA_TILE_ROWS;
+static_assert((kFTile / kGroup) % LPMM_FA_TILE_ROWS == 0, "a tile is a whole number of groups per row");
 constexpr uint32_t kFaUpdLds = LPMM_FA_UPD_LDS_KB * 1024u > kLdsBytes ? LPMM_FA_UPD_LDS_KB * 1024u : kLdsBytes;
 
 __device__ __forceinline__ void update_rows128_body(
@@ -331,21 +337,15 @@ __device__ __forceinline__ void update_rows128_body(
     const int64_t n = R * C;
     const int lane16 = threadIdx.x & 15;
     const uint32_t col_blocks = (uint32_t)(C / kGroup);
-    const int64_t g0 = (int64_t)tile * (kFTile / kGroup);   // first group of the tile (uniform)
-    const int64_t r0 = g0 / col_blocks;
-    uint32_t cb = (uint32_t)(g0 - r0 * col_blocks) + (threadIdx.x >> 4);
-    int64_t r = r0;
-    if (col_blocks >= kFTile / kGroup) {  // uniform: a tile spans at most two rows
-        if (cb >= col_blocks) {
-            cb -= col_blocks;
-            ++r;
-        }
-    } else {
-        r += cb / col_blocks;
-        cb = cb % col_blocks;
-    }
-    const int64_t grp = g0 + (threadIdx.x >> 4);
-    const bool live = grp * kGroup < n;  // uniform over the 16 lanes of the group
+    // tile = kFaTileRows rows by 16 / kFaTileRows adjacent groups
+    constexpr uint32_t kGPS = (kFTile / kGroup) / kFaTileRows;
+    const uint32_t col_tiles = (col_blocks + kGPS - 1) / kGPS;
+    const uint32_t rb = tile / col_tiles, ct = tile - rb * col_tiles;
+    const uint32_t drow = threadIdx.x >> 4;
+    const int64_t r = (int64_t)rb * kFaTileRows + drow / kGPS;
+    const uint32_t cb = ct * kGPS + drow % kGPS;
+    const bool live = r < R && cb < col_blocks;  // uniform over the 16 lanes of the group
+    const int64_t grp = r * col_blocks + cb;
     const int64_t gbase = grp * kGroup;
     float *pp = p + gbase + lane16 * 4;
     uint16_t *mcp = reinterpret_cast<uint16_t *>(m_codes + (gbase >> 1)) + lane16;
@@ -543,6 +543,13 @@ __global__ __launch_bounds__(kFThreads) void factored_update_multi_kernel(const 
 
 inline int64_t round_up(int64_t a, int64_t b) { return (a + b - 1) / b * b; }
 
+// update tiles of a rows x cols tensor (cols a multiple of 128)
+inline uint64_t update_tiles(int64_t rows, int64_t cols)
+{
+    constexpr int64_t kTR = kFaTileRows, kGPS = (kFTile / kGroup) / kTR;
+    return (uint64_t)(((rows + kTR - 1) / kTR) * ((cols / kGroup + kGPS - 1) / kGPS));
+}
+
 }  // namespace lpmm
 
 using namespace lpmm;
@@ -718,7 +725,10 @@ extern "C" int lpmm_factored_update(float *p, const float *g, uint8_t *m_codes, 
     const bool vec = aligned_to(p, 16) && aligned_to(g, 16);
     const NfHyper h = make_nf_hyper(beta1, beta2, lr, weight_decay, eps, step);
     if ((cols % kGroup) == 0 && vec && aligned_to(col, 16) && aligned_to(m_codes, 4)) {
-        hipLaunchKernelGGL(factored_update_rows128_kernel, dim3((uint32_t)tiles), dim3(kFThreads), 0,
+        const uint64_t row_tiles = update_tiles(rows, cols);
+        if (row_tiles > 0x7fffffffULL)
+            return LPMM_ERR_SIZE;
+        hipLaunchKernelGGL(factored_update_rows128_kernel, dim3((uint32_t)row_tiles), dim3(kFThreads), 0,
                            (hipStream_t)stream, p, g, m_codes, m_max1, qmap_m, row, col, row_mean_all, rows, cols,
                            n_padded, h, first_step != 0);
     } else if ((cols % 8) == 0 && aligned_to(col, 16))
@@ -777,7 +787,7 @@ extern "C" int lpmm_factored_step_multi(const lpmm_factored_tensor *tensors, int
         if (t.rows <= 0 || t.cols <= 0 || t.cols % kGroup != 0 || t.rows > INT64_MAX / t.cols)
             return LPMM_ERR_SIZE;
         const int64_t ty = (t.rows + kSRows - 1) / kSRows, tx = (t.cols + kSCols - 1) / kSCols;
-        const int64_t ux = (t.cols + kFTile - 1) / kFTile;
+        const int64_t ux = (t.cols + kFTile - 1) / kFTile + 1;  // per row: an upper bound for any tile shape
         if (tx > 0x7fffffffLL / ty || ux > 0x7fffffffLL / t.rows ||
             (t.rows + kFThreads - 1) / kFThreads + (t.cols + 63) / 64 > 0x7fffffffLL)
             return LPMM_ERR_SIZE;
@@ -814,7 +824,7 @@ extern "C" int lpmm_factored_step_multi(const lpmm_factored_tensor *tensors, int
             const uint64_t ty = (uint64_t)((t.rows + kSRows - 1) / kSRows), tx = (uint64_t)((t.cols + kSCols - 1) / kSCols);
             const uint64_t row_blocks = (uint64_t)((t.rows + kFThreads - 1) / kFThreads);
             const uint64_t fin = row_blocks + (uint64_t)((t.cols + 63) / 64);
-            const uint64_t ux = (uint64_t)(round_up(t.rows * t.cols, kFTile) / kFTile);  // update tiles of the tensor
+            const uint64_t ux = update_tiles(t.rows, t.cols);
             if (n_stats + tx * ty > 0x7fffffffULL || n_fin + fin > 0x7fffffffULL ||
                 n_upd + ux > 0x7fffffffULL) {
                 if (k == 0)
