@@ -108,6 +108,22 @@ def test_rank1_two_pass_matches_staged_oracle(oracle, qmaps):
             t.check(f"{t.rows}x{t.cols} step {step}")
 
 
+def test_rank1_interleaved_row_blocks_with_ragged_last_group(oracle, qmaps):
+    """Tensors with more row blocks than interleave in one group: several groups, the last one
+    short of blocks and ending in a ragged block (2500 = 39 * 64 + 4 rows over 16 column tiles,
+    1100 = 17 * 64 + 12 rows over 32 column tiles, 64 * 11 + 1 rows over 43 column tiles of which
+    the last is half empty)."""
+    qm, qv = qmaps
+    dqm, dqv = to_dev(qm), to_dev(qv)
+    rng = np.random.default_rng(23)
+    tensors = [_Tensor(r, c, rng) for r, c in [(2500, 4096), (1100, 8192), (705, 11008)]]
+    for step in (1, 2):
+        grads = [_grad(rng, t) for t in tensors]
+        _step_all(oracle, tensors, grads, qm, qv, dqm, dqv, step)
+        for t in tensors:
+            t.check(f"{t.rows}x{t.cols} step {step}")
+
+
 def test_rank1_more_tensors_than_one_launch(oracle, qmaps):
     qm, qv = qmaps
     dqm, dqv = to_dev(qm), to_dev(qv)
