@@ -416,7 +416,7 @@ def run_factored(torch, args):
 def run_nonfused(torch, args, v_scale):
     """fused=False on the LLaMA-7B-shaped set.  v_scale 'group': both moments block-wise over
     128 values, one kernel per launch group of tensors; 'rank1' (the reference's default
-    configuration): dequantise, update, statistics and re-quantise kernels per tensor."""
+    configuration): an update pass and a re-quantise pass per launch group of tensors."""
     import lpmm
 
     dev = torch.device("cuda:0")
