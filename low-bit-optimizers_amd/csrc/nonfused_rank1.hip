@@ -39,8 +39,6 @@ constexpr int kThreads = 256;
 constexpr int kEltsPerLane = 8;
 constexpr int kDppRows = kThreads / 16;  // 128-column groups a workgroup handles per pass
 constexpr int kR1Max = 32;               // tensors per launch
-constexpr int kMaxLgWide = 3;
-constexpr int kMaxWide = 1 << kMaxLgWide;
 // Tile policy: widest tile (lg of 128-column groups), tensor rows per workgroup (more where one pass
 // of a narrow tile covers more), workgroups taken to be resident together.
 #ifndef LPMM_R1_LG
@@ -54,7 +52,9 @@ constexpr int kMaxWide = 1 << kMaxLgWide;
 #endif
 constexpr int kPolicyLgWide = LPMM_R1_LG;
 constexpr uint32_t kPolicyRows = LPMM_R1_ROWS, kPolicyResident = LPMM_R1_RESIDENT;
-static_assert(LPMM_R1_LG <= kMaxLgWide, "the LDS column arrays hold 128 << 3 columns");
+static_assert(LPMM_R1_LG >= 1 && LPMM_R1_LG <= 3, "a tile is 256 to 1024 columns wide at most");
+constexpr int kMaxLgWide = kPolicyLgWide;   // the LDS column arrays hold 128 << kMaxLgWide columns
+constexpr int kMaxWide = 1 << kMaxLgWide;
 // Per-column data of a tile lives in LDS, not in registers (occupancy): the current column
 // statistics in the unused bytes between the maps and the encode table, further arrays after
 // the table.
