@@ -520,8 +520,7 @@ def main():
     n_quant_tensors = sum(1 for p in params if p.numel() > 4096)
     launches_per_step = math.ceil(n_quant_tensors / MULTI_MAX)
 
-    # events around the dominant kernel's launches (same stream as the launches); a call is one launch when
-    # every tensor is a whole number of tiles (the LLaMA-7B set), else a second short launch takes the ragged tails
+    # events around the dominant kernel's launches (same stream as the launches)
     events = []
     real_call = lib.lpmm_adamw4bit_step_multi
     recording = {"on": False}

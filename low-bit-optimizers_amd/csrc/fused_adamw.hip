@@ -73,7 +73,7 @@ struct Tensor4 {
     float c1;    // 1 - beta1^step
     float c2s;   // sqrt(1 - beta2^step)
     float rc2s;  // 1 / c2s, correctly rounded (host division)
-    uint32_t owns_end;  // padded layout: this record ends where its tensor ends (its last tile writes the extra byte)
+    float pad;
 };
 
 constexpr int kStartSlots = LPMM_MULTI_MAX + 8;   // tile_start is read 8 entries at a time
@@ -348,7 +348,7 @@ __global__ __launch_bounds__(kThreads) void adamw4bit_kernel(const Multi4 args,
     // the loaded words stay as they are until here, so that nothing above waits for them
     asm volatile("" : "+v"(regs.m0), "+v"(regs.m1), "+v"(regs.v0), "+v"(regs.v1));
 
-    if (Arith::kPadded && threadIdx.x == 0 && t.owns_end != 0 && blockIdx.x + 1 == args.tile_start[lo + 1]) {
+    if (Arith::kPadded && threadIdx.x == 0 && blockIdx.x + 1 == args.tile_start[lo + 1]) {
         // the tensor's last tile also owns the extra byte at the end of each code buffer
         const int64_t end = (int64_t)(args.tile_start[lo + 1] - args.tile_start[lo]) * (kTile / 2);
         t.mc[end] = 0;
@@ -506,70 +506,59 @@ static int step_multi4(const lpmm_adamw4bit_tensor *tensors, int64_t count, cons
     Multi4 args;
     for (int j = 0; j < 7; ++j)
         args.s[j] = scalars[j];
-    // Two rounds over the list.  The first takes the whole tiles of every tensor whose pointers allow
-    // vector access and launches the straight-line variant of the kernel; the second takes what is left
-    // -- the ragged last tile of a tensor (tiles are independent, so it is a tensor of its own that
-    // starts at a tile boundary) and tensors with unaligned pointers -- and launches the guarded variants.
-    // A set in which a few tensors are ragged (GPT-2-XL: the embedding and the 4800- and 6400-long
-    // biases) thus runs all but a few thousand of its elements through the fast variant.
-    for (int round = 0; round < 2; ++round) {
-        int64_t i = 0;
-        while (i < count) {
-            int k = 0;
-            uint64_t tiles = 0;
-            bool aligned = true;  // per launch: do all pointers allow vector access
-            args.tile_start[0] = 0;
-            while (i < count && k < LPMM_MULTI_MAX) {
-                const lpmm_adamw4bit_tensor &t = tensors[i];
-                const bool vec = aligned_to(t.p, 16) && aligned_to(t.g, 16) && aligned_to(t.m_codes, 2) &&
-                                 aligned_to(t.v_codes, 2);
-                // this round's share of the tensor: elements [first, first + n)
-                const int64_t whole = vec ? t.n - t.n % kTile : 0;
-                const int64_t first = round == 0 ? 0 : whole;
-                const int64_t n = round == 0 ? whole : t.n - whole;
-                if (n == 0) {
-                    ++i;
-                    continue;
-                }
-                const uint64_t nt = (uint64_t)((n + kTile - 1) / kTile);
-                if (tiles + nt > 0x7fffffffULL)
-                    break;
-                aligned = aligned && vec;
-                Tensor4 &d = args.t[k];
-                d.p = t.p + first;
-                d.g = t.g + first;
-                d.mc = t.m_codes + first / 2;
-                d.vc = t.v_codes + first / 2;
-                d.ms = t.m_scale + first / kGroup;
-                d.vs = t.v_scale + first / kGroup;
-                d.n = n;
-                per_tensor(t.step, &d.c1, &d.c2s, &d.rc2s);
-                d.owns_end = first + n == t.n;
-                tiles += nt;
-                args.tile_start[++k] = (uint32_t)tiles;
+    int64_t i = 0;
+    while (i < count) {
+        int k = 0;
+        uint64_t tiles = 0;
+        // per launch: do all pointers allow vector access, is every tensor a whole number of tiles
+        bool aligned = true, allfull = true;
+        args.tile_start[0] = 0;
+        while (i < count && k < LPMM_MULTI_MAX) {
+            const lpmm_adamw4bit_tensor &t = tensors[i];
+            if (t.n == 0) {
                 ++i;
-            }
-            if (k == 0)
                 continue;
-            args.count = k;
-            for (int j = k + 1; j < kStartSlots; ++j)
-                args.tile_start[j] = (uint32_t)tiles;
-            for (int j = 0; j < kCoarseSlots; ++j)
-                args.coarse[j] = args.tile_start[8 * (j + 1)];
-            const dim3 grid((uint32_t)tiles), block(kThreads);
-            if (round == 0)
-                hipLaunchKernelGGL((adamw4bit_kernel<true, true, Arith>), grid, block, 0, (hipStream_t)stream, args,
-                                   qmap_m, qmap_v);
-            else if (aligned)
-                hipLaunchKernelGGL((adamw4bit_kernel<true, false, Arith>), grid, block, 0, (hipStream_t)stream, args,
-                                   qmap_m, qmap_v);
-            else
-                hipLaunchKernelGGL((adamw4bit_kernel<false, false, Arith>), grid, block, 0, (hipStream_t)stream, args,
-                                   qmap_m, qmap_v);
-            const int st = launch_status();
-            if (st != LPMM_OK)
-                return st;
+            }
+            const uint64_t nt = (uint64_t)((t.n + kTile - 1) / kTile);
+            if (tiles + nt > 0x7fffffffULL)
+                break;
+            allfull = allfull && (t.n % kTile) == 0;
+            aligned = aligned && aligned_to(t.p, 16) && aligned_to(t.g, 16) && aligned_to(t.m_codes, 2) &&
+                      aligned_to(t.v_codes, 2);
+            Tensor4 &d = args.t[k];
+            d.p = t.p;
+            d.g = t.g;
+            d.mc = t.m_codes;
+            d.vc = t.v_codes;
+            d.ms = t.m_scale;
+            d.vs = t.v_scale;
+            d.n = t.n;
+            per_tensor(t.step, &d.c1, &d.c2s, &d.rc2s);
+            d.pad = 0.0f;
+            tiles += nt;
+            args.tile_start[++k] = (uint32_t)tiles;
+            ++i;
         }
+        if (k == 0)
+            continue;
+        args.count = k;
+        for (int j = k + 1; j < kStartSlots; ++j)
+            args.tile_start[j] = (uint32_t)tiles;
+        for (int j = 0; j < kCoarseSlots; ++j)
+            args.coarse[j] = args.tile_start[8 * (j + 1)];
+        const dim3 grid((uint32_t)tiles), block(kThreads);
+        if (aligned && allfull)
+            hipLaunchKernelGGL((adamw4bit_kernel<true, true, Arith>), grid, block, 0, (hipStream_t)stream, args,
+                               qmap_m, qmap_v);
+        else if (aligned)
+            hipLaunchKernelGGL((adamw4bit_kernel<true, false, Arith>), grid, block, 0, (hipStream_t)stream, args,
+                               qmap_m, qmap_v);
+        else
+            hipLaunchKernelGGL((adamw4bit_kernel<false, false, Arith>), grid, block, 0, (hipStream_t)stream, args,
+                               qmap_m, qmap_v);
+        const int st = launch_status();
+        if (st != LPMM_OK)
+            return st;
     }
     return LPMM_OK;
 }
