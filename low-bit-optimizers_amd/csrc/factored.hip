@@ -349,7 +349,8 @@ __device__ __forceinline__ void update_rows128_body(
     const int64_t gbase = grp * kGroup;
     float *pp = p + gbase + lane16 * 4;
     uint16_t *mcp = reinterpret_cast<uint16_t *>(m_codes + (gbase >> 1)) + lane16;
-    // the group's loads first, the LDS tables afterwards
+    // the small loads that feed LDS first (they return first), then the group's loads
+    const LdsFill fill = lds_fill_load(qmap_m, qmap_m);
     float4 a0, a1, b0, b1, c_lo, c_hi;
     uint32_t w0 = 0, w1 = 0;
     float sm = 0.0f, row_r = 0.0f, mean_all = 1.0f;
@@ -370,7 +371,7 @@ __device__ __forceinline__ void update_rows128_body(
         row_r = row[r];
         mean_all = *row_mean_all;
     }
-    lds_fill(lds, qmap_m, nullptr);
+    lds_fill_store(lds, fill);
     const int kind = classify_map(qmap_m);
     lds_barrier();
     if (tile == 0) {

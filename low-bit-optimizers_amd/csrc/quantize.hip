@@ -13,6 +13,7 @@
 namespace lpmm {
 
 constexpr int kQThreads = 256;
+static_assert(kQThreads == kEncEntries, "lds_fill_load / lds_fill_store: one encode-table entry per thread");
 constexpr int kQElts = 8;
 constexpr int kQTile = kQThreads * kQElts;  // 2048
 
@@ -137,6 +138,11 @@ __global__ __launch_bounds__(THREADS) void quant_group_kernel(const float *__res
 
     if (vec && tile0 + (int64_t)T * kTileElts <= n) {  // uniform over the workgroup
         float v[T][kQElts];
+        // the small loads that feed LDS first (they return first), then the tiles' loads (workgroups
+        // of one thread per encode-table entry; larger ones fill the tables after their loads)
+        LdsFill fill;
+        if (THREADS == kEncEntries)
+            fill = lds_fill_load(qmap, qmap);
 #pragma unroll
         for (int t = 0; t < T; ++t) {
             const float *p = x + tile0 + (int64_t)t * kTileElts + wrow * kGroup + lane16 * 4;
@@ -144,7 +150,10 @@ __global__ __launch_bounds__(THREADS) void quant_group_kernel(const float *__res
             v[t][0] = a.x; v[t][1] = a.y; v[t][2] = a.z; v[t][3] = a.w;
             v[t][4] = b.x; v[t][5] = b.y; v[t][6] = b.z; v[t][7] = b.w;
         }
-        lds_fill(lds, qmap, nullptr);
+        if (THREADS == kEncEntries)
+            lds_fill_store(lds, fill);
+        else
+            lds_fill(lds, qmap, nullptr);
         const int kind = classify_map(qmap);
         if (tile0 == 0 && threadIdx.x == 0)
             codes[n_padded / 2] = 0;
@@ -573,6 +582,8 @@ __global__ __launch_bounds__(kQThreads) void quant_rank1_rows128_kernel(const fl
     const int64_t r0 = (int64_t)blockIdx.y * T;
     const int64_t c0 = (int64_t)blockIdx.x * kR1Cols + (int64_t)(threadIdx.x >> 4) * kGroup;
     const bool live = c0 < C;  // uniform over the 16 lanes of a group
+    // the small loads that feed LDS first (they return first), then the rows' loads
+    const LdsFill fill = lds_fill_load(qmap, qmap);
     float4 a[T], b[T], ca, cb;
     float rm[T];
     if (live) {
@@ -589,7 +600,7 @@ __global__ __launch_bounds__(kQThreads) void quant_rank1_rows128_kernel(const fl
             }
         }
     }
-    lds_fill(lds, qmap, nullptr);
+    lds_fill_store(lds, fill);
     const int kind = classify_map(qmap);
     lds_barrier();
     if (blockIdx.x == 0 && blockIdx.y == 0) {
