@@ -16,7 +16,8 @@ prints the full table alone).
 Two further workloads measure the other kernels of the path with the same JSON shape:
 `--workload quant64m` (stand-alone quantise/dequantise round trip on 2^26 values) and
 `--workload factored` (factored second moment on LLaMA-7B MLP/attention shapes) and
-`--workload nonfused_group|nonfused_rank1` (fused=False on the LLaMA-7B-shaped set).
+`--workload nonfused_group|nonfused_rank1` (fused=False on the LLaMA-7B-shaped set) and
+`--workload sgd` (4-bit SGD momentum on the same set).
 """
 import argparse
 import contextlib
@@ -413,6 +414,39 @@ def run_factored(torch, args):
                      "traffic": None, "bytes_per_param": 17.0625}}))
 
 
+def run_sgd(torch, args):
+    """lpmm.optim.SGD (momentum 0.9, 4-bit momentum buffer) on the LLaMA-7B-shaped set: one pass
+    per launch group of 64 tensors, 13.0625 B per quantised parameter (p read and written 8, g 4,
+    codes read and written 1, scales 8/128); the 65 norm vectors keep fp32 buffers and take the
+    reference's chain of PyTorch ops."""
+    import lpmm
+
+    dev = torch.device("cuda:0")
+    params = make_params(torch, llama7b_shapes(), dev, heavy_tailed=True)
+    opt = lpmm.optim.SGD(params, lr=1e-3, momentum=0.9, weight_decay=1e-4)
+    n_total = sum(p.numel() for p in params)
+    for _ in range(args.warmup):
+        opt.step()
+    torch.cuda.synchronize()
+    with _gc_paused():
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            opt.step()
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - t0) / args.steps
+    bytes_per_param = 13.0625
+    achieved = n_total * bytes_per_param / dt / 1e9
+    print(json.dumps({
+        "metric": "4-bit SGD-momentum step: params/sec, 1 MI355X", "value": n_total / dt,
+        "unit": "params/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": dt * 1e3,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "SGD, momentum 0.9, 4-bit momentum buffer, LLaMA-7B-shaped fp32 set",
+                   "tensors": len(params), "params": n_total},
+        "roofline": {"bound": "hbm", "kernel": "whole step", "achieved": achieved, "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "bytes_per_param": bytes_per_param}}))
+
+
 def run_nonfused(torch, args, v_scale):
     """fused=False on the LLaMA-7B-shaped set.  v_scale 'group': both moments block-wise over
     128 values, one kernel per launch group of tensors; 'rank1' (the reference's default
@@ -455,7 +489,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="llama7b", choices=sorted(WORKLOADS) + ["quant64m", "factored", "nonfused_group", "nonfused_rank1", "calibrate"])
+    ap.add_argument("--workload", default="llama7b", choices=sorted(WORKLOADS) + ["quant64m", "factored", "nonfused_group", "nonfused_rank1", "sgd", "calibrate"])
     ap.add_argument("--bits", type=int, default=4, choices=range(1, 9), help="code width of --workload quant64m")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--interleaved-grads", action="store_true",
@@ -506,6 +540,8 @@ def main():
         return run_quant_roundtrip(torch, args)
     if args.workload == "factored":
         return run_factored(torch, args)
+    if args.workload == "sgd":
+        return run_sgd(torch, args)
     if args.workload.startswith("nonfused_"):
         return run_nonfused(torch, args, args.workload.split("_")[1])
 

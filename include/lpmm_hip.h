@@ -349,6 +349,33 @@ int lpmm_factored_update_fp32m(float *p, const float *g, float *m, const float *
                                double weight_decay, double eps, double step, void *stream);
 
 /* ---------------------------------------------------------------------------------------
+ * (d) SGD with a 4-bit momentum buffer, one pass, for a list of tensors.
+ * Replaces the per-tensor op chain of _single_tensor_sgd4bit (lpmm/optim/sgd.py:133-187) for
+ * tensors whose buffer is quantised with 4 bits, 'group' scaling, gp_sz 128, round to nearest:
+ *   d = -g if maximize else g;  d += weight_decay * p (if weight_decay != 0)     (:152-155)
+ *   buf = d on the first step, else buf = dequant(codes) * momentum + (1 - dampening) * d  (:161-173)
+ *   d = d + momentum * buf if nesterov else buf;  p += -lr * d                   (:176-181)
+ *   codes, max1 = quantise(buf)                                                  (:184-187)
+ * Every multiply-add of the chain is one fused operation with the float-cast scalar, as in
+ * PyTorch's kernels.  m_codes: int8[ceil(n / 2048) * 1024 + 1] (the packed layout of
+ * vectorwise_quant), m_max1: float[ceil(n / 128)]; first_step != 0 means the buffer does not
+ * exist yet and both are only written.  momentum must not be 0 (the reference keeps no buffer
+ * then).  Up to 64 tensors per launch. */
+typedef struct lpmm_sgd4bit_tensor {
+    float *p;
+    const float *g;
+    uint8_t *m_codes;
+    float *m_max1;
+    int64_t n;
+    int32_t first_step;
+    int32_t reserved;
+} lpmm_sgd4bit_tensor;
+
+int lpmm_sgd4bit_step_multi(const lpmm_sgd4bit_tensor *tensors, int64_t count, const float *qmap,
+                            double momentum, double dampening, double lr, double weight_decay,
+                            int nesterov, int maximize, void *stream);
+
+/* ---------------------------------------------------------------------------------------
  * Diagnostic (no counterpart in the reference): compares the library's near-exact sqrt and
  * division sequences (hardware approximation + one fma correction of the residual) with the
  * correctly rounded operations on the device.  counts: 11 zero-initialised device uint64:

@@ -11,6 +11,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "liblpmm_hip.so")
 MULTI_MAX = 48  # tensors per launch of the fused step (LPMM_MULTI_MAX in include/lpmm_hip.h)
 RANK1_MULTI_MAX = 32  # tensors per launch of the two-pass rank-1 step (kR1Max in csrc/nonfused_rank1.hip)
+SGD_MULTI_MAX = 64  # tensors per launch of the one-pass SGD step (kSgdMax in csrc/sgd.hip)
 ABI_VERSION = 1
 
 _vp = ctypes.c_void_p
@@ -54,6 +55,7 @@ PROTOTYPES = {
     "lpmm_factored_update": (_int, [_vp] * 8 + [_i64, _i64] + [_d] * 6 + [_int, _vp]),
     "lpmm_factored_step_multi": (_int, [_vp, _i64, _vp] + [_d] * 5 + [_vp]),
     "lpmm_factored_update_fp32m": (_int, [_vp] * 6 + [_i64, _i64] + [_d] * 6 + [_vp]),
+    "lpmm_sgd4bit_step_multi": (_int, [_vp, _i64, _vp] + [_d] * 4 + [_int, _int, _vp]),
     "lpmm_stream_probe": (_int, [_int] + [_vp] * 6 + [_i64, _i64, _vp]),
     "lpmm_selftest_encoders": (_int, [_vp, _vp]),
     "lpmm_selftest_arithmetic": (_int, [_vp, ctypes.c_uint32, ctypes.c_uint64, ctypes.c_uint32, _vp]),
@@ -70,6 +72,8 @@ NONFUSED_RANK1_TENSOR = np.dtype([("p", "<u8"), ("g", "<u8"), ("m_codes", "<u8")
 FACTORED_TENSOR = np.dtype([("p", "<u8"), ("g", "<u8"), ("m_codes", "<u8"), ("m_max1", "<u8"), ("row", "<u8"),
                             ("col", "<u8"), ("workspace", "<u8"), ("rows", "<i8"), ("cols", "<i8"), ("step", "<f4"),
                             ("first_step", "<i4")])
+SGD4BIT_TENSOR = np.dtype([("p", "<u8"), ("g", "<u8"), ("m_codes", "<u8"), ("m_max1", "<u8"), ("n", "<i8"),
+                           ("first_step", "<i4"), ("reserved", "<i4")])
 ADAMW_FP32_TENSOR = np.dtype([("p", "<u8"), ("g", "<u8"), ("m", "<u8"), ("v", "<u8"), ("n", "<i8"),
                               ("step", "<f4"), ("reserved", "<f4")])
 

@@ -2,15 +2,21 @@
 
 Drop-in for lpmm.optim.SGD (lpmm/optim/sgd.py:11-187): same constructor and state keys
 (`momentum_buffer`, `momentum_buffer_qstate`), non-fused only (fused=True raises, as there).
-The momentum buffer uses the first-moment quantisation config (QUANT.M); dequantise and
-quantise are the one-pass HIP kernels of lpmm.functional, the update itself is the same
-short chain of PyTorch ops on the device as in the reference (lpmm/optim/sgd.py:152-187).
+The momentum buffer uses the first-moment quantisation config (QUANT.M).  Contiguous float32
+tensors whose buffer is quantised with 4 bits, 'group' scaling over 128 values and round to
+nearest (the default configuration) take one HIP kernel per 64 tensors that reads p, g and the
+packed buffer once and writes p and the buffer back (lpmm_sgd4bit_step_multi: 13 bytes per
+parameter).  Every other case runs the reference's own chain of PyTorch ops on the device
+(lpmm/optim/sgd.py:152-187) around the HIP dequantise / quantise kernels of lpmm.functional.
+Both produce the same state layout.
 """
 from typing import Optional
 
+import numpy as np
 import torch
 
-from ..functional import vectorwise_dequant, vectorwise_quant
+from .. import _native
+from ..functional import packed_nbytes, vectorwise_dequant, vectorwise_quant
 from .optimizer import LowBitOptimizer
 
 __all__ = ["SGD"]
@@ -56,8 +62,11 @@ class SGD(LowBitOptimizer):
                 loss = closure()
 
         md = self.get_qmetadata_by_state_name("momentum_buffer")
+        one_pass_config = (md["b"] == 4 and md["scale_type"] == "group" and md["gp_sz"] == 128
+                           and md["round_type"] == "real-nearest")
         for group in self.param_groups:
             momentum, dampening = group["momentum"], group["dampening"]
+            batched = {}  # (device, map address) -> records of the one-pass kernel
             for p in group["params"]:
                 if p.grad is None:
                     continue
@@ -69,6 +78,22 @@ class SGD(LowBitOptimizer):
                     self.init_qstate(p, "momentum_buffer")
                 qstate = state["momentum_buffer_qstate"]
                 enabled = self.override_q_enable.get(id(p), qstate["enable"])
+
+                if (one_pass_config and enabled and momentum != 0 and p.is_cuda and p.dtype is torch.float32
+                        and p.grad.dtype is torch.float32 and p.is_contiguous() and p.grad.is_contiguous()):
+                    first = state["momentum_buffer"].numel() <= 1
+                    if first:
+                        groups = (p.numel() + 127) // 128
+                        state["momentum_buffer"] = torch.empty((packed_nbytes(groups * 128),), dtype=torch.int8,
+                                                               device=p.device)
+                        qstate["overhead"].clear()
+                        qstate["overhead"].update({"dtype": p.dtype, "stride": p.stride(),
+                                                   "max1": torch.empty((groups, 1), dtype=torch.float32, device=p.device),
+                                                   "scaled_shape": torch.Size((groups, 128))})
+                    batched.setdefault((p.device, qstate["qmap"].data_ptr()), []).append(
+                        (p.data_ptr(), p.grad.data_ptr(), state["momentum_buffer"].data_ptr(),
+                         qstate["overhead"]["max1"].data_ptr(), p.numel(), 1 if first else 0, 0))
+                    continue
 
                 d_p = p.grad if not group["maximize"] else -p.grad
                 if group["weight_decay"] != 0:
@@ -95,4 +120,13 @@ class SGD(LowBitOptimizer):
                     else:
                         state["momentum_buffer"] = buf
                 p.add_(d_p, alpha=-group["lr"])
+
+            for (dev, qmap_ptr), records in batched.items():
+                table = np.array(records, dtype=_native.SGD4BIT_TENSOR)
+                with torch.cuda.device(dev):
+                    st = _native.lib().lpmm_sgd4bit_step_multi(
+                        table.ctypes.data, len(records), qmap_ptr, momentum, dampening, group["lr"],
+                        group["weight_decay"], int(bool(group["nesterov"])), int(bool(group["maximize"])),
+                        _native.current_stream(dev))
+                _native.check(st, "SGD step")
         return loss

@@ -28,6 +28,8 @@
  *   nonfused_step       PyTorch CPU op sequence (library ops) of the reference's
  *                       _single_tensor_adamw4bit, to 1e-6 relative.
  *   factored_step       closed form v = row*col/mean(row) (Adafactor); rank-one g^2 case.
+ *   sgd_update          PyTorch CPU op sequence (library ops) of the reference's
+ *                       _single_tensor_sgd4bit, bit for bit.
  *   philox / SR pack    Random123's known-answer vectors for philox4x32-10; torch.randint on
  *                       the GPU for cuRAND's state conventions; noise = 0.5 reduces the
  *                       stochastic search to round-to-nearest on the linear scale; the
@@ -501,6 +503,44 @@ void lpmm_oracle_nonfused_update(float *p, const float *g, float *m, float *v, i
         p[i] = pi;
         m[i] = mi;
         v[i] = vi;
+    }
+}
+
+/* ------------------------------------------------------------------------------------ */
+/* 4-bit SGD with momentum: the elementwise part of lpmm/optim/sgd.py:133-187            */
+/* (_single_tensor_sgd4bit) on fp32 buffers, with the roundings of the PyTorch kernels   */
+/* its op sequence runs: Tensor.add(other, alpha=s) is fma(s, other, self) with s cast   */
+/* to float (alpha = 1 gives the same value as a plain add), mul_ is one multiply.       */
+/*   d = -g if maximize else g;  d = d.add(p, alpha=wd) if wd != 0          (:152-155)   */
+/*   first step: buf = d                                                    (:161-163)   */
+/*   else:       buf.mul_(momentum).add_(d, alpha=1-dampening)              (:173)       */
+/*   d = d.add(buf, alpha=momentum) if nesterov else buf                    (:176-179)   */
+/*   p.add_(d, alpha=-lr)                                                   (:181)       */
+/* buf is a full fp32 tensor here (already dequantised / to be quantised).               */
+/* ------------------------------------------------------------------------------------ */
+void lpmm_oracle_sgd_update(float *p, const float *g, float *buf, int64_t n, double momentum,
+                            double dampening, double lr, double weight_decay, int nesterov,
+                            int maximize, int first_step)
+{
+    const float mom = (float)momentum;
+    const float w = (float)(1.0 - dampening);
+    const float wd = (float)weight_decay;
+    const float neg_lr = (float)(-lr);
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < n; ++i) {
+        float d = maximize ? -g[i] : g[i];
+        if (weight_decay != 0.0)
+            d = fmaf(wd, p[i], d);
+        float b;
+        if (first_step) {
+            b = d;
+        } else {
+            b = buf[i] * mom;
+            b = fmaf(w, d, b);
+        }
+        const float u = nesterov ? fmaf(mom, b, d) : b;
+        p[i] = fmaf(neg_lr, u, p[i]);
+        buf[i] = b;
     }
 }
 

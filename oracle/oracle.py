@@ -82,6 +82,8 @@ _dequant_rank1 = _sig("lpmm_oracle_dequant_rank1", None, _u8p, _f32p, _f32p, _f3
                       _f32p)
 _nonfused_update = _sig("lpmm_oracle_nonfused_update", None, _f32p, _f32p, _f32p, _f32p, _i64,
                         _d, _d, _d, _d, _d, _d)
+_sgd_update = _sig("lpmm_oracle_sgd_update", None, _f32p, _f32p, _f32p, _i64, _d, _d, _d, _d, ctypes.c_int,
+                   ctypes.c_int, ctypes.c_int)
 _factored_stats = _sig("lpmm_oracle_factored_stats", None, _f32p, _i64, _i64, _f32p, _f32p)
 _factored_ema = _sig("lpmm_oracle_factored_ema", _f, _f32p, _f32p, _f32p, _f32p, _i64, _i64, _d)
 _factored_update = _sig("lpmm_oracle_factored_update", None, _f32p, _f32p, _f32p, _f32p, _f32p,
@@ -433,6 +435,12 @@ def dequant_rank1(codes, rowmax, colmax, qmap, r, c):
 
 def nonfused_update(p, g, m, v, beta1, beta2, lr, wd, eps, step):
     _nonfused_update(p, g, m, v, p.size, beta1, beta2, lr, wd, eps, step)
+
+
+def sgd_update(p, g, buf, momentum, dampening, lr, wd, nesterov, maximize, first_step):
+    """Elementwise part of _single_tensor_sgd4bit (lpmm/optim/sgd.py:133-187) on fp32 buffers, in place."""
+    _sgd_update(p, g, buf, p.size, momentum, dampening, lr, wd, int(bool(nesterov)), int(bool(maximize)),
+                int(bool(first_step)))
 
 
 def factored_stats(g):

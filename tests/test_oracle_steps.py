@@ -304,6 +304,37 @@ def test_nonfused_c_update_follows_torch_cpu_ops(oracle, qmaps):
     assert flips <= 2, flips
 
 
+@pytest.mark.parametrize("nesterov", [False, True])
+@pytest.mark.parametrize("maximize", [False, True])
+@pytest.mark.parametrize("dampening, wd", [(0.0, 0.0), (0.1, 1e-4), (0.0, 0.05)])
+def test_sgd_c_update_follows_torch_cpu_ops(oracle, nesterov, maximize, dampening, wd):
+    """The elementwise part of the 4-bit SGD step against the reference's own op sequence
+    (lpmm/optim/sgd.py:152-181) run by PyTorch's CPU kernels, bit for bit, over three steps
+    (the first stores the decayed gradient itself): Tensor.add(alpha=) is one fused
+    multiply-add with the float-cast scalar, mul_ one multiply.  Sizes cover the vectorised
+    body of the library kernels and their scalar tails."""
+    rng = np.random.default_rng(31)
+    lr, mom = 0.05, 0.9
+    for n in (1, 7, 64, 1000, 4099):
+        p = rng.standard_normal(n).astype(f32)
+        tp, tbuf, buf = torch.from_numpy(p.copy()), None, np.zeros(n, f32)
+        for step in range(3):
+            g = (rng.standard_normal(n) * 1e-2).astype(f32)
+            tg = torch.from_numpy(g)
+            d_p = tg if not maximize else -tg
+            if wd != 0:
+                d_p = d_p.add(tp, alpha=wd)
+            if tbuf is None:
+                tbuf = torch.clone(d_p).detach()
+            else:
+                tbuf.mul_(mom).add_(d_p, alpha=1 - dampening)
+            d_p = d_p.add(tbuf, alpha=mom) if nesterov else tbuf
+            tp.add_(d_p, alpha=-lr)
+            oracle.sgd_update(p, g, buf, mom, dampening, lr, wd, nesterov, maximize, step == 0)
+            assert np.array_equal(buf, tbuf.numpy()), (n, step)
+            assert np.array_equal(p, tp.numpy()), (n, step)
+
+
 def test_factored_closed_forms(oracle):
     rng = np.random.default_rng(7)
     r, c = 24, 40
