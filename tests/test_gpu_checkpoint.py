@@ -121,6 +121,62 @@ def test_resume_through_a_file_equals_uninterrupted_run(mode, map_location, tmp_
             assert torch.equal(sa[name], sc[name].to(sa[name].device)), f"state {name} differs after the resumed run"
 
 
+@pytest.mark.parametrize("map_location", [None, "cpu"])
+def test_sgd_resume_through_a_file_equals_uninterrupted_run(map_location, tmp_path):
+    """lpmm.optim.SGD with a 4-bit momentum buffer: tensors on the one-pass kernel (contiguous, quantised),
+    a strided one on the chain of PyTorch ops, and one with an fp32 buffer."""
+    import lpmm
+
+    shapes = [(96, 256), (8192,), (70, 130), (1600,)]
+    rng = np.random.default_rng(13)
+    start = [(rng.standard_normal(s) * 0.02).astype(np.float32) for s in shapes]
+    grads = [[(rng.standard_normal(s) * 1e-2).astype(np.float32) for s in shapes] for _ in range(6)]
+
+    def make(params):
+        return lpmm.optim.SGD(params, lr=0.05, momentum=0.9, dampening=0.1, weight_decay=1e-4, nesterov=True)
+
+    def fresh(values):
+        params = [torch.nn.Parameter(to_dev(x)) for x in values]
+        # the third tensor lives transposed in its storage: not contiguous
+        params[2] = torch.nn.Parameter(to_dev(np.ascontiguousarray(values[2].T)).t())
+        assert not params[2].is_contiguous()
+        return params
+
+    def run(opt, params, steps):
+        for k in steps:
+            for i, (p, g) in enumerate(zip(params, grads[k])):
+                p.grad = to_dev(np.ascontiguousarray(g.T)).t() if i == 2 else to_dev(g)
+            opt.step()
+
+    params_a = fresh(start)
+    opt_a = make(params_a)
+    run(opt_a, params_a, range(6))
+
+    params_b = fresh(start)
+    opt_b = make(params_b)
+    run(opt_b, params_b, range(3))
+    path = str(tmp_path / "sgd.pt")
+    torch.save({"opt": opt_b.state_dict(), "params": [p.detach().contiguous() for p in params_b]}, path)
+    del opt_b
+
+    ckpt = torch.load(path, weights_only=True, map_location=map_location)
+    params_c = fresh([to_np(p) for p in ckpt["params"]])
+    opt_c = make(params_c)
+    opt_c.load_state_dict(ckpt["opt"])
+    run(opt_c, params_c, range(3, 6))
+    torch.cuda.synchronize()
+
+    for i, (pa, pc) in enumerate(zip(params_a, params_c)):
+        assert torch.equal(pa, pc), f"parameter {i} {tuple(pa.shape)} differs after the resumed run"
+    sa, sc = _flat_state(opt_a, params_a), _flat_state(opt_c, params_c)
+    assert sa.keys() == sc.keys()
+    for name in sa:
+        assert sa[name].dtype == sc[name].dtype and sa[name].shape == sc[name].shape, name
+        assert torch.equal(sa[name], sc[name].to(sa[name].device)), f"state {name} differs after the resumed run"
+    assert opt_c.state[params_c[0]]["momentum_buffer"].dtype == torch.int8
+    assert opt_c.state[params_c[3]]["momentum_buffer"].dtype == torch.float32
+
+
 def test_reference_shaped_fused_checkpoint_continues_like_the_oracle(oracle, qmaps):
     import lpmm
 
