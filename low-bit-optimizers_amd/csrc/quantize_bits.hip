@@ -65,6 +65,39 @@ __device__ __forceinline__ void fill_search(SearchLds &t, const float *__restric
     }
 }
 
+// The same in two halves for workgroups of at least 2^bits threads (one entry per thread), so that a
+// kernel can issue these small loads first, start its streaming loads, and write LDS once the small
+// ones have arrived (loads return in order).
+struct SearchFill {
+    float tree, mid;
+};
+
+__device__ __forceinline__ SearchFill fill_search_load(const float *__restrict__ qmap, int bits)
+{
+    SearchFill f;
+    const uint32_t n = 1u << bits, j = threadIdx.x;
+    f.tree = f.mid = 0.0f;
+    if (j == 0) {
+        f.tree = qmap[0];
+        f.mid = qmap[n - 1];
+    } else if (j < n) {
+        const uint32_t level = 31u - (uint32_t)__clz((int)j);
+        const uint32_t k = j - (1u << level);
+        f.tree = qmap[(((2u * k + 1u) << (bits - 1 - level))) - 1u];
+        f.mid = (qmap[j - 1] + qmap[j]) * 0.5f;
+    }
+    return f;
+}
+
+__device__ __forceinline__ void fill_search_store(SearchLds &t, const SearchFill &f, int bits)
+{
+    if (threadIdx.x < (1u << bits)) {
+        t.tree[threadIdx.x] = f.tree;
+        t.mid[threadIdx.x] = f.mid;
+    }
+}
+static_assert(kBThreads >= 256, "fill_search_load: one map entry per thread for up to 8 bits");
+
 __device__ __forceinline__ uint32_t search_code(const SearchLds &t, int bits, float x)
 {
     const uint32_t n = 1u << bits;
@@ -554,6 +587,8 @@ __global__ __launch_bounds__(kBThreads) void quant_group_bits_rows_kernel(const 
     __shared__ float s_row[T][kBThreads / 16];
     const int lane16 = threadIdx.x & 15, wrow = threadIdx.x >> 4;
     const int64_t tile0 = (int64_t)blockIdx.x * T;
+    // the small loads that feed LDS first (they return first), then the tiles' loads
+    const SearchFill fill = fill_search_load(qmap, bits);
     float v[T][kBElts];
 #pragma unroll
     for (int t = 0; t < T; ++t) {
@@ -565,7 +600,7 @@ __global__ __launch_bounds__(kBThreads) void quant_group_bits_rows_kernel(const 
         }
         unpack8(a, b, v[t]);
     }
-    fill_search(lds_map, qmap, bits);
+    fill_search_store(lds_map, fill, bits);
     if (blockIdx.x == 0 && threadIdx.x == 0)
         codes[trailing] = 0;
     float amax[T];
@@ -673,6 +708,8 @@ __global__ __launch_bounds__(kBThreads) void quant_rank1_bits_rows128_kernel(con
     const int64_t r0 = (int64_t)blockIdx.y * T;
     const int64_t c0 = (int64_t)blockIdx.x * kBTile + (int64_t)(threadIdx.x >> 4) * kGroup;
     const bool live = c0 < C;  // uniform over the 16 lanes of a group
+    // the small loads that feed LDS first (they return first), then the rows' loads
+    const SearchFill fill = fill_search_load(qmap, bits);
     float4 a[T], b[T], ca, cb;
     float rm[T];
     if (live) {
@@ -689,7 +726,7 @@ __global__ __launch_bounds__(kBThreads) void quant_rank1_bits_rows128_kernel(con
             }
         }
     }
-    fill_search(lds_map, qmap, bits);
+    fill_search_store(lds_map, fill, bits);
     lds_barrier();
     if (blockIdx.x == 0 && blockIdx.y == 0) {
         // the padding added by the re-grouping to 2048: plain zeros, not divided by anything
