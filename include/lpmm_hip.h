@@ -279,6 +279,54 @@ int lpmm_nonfused_adamw4bit_rank1_step_multi(const lpmm_nonfused_rank1_tensor *t
                                              double beta2, double lr, double weight_decay, double eps,
                                              void *stream);
 
+/* The non-fused step with an fp32 first moment and a 4-bit second moment: the configurations
+ * that quantise the second moment only (QUANT.M.ENABLE False: lpmm/configs/
+ * 2nd_moment_only_group_128.yml and 2nd_moment_only_default.yml).  In _single_tensor_adamw4bit
+ * exp_avg then is the state tensor itself, updated in place by lerp_ (lpmm/optim/adamw.py:397-399,
+ * :412), and only exp_avg_sq is dequantised and quantised again (:402-409, :430-434).  Same
+ * arithmetic, state layouts and first-step convention as the two entry points above, with
+ * m: float[n] in place of the first moment's codes and scales.
+ *
+ * lpmm_nonfused_adamw_v4bit_step_multi: second moment with 'group' scaling, gp_sz 128; one
+ * pass; any n; up to 48 tensors per launch.
+ * lpmm_nonfused_adamw_v4bit_rank1_step_multi: second moment with 'rank1' scaling on row-major
+ * R x C tensors whose column count is a multiple of 128; two passes; the statistics trade
+ * places as in lpmm_nonfused_adamw4bit_rank1_step_multi; p, g and m 16-byte aligned. */
+typedef struct lpmm_adamw_v4bit_tensor {
+    float *p;
+    const float *g;
+    float *m;
+    uint8_t *v_codes;
+    float *v_max1;
+    int64_t n;
+    float step;
+    float reserved;
+} lpmm_adamw_v4bit_tensor;
+
+int lpmm_nonfused_adamw_v4bit_step_multi(const lpmm_adamw_v4bit_tensor *tensors, int64_t count,
+                                         const float *qmap_v, double beta1, double beta2, double lr,
+                                         double weight_decay, double eps, void *stream);
+
+typedef struct lpmm_rank1_v4bit_tensor {
+    float *p;
+    const float *g;
+    float *m;
+    uint8_t *v_codes;
+    const float *v_rowmax;
+    const float *v_colmax;
+    float *v_rowmax_next;
+    float *v_colmax_next;
+    int64_t rows;
+    int64_t cols;
+    float step;
+    float reserved;
+} lpmm_rank1_v4bit_tensor;
+
+int lpmm_nonfused_adamw_v4bit_rank1_step_multi(const lpmm_rank1_v4bit_tensor *tensors, int64_t count,
+                                               const float *qmap_v, double beta1, double beta2,
+                                               double lr, double weight_decay, double eps,
+                                               void *stream);
+
 /* ---------------------------------------------------------------------------------------
  * (c) Factored second moment on a row-major R x C tensor.
  * Replaces _single_quantized_factored_update (lpmm/optim/adamw.py:579-627) and

@@ -78,7 +78,7 @@ struct TileShape {
 struct TensorR1 {
     float *p;
     const float *g;
-    uint8_t *mc;
+    uint8_t *mc;  // fp32 first moment: the moment itself (float[rows * cols]), ms unused
     float *ms;
     uint8_t *vc;
     const float *row_old;
@@ -166,10 +166,13 @@ __global__ __launch_bounds__(kThreads) void rank1_clear_kernel(const MultiR1 arg
 // operands of one pass of a DPP row, as loaded
 struct PassRegs {
     float4 a0, a1, b0, b1;
+    float4 c0, c1;  // fp32 first moment only
     uint32_t m0, m1, v0, v1;
     float sm, ro;
 };
 
+// M32: the first moment is kept in fp32 (read and written as floats) instead of as 4-bit codes
+template <bool M32>
 __device__ __forceinline__ void pass_fetch(const TensorR1 &t, uint32_t cg, int lane16, int64_t r, PassRegs &x)
 {
     const int64_t grp = r * t.col_blocks + cg;
@@ -180,13 +183,19 @@ __device__ __forceinline__ void pass_fetch(const TensorR1 &t, uint32_t cg, int l
     x.a1 = load4(pp + 64);
     x.b0 = load4(gp);
     x.b1 = load4(gp + 64);
-    const uint16_t *mcp = reinterpret_cast<const uint16_t *>(t.mc + (gbase >> 1)) + lane16;
     const uint16_t *vcp = reinterpret_cast<const uint16_t *>(t.vc + (gbase >> 1)) + lane16;
-    x.m0 = load_u16(mcp);
-    x.m1 = load_u16(mcp + 16);
+    if (M32) {
+        const float *mp = reinterpret_cast<const float *>(t.mc) + gbase + lane16 * 4;
+        x.c0 = load4(mp);
+        x.c1 = load4(mp + 64);
+    } else {
+        const uint16_t *mcp = reinterpret_cast<const uint16_t *>(t.mc + (gbase >> 1)) + lane16;
+        x.m0 = load_u16(mcp);
+        x.m1 = load_u16(mcp + 16);
+        x.sm = t.ms[grp];
+    }
     x.v0 = load_u16(vcp);
     x.v1 = load_u16(vcp + 16);
-    x.sm = t.ms[grp];
     x.ro = t.row_old[r];
 }
 
@@ -195,6 +204,7 @@ __device__ __forceinline__ void pass_fetch(const TensorR1 &t, uint32_t cg, int l
 #endif
 // 4 waves per SIMD, up to 128 registers: the first pass's operands stay live across the prologue and
 // the lane's column statistics across the passes (with 5 or 6 the compiler spills or re-reads)
+template <bool M32>
 __global__ __launch_bounds__(kThreads, LPMM_R1_WAVES) void rank1_update_kernel(const MultiR1 args, const float *__restrict__ qmap_m,
                                                                 const float *__restrict__ qmap_v)
 {
@@ -223,7 +233,7 @@ __global__ __launch_bounds__(kThreads, LPMM_R1_WAVES) void rank1_update_kernel(c
     const bool row_live = q.cg < t.col_blocks;  // the whole DPP row
     PassRegs x;
     if (row_live && q.row0 < t.rows)
-        pass_fetch(t, q.cg, lane16, q.row0, x);
+        pass_fetch<M32>(t, q.cg, lane16, q.row0, x);
     lds_fill_store(lds, fill);
     for (int j = threadIdx.x; j < kMaxWide * (int)kRedSlotWords; j += kThreads)
         colred[j] = 0u;
@@ -242,7 +252,7 @@ __global__ __launch_bounds__(kThreads, LPMM_R1_WAVES) void rank1_update_kernel(c
     h.rbc2_sqrt = t.rbc2_sqrt;
     lds_barrier();
 
-    if (tl == 0) {
+    if (!M32 && tl == 0) {
         const float z[kEltsPerLane] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
         const int64_t n = t.rows * cols;
         write_padding(t.mc, n, (n + LPMM_PACK_GROUP - 1) / LPMM_PACK_GROUP * LPMM_PACK_GROUP,
@@ -262,40 +272,55 @@ __global__ __launch_bounds__(kThreads, LPMM_R1_WAVES) void rank1_update_kernel(c
             if (r >= t.rows)
                 break;
             if (it > 0)
-                pass_fetch(t, q.cg, lane16, r, x);
+                pass_fetch<M32>(t, q.cg, lane16, r, x);
             const int64_t grp = r * t.col_blocks + q.cg;
             const int64_t gbase = grp * kGroup;
             float *pp = t.p + gbase + lane16 * 4;
-            uint16_t *mcp = reinterpret_cast<uint16_t *>(t.mc + (gbase >> 1)) + lane16;
-            const uint32_t wm = x.m0 | (x.m1 << 16);
             const uint32_t wv = x.v0 | (x.v1 << 16);
-            const float sm = x.sm, ro = x.ro;
+            const float ro = x.ro;
             float pv[kEltsPerLane], gv[kEltsPerLane], m[kEltsPerLane], v[kEltsPerLane];
             unpack8(x.a0, x.a1, pv);
             unpack8(x.b0, x.b1, gv);
+            const Nibbles nm = split_nibbles(M32 ? 0u : (x.m0 | (x.m1 << 16)));
+            const float sm = M32 ? 0.0f : x.sm;
+            if (M32)
+                unpack8(x.c0, x.c1, m);
 
-            const Nibbles nm = split_nibbles(wm), nv = split_nibbles(wv);
+            const Nibbles nv = split_nibbles(wv);
             float amax_m = 0.0f, vmax = 0.0f;
 #pragma unroll
             for (int k = 0; k < kEltsPerLane; ++k) {
-                m[k] = decode_nibble(lds, kLdsQ0, nm, k) * sm;
+                if (!M32)
+                    m[k] = decode_nibble(lds, kLdsQ0, nm, k) * sm;
                 v[k] = decode_nibble(lds, kLdsQ1, nv, k) * ((co[k] < ro) ? co[k] : ro);
                 nonfused_elt(pv[k], gv[k], m[k], v[k], h);
                 amax_m = fmaxf(amax_m, fabsf(m[k]));
                 vmax = fmaxf(vmax, v[k]);
                 atomicMax(red + k * 16, __float_as_uint(v[k]));
             }
-            row16_max2(amax_m, vmax);
-            const uint32_t cm = encode8_scaled(lds, kLdsQ0, kind_m, m, amax_m);
+            uint32_t cm = 0;
+            if (M32) {
+                vmax = row16_max(vmax);
+            } else {
+                row16_max2(amax_m, vmax);
+                cm = encode8_scaled(lds, kLdsQ0, kind_m, m, amax_m);
+            }
 
             store4(pp, make_float4(pv[0], pv[1], pv[2], pv[3]));
             store4(pp + 64, make_float4(pv[4], pv[5], pv[6], pv[7]));
-            store_u16(mcp, cm & 0xFFFFu);
-            store_u16(mcp + 16, cm >> 16);
-            if (lane16 == 0) {
-                t.ms[grp] = amax_m;
-                atomic_max_nonneg(t.row_new + r, vmax);
+            if (M32) {
+                float *mp = reinterpret_cast<float *>(t.mc) + gbase + lane16 * 4;
+                store4(mp, make_float4(m[0], m[1], m[2], m[3]));
+                store4(mp + 64, make_float4(m[4], m[5], m[6], m[7]));
+            } else {
+                uint16_t *mcp = reinterpret_cast<uint16_t *>(t.mc + (gbase >> 1)) + lane16;
+                store_u16(mcp, cm & 0xFFFFu);
+                store_u16(mcp + 16, cm >> 16);
+                if (lane16 == 0)
+                    t.ms[grp] = amax_m;
             }
+            if (lane16 == 0)
+                atomic_max_nonneg(t.row_new + r, vmax);
         }
     }
     // the column maxima meet in LDS: nothing below depends on the global stores still in flight
@@ -439,10 +464,16 @@ static uint64_t shape_tiles(int64_t rows, uint32_t col_blocks, TileShape &ts)
     return (row_blocks + comb - 1) / comb * comb * col_tiles;  // whole groups: the last may hold empty blocks
 }
 
-extern "C" int lpmm_nonfused_adamw4bit_rank1_step_multi(const lpmm_nonfused_rank1_tensor *tensors, int64_t count,
-                                                        const float *qmap_m, const float *qmap_v, double beta1,
-                                                        double beta2, double lr, double weight_decay,
-                                                        double eps, void *stream)
+// The first moment of a record: its codes and scales, or the fp32 moment itself.
+static uint8_t *first_moment(const lpmm_nonfused_rank1_tensor &t) { return t.m_codes; }
+static float *first_moment_scales(const lpmm_nonfused_rank1_tensor &t) { return t.m_max1; }
+static uint8_t *first_moment(const lpmm_rank1_v4bit_tensor &t) { return reinterpret_cast<uint8_t *>(t.m); }
+static float *first_moment_scales(const lpmm_rank1_v4bit_tensor &) { return nullptr; }
+
+// Validation, batching into launches of at most kR1Max tensors, and the three launches.
+template <bool M32, class Record>
+static int rank1_step_multi(const Record *tensors, int64_t count, const float *qmap_m, const float *qmap_v,
+                            double beta1, double beta2, double lr, double weight_decay, double eps, void *stream)
 {
     if (count < 0)
         return LPMM_ERR_SIZE;
@@ -454,7 +485,7 @@ extern "C" int lpmm_nonfused_adamw4bit_rank1_step_multi(const lpmm_nonfused_rank
     LPMM_REQUIRE_ALIGN(qmap_m, 4);
     LPMM_REQUIRE_ALIGN(qmap_v, 4);
     for (int64_t i = 0; i < count; ++i) {
-        const lpmm_nonfused_rank1_tensor &t = tensors[i];
+        const Record &t = tensors[i];
         if (t.rows < 0 || t.cols < 0 || t.cols % kGroup != 0)
             return LPMM_ERR_SIZE;
         if (t.rows == 0 || t.cols == 0)
@@ -467,8 +498,9 @@ extern "C" int lpmm_nonfused_adamw4bit_rank1_step_multi(const lpmm_nonfused_rank
             return LPMM_ERR_SIZE;
         LPMM_REQUIRE_PTR(t.p);
         LPMM_REQUIRE_PTR(t.g);
-        LPMM_REQUIRE_PTR(t.m_codes);
-        LPMM_REQUIRE_PTR(t.m_max1);
+        LPMM_REQUIRE_PTR(first_moment(t));
+        if (!M32)
+            LPMM_REQUIRE_PTR(first_moment_scales(t));
         LPMM_REQUIRE_PTR(t.v_codes);
         LPMM_REQUIRE_PTR(t.v_rowmax);
         LPMM_REQUIRE_PTR(t.v_colmax);
@@ -476,9 +508,9 @@ extern "C" int lpmm_nonfused_adamw4bit_rank1_step_multi(const lpmm_nonfused_rank
         LPMM_REQUIRE_PTR(t.v_colmax_next);
         LPMM_REQUIRE_ALIGN(t.p, 16);
         LPMM_REQUIRE_ALIGN(t.g, 16);
-        LPMM_REQUIRE_ALIGN(t.m_codes, 4);
+        LPMM_REQUIRE_ALIGN(first_moment(t), M32 ? 16 : 4);
         LPMM_REQUIRE_ALIGN(t.v_codes, 4);
-        LPMM_REQUIRE_ALIGN(t.m_max1, 4);
+        LPMM_REQUIRE_ALIGN(first_moment_scales(t), 4);
         LPMM_REQUIRE_ALIGN(t.v_rowmax, 4);
         LPMM_REQUIRE_ALIGN(t.v_colmax, 16);
         LPMM_REQUIRE_ALIGN(t.v_rowmax_next, 4);
@@ -501,7 +533,7 @@ extern "C" int lpmm_nonfused_adamw4bit_rank1_step_multi(const lpmm_nonfused_rank
         int64_t longest = 0;
         args.tile_start[0] = 0;
         while (i < count && k < kR1Max) {
-            const lpmm_nonfused_rank1_tensor &t = tensors[i];
+            const Record &t = tensors[i];
             if (t.rows == 0 || t.cols == 0) {
                 ++i;
                 continue;
@@ -513,8 +545,8 @@ extern "C" int lpmm_nonfused_adamw4bit_rank1_step_multi(const lpmm_nonfused_rank
                 break;
             d.p = t.p;
             d.g = t.g;
-            d.mc = t.m_codes;
-            d.ms = t.m_max1;
+            d.mc = first_moment(t);
+            d.ms = first_moment_scales(t);
             d.vc = t.v_codes;
             d.row_old = t.v_rowmax;
             d.col_old = t.v_colmax;
@@ -543,8 +575,8 @@ extern "C" int lpmm_nonfused_adamw4bit_rank1_step_multi(const lpmm_nonfused_rank
         clear_blocks = clear_blocks > 64 ? 64 : clear_blocks;
         hipLaunchKernelGGL(rank1_clear_kernel, dim3((uint32_t)clear_blocks, (uint32_t)k), dim3(kThreads), 0,
                            (hipStream_t)stream, args);
-        hipLaunchKernelGGL(rank1_update_kernel, dim3((uint32_t)tiles), dim3(kThreads), 0, (hipStream_t)stream, args,
-                           qmap_m, qmap_v);
+        hipLaunchKernelGGL(rank1_update_kernel<M32>, dim3((uint32_t)tiles), dim3(kThreads), 0, (hipStream_t)stream,
+                           args, qmap_m, qmap_v);
         hipLaunchKernelGGL(rank1_requant_kernel, dim3((uint32_t)tiles), dim3(kThreads), 0, (hipStream_t)stream, args,
                            qmap_v);
         const int st = launch_status();
@@ -552,4 +584,21 @@ extern "C" int lpmm_nonfused_adamw4bit_rank1_step_multi(const lpmm_nonfused_rank
             return st;
     }
     return LPMM_OK;
+}
+
+extern "C" int lpmm_nonfused_adamw4bit_rank1_step_multi(const lpmm_nonfused_rank1_tensor *tensors, int64_t count,
+                                                        const float *qmap_m, const float *qmap_v, double beta1,
+                                                        double beta2, double lr, double weight_decay,
+                                                        double eps, void *stream)
+{
+    return rank1_step_multi<false>(tensors, count, qmap_m, qmap_v, beta1, beta2, lr, weight_decay, eps, stream);
+}
+
+extern "C" int lpmm_nonfused_adamw_v4bit_rank1_step_multi(const lpmm_rank1_v4bit_tensor *tensors, int64_t count,
+                                                          const float *qmap_v, double beta1, double beta2,
+                                                          double lr, double weight_decay, double eps,
+                                                          void *stream)
+{
+    // the update kernel keeps the second moment's map in both map slots; only the second is read
+    return rank1_step_multi<true>(tensors, count, qmap_v, qmap_v, beta1, beta2, lr, weight_decay, eps, stream);
 }

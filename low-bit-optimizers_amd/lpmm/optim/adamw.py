@@ -337,6 +337,7 @@ class AdamW(LowBitOptimizer):
         v_group128 = fits(md_v) and md_v["scale_type"] == "group" and md_v["gp_sz"] == 128
         v_rank1 = fits(md_v) and md_v["scale_type"] == "rank1"
         batched, batched_rank1, plain = {}, {}, {}
+        batched_m32, batched_rank1_m32 = {}, {}  # fp32 first moment, quantised second moment
         factored_work = []
         held = []  # contiguous copies of strided operands
 
@@ -356,6 +357,22 @@ class AdamW(LowBitOptimizer):
                                                                   beta1, beta2, lr, wd, eps,
                                                                   _native.current_stream(dev))
             _native.check(st, "non-fused 4-bit AdamW step (rank-1 second moment)")
+
+        def launch_group_m32(key, records):
+            dev, qv_ptr = key
+            table = np.array(records, dtype=_native.ADAMW_V4BIT_TENSOR)
+            with torch.cuda.device(dev):
+                st = lib.lpmm_nonfused_adamw_v4bit_step_multi(table.ctypes.data, len(records), qv_ptr, beta1, beta2,
+                                                              lr, wd, eps, _native.current_stream(dev))
+            _native.check(st, "non-fused AdamW step (fp32 first moment, 4-bit second moment)")
+
+        def launch_rank1_m32(key, records):
+            dev, qv_ptr = key
+            table = np.array(records, dtype=_native.RANK1_V4BIT_TENSOR)
+            with torch.cuda.device(dev):
+                st = lib.lpmm_nonfused_adamw_v4bit_rank1_step_multi(table.ctypes.data, len(records), qv_ptr, beta1,
+                                                                    beta2, lr, wd, eps, _native.current_stream(dev))
+            _native.check(st, "non-fused AdamW step (fp32 first moment, rank-1 4-bit second moment)")
 
         for p, grad, state, factored in work:
             step = self._next_step(state)
@@ -385,6 +402,25 @@ class AdamW(LowBitOptimizer):
                         pending.clear()
                     continue
             m = self._materialise(p, state, "exp_avg", en_m, md_m)
+            if not en_m and en_v:
+                # only the second moment is quantised: the first is read and written as floats
+                key = (p.device, state["exp_avg_sq_qstate"]["qmap"].data_ptr())
+                if v_group128:
+                    pending = batched_m32.setdefault(key, [])
+                    pending.append((dense.data_ptr(), grad.data_ptr(), m.data_ptr())
+                                   + self._group_state(p, state, "exp_avg_sq") + (p.numel(), step, 0.0))
+                    if len(pending) == _native.V4BIT_MULTI_MAX:
+                        launch_group_m32(key, pending)
+                        pending.clear()
+                    continue
+                if v_rank1 and p.dim() == 2 and p.shape[1] % 128 == 0 and m.data_ptr() % 16 == 0:
+                    pending = batched_rank1_m32.setdefault(key, [])
+                    pending.append((dense.data_ptr(), grad.data_ptr(), m.data_ptr()) + self._rank1_state(p, state)
+                                   + (p.shape[0], p.shape[1], step, 0.0))
+                    if len(pending) == _native.RANK1_MULTI_MAX:
+                        launch_rank1_m32(key, pending)
+                        pending.clear()
+                    continue
             v = self._materialise(p, state, "exp_avg_sq", en_v, md_v)
             if not en_m and not en_v and m.is_contiguous() and v.is_contiguous():
                 # fp32 states (small tensors): all of them in one launch
@@ -412,6 +448,12 @@ class AdamW(LowBitOptimizer):
         for key, records in batched_rank1.items():
             if records:
                 launch_rank1(key, records)
+        for key, records in batched_m32.items():
+            if records:
+                launch_group_m32(key, records)
+        for key, records in batched_rank1_m32.items():
+            if records:
+                launch_rank1_m32(key, records)
         self._write_back(held)
 
     def _half_step(self, group, p, grad, state, step, md_m, md_v):
@@ -456,44 +498,33 @@ class AdamW(LowBitOptimizer):
             else:
                 state[name] = t
 
-    def _nonfused_record(self, p, dense, grad, state, step):
-        """The tensor's record for the one-pass non-fused step; creates the quantised states
-        on first use: all-zero moments in the layout and with the metadata vectorwise_quant
-        gives them (lpmm/optim/adamw.py:425-434)."""
-        n = p.numel()
-        groups = (n + 127) // 128
-        ptrs = []
-        for name in ("exp_avg", "exp_avg_sq"):
-            qstate = state[f"{name}_qstate"]
-            if _is_placeholder(state[name]):
-                state[name] = torch.full((packed_nbytes(groups * 128),), _zero_byte(qstate["qmap"]),
-                                         dtype=torch.int8, device=p.device)
-                oh = qstate["overhead"]
-                oh.clear()
-                oh.update({"dtype": p.dtype, "stride": self._state_stride(p),
-                           "max1": torch.zeros((groups, 1), dtype=torch.float32, device=p.device),
-                           "scaled_shape": torch.Size((groups, 128))})
-            ptrs.append((state[name].data_ptr(), qstate["overhead"]["max1"].data_ptr()))
-        return (dense.data_ptr(), grad.data_ptr(), ptrs[0][0], ptrs[1][0], ptrs[0][1], ptrs[1][1], n, step, 0.0)
+    def _group_state(self, p, state, name):
+        """Pointers to the codes and scales of a state with block-wise scaling over 128 values;
+        creates the state on first use: an all-zero moment in the layout and with the metadata
+        vectorwise_quant gives it (lpmm/optim/adamw.py:425-434)."""
+        groups = (p.numel() + 127) // 128
+        qstate = state[f"{name}_qstate"]
+        if _is_placeholder(state[name]):
+            state[name] = torch.full((packed_nbytes(groups * 128),), _zero_byte(qstate["qmap"]),
+                                     dtype=torch.int8, device=p.device)
+            oh = qstate["overhead"]
+            oh.clear()
+            oh.update({"dtype": p.dtype, "stride": self._state_stride(p),
+                       "max1": torch.zeros((groups, 1), dtype=torch.float32, device=p.device),
+                       "scaled_shape": torch.Size((groups, 128))})
+        return state[name].data_ptr(), qstate["overhead"]["max1"].data_ptr()
 
-    def _nonfused_rank1_record(self, p, dense, grad, state, step):
-        """The tensor's record for the two-pass step with a rank-1 second moment.  The kernels
-        leave the statistics of the new second moment in a second pair of buffers; the pairs
-        trade places here, so that the state's `max_dims` always are the statistics its codes
-        are scaled by."""
+    def _rank1_state(self, p, state):
+        """Pointers to the codes of a rank-1 scaled second moment, the statistics they are scaled
+        by and the pair of buffers that receives the next statistics; creates the state on first
+        use.  The kernels leave the statistics of the new second moment in the second pair; the
+        pairs trade places here, so that the state's `max_dims` always are the statistics its
+        codes are scaled by."""
         rows, cols = p.shape
-        n = p.numel()
-        groups = n // 128
         dev = p.device
-        qs_m, qs_v = state["exp_avg_qstate"], state["exp_avg_sq_qstate"]
-        if _is_placeholder(state["exp_avg"]):
-            state["exp_avg"] = torch.full((packed_nbytes(n),), _zero_byte(qs_m["qmap"]), dtype=torch.int8, device=dev)
-            qs_m["overhead"].clear()
-            qs_m["overhead"].update({"dtype": p.dtype, "stride": self._state_stride(p),
-                                     "max1": torch.zeros((groups, 1), dtype=torch.float32, device=dev),
-                                     "scaled_shape": torch.Size((groups, 128))})
+        qs_v = state["exp_avg_sq_qstate"]
         if _is_placeholder(state["exp_avg_sq"]):
-            state["exp_avg_sq"] = torch.full((packed_nbytes(n),), _zero_byte(qs_v["qmap"]), dtype=torch.int8,
+            state["exp_avg_sq"] = torch.full((packed_nbytes(p.numel()),), _zero_byte(qs_v["qmap"]), dtype=torch.int8,
                                              device=dev)
             qs_v["overhead"].clear()
             qs_v["overhead"].update({"dtype": p.dtype, "stride": self._state_stride(p), "dim": 2, "max1": None,
@@ -507,9 +538,20 @@ class AdamW(LowBitOptimizer):
             nxt = [torch.empty_like(cur[0]), torch.empty_like(cur[1])]
         self._spare_stats[p] = cur
         oh["max_dims"] = nxt
-        return (dense.data_ptr(), grad.data_ptr(), state["exp_avg"].data_ptr(), qs_m["overhead"]["max1"].data_ptr(),
-                state["exp_avg_sq"].data_ptr(), cur[0].data_ptr(), cur[1].data_ptr(), nxt[0].data_ptr(),
-                nxt[1].data_ptr(), rows, cols, step, 0.0)
+        return (state["exp_avg_sq"].data_ptr(), cur[0].data_ptr(), cur[1].data_ptr(), nxt[0].data_ptr(),
+                nxt[1].data_ptr())
+
+    def _nonfused_record(self, p, dense, grad, state, step):
+        """The tensor's record for the one-pass non-fused step."""
+        mc, ms = self._group_state(p, state, "exp_avg")
+        vc, vs = self._group_state(p, state, "exp_avg_sq")
+        return (dense.data_ptr(), grad.data_ptr(), mc, vc, ms, vs, p.numel(), step, 0.0)
+
+    def _nonfused_rank1_record(self, p, dense, grad, state, step):
+        """The tensor's record for the two-pass step with a rank-1 second moment."""
+        mc, ms = self._group_state(p, state, "exp_avg")
+        return (dense.data_ptr(), grad.data_ptr(), mc, ms) + self._rank1_state(p, state) + (
+            p.shape[0], p.shape[1], step, 0.0)
 
     @property
     def _spare_stats(self):
