@@ -17,7 +17,8 @@ Two further workloads measure the other kernels of the path with the same JSON s
 `--workload quant64m` (stand-alone quantise/dequantise round trip on 2^26 values) and
 `--workload factored` (factored second moment on LLaMA-7B MLP/attention shapes) and
 `--workload nonfused_group|nonfused_rank1` (fused=False on the LLaMA-7B-shaped set; with the suffix
-`_m32` under the configurations that quantise the second moment only: fp32 first moment) and
+`_m32` under the configurations that quantise the second moment only: fp32 first moment;
+`nonfused_rank1_mgroup`: first-moment groups of 1024 values) and
 `--workload sgd` (4-bit SGD momentum on the same set).
 """
 import argparse
@@ -448,17 +449,20 @@ def run_sgd(torch, args):
                      "bytes_per_param": bytes_per_param}}))
 
 
-def run_nonfused(torch, args, v_scale, m32=False):
+def run_nonfused(torch, args, v_scale, m32=False, mgroup=False):
     """fused=False on the LLaMA-7B-shaped set.  v_scale 'group': both moments block-wise over
     128 values, one kernel per launch group of tensors; 'rank1' (the reference's default
     configuration): an update pass and a re-quantise pass per launch group of tensors.
     m32: the configurations that quantise the second moment only (the first moment is an fp32
-    state, read and written as floats by the same passes)."""
+    state, read and written as floats by the same passes).  mgroup: first-moment groups of 1024
+    values with the rank-1 second moment (the first moment's codes are written by the second pass)."""
     import lpmm
 
     dev = torch.device("cuda:0")
     params = make_params(torch, llama7b_shapes(), dev, heavy_tailed=True)
-    if m32:
+    if mgroup:
+        name = "1st_moment_group_1024.yml"
+    elif m32:
         name = "2nd_moment_only_group_128.yml" if v_scale == "group" else "2nd_moment_only_default.yml"
     else:
         name = "2nd_moment_group_128.yml" if v_scale == "group" else "default.yml"
@@ -480,12 +484,14 @@ def run_nonfused(torch, args, v_scale, m32=False):
     bytes_per_param = BYTES_PER_PARAM_4BIT if v_scale == "group" else 18.5625
     if m32:  # m read and written as floats (8) instead of codes and scales (1.0625)
         bytes_per_param += 8.0 - 1.0625
+    if mgroup:  # update pass: p 8, g 4, both codes read 1; second pass: g 4, both codes read and written 2
+        bytes_per_param = 19.0 + 12.0 / 1024
     achieved = n_total * bytes_per_param / dt / 1e9
     print(json.dumps({
         "metric": "non-fused 4-bit AdamW step: params/sec, 1 MI355X", "value": n_total / dt,
         "unit": "params/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": dt * 1e3,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": f"fused=False, {'fp32 first moment, ' if m32 else ''}second moment '{v_scale}' scaling, "
+        "config": {"workload": f"fused=False, {'fp32 first moment, ' if m32 else ''}{'first-moment groups of 1024, ' if mgroup else ''}second moment '{v_scale}' scaling, "
                                "LLaMA-7B-shaped fp32 set", "qconfig": name,
                    "tensors": len(params), "params": n_total},
         "roofline": {"bound": "hbm", "kernel": "whole step", "achieved": achieved, "peak": HBM_PEAK_GBS,
@@ -498,7 +504,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="llama7b", choices=sorted(WORKLOADS) + ["quant64m", "factored", "nonfused_group", "nonfused_rank1", "nonfused_group_m32", "nonfused_rank1_m32", "sgd", "calibrate"])
+    ap.add_argument("--workload", default="llama7b", choices=sorted(WORKLOADS) + ["quant64m", "factored", "nonfused_group", "nonfused_rank1", "nonfused_group_m32", "nonfused_rank1_m32", "nonfused_rank1_mgroup", "sgd", "calibrate"])
     ap.add_argument("--bits", type=int, default=4, choices=range(1, 9), help="code width of --workload quant64m")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--interleaved-grads", action="store_true",
@@ -552,7 +558,8 @@ def main():
     if args.workload == "sgd":
         return run_sgd(torch, args)
     if args.workload.startswith("nonfused_"):
-        return run_nonfused(torch, args, args.workload.split("_")[1], m32=args.workload.endswith("_m32"))
+        return run_nonfused(torch, args, args.workload.split("_")[1], m32=args.workload.endswith("_m32"),
+                            mgroup=args.workload.endswith("_mgroup"))
 
     desc, shape_fn = WORKLOADS[args.workload]
     shapes = shape_fn()

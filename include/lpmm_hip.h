@@ -327,6 +327,40 @@ int lpmm_nonfused_adamw_v4bit_rank1_step_multi(const lpmm_rank1_v4bit_tensor *te
                                                double lr, double weight_decay, double eps,
                                                void *stream);
 
+/* The two-pass step above with a first moment whose 'group' scaling spans m_group_size =
+ * 256, 512, 1024, 2048 or 4096 values of the flattened tensor (lpmm/configs/
+ * 1st_moment_group_{256,512,1024,2048,4096}.yml; group_tensor, lpmm/functional.py:404-422).
+ * A group then spans several 128-column pieces and, where the column count is not a multiple
+ * of the group size, tensor rows: the update pass merges the groups' maxima of the new first
+ * moment into m_max1_next (cleared by the call, must not alias m_max1), and the second pass
+ * recomputes the first moment from g and the old codes and scales, bit-identically, and
+ * overwrites its codes scaled by m_max1_next -- the caller swaps m_max1 / m_max1_next like the
+ * statistics of the second moment.  m_codes: ceil(ceil(R*C / m_group_size) * m_group_size / 2048)
+ * * 1024 + 1 bytes, 4-byte aligned, written in full; m_max1, m_max1_next: float[ceil(R*C /
+ * m_group_size)].  Everything else as in lpmm_nonfused_adamw4bit_rank1_step_multi. */
+typedef struct lpmm_rank1_mgroup_tensor {
+    float *p;
+    const float *g;
+    uint8_t *m_codes;
+    const float *m_max1;
+    float *m_max1_next;
+    uint8_t *v_codes;
+    const float *v_rowmax;
+    const float *v_colmax;
+    float *v_rowmax_next;
+    float *v_colmax_next;
+    int64_t rows;
+    int64_t cols;
+    float step;
+    float reserved;
+} lpmm_rank1_mgroup_tensor;
+
+int lpmm_nonfused_adamw4bit_rank1_mgroup_step_multi(const lpmm_rank1_mgroup_tensor *tensors,
+                                                    int64_t count, const float *qmap_m,
+                                                    const float *qmap_v, int64_t m_group_size,
+                                                    double beta1, double beta2, double lr,
+                                                    double weight_decay, double eps, void *stream);
+
 /* ---------------------------------------------------------------------------------------
  * (c) Factored second moment on a row-major R x C tensor.
  * Replaces _single_quantized_factored_update (lpmm/optim/adamw.py:579-627) and

@@ -80,6 +80,7 @@ struct TensorR1 {
     const float *g;
     uint8_t *mc;  // fp32 first moment: the moment itself (float[rows * cols]), ms unused
     float *ms;
+    float *ms_new;  // first-moment groups wider than 128 values: the scales of the new first moment
     uint8_t *vc;
     const float *row_old;
     const float *col_old;
@@ -88,8 +89,17 @@ struct TensorR1 {
     int64_t rows;
     uint32_t col_blocks;  // columns / 128
     float neg_step_size, bc2_sqrt, rbc2_sqrt;
+    uint32_t m_lg;  // the first moment's group holds 128 << m_lg values
     TileShape tile;
 };
+
+// How the first moment is kept: 4-bit codes in groups of 128 values (re-quantised where it is
+// updated), fp32 (read and written as floats), or 4-bit codes in wider groups (256 .. 4096
+// values of the flattened tensor: a group spans several DPP rows, tiles and, where the column
+// count is not a multiple of the group size, tensor rows.  The update pass only merges the
+// groups' maxima into the next scales, the second pass recomputes the moment from g and the old
+// codes, bit-identically, and writes its codes -- what both passes do for the second moment).
+enum MomentMode { kMCodes128 = 0, kMFloat = 1, kMCodesWide = 2 };
 
 struct MultiR1 {
     TensorR1 t[kR1Max];
@@ -155,11 +165,16 @@ __global__ __launch_bounds__(kThreads) void rank1_clear_kernel(const MultiR1 arg
 {
     const TensorR1 &t = args.t[blockIdx.y];
     const int64_t cols = (int64_t)t.col_blocks * kGroup;
-    for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < t.rows + cols; i += (int64_t)gridDim.x * kThreads) {
+    // wide first-moment groups: their next scales are merged with atomic maxima as well
+    const int64_t m_groups = t.m_lg ? ((t.rows * t.col_blocks + (1 << t.m_lg) - 1) >> t.m_lg) : 0;
+    for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < t.rows + cols + m_groups;
+         i += (int64_t)gridDim.x * kThreads) {
         if (i < t.rows)
             t.row_new[i] = 0.0f;
-        else
+        else if (i < t.rows + cols)
             t.col_new[i - t.rows] = 0.0f;
+        else
+            t.ms_new[i - t.rows - cols] = 0.0f;
     }
 }
 
@@ -171,8 +186,7 @@ struct PassRegs {
     float sm, ro;
 };
 
-// M32: the first moment is kept in fp32 (read and written as floats) instead of as 4-bit codes
-template <bool M32>
+template <int MODE>
 __device__ __forceinline__ void pass_fetch(const TensorR1 &t, uint32_t cg, int lane16, int64_t r, PassRegs &x)
 {
     const int64_t grp = r * t.col_blocks + cg;
@@ -184,7 +198,7 @@ __device__ __forceinline__ void pass_fetch(const TensorR1 &t, uint32_t cg, int l
     x.b0 = load4(gp);
     x.b1 = load4(gp + 64);
     const uint16_t *vcp = reinterpret_cast<const uint16_t *>(t.vc + (gbase >> 1)) + lane16;
-    if (M32) {
+    if (MODE == kMFloat) {
         const float *mp = reinterpret_cast<const float *>(t.mc) + gbase + lane16 * 4;
         x.c0 = load4(mp);
         x.c1 = load4(mp + 64);
@@ -192,7 +206,7 @@ __device__ __forceinline__ void pass_fetch(const TensorR1 &t, uint32_t cg, int l
         const uint16_t *mcp = reinterpret_cast<const uint16_t *>(t.mc + (gbase >> 1)) + lane16;
         x.m0 = load_u16(mcp);
         x.m1 = load_u16(mcp + 16);
-        x.sm = t.ms[grp];
+        x.sm = t.ms[MODE == kMCodesWide ? grp >> t.m_lg : grp];
     }
     x.v0 = load_u16(vcp);
     x.v1 = load_u16(vcp + 16);
@@ -204,7 +218,7 @@ __device__ __forceinline__ void pass_fetch(const TensorR1 &t, uint32_t cg, int l
 #endif
 // 4 waves per SIMD, up to 128 registers: the first pass's operands stay live across the prologue and
 // the lane's column statistics across the passes (with 5 or 6 the compiler spills or re-reads)
-template <bool M32>
+template <int MODE>
 __global__ __launch_bounds__(kThreads, LPMM_R1_WAVES) void rank1_update_kernel(const MultiR1 args, const float *__restrict__ qmap_m,
                                                                 const float *__restrict__ qmap_v)
 {
@@ -233,7 +247,7 @@ __global__ __launch_bounds__(kThreads, LPMM_R1_WAVES) void rank1_update_kernel(c
     const bool row_live = q.cg < t.col_blocks;  // the whole DPP row
     PassRegs x;
     if (row_live && q.row0 < t.rows)
-        pass_fetch<M32>(t, q.cg, lane16, q.row0, x);
+        pass_fetch<MODE>(t, q.cg, lane16, q.row0, x);
     lds_fill_store(lds, fill);
     for (int j = threadIdx.x; j < kMaxWide * (int)kRedSlotWords; j += kThreads)
         colred[j] = 0u;
@@ -252,7 +266,7 @@ __global__ __launch_bounds__(kThreads, LPMM_R1_WAVES) void rank1_update_kernel(c
     h.rbc2_sqrt = t.rbc2_sqrt;
     lds_barrier();
 
-    if (!M32 && tl == 0) {
+    if (MODE == kMCodes128 && tl == 0) {
         const float z[kEltsPerLane] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
         const int64_t n = t.rows * cols;
         write_padding(t.mc, n, (n + LPMM_PACK_GROUP - 1) / LPMM_PACK_GROUP * LPMM_PACK_GROUP,
@@ -272,7 +286,7 @@ __global__ __launch_bounds__(kThreads, LPMM_R1_WAVES) void rank1_update_kernel(c
             if (r >= t.rows)
                 break;
             if (it > 0)
-                pass_fetch<M32>(t, q.cg, lane16, r, x);
+                pass_fetch<MODE>(t, q.cg, lane16, r, x);
             const int64_t grp = r * t.col_blocks + q.cg;
             const int64_t gbase = grp * kGroup;
             float *pp = t.p + gbase + lane16 * 4;
@@ -281,6 +295,7 @@ __global__ __launch_bounds__(kThreads, LPMM_R1_WAVES) void rank1_update_kernel(c
             float pv[kEltsPerLane], gv[kEltsPerLane], m[kEltsPerLane], v[kEltsPerLane];
             unpack8(x.a0, x.a1, pv);
             unpack8(x.b0, x.b1, gv);
+            constexpr bool M32 = MODE == kMFloat;
             const Nibbles nm = split_nibbles(M32 ? 0u : (x.m0 | (x.m1 << 16)));
             const float sm = M32 ? 0.0f : x.sm;
             if (M32)
@@ -303,7 +318,8 @@ __global__ __launch_bounds__(kThreads, LPMM_R1_WAVES) void rank1_update_kernel(c
                 vmax = row16_max(vmax);
             } else {
                 row16_max2(amax_m, vmax);
-                cm = encode8_scaled(lds, kLdsQ0, kind_m, m, amax_m);
+                if (MODE == kMCodes128)
+                    cm = encode8_scaled(lds, kLdsQ0, kind_m, m, amax_m);
             }
 
             store4(pp, make_float4(pv[0], pv[1], pv[2], pv[3]));
@@ -312,12 +328,14 @@ __global__ __launch_bounds__(kThreads, LPMM_R1_WAVES) void rank1_update_kernel(c
                 float *mp = reinterpret_cast<float *>(t.mc) + gbase + lane16 * 4;
                 store4(mp, make_float4(m[0], m[1], m[2], m[3]));
                 store4(mp + 64, make_float4(m[4], m[5], m[6], m[7]));
-            } else {
+            } else if (MODE == kMCodes128) {
                 uint16_t *mcp = reinterpret_cast<uint16_t *>(t.mc + (gbase >> 1)) + lane16;
                 store_u16(mcp, cm & 0xFFFFu);
                 store_u16(mcp + 16, cm >> 16);
                 if (lane16 == 0)
                     t.ms[grp] = amax_m;
+            } else if (lane16 == 0) {
+                atomic_max_nonneg(t.ms_new + (grp >> t.m_lg), amax_m);
             }
             if (lane16 == 0)
                 atomic_max_nonneg(t.row_new + r, vmax);
@@ -334,12 +352,20 @@ __global__ __launch_bounds__(kThreads, LPMM_R1_WAVES) void rank1_update_kernel(c
     }
 }
 
-__global__ __launch_bounds__(kThreads) void rank1_requant_kernel(const MultiR1 args, const float *__restrict__ qmap_v)
+// MWIDE: the first moment's groups are wider than 128 values; its codes are written here too.
+template <bool MWIDE>
+__global__ __launch_bounds__(kThreads) void rank1_requant_kernel(const MultiR1 args, const float *__restrict__ qmap_m,
+                                                                 const float *__restrict__ qmap_v)
 {
     __shared__ __align__(16) uint32_t lds[(kColExtra + 2 * kColBytes) / 4];
     constexpr uint32_t kColNew = kColExtra, kColRcp = kColExtra + kColBytes;
-    lds_fill(lds, qmap_v, nullptr);
+    constexpr uint32_t kVMap = MWIDE ? kLdsQ1 : kLdsQ0;  // where the second moment's map sits in LDS
+    if (MWIDE)
+        lds_fill(lds, qmap_m, qmap_v);
+    else
+        lds_fill(lds, qmap_v, nullptr);
     const int kind = classify_map(qmap_v);
+    const int kind_m = MWIDE ? classify_map(qmap_m) : kMapGeneric;
     const int lo = find_tensor(args);
     const TensorR1 &t = args.t[lo];
     const uint32_t tl = blockIdx.x - args.tile_start[lo];
@@ -357,13 +383,35 @@ __global__ __launch_bounds__(kThreads) void rank1_requant_kernel(const MultiR1 a
     NfHyper h;
     h.b2 = args.b2;
     h.w2 = args.w2;
+    h.w1 = args.w1;
     __syncthreads();
 
     if (tl == 0) {
         const float z[kEltsPerLane] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
         const int64_t n = t.rows * cols;
-        write_padding(t.vc, n, (n + LPMM_PACK_GROUP - 1) / LPMM_PACK_GROUP * LPMM_PACK_GROUP,
-                      encode8_plain(lds, kLdsQ0, kind, z));
+        const int64_t n_pack = (n + LPMM_PACK_GROUP - 1) / LPMM_PACK_GROUP * LPMM_PACK_GROUP;
+        write_padding(t.vc, n, n_pack, encode8_plain(lds, kVMap, kind, z));
+        if (MWIDE) {
+            // The quantiser pads the flattened tensor with zeros to whole groups (functional.py:404-422),
+            // the packing pads to whole pack groups of 2048 values.  The zeros that fill up the last
+            // group are divided by its scale like its other values (0/0 -> NaN -> code 15 when the
+            // group is all zero), those behind it are plain zeros.
+            const int64_t group = (int64_t)kGroup << t.m_lg;
+            const int64_t n_grp = (n + group - 1) / group * group;
+            const int64_t n_all = (n_grp + LPMM_PACK_GROUP - 1) / LPMM_PACK_GROUP * LPMM_PACK_GROUP;
+            const uint32_t zero_word = encode8_plain(lds, kLdsQ0, kind_m, z);
+            uint32_t last_word = zero_word;
+            if (n_grp > n) {
+                const float last = t.ms_new[(n - 1) >> (7 + t.m_lg)];
+                const float zs[kEltsPerLane] = {0.0f / last, 0.0f / last, 0.0f / last, 0.0f / last,
+                                                0.0f / last, 0.0f / last, 0.0f / last, 0.0f / last};
+                last_word = encode8_plain(lds, kLdsQ0, kind_m, zs);
+            }
+            for (int64_t i = n + (int64_t)threadIdx.x * kEltsPerLane; i < n_all; i += kThreads * kEltsPerLane)
+                *reinterpret_cast<uint32_t *>(t.mc + (i >> 1)) = i < n_grp ? last_word : zero_word;
+            if (threadIdx.x == 0)
+                t.mc[n_all / 2] = 0;
+        }
     }
     if (q.cg >= t.col_blocks)
         return;
@@ -392,14 +440,33 @@ __global__ __launch_bounds__(kThreads) void rank1_requant_kernel(const MultiR1 a
         const float4 b0 = load4(gp), b1 = load4(gp + 64);
         uint32_t *vcp = reinterpret_cast<uint32_t *>(t.vc + (gbase >> 1)) + code_dword;
         const uint32_t wv = swap_code_halves(load_u32(vcp), code_sel);
+        uint32_t *mcp = nullptr;
+        uint32_t wm = 0;
+        float ms_old = 0.0f, ms_new = 0.0f;
+        if (MWIDE) {
+            mcp = reinterpret_cast<uint32_t *>(t.mc + (gbase >> 1)) + code_dword;
+            wm = swap_code_halves(load_u32(mcp), code_sel);
+            const int64_t mg = gbase >> (7 + t.m_lg);
+            ms_old = t.ms[mg];
+            ms_new = t.ms_new[mg];
+        }
         const float ro = t.row_old[r], rn = t.row_new[r];
         float gv[kEltsPerLane], v[kEltsPerLane], x[kEltsPerLane];
         unpack8(b0, b1, gv);
         const Nibbles nv = split_nibbles(wv);
 #pragma unroll
         for (int k = 0; k < kEltsPerLane; ++k) {
-            v[k] = decode_nibble(lds, kLdsQ0, nv, k) * ((co[k] < ro) ? co[k] : ro);
+            v[k] = decode_nibble(lds, kVMap, nv, k) * ((co[k] < ro) ? co[k] : ro);
             nonfused_second_moment(v[k], gv[k], h);
+        }
+        if (MWIDE) {
+            // the first moment as the update pass computed it, with the scale of its whole group
+            const Nibbles nm = split_nibbles(wm);
+            float m[kEltsPerLane];
+#pragma unroll
+            for (int k = 0; k < kEltsPerLane; ++k)
+                m[k] = lerp_w(decode_nibble(lds, kLdsQ0, nm, k) * ms_old, gv[k], h.w1);
+            store_u32(mcp, swap_code_halves(encode8_scaled(lds, kLdsQ0, kind_m, m, ms_new), code_sel));
         }
         uint32_t w;
         // every scale the wave divides by is a column or the row statistic: all in the range in
@@ -418,7 +485,7 @@ __global__ __launch_bounds__(kThreads) void rank1_requant_kernel(const MultiR1 a
 #pragma unroll
             for (int k = 0; k < kEltsPerLane; ++k)
                 x[k] = v[k] / ((cn[k] < rn) ? cn[k] : rn);
-            w = encode8_plain(lds, kLdsQ0, kind, x);
+            w = encode8_plain(lds, kVMap, kind, x);
         }
         store_u32(vcp, swap_code_halves(w, code_sel));
     }
@@ -469,12 +536,20 @@ static uint8_t *first_moment(const lpmm_nonfused_rank1_tensor &t) { return t.m_c
 static float *first_moment_scales(const lpmm_nonfused_rank1_tensor &t) { return t.m_max1; }
 static uint8_t *first_moment(const lpmm_rank1_v4bit_tensor &t) { return reinterpret_cast<uint8_t *>(t.m); }
 static float *first_moment_scales(const lpmm_rank1_v4bit_tensor &) { return nullptr; }
+static uint8_t *first_moment(const lpmm_rank1_mgroup_tensor &t) { return t.m_codes; }
+static float *first_moment_scales(const lpmm_rank1_mgroup_tensor &t) { return const_cast<float *>(t.m_max1); }
+static float *next_scales(const lpmm_nonfused_rank1_tensor &) { return nullptr; }
+static float *next_scales(const lpmm_rank1_v4bit_tensor &) { return nullptr; }
+static float *next_scales(const lpmm_rank1_mgroup_tensor &t) { return t.m_max1_next; }
 
 // Validation, batching into launches of at most kR1Max tensors, and the three launches.
-template <bool M32, class Record>
+// m_lg: the first moment's group holds 128 << m_lg values (MODE kMCodesWide only).
+template <int MODE, class Record>
 static int rank1_step_multi(const Record *tensors, int64_t count, const float *qmap_m, const float *qmap_v,
-                            double beta1, double beta2, double lr, double weight_decay, double eps, void *stream)
+                            uint32_t m_lg, double beta1, double beta2, double lr, double weight_decay, double eps,
+                            void *stream)
 {
+    constexpr bool M32 = MODE == kMFloat;
     if (count < 0)
         return LPMM_ERR_SIZE;
     if (count == 0)
@@ -511,6 +586,12 @@ static int rank1_step_multi(const Record *tensors, int64_t count, const float *q
         LPMM_REQUIRE_ALIGN(first_moment(t), M32 ? 16 : 4);
         LPMM_REQUIRE_ALIGN(t.v_codes, 4);
         LPMM_REQUIRE_ALIGN(first_moment_scales(t), 4);
+        if (MODE == kMCodesWide) {
+            LPMM_REQUIRE_PTR(next_scales(t));
+            LPMM_REQUIRE_ALIGN(next_scales(t), 4);
+            if (next_scales(t) == first_moment_scales(t))
+                return LPMM_ERR_ARG;
+        }
         LPMM_REQUIRE_ALIGN(t.v_rowmax, 4);
         LPMM_REQUIRE_ALIGN(t.v_colmax, 16);
         LPMM_REQUIRE_ALIGN(t.v_rowmax_next, 4);
@@ -547,6 +628,8 @@ static int rank1_step_multi(const Record *tensors, int64_t count, const float *q
             d.g = t.g;
             d.mc = first_moment(t);
             d.ms = first_moment_scales(t);
+            d.ms_new = next_scales(t);
+            d.m_lg = m_lg;
             d.vc = t.v_codes;
             d.row_old = t.v_rowmax;
             d.col_old = t.v_colmax;
@@ -575,10 +658,10 @@ static int rank1_step_multi(const Record *tensors, int64_t count, const float *q
         clear_blocks = clear_blocks > 64 ? 64 : clear_blocks;
         hipLaunchKernelGGL(rank1_clear_kernel, dim3((uint32_t)clear_blocks, (uint32_t)k), dim3(kThreads), 0,
                            (hipStream_t)stream, args);
-        hipLaunchKernelGGL(rank1_update_kernel<M32>, dim3((uint32_t)tiles), dim3(kThreads), 0, (hipStream_t)stream,
+        hipLaunchKernelGGL(rank1_update_kernel<MODE>, dim3((uint32_t)tiles), dim3(kThreads), 0, (hipStream_t)stream,
                            args, qmap_m, qmap_v);
-        hipLaunchKernelGGL(rank1_requant_kernel, dim3((uint32_t)tiles), dim3(kThreads), 0, (hipStream_t)stream, args,
-                           qmap_v);
+        hipLaunchKernelGGL(rank1_requant_kernel<MODE == kMCodesWide>, dim3((uint32_t)tiles), dim3(kThreads), 0,
+                           (hipStream_t)stream, args, qmap_m, qmap_v);
         const int st = launch_status();
         if (st != LPMM_OK)
             return st;
@@ -591,7 +674,7 @@ extern "C" int lpmm_nonfused_adamw4bit_rank1_step_multi(const lpmm_nonfused_rank
                                                         double beta2, double lr, double weight_decay,
                                                         double eps, void *stream)
 {
-    return rank1_step_multi<false>(tensors, count, qmap_m, qmap_v, beta1, beta2, lr, weight_decay, eps, stream);
+    return rank1_step_multi<kMCodes128>(tensors, count, qmap_m, qmap_v, 0, beta1, beta2, lr, weight_decay, eps, stream);
 }
 
 extern "C" int lpmm_nonfused_adamw_v4bit_rank1_step_multi(const lpmm_rank1_v4bit_tensor *tensors, int64_t count,
@@ -600,5 +683,20 @@ extern "C" int lpmm_nonfused_adamw_v4bit_rank1_step_multi(const lpmm_rank1_v4bit
                                                           void *stream)
 {
     // the update kernel keeps the second moment's map in both map slots; only the second is read
-    return rank1_step_multi<true>(tensors, count, qmap_v, qmap_v, beta1, beta2, lr, weight_decay, eps, stream);
+    return rank1_step_multi<kMFloat>(tensors, count, qmap_v, qmap_v, 0, beta1, beta2, lr, weight_decay, eps, stream);
+}
+
+extern "C" int lpmm_nonfused_adamw4bit_rank1_mgroup_step_multi(const lpmm_rank1_mgroup_tensor *tensors, int64_t count,
+                                                               const float *qmap_m, const float *qmap_v,
+                                                               int64_t m_group_size, double beta1, double beta2,
+                                                               double lr, double weight_decay, double eps,
+                                                               void *stream)
+{
+    uint32_t m_lg = 0;
+    while (m_lg < 5 && ((int64_t)kGroup << m_lg) < m_group_size)
+        ++m_lg;
+    if (m_lg == 0 || ((int64_t)kGroup << m_lg) != m_group_size)
+        return LPMM_ERR_SIZE;  // 256, 512, 1024, 2048 or 4096
+    return rank1_step_multi<kMCodesWide>(tensors, count, qmap_m, qmap_v, m_lg, beta1, beta2, lr, weight_decay, eps,
+                                         stream);
 }

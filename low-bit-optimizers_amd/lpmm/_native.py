@@ -52,6 +52,7 @@ PROTOTYPES = {
     "lpmm_nonfused_adamw4bit_rank1_step_multi": (_int, [_vp, _i64, _vp, _vp] + [_d] * 5 + [_vp]),
     "lpmm_nonfused_adamw_v4bit_step_multi": (_int, [_vp, _i64, _vp] + [_d] * 5 + [_vp]),
     "lpmm_nonfused_adamw_v4bit_rank1_step_multi": (_int, [_vp, _i64, _vp] + [_d] * 5 + [_vp]),
+    "lpmm_nonfused_adamw4bit_rank1_mgroup_step_multi": (_int, [_vp, _i64, _vp, _vp, _i64] + [_d] * 5 + [_vp]),
     "lpmm_factored_workspace_bytes": (_i64, [_i64, _i64]),
     "lpmm_factored_stats": (_int, [_vp, _i64, _i64, _vp, _vp, _vp, _d, _vp, _vp]),
     "lpmm_factored_stats_static": (_int, [_vp, _i64, _i64, _vp, _vp, _vp, _d, _vp]),
@@ -77,6 +78,10 @@ ADAMW_V4BIT_TENSOR = np.dtype([("p", "<u8"), ("g", "<u8"), ("m", "<u8"), ("v_cod
 RANK1_V4BIT_TENSOR = np.dtype([("p", "<u8"), ("g", "<u8"), ("m", "<u8"), ("v_codes", "<u8"), ("v_rowmax", "<u8"),
                                ("v_colmax", "<u8"), ("v_rowmax_next", "<u8"), ("v_colmax_next", "<u8"),
                                ("rows", "<i8"), ("cols", "<i8"), ("step", "<f4"), ("reserved", "<f4")])
+RANK1_MGROUP_TENSOR = np.dtype([("p", "<u8"), ("g", "<u8"), ("m_codes", "<u8"), ("m_max1", "<u8"),
+                                ("m_max1_next", "<u8"), ("v_codes", "<u8"), ("v_rowmax", "<u8"), ("v_colmax", "<u8"),
+                                ("v_rowmax_next", "<u8"), ("v_colmax_next", "<u8"), ("rows", "<i8"), ("cols", "<i8"),
+                                ("step", "<f4"), ("reserved", "<f4")])
 FACTORED_TENSOR = np.dtype([("p", "<u8"), ("g", "<u8"), ("m_codes", "<u8"), ("m_max1", "<u8"), ("row", "<u8"),
                             ("col", "<u8"), ("workspace", "<u8"), ("rows", "<i8"), ("cols", "<i8"), ("step", "<f4"),
                             ("first_step", "<i4")])

@@ -336,8 +336,11 @@ class AdamW(LowBitOptimizer):
         m_group128 = fits(md_m) and md_m["scale_type"] == "group" and md_m["gp_sz"] == 128
         v_group128 = fits(md_v) and md_v["scale_type"] == "group" and md_v["gp_sz"] == 128
         v_rank1 = fits(md_v) and md_v["scale_type"] == "rank1"
+        # first-moment groups of 256 .. 4096 values (configs/1st_moment_group_*.yml)
+        m_group_wide = fits(md_m) and md_m["scale_type"] == "group" and md_m["gp_sz"] in (256, 512, 1024, 2048, 4096)
         batched, batched_rank1, plain = {}, {}, {}
         batched_m32, batched_rank1_m32 = {}, {}  # fp32 first moment, quantised second moment
+        batched_rank1_mgroup = {}
         factored_work = []
         held = []  # contiguous copies of strided operands
 
@@ -374,6 +377,15 @@ class AdamW(LowBitOptimizer):
                                                                     beta2, lr, wd, eps, _native.current_stream(dev))
             _native.check(st, "non-fused AdamW step (fp32 first moment, rank-1 4-bit second moment)")
 
+        def launch_rank1_mgroup(key, records):
+            dev, qm_ptr, qv_ptr = key
+            table = np.array(records, dtype=_native.RANK1_MGROUP_TENSOR)
+            with torch.cuda.device(dev):
+                st = lib.lpmm_nonfused_adamw4bit_rank1_mgroup_step_multi(
+                    table.ctypes.data, len(records), qm_ptr, qv_ptr, md_m["gp_sz"], beta1, beta2, lr, wd, eps,
+                    _native.current_stream(dev))
+            _native.check(st, "non-fused 4-bit AdamW step (wide first-moment groups, rank-1 second moment)")
+
         for p, grad, state, factored in work:
             step = self._next_step(state)
             if factored:
@@ -401,6 +413,25 @@ class AdamW(LowBitOptimizer):
                         launch_rank1(key, pending)
                         pending.clear()
                     continue
+            if m_group_wide and en_m and en_v and v_rank1 and p.dim() == 2 and p.shape[1] % 128 == 0:
+                key = (p.device, state["exp_avg_qstate"]["qmap"].data_ptr(),
+                       state["exp_avg_sq_qstate"]["qmap"].data_ptr())
+                pending = batched_rank1_mgroup.setdefault(key, [])
+                mc, _ = self._group_state(p, state, "exp_avg", md_m["gp_sz"])
+                # the scales trade places with a second buffer, like the second moment's statistics
+                oh = state["exp_avg_qstate"]["overhead"]
+                cur = oh["max1"]
+                nxt = self._spare_scales.pop(p, None)
+                if nxt is None or nxt.device != cur.device or nxt.shape != cur.shape:
+                    nxt = torch.empty_like(cur)
+                self._spare_scales[p] = cur
+                oh["max1"] = nxt
+                pending.append((dense.data_ptr(), grad.data_ptr(), mc, cur.data_ptr(), nxt.data_ptr())
+                               + self._rank1_state(p, state) + (p.shape[0], p.shape[1], step, 0.0))
+                if len(pending) == _native.RANK1_MULTI_MAX:
+                    launch_rank1_mgroup(key, pending)
+                    pending.clear()
+                continue
             m = self._materialise(p, state, "exp_avg", en_m, md_m)
             if not en_m and en_v:
                 # only the second moment is quantised: the first is read and written as floats
@@ -448,6 +479,9 @@ class AdamW(LowBitOptimizer):
         for key, records in batched_rank1.items():
             if records:
                 launch_rank1(key, records)
+        for key, records in batched_rank1_mgroup.items():
+            if records:
+                launch_rank1_mgroup(key, records)
         for key, records in batched_m32.items():
             if records:
                 launch_group_m32(key, records)
@@ -498,20 +532,20 @@ class AdamW(LowBitOptimizer):
             else:
                 state[name] = t
 
-    def _group_state(self, p, state, name):
-        """Pointers to the codes and scales of a state with block-wise scaling over 128 values;
+    def _group_state(self, p, state, name, gp_sz=128):
+        """Pointers to the codes and scales of a state with block-wise scaling over gp_sz values;
         creates the state on first use: an all-zero moment in the layout and with the metadata
         vectorwise_quant gives it (lpmm/optim/adamw.py:425-434)."""
-        groups = (p.numel() + 127) // 128
+        groups = (p.numel() + gp_sz - 1) // gp_sz
         qstate = state[f"{name}_qstate"]
         if _is_placeholder(state[name]):
-            state[name] = torch.full((packed_nbytes(groups * 128),), _zero_byte(qstate["qmap"]),
+            state[name] = torch.full((packed_nbytes(groups * gp_sz),), _zero_byte(qstate["qmap"]),
                                      dtype=torch.int8, device=p.device)
             oh = qstate["overhead"]
             oh.clear()
             oh.update({"dtype": p.dtype, "stride": self._state_stride(p),
                        "max1": torch.zeros((groups, 1), dtype=torch.float32, device=p.device),
-                       "scaled_shape": torch.Size((groups, 128))})
+                       "scaled_shape": torch.Size((groups, gp_sz))})
         return state[name].data_ptr(), qstate["overhead"]["max1"].data_ptr()
 
     def _rank1_state(self, p, state):
@@ -560,6 +594,14 @@ class AdamW(LowBitOptimizer):
         d = self.__dict__.get("_spare_stats_by_param")
         if d is None:
             d = self.__dict__["_spare_stats_by_param"] = {}
+        return d
+
+    @property
+    def _spare_scales(self):
+        # second buffer of first-moment scales per parameter (wide groups); not part of the state
+        d = self.__dict__.get("_spare_scales_by_param")
+        if d is None:
+            d = self.__dict__["_spare_scales_by_param"] = {}
         return d
 
     def _materialise(self, p, state, name, enabled, md):
