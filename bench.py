@@ -18,7 +18,8 @@ Two further workloads measure the other kernels of the path with the same JSON s
 `--workload factored` (factored second moment on LLaMA-7B MLP/attention shapes) and
 `--workload nonfused_group|nonfused_rank1` (fused=False on the LLaMA-7B-shaped set; with the suffix
 `_m32` under the configurations that quantise the second moment only: fp32 first moment;
-`nonfused_rank1_mgroup`: first-moment groups of 1024 values) and
+`nonfused_rank1_mgroup`: first-moment groups of 1024 values; `nonfused_rank1 --bits 5..8`: the
+configurations with wider codes) and
 `--workload sgd` (4-bit SGD momentum on the same set).
 """
 import argparse
@@ -460,7 +461,12 @@ def run_nonfused(torch, args, v_scale, m32=False, mgroup=False):
 
     dev = torch.device("cuda:0")
     params = make_params(torch, llama7b_shapes(), dev, heavy_tailed=True)
-    if mgroup:
+    bits = args.bits if (v_scale == "rank1" and not m32 and not mgroup) else 4
+    if bits != 4:
+        if bits < 5:
+            sys.exit("bench.py: --workload nonfused_rank1 takes --bits 4 (default) to 8")
+        name = f"default_{bits}b.yml"
+    elif mgroup:
         name = "1st_moment_group_1024.yml"
     elif m32:
         name = "2nd_moment_only_group_128.yml" if v_scale == "group" else "2nd_moment_only_default.yml"
@@ -486,6 +492,8 @@ def run_nonfused(torch, args, v_scale, m32=False, mgroup=False):
         bytes_per_param += 8.0 - 1.0625
     if mgroup:  # update pass: p 8, g 4, both codes read 1; second pass: g 4, both codes read and written 2
         bytes_per_param = 19.0 + 12.0 / 1024
+    if bits != 4:  # one code per byte: p 8, g 4 + 4, m codes 2, v codes 1 + 2, scales 8/128
+        bytes_per_param = 21.0625
     achieved = n_total * bytes_per_param / dt / 1e9
     print(json.dumps({
         "metric": "non-fused 4-bit AdamW step: params/sec, 1 MI355X", "value": n_total / dt,
@@ -505,7 +513,8 @@ def main():
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="llama7b", choices=sorted(WORKLOADS) + ["quant64m", "factored", "nonfused_group", "nonfused_rank1", "nonfused_group_m32", "nonfused_rank1_m32", "nonfused_rank1_mgroup", "sgd", "calibrate"])
-    ap.add_argument("--bits", type=int, default=4, choices=range(1, 9), help="code width of --workload quant64m")
+    ap.add_argument("--bits", type=int, default=4, choices=range(1, 9),
+                    help="code width of --workload quant64m (1-8) and nonfused_rank1 (4-8)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--interleaved-grads", action="store_true",
                     help="allocate each gradient right behind its parameter instead of all parameters first")

@@ -361,6 +361,18 @@ int lpmm_nonfused_adamw4bit_rank1_mgroup_step_multi(const lpmm_rank1_mgroup_tens
                                                     double beta1, double beta2, double lr,
                                                     double weight_decay, double eps, void *stream);
 
+/* lpmm_nonfused_adamw4bit_rank1_step_multi for code widths of 5 to 8 bits (lpmm/configs/
+ * default_{5,6,7,8}b.yml): qmap_m / qmap_v hold 2^bits_m / 2^bits_v entries; the code arrays hold
+ * one code per byte (lpmm/cpp_extension/quantization_kernel.cu:516-533, :656-669):
+ * ceil(R*C/2048)*2048 + 1 bytes each, 4-byte aligned, written in full.  Codes are found by the
+ * reference's search (:397-427), so maps with repeated entries behave as there.  Everything
+ * else (records, statistics, first-step convention) as in the 4-bit entry point. */
+int lpmm_nonfused_adamw_bits_rank1_step_multi(const lpmm_nonfused_rank1_tensor *tensors,
+                                              int64_t count, const float *qmap_m, int bits_m,
+                                              const float *qmap_v, int bits_v, double beta1,
+                                              double beta2, double lr, double weight_decay,
+                                              double eps, void *stream);
+
 /* ---------------------------------------------------------------------------------------
  * (c) Factored second moment on a row-major R x C tensor.
  * Replaces _single_quantized_factored_update (lpmm/optim/adamw.py:579-627) and

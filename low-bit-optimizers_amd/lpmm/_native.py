@@ -53,6 +53,7 @@ PROTOTYPES = {
     "lpmm_nonfused_adamw_v4bit_step_multi": (_int, [_vp, _i64, _vp] + [_d] * 5 + [_vp]),
     "lpmm_nonfused_adamw_v4bit_rank1_step_multi": (_int, [_vp, _i64, _vp] + [_d] * 5 + [_vp]),
     "lpmm_nonfused_adamw4bit_rank1_mgroup_step_multi": (_int, [_vp, _i64, _vp, _vp, _i64] + [_d] * 5 + [_vp]),
+    "lpmm_nonfused_adamw_bits_rank1_step_multi": (_int, [_vp, _i64, _vp, _int, _vp, _int] + [_d] * 5 + [_vp]),
     "lpmm_factored_workspace_bytes": (_i64, [_i64, _i64]),
     "lpmm_factored_stats": (_int, [_vp, _i64, _i64, _vp, _vp, _vp, _d, _vp, _vp]),
     "lpmm_factored_stats_static": (_int, [_vp, _i64, _i64, _vp, _vp, _vp, _d, _vp]),

@@ -341,6 +341,13 @@ class AdamW(LowBitOptimizer):
         batched, batched_rank1, plain = {}, {}, {}
         batched_m32, batched_rank1_m32 = {}, {}  # fp32 first moment, quantised second moment
         batched_rank1_mgroup = {}
+        # 5 to 8 bits (configs/default_{5,6,7,8}b.yml): one code per byte, the same two passes
+        def wide_codes(md):
+            return md["b"] in (5, 6, 7, 8) and md["round_type"] == "real-nearest"
+
+        bits_rank1 = (wide_codes(md_m) and md_m["scale_type"] == "group" and md_m["gp_sz"] == 128
+                      and wide_codes(md_v) and md_v["scale_type"] == "rank1")
+        batched_rank1_bits = {}
         factored_work = []
         held = []  # contiguous copies of strided operands
 
@@ -386,6 +393,15 @@ class AdamW(LowBitOptimizer):
                     _native.current_stream(dev))
             _native.check(st, "non-fused 4-bit AdamW step (wide first-moment groups, rank-1 second moment)")
 
+        def launch_rank1_bits(key, records):
+            dev, qm_ptr, qv_ptr = key
+            table = np.array(records, dtype=_native.NONFUSED_RANK1_TENSOR)
+            with torch.cuda.device(dev):
+                st = lib.lpmm_nonfused_adamw_bits_rank1_step_multi(
+                    table.ctypes.data, len(records), qm_ptr, md_m["b"], qv_ptr, md_v["b"], beta1, beta2, lr, wd, eps,
+                    _native.current_stream(dev))
+            _native.check(st, "non-fused AdamW step (5-8-bit states, rank-1 second moment)")
+
         for p, grad, state, factored in work:
             step = self._next_step(state)
             if factored:
@@ -413,6 +429,17 @@ class AdamW(LowBitOptimizer):
                         launch_rank1(key, pending)
                         pending.clear()
                     continue
+            if bits_rank1 and en_m and en_v and p.dim() == 2 and p.shape[1] % 128 == 0:
+                key = (p.device, state["exp_avg_qstate"]["qmap"].data_ptr(),
+                       state["exp_avg_sq_qstate"]["qmap"].data_ptr())
+                pending = batched_rank1_bits.setdefault(key, [])
+                mc, ms = self._group_state(p, state, "exp_avg", b=md_m["b"])
+                pending.append((dense.data_ptr(), grad.data_ptr(), mc, ms) + self._rank1_state(p, state, b=md_v["b"])
+                               + (p.shape[0], p.shape[1], step, 0.0))
+                if len(pending) == _native.RANK1_MULTI_MAX:
+                    launch_rank1_bits(key, pending)
+                    pending.clear()
+                continue
             if m_group_wide and en_m and en_v and v_rank1 and p.dim() == 2 and p.shape[1] % 128 == 0:
                 key = (p.device, state["exp_avg_qstate"]["qmap"].data_ptr(),
                        state["exp_avg_sq_qstate"]["qmap"].data_ptr())
@@ -482,6 +509,9 @@ class AdamW(LowBitOptimizer):
         for key, records in batched_rank1_mgroup.items():
             if records:
                 launch_rank1_mgroup(key, records)
+        for key, records in batched_rank1_bits.items():
+            if records:
+                launch_rank1_bits(key, records)
         for key, records in batched_m32.items():
             if records:
                 launch_group_m32(key, records)
@@ -532,14 +562,16 @@ class AdamW(LowBitOptimizer):
             else:
                 state[name] = t
 
-    def _group_state(self, p, state, name, gp_sz=128):
+    def _group_state(self, p, state, name, gp_sz=128, b=4):
         """Pointers to the codes and scales of a state with block-wise scaling over gp_sz values;
         creates the state on first use: an all-zero moment in the layout and with the metadata
-        vectorwise_quant gives it (lpmm/optim/adamw.py:425-434)."""
+        vectorwise_quant gives it (lpmm/optim/adamw.py:425-434).  With zero scales every code decodes
+        to zero, and the first step overwrites the codes in full: for widths other than 4 bits the
+        array starts as zero bytes."""
         groups = (p.numel() + gp_sz - 1) // gp_sz
         qstate = state[f"{name}_qstate"]
         if _is_placeholder(state[name]):
-            state[name] = torch.full((packed_nbytes(groups * gp_sz),), _zero_byte(qstate["qmap"]),
+            state[name] = torch.full((packed_nbytes(groups * gp_sz, b),), _zero_byte(qstate["qmap"]) if b == 4 else 0,
                                      dtype=torch.int8, device=p.device)
             oh = qstate["overhead"]
             oh.clear()
@@ -548,7 +580,7 @@ class AdamW(LowBitOptimizer):
                        "scaled_shape": torch.Size((groups, gp_sz))})
         return state[name].data_ptr(), qstate["overhead"]["max1"].data_ptr()
 
-    def _rank1_state(self, p, state):
+    def _rank1_state(self, p, state, b=4):
         """Pointers to the codes of a rank-1 scaled second moment, the statistics they are scaled
         by and the pair of buffers that receives the next statistics; creates the state on first
         use.  The kernels leave the statistics of the new second moment in the second pair; the
@@ -558,8 +590,8 @@ class AdamW(LowBitOptimizer):
         dev = p.device
         qs_v = state["exp_avg_sq_qstate"]
         if _is_placeholder(state["exp_avg_sq"]):
-            state["exp_avg_sq"] = torch.full((packed_nbytes(p.numel()),), _zero_byte(qs_v["qmap"]), dtype=torch.int8,
-                                             device=dev)
+            state["exp_avg_sq"] = torch.full((packed_nbytes(p.numel(), b),), _zero_byte(qs_v["qmap"]) if b == 4 else 0,
+                                             dtype=torch.int8, device=dev)
             qs_v["overhead"].clear()
             qs_v["overhead"].update({"dtype": p.dtype, "stride": self._state_stride(p), "dim": 2, "max1": None,
                                      "max_dims": [torch.zeros((rows, 1), dtype=torch.float32, device=dev),

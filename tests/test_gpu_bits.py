@@ -155,7 +155,8 @@ def test_nonfused_optimizer_other_widths(oracle, bits):
 
     H = dict(lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01)
     rng = np.random.default_rng(bits)
-    shapes = [(96, 160), (11008,)]
+    # a ragged matrix and a vector (staged path), a matrix the two-pass kernels take
+    shapes = [(96, 160), (11008,), (64, 256)]
     host = [(rng.standard_normal(s) * 0.02).astype(np.float32) for s in shapes]
     params = [torch.nn.Parameter(to_dev(h)) for h in host]
     cfg = os.path.join(os.path.dirname(lpmm.config.__file__), "configs", f"default_{bits}b.yml")
