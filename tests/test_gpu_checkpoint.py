@@ -32,6 +32,10 @@ MODES = {
     "fused": dict(fused=True),
     "nonfused_rank1": dict(fused=False, qconfig="default.yml"),
     "nonfused_group": dict(fused=False, qconfig="2nd_moment_group_128.yml"),
+    "nonfused_rank1_fp32_m": dict(fused=False, qconfig="2nd_moment_only_default.yml"),
+    "nonfused_group_fp32_m": dict(fused=False, qconfig="2nd_moment_only_group_128.yml"),
+    "nonfused_rank1_m_group_512": dict(fused=False, qconfig="1st_moment_group_512.yml"),
+    "nonfused_rank1_6bit": dict(fused=False, qconfig="default_6b.yml"),
     "factored": dict(fused=False, factor_second_moment=True),
     "factored_fused": dict(fused=True, factor_second_moment=True),
 }
