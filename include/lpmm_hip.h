@@ -337,7 +337,12 @@ int lpmm_nonfused_adamw_v4bit_rank1_step_multi(const lpmm_rank1_v4bit_tensor *te
  * overwrites its codes scaled by m_max1_next -- the caller swaps m_max1 / m_max1_next like the
  * statistics of the second moment.  m_codes: ceil(ceil(R*C / m_group_size) * m_group_size / 2048)
  * * 1024 + 1 bytes, 4-byte aligned, written in full; m_max1, m_max1_next: float[ceil(R*C /
- * m_group_size)].  Everything else as in lpmm_nonfused_adamw4bit_rank1_step_multi. */
+ * m_group_size)].  Everything else as in lpmm_nonfused_adamw4bit_rank1_step_multi.
+ *
+ * This entry point also takes column counts that are no multiple of 128 (any multiple of 8, e.g.
+ * 1600 or 1000), with m_group_size 128 as well: the 128-value groups of the flattened tensor then
+ * straddle tensor rows, which is the same global dependency.  A call with such a tensor runs
+ * more general (somewhat slower) kernels on all its tensors. */
 typedef struct lpmm_rank1_mgroup_tensor {
     float *p;
     const float *g;

@@ -385,7 +385,7 @@ class AdamW(LowBitOptimizer):
             _native.check(st, "non-fused AdamW step (fp32 first moment, rank-1 4-bit second moment)")
 
         def launch_rank1_mgroup(key, records):
-            dev, qm_ptr, qv_ptr = key
+            dev, qm_ptr, qv_ptr = key[:3]
             table = np.array(records, dtype=_native.RANK1_MGROUP_TENSOR)
             with torch.cuda.device(dev):
                 st = lib.lpmm_nonfused_adamw4bit_rank1_mgroup_step_multi(
@@ -415,9 +415,10 @@ class AdamW(LowBitOptimizer):
             if m_group128 and en_m and en_v:
                 key = (p.device, state["exp_avg_qstate"]["qmap"].data_ptr(),
                        state["exp_avg_sq_qstate"]["qmap"].data_ptr())
-                if v_group128:
+                # a vector under 'rank1' is scaled block-wise over 128 values (lpmm/functional.py:192-197)
+                if v_group128 or (v_rank1 and p.dim() == 1):
                     pending = batched.setdefault(key, [])
-                    pending.append(self._nonfused_record(p, dense, grad, state, step))
+                    pending.append(self._nonfused_record(p, dense, grad, state, step, v_rank1))
                     if len(pending) == _native.MULTI_MAX:  # one launch's worth: enqueue it now
                         launch_group(key, pending)
                         pending.clear()
@@ -440,9 +441,13 @@ class AdamW(LowBitOptimizer):
                     launch_rank1_bits(key, pending)
                     pending.clear()
                 continue
-            if m_group_wide and en_m and en_v and v_rank1 and p.dim() == 2 and p.shape[1] % 128 == 0:
+            # wide first-moment groups, or rows that are no whole number of 128-value groups (a multiple
+            # of 8 columns; the two kinds go to different launches: the second takes more general kernels)
+            ragged = p.dim() == 2 and p.shape[1] % 128 != 0 and p.shape[1] % 8 == 0
+            if (en_m and en_v and v_rank1 and p.dim() == 2
+                    and ((m_group_wide and p.shape[1] % 128 == 0) or ((m_group_wide or m_group128) and ragged))):
                 key = (p.device, state["exp_avg_qstate"]["qmap"].data_ptr(),
-                       state["exp_avg_sq_qstate"]["qmap"].data_ptr())
+                       state["exp_avg_sq_qstate"]["qmap"].data_ptr(), ragged)
                 pending = batched_rank1_mgroup.setdefault(key, [])
                 mc, _ = self._group_state(p, state, "exp_avg", md_m["gp_sz"])
                 # the scales trade places with a second buffer, like the second moment's statistics
@@ -463,10 +468,11 @@ class AdamW(LowBitOptimizer):
             if not en_m and en_v:
                 # only the second moment is quantised: the first is read and written as floats
                 key = (p.device, state["exp_avg_sq_qstate"]["qmap"].data_ptr())
-                if v_group128:
+                if v_group128 or (v_rank1 and p.dim() == 1):
                     pending = batched_m32.setdefault(key, [])
                     pending.append((dense.data_ptr(), grad.data_ptr(), m.data_ptr())
-                                   + self._group_state(p, state, "exp_avg_sq") + (p.numel(), step, 0.0))
+                                   + self._group_state(p, state, "exp_avg_sq", rank1_vector=v_rank1)
+                                   + (p.numel(), step, 0.0))
                     if len(pending) == _native.V4BIT_MULTI_MAX:
                         launch_group_m32(key, pending)
                         pending.clear()
@@ -562,7 +568,7 @@ class AdamW(LowBitOptimizer):
             else:
                 state[name] = t
 
-    def _group_state(self, p, state, name, gp_sz=128, b=4):
+    def _group_state(self, p, state, name, gp_sz=128, b=4, rank1_vector=False):
         """Pointers to the codes and scales of a state with block-wise scaling over gp_sz values;
         creates the state on first use: an all-zero moment in the layout and with the metadata
         vectorwise_quant gives it (lpmm/optim/adamw.py:425-434).  With zero scales every code decodes
@@ -578,6 +584,8 @@ class AdamW(LowBitOptimizer):
             oh.update({"dtype": p.dtype, "stride": self._state_stride(p),
                        "max1": torch.zeros((groups, 1), dtype=torch.float32, device=p.device),
                        "scaled_shape": torch.Size((groups, gp_sz))})
+            if rank1_vector:  # the 'rank1' branch records the dimension count (lpmm/functional.py:191)
+                oh["dim"] = 1
         return state[name].data_ptr(), qstate["overhead"]["max1"].data_ptr()
 
     def _rank1_state(self, p, state, b=4):
@@ -607,10 +615,10 @@ class AdamW(LowBitOptimizer):
         return (state["exp_avg_sq"].data_ptr(), cur[0].data_ptr(), cur[1].data_ptr(), nxt[0].data_ptr(),
                 nxt[1].data_ptr())
 
-    def _nonfused_record(self, p, dense, grad, state, step):
+    def _nonfused_record(self, p, dense, grad, state, step, rank1_vector=False):
         """The tensor's record for the one-pass non-fused step."""
         mc, ms = self._group_state(p, state, "exp_avg")
-        vc, vs = self._group_state(p, state, "exp_avg_sq")
+        vc, vs = self._group_state(p, state, "exp_avg_sq", rank1_vector=rank1_vector)
         return (dense.data_ptr(), grad.data_ptr(), mc, vc, ms, vs, p.numel(), step, 0.0)
 
     def _nonfused_rank1_record(self, p, dense, grad, state, step):

@@ -141,6 +141,74 @@ def test_mgroup_all_zero_groups(oracle, qmaps, gp):
             t.check(f"group {gp}, {t.rows}x{t.cols} step {step}")
 
 
+@pytest.mark.parametrize("gp", [128, 512, 4096])
+def test_ragged_columns_match_staged_oracle(oracle, qmaps, gp):
+    """Column counts that are no multiple of 128 (multiples of 8): the first moment's groups
+    straddle rows, the last 128-column block of a row is cut, and the end of the tensor cuts a
+    group (its padding takes the group's scale).  With whole tiles, ragged row counts, fewer
+    columns than one block, and a tensor that is a multiple of 128 columns in the same call."""
+    qm, qv = qmaps
+    dqm, dqv = to_dev(qm), to_dev(qv)
+    rng = np.random.default_rng(66)
+    shapes = [(5, 136), (7, 72), (1, 8), (40, 1600), (130, 200), (300, 1000), (64, 4800), (2500, 328), (33, 256),
+              (513, 1096)]
+    tensors = [_Tensor(r, c, gp, rng) for r, c in shapes]
+    for step in range(1, 4):
+        grads = [_grad(rng, t) for t in tensors]
+        _step_all(oracle, tensors, grads, gp, qm, qv, dqm, dqv, step)
+        for t in tensors:
+            t.check(f"group {gp}, {t.rows}x{t.cols} step {step}")
+
+
+def test_ragged_columns_all_zero_groups(oracle, qmaps):
+    qm, qv = qmaps
+    dqm, dqv = to_dev(qm), to_dev(qv)
+    rng = np.random.default_rng(67)
+    tensors = [_Tensor(r, c, 128, rng) for r, c in [(40, 200), (70, 72), (9, 1608)]]
+    zero_rows = [34, 66, 3]
+    for step in (1, 2):
+        grads = [_grad(rng, t, z) for t, z in zip(tensors, zero_rows)]
+        _step_all(oracle, tensors, grads, 128, qm, qv, dqm, dqv, step)
+        for t in tensors:
+            t.check(f"{t.rows}x{t.cols} step {step}")
+
+
+def test_ragged_columns_optimizer_with_the_default_configuration(oracle, qmaps):
+    """lpmm.optim.AdamW(fused=False, qconfig=default.yml) on GPT-2-XL-like shapes (d = 1600): the
+    two-pass kernels for ragged rows; states in the reference's layout, equal to the oracle."""
+    import lpmm
+
+    qm, qv = qmaps
+    rng = np.random.default_rng(68)
+    shapes = [(48, 1600), (1600, 200), (10, 4800)]
+    holders = [_Tensor(r, c, 128, rng) for r, c in shapes]
+    params = [torch.nn.Parameter(to_dev(h.host_p)) for h in holders]
+    cfg = os.path.join(os.path.dirname(lpmm.config.__file__), "configs", "default.yml")
+    opt = lpmm.optim.AdamW(params, fused=False, qconfig=cfg, lr=H["lr"], betas=(H["beta1"], H["beta2"]),
+                           eps=H["eps"], weight_decay=H["wd"])
+    for step in range(1, 4):
+        grads = [_grad(rng, h) for h in holders]
+        for p, g in zip(params, grads):
+            p.grad = to_dev(g)
+        opt.step()
+        torch.cuda.synchronize()
+        for i, (h, p, g) in enumerate(zip(holders, params, grads)):
+            h.oracle_step(oracle, g, qm, qv, step)
+            st = opt.state[p]
+            what = f"tensor {i} step {step}"
+            oh = st["exp_avg_qstate"]["overhead"]
+            assert tuple(oh["max1"].shape) == ((h.n + 127) // 128, 1), what
+            np.testing.assert_array_equal(to_np(st["exp_avg"]).view(np.uint8), h.ref_m[0], err_msg=f"{what}: m codes")
+            np.testing.assert_array_equal(to_np(oh["max1"]).reshape(-1), h.ref_m[1], err_msg=f"{what}: m max1")
+            ov = st["exp_avg_sq_qstate"]["overhead"]
+            np.testing.assert_array_equal(to_np(st["exp_avg_sq"]).view(np.uint8), h.ref_v[0], err_msg=f"{what}: v codes")
+            np.testing.assert_array_equal(to_np(ov["max_dims"][0]).reshape(-1), h.ref_v[1], err_msg=what)
+            np.testing.assert_array_equal(to_np(ov["max_dims"][1]).reshape(-1), h.ref_v[2], err_msg=what)
+            assert_rel(to_np(p), h.host_p, f"{what}: p", scale=h.host_p)
+            with torch.no_grad():
+                p.copy_(torch.from_numpy(h.host_p))
+
+
 def test_mgroup_more_tensors_than_one_launch(oracle, qmaps):
     qm, qv = qmaps
     dqm, dqv = to_dev(qm), to_dev(qv)
@@ -225,10 +293,10 @@ def test_mgroup_argument_checks(qmaps):
         return lib.lpmm_nonfused_adamw4bit_rank1_mgroup_step_multi(table.ctypes.data, len(records), dqm.data_ptr(),
                                                                    dqv.data_ptr(), gp, *f5, stream)
 
-    for gp in (0, 128, 300, 384, 8192):
-        assert call([ok], gp) != 0, gp  # 256 .. 4096 in powers of two only
+    for gp in (0, 64, 300, 384, 8192):
+        assert call([ok], gp) != 0, gp  # 128 .. 4096 in powers of two only
     assert call([ok[:4] + (0,) + ok[5:]]) != 0  # no buffer for the next scales
     assert call([ok[:4] + (ms[0].data_ptr(),) + ok[5:]]) != 0  # the scales alias
-    assert call([ok[:11] + (100, 1.0, 0.0)]) != 0  # columns not a multiple of 128
+    assert call([ok[:11] + (100, 1.0, 0.0)]) != 0  # columns not a multiple of 8
     assert call([ok[:10] + (0, 128, 1.0, 0.0)]) == 0  # an empty tensor is skipped
     torch.cuda.synchronize()

@@ -127,6 +127,8 @@ def test_nonfused_optimizer_matches_oracle(oracle, qmaps, v_scale):
     assert_rel(to_np(params[0]), host[0], 'p 2-D', scale=host[0])
     # 1-D tensor: rank1 falls back to group-128
     s1 = opt.state[params[1]]
+    if v_scale == "rank1":
+        assert s1["exp_avg_sq_qstate"]["overhead"]["dim"] == 1  # as the reference's 'rank1' branch records it
     np.testing.assert_array_equal(to_np(s1["exp_avg_sq"]).view(np.uint8), states[1].v[0])
     np.testing.assert_array_equal(to_np(s1["exp_avg_sq_qstate"]["overhead"]["max1"]).reshape(-1), states[1].v[1])
     assert_rel(to_np(params[1]), host[1], 'p 1-D', scale=host[1])
