@@ -460,7 +460,8 @@ def run_nonfused(torch, args, v_scale, m32=False, mgroup=False):
     import lpmm
 
     dev = torch.device("cuda:0")
-    params = make_params(torch, llama7b_shapes(), dev, heavy_tailed=True)
+    shapes = gpt2xl_shapes() if args.shapes == "gpt2xl" else llama7b_shapes()
+    params = make_params(torch, shapes, dev, heavy_tailed=True)
     bits = args.bits if (v_scale == "rank1" and not m32 and not mgroup) else 4
     if bits != 4:
         if bits < 5:
@@ -494,13 +495,28 @@ def run_nonfused(torch, args, v_scale, m32=False, mgroup=False):
         bytes_per_param = 19.0 + 12.0 / 1024
     if bits != 4:  # one code per byte: p 8, g 4 + 4, m codes 2, v codes 1 + 2, scales 8/128
         bytes_per_param = 21.0625
+    if args.shapes != "llama7b":
+        # a mix of paths: per tensor, what its path moves (rank-1: matrices with a multiple of 128 columns
+        # as above, other multiples of 8 through the kernels for ragged rows 19.0625, quantised vectors one
+        # pass 14.125; fp32 states 28)
+        total = 0.0
+        for p in params:
+            if p.numel() <= 4096:
+                total += 28.0 * p.numel()
+            elif v_scale == "group" or p.dim() == 1:
+                total += BYTES_PER_PARAM_4BIT * p.numel()
+            elif p.shape[1] % 128 == 0:
+                total += 18.5625 * p.numel()
+            else:
+                total += 19.0625 * p.numel()
+        bytes_per_param = total / n_total
     achieved = n_total * bytes_per_param / dt / 1e9
     print(json.dumps({
         "metric": "non-fused 4-bit AdamW step: params/sec, 1 MI355X", "value": n_total / dt,
         "unit": "params/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": dt * 1e3,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": f"fused=False, {'fp32 first moment, ' if m32 else ''}{'first-moment groups of 1024, ' if mgroup else ''}second moment '{v_scale}' scaling, "
-                               "LLaMA-7B-shaped fp32 set", "qconfig": name,
+                               f"{'GPT-2-XL' if args.shapes == 'gpt2xl' else 'LLaMA-7B'}-shaped fp32 set", "qconfig": name,
                    "tensors": len(params), "params": n_total},
         "roofline": {"bound": "hbm", "kernel": "whole step", "achieved": achieved, "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None,
@@ -515,6 +531,8 @@ def main():
     ap.add_argument("--workload", default="llama7b", choices=sorted(WORKLOADS) + ["quant64m", "factored", "nonfused_group", "nonfused_rank1", "nonfused_group_m32", "nonfused_rank1_m32", "nonfused_rank1_mgroup", "sgd", "calibrate"])
     ap.add_argument("--bits", type=int, default=4, choices=range(1, 9),
                     help="code width of --workload quant64m (1-8) and nonfused_rank1 (4-8)")
+    ap.add_argument("--shapes", default="llama7b", choices=["llama7b", "gpt2xl"],
+                    help="parameter set of the nonfused_* workloads")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--interleaved-grads", action="store_true",
                     help="allocate each gradient right behind its parameter instead of all parameters first")
