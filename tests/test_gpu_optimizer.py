@@ -181,6 +181,10 @@ def test_nonfused_rank1_on_tensors_of_more_than_two_dimensions(oracle, qmaps):
 STRIDED_MODES = {
     "rank1": dict(fused=False, qconfig="default.yml"),
     "group": dict(fused=False, qconfig="2nd_moment_group_128.yml"),
+    "rank1_fp32_m": dict(fused=False, qconfig="2nd_moment_only_default.yml"),
+    "group_fp32_m": dict(fused=False, qconfig="2nd_moment_only_group_128.yml"),
+    "rank1_m_group_512": dict(fused=False, qconfig="1st_moment_group_512.yml"),
+    "rank1_6bit": dict(fused=False, qconfig="default_6b.yml"),
     "factored": dict(fused=False, factor_second_moment=True),
     "factored_on_fused": dict(fused=True, factor_second_moment=True),
 }
@@ -201,13 +205,16 @@ def test_strided_parameters_equal_their_contiguous_twins(mode):
     rng = np.random.default_rng(8)
     dev = "cuda"
     # a transposed matrix (dense, permuted strides), every other column of a wider matrix (gaps),
-    # a permuted 3-D tensor, a strided small vector with fp32 states, a transposed ragged matrix
+    # a permuted 3-D tensor, a strided small vector with fp32 states, a transposed ragged matrix, a
+    # transposed matrix whose rows are a multiple of 8 but not of 128 values long
     bases = [to_dev((rng.standard_normal((256, 96)) * 0.02).astype(np.float32)),
              to_dev((rng.standard_normal((64, 512)) * 0.02).astype(np.float32)),
              to_dev((rng.standard_normal((40, 6, 64)) * 0.02).astype(np.float32)),
              to_dev((rng.standard_normal((4000,)) * 0.02).astype(np.float32)),
-             to_dev((rng.standard_normal((130, 70)) * 0.02).astype(np.float32))]
-    views = [lambda t: t.t(), lambda t: t[:, ::2], lambda t: t.permute(1, 0, 2), lambda t: t[::2], lambda t: t.t()]
+             to_dev((rng.standard_normal((130, 70)) * 0.02).astype(np.float32)),
+             to_dev((rng.standard_normal((136, 64)) * 0.02).astype(np.float32))]
+    views = [lambda t: t.t(), lambda t: t[:, ::2], lambda t: t.permute(1, 0, 2), lambda t: t[::2], lambda t: t.t(),
+             lambda t: t.t()]
     if mode == "factored":
         bases, views = bases[:2] + bases[3:], views[:2] + views[3:]
     elif mode == "factored_on_fused":
@@ -257,10 +264,12 @@ def test_strided_parameters_equal_their_contiguous_twins(mode):
     import lpmm.functional as F
 
     s0 = opt_s.state[strided[0]]
-    md = opt_s.get_qmetadata_by_state_name("exp_avg")
-    m = F.vectorwise_dequant(s0["exp_avg"], qmap=s0["exp_avg_qstate"]["qmap"], shape=strided[0].shape,
-                             **{**s0["exp_avg_qstate"]["overhead"], **md})
-    assert m.stride() == strided[0].stride() and m.shape == strided[0].shape
+    name = "exp_avg" if s0["exp_avg"].dtype == torch.int8 else "exp_avg_sq"  # a quantised state of this mode
+    if s0[name].dtype == torch.int8:
+        md = opt_s.get_qmetadata_by_state_name(name)
+        m = F.vectorwise_dequant(s0[name], qmap=s0[f"{name}_qstate"]["qmap"], shape=strided[0].shape,
+                                 **{**s0[f"{name}_qstate"]["overhead"], **md})
+        assert m.stride() == strided[0].stride() and m.shape == strided[0].shape
 
 
 @pytest.mark.parametrize("fused", [False, True])
