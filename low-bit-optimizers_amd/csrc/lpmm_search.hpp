@@ -28,26 +28,60 @@ __device__ __forceinline__ void fill_map(float *lds_map, const float *__restrict
 // breadth-first order the nodes of a level are neighbours, so up to 32 of them sit in 32
 // different banks (and lanes that read the same node share one access).  The midpoints are
 // formed once per workgroup with the reference's expression.
+//
+// The evenly spaced map without zero, q[k] = (k + 1) / N (create_pow_map(b, False, 1),
+// lpmm/functional.py:303-315: the second moment's map of every shipped configuration), needs no
+// search: its midpoints are (2j + 1) / 2N, and the number of them below x is
+// ceil(x * N - 1.5) clamped to [0, N - 1] -- exact in float arithmetic (x * N is a scaling by a
+// power of two, and the fused subtraction rounds once).  The stored code depends on the map only
+// through its first and last entry and its midpoints (the entries themselves only select which
+// midpoint decides), so the closed form applies whenever those have the values of that map, which
+// is checked while the tables are filled: every wave records whether its entries match.
 struct SearchLds {
     float tree[256];  // [1, N): breadth-first; [0]: q[0]
     float mid[256];   // [1, N): (q[lo-1] + q[lo]) * 0.5f; [0]: q[N-1]
+    uint32_t even[16];  // per wave of the workgroup: do the entries it filled match the evenly spaced map
 };
+
+// does entry j (as stored: tree[0] = q[0], mid[0] = q[N-1], mid[j] for j >= 1) match the evenly spaced map
+__device__ __forceinline__ bool matches_even_map(uint32_t j, float tree, float mid, int bits)
+{
+    const float step = __uint_as_float((127u - (uint32_t)bits) << 23);  // 1 / N
+    return j == 0 ? (tree == step && mid == 1.0f) : mid == (float)(2u * j + 1u) * (0.5f * step);
+}
+
+// all waves' records (after the barrier that follows the fill); uniform over the workgroup, in a scalar register
+__device__ __forceinline__ bool map_is_even(const SearchLds &t)
+{
+    uint32_t ok = 1u;
+    for (uint32_t w = 0; w < (blockDim.x + kWave - 1) / kWave; ++w)
+        ok &= t.even[w];
+    return __builtin_amdgcn_readfirstlane((int)ok) != 0;
+}
 
 // the caller synchronises
 __device__ __forceinline__ void fill_search(SearchLds &t, const float *__restrict__ qmap, int bits)
 {
     const uint32_t n = 1u << bits;
+    bool even = true;
     for (uint32_t j = threadIdx.x; j < n; j += blockDim.x) {
+        float tree, mid;
         if (j == 0) {
-            t.tree[0] = qmap[0];
-            t.mid[0] = qmap[n - 1];
+            tree = qmap[0];
+            mid = qmap[n - 1];
         } else {
             const uint32_t level = 31u - (uint32_t)__clz((int)j);
             const uint32_t k = j - (1u << level);
-            t.tree[j] = qmap[(((2u * k + 1u) << (bits - 1 - level))) - 1u];
-            t.mid[j] = (qmap[j - 1] + qmap[j]) * 0.5f;
+            tree = qmap[(((2u * k + 1u) << (bits - 1 - level))) - 1u];
+            mid = (qmap[j - 1] + qmap[j]) * 0.5f;
         }
+        t.tree[j] = tree;
+        t.mid[j] = mid;
+        even = even && matches_even_map(j, tree, mid, bits);
     }
+    const bool wave_even = __all(even);
+    if ((threadIdx.x & (kWave - 1)) == 0)
+        t.even[threadIdx.x / kWave] = wave_even;
 }
 
 // The same in two halves for workgroups of at least 2^bits threads (one entry per thread), so that a
@@ -76,10 +110,14 @@ __device__ __forceinline__ SearchFill fill_search_load(const float *__restrict__
 
 __device__ __forceinline__ void fill_search_store(SearchLds &t, const SearchFill &f, int bits)
 {
-    if (threadIdx.x < (1u << bits)) {
+    const bool mine = threadIdx.x < (1u << bits);
+    if (mine) {
         t.tree[threadIdx.x] = f.tree;
         t.mid[threadIdx.x] = f.mid;
     }
+    const bool wave_even = __all(!mine || matches_even_map(threadIdx.x, f.tree, f.mid, bits));
+    if ((threadIdx.x & (kWave - 1)) == 0)
+        t.even[threadIdx.x / kWave] = wave_even;
 }
 
 __device__ __forceinline__ uint32_t search_code(const SearchLds &t, int bits, float x)
@@ -98,11 +136,23 @@ __device__ __forceinline__ uint32_t search_code(const SearchLds &t, int bits, fl
     return (x != x) ? nan_code : code;
 }
 
-// The same for a lane's 8 values at once: the levels are the outer loop, so that the 8 reads of
+// The same for a lane's 8 values at once (even: map_is_even(t), read once per kernel after the
+// barrier that follows the fill): the levels are the outer loop, so that the 8 reads of
 // a level are in flight together instead of 8 x `bits` dependent ones in a row.
-__device__ __forceinline__ void search_codes8(const SearchLds &t, int bits, const float (&x)[8], uint32_t (&code)[8])
+__device__ __forceinline__ void search_codes8(const SearchLds &t, int bits, bool even, const float (&x)[8],
+                                              uint32_t (&code)[8])
 {
     const uint32_t n = 1u << bits;
+    if (even) {
+        const float scale = (float)n, top = (float)(n - 1u);
+        const uint32_t nan = codes_per_byte(bits) == 1 ? 255u : n - 1u;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const float c = fminf(fmaxf(__builtin_ceilf(__builtin_fmaf(x[k], scale, -1.5f)), 0.0f), top);
+            code[k] = (x[k] != x[k]) ? nan : (uint32_t)c;
+        }
+        return;
+    }
     // a = byte offset of the node (4 i): one shift-or per level, no separate address computation
     uint32_t a[8];
 #pragma unroll

@@ -501,8 +501,9 @@ __global__ __launch_bounds__(kThreads) void rank1_requant_kernel(const MultiR1 a
 // entries in LDS, decoded by indexing and encoded by the reference's search (:397-427) as the
 // stand-alone quantisers of these widths do it.  Same tiles and statistics as above; a lane's
 // eight codes are two dwords.  21.06 bytes per parameter cross HBM (p 8, g 4 + 4, m codes 2,
-// v codes 1 + 2, scales).  LLaMA-7B-shaped set: 27.6 ms per step with 5 bits, 29.5 ms with 8
-// (the staged path 67.6 ms).
+// v codes 1 + 2, scales).  LLaMA-7B-shaped set: 25.1 ms per step with 5 bits, 25.3 ms with 8
+// (the staged path 67.6 ms); the second moment's evenly spaced map takes the closed form of
+// lpmm_search.hpp, so only the first moment is searched.
 // ---------------------------------------------------------------------------------------
 __device__ __forceinline__ uint32_t byte_of(uint32_t w0, uint32_t w1, int k)
 {
@@ -556,6 +557,7 @@ __global__ __launch_bounds__(kThreads) void rank1_update_bits_kernel(const Multi
     h.bc2_sqrt = t.bc2_sqrt;
     h.rbc2_sqrt = t.rbc2_sqrt;
     __syncthreads();
+    const bool map_even = map_is_even(search_m);
 
     if (tl == 0) {
         const int64_t n = t.rows * cols;
@@ -613,7 +615,7 @@ __global__ __launch_bounds__(kThreads) void rank1_update_bits_kernel(const Multi
                     xs[k] = m[k] / amax_m;
             }
             uint32_t c[kEltsPerLane];
-            search_codes8(search_m, bits_m, xs, c);
+            search_codes8(search_m, bits_m, map_even, xs, c);
             store4(pp, make_float4(pv[0], pv[1], pv[2], pv[3]));
             store4(pp + 64, make_float4(pv[4], pv[5], pv[6], pv[7]));
             store_u32(mcp, pack4(c, 0));
@@ -658,6 +660,7 @@ __global__ __launch_bounds__(kThreads) void rank1_requant_bits_kernel(const Mult
     h.b2 = args.b2;
     h.w2 = args.w2;
     __syncthreads();
+    const bool map_even = map_is_even(search_v);
 
     if (tl == 0) {
         const int64_t n = t.rows * cols;
@@ -691,7 +694,7 @@ __global__ __launch_bounds__(kThreads) void rank1_requant_bits_kernel(const Mult
             x[k] = v / ((cn[k] < rn) ? cn[k] : rn);
         }
         uint32_t c[kEltsPerLane];
-        search_codes8(search_v, bits_v, x, c);
+        search_codes8(search_v, bits_v, map_even, x, c);
         store_u32(vcp, pack4(c, 0));
         store_u32(vcp + 16, pack4(c, 1));
     }

@@ -112,6 +112,7 @@ __global__ __launch_bounds__(kBThreads) void pack_bits_kernel(const float *__res
     __shared__ SearchLds lds_map;
     fill_search(lds_map, qmap, bits);
     __syncthreads();
+    const bool map_even = map_is_even(lds_map);
     const int64_t base = ((int64_t)blockIdx.x * kBThreads + threadIdx.x) * kBElts;
     if (base == 0)
         out[last_byte(n_padded, bits)] = 0;
@@ -120,7 +121,7 @@ __global__ __launch_bounds__(kBThreads) void pack_bits_kernel(const float *__res
     float v[kBElts];
     load_values(x, base, n_padded, vec, v);
     uint32_t c[kBElts];
-    search_codes8(lds_map, bits, v, c);
+    search_codes8(lds_map, bits, map_even, v, c);
     store_codes(out, base, bits, c);
 }
 
@@ -270,6 +271,7 @@ __global__ __launch_bounds__(THREADS) void quant_group_bits_kernel(const float *
     if ((threadIdx.x & 15) == 0)
         s_row[threadIdx.x >> 4] = amax;
     __syncthreads();
+    const bool map_even = map_is_even(lds_map);
     if (rows_per_group > 1) {
         const int first = (threadIdx.x >> 4) & ~(rows_per_group - 1);
         amax = s_row[first];
@@ -298,7 +300,7 @@ __global__ __launch_bounds__(THREADS) void quant_group_bits_kernel(const float *
             for (int k = 0; k < kBElts; ++k)
                 xs[k] = v[k] / amax;
         }
-        search_codes8(lds_map, bits, xs, c);
+        search_codes8(lds_map, bits, map_even, xs, c);
     } else {
         // padding added by the re-grouping to 2048: plain zeros, not divided by anything
         const uint32_t z = search_code(lds_map, bits, 0.0f);
@@ -342,6 +344,7 @@ __global__ __launch_bounds__(kBThreads) void quant_rank1_bits_kernel(const float
     __shared__ SearchLds lds_map;
     fill_search(lds_map, qmap, bits);
     __syncthreads();
+    const bool map_even = map_is_even(lds_map);
     const int64_t base = ((int64_t)blockIdx.x * kBThreads + threadIdx.x) * kBElts;
     if (base == 0)
         codes[last_byte(n_padded, bits)] = 0;
@@ -367,7 +370,7 @@ __global__ __launch_bounds__(kBThreads) void quant_rank1_bits_kernel(const float
             }
         }
     }
-    search_codes8(lds_map, bits, xs, code);
+    search_codes8(lds_map, bits, map_even, xs, code);
     store_codes(codes, base, bits, code);
 }
 
@@ -475,6 +478,7 @@ __global__ __launch_bounds__(kBThreads) void quant_group_bits_rows_kernel(const 
             s_row[t][wrow] = amax[t];
     }
     lds_barrier();
+    const bool map_even = map_is_even(lds_map);
     const int first = wrow & ~(rows_per_group - 1);
     const int64_t gp_sz = (int64_t)rows_per_group * kGroup;
 #pragma unroll
@@ -501,7 +505,7 @@ __global__ __launch_bounds__(kBThreads) void quant_group_bits_rows_kernel(const 
                 xs[k] = v[t][k] / amax[t];
         }
         uint32_t c[kBElts];
-        search_codes8(lds_map, bits, xs, c);
+        search_codes8(lds_map, bits, map_even, xs, c);
         uint32_t *cp = reinterpret_cast<uint32_t *>(codes + base) + lane16;
         store_u32(cp, bytes4(c[0], c[1], c[2], c[3]));
         store_u32(cp + 16, bytes4(c[4], c[5], c[6], c[7]));
@@ -588,6 +592,7 @@ __global__ __launch_bounds__(kBThreads) void quant_rank1_bits_rows128_kernel(con
     }
     fill_search_store(lds_map, fill, bits);
     lds_barrier();
+    const bool map_even = map_is_even(lds_map);
     if (blockIdx.x == 0 && blockIdx.y == 0) {
         // the padding added by the re-grouping to 2048: plain zeros, not divided by anything
         const uint32_t z = search_code(lds_map, bits, 0.0f);
@@ -626,7 +631,7 @@ __global__ __launch_bounds__(kBThreads) void quant_rank1_bits_rows128_kernel(con
                 xs[k] = v[k] / ((cmx[k] < rm[t]) ? cmx[k] : rm[t]);
         }
         uint32_t c[kBElts];
-        search_codes8(lds_map, bits, xs, c);
+        search_codes8(lds_map, bits, map_even, xs, c);
         uint32_t *cp = reinterpret_cast<uint32_t *>(codes + (r0 + t) * C + c0) + lane16;
         store_u32(cp, bytes4(c[0], c[1], c[2], c[3]));
         store_u32(cp + 16, bytes4(c[4], c[5], c[6], c[7]));
