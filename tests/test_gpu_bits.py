@@ -50,6 +50,30 @@ def test_pack_unpack_bits(oracle, bits):
         np.testing.assert_array_equal(to_np(back), oracle.unpack_nonlinear(want, qmap, bits, n))
 
 
+@pytest.mark.parametrize("bits", [1, 2, 3, 5, 6, 7, 8])
+def test_evenly_spaced_map_closed_form_on_a_dense_sample(oracle, bits):
+    """The evenly spaced map without zero takes a closed form instead of the search: every 251st
+    float bit pattern (negative values, infinities and NaNs included) and the 17 floats around
+    every midpoint and every entry of the map, against the oracle's search."""
+    lib = _lib()
+    qmap = oracle.create_pow_map(bits, False, 1)
+    assert np.array_equal(qmap, (np.arange(1, 2 ** bits + 1) / 2 ** bits).astype(np.float32))
+    mids = oracle.midpoints(qmap)
+    sample = np.arange(0, 2 ** 32, 251, dtype=np.uint64).astype(np.uint32)
+    near = (np.concatenate([mids, qmap]).view(np.uint32)[:, None].astype(np.int64) + np.arange(-8, 9)[None, :]).reshape(-1)
+    bitsx = np.concatenate([sample, near.astype(np.uint32)])
+    bitsx = np.concatenate([bitsx, np.zeros((-bitsx.size) % 2048, np.uint32)])
+    x = bitsx.view(np.float32)
+    want = oracle.pack_nonlinear(x, qmap, bits)
+    out = torch.full((want.size,), 0x5A, dtype=torch.uint8, device="cuda")
+    assert lib.lpmm_pack_nonlinear(to_dev(x).data_ptr(), to_dev(qmap).data_ptr(), bits, x.size, out.data_ptr(),
+                                   _stream()) == 0
+    torch.cuda.synchronize()
+    got = to_np(out)
+    bad = np.flatnonzero(got != want)
+    assert bad.size == 0, (bits, bad[:5], got[bad[:5]], want[bad[:5]])
+
+
 @pytest.mark.parametrize("bits", BITS)
 @pytest.mark.parametrize("n,gp_sz", [(4097, 128), (2048 * 5 + 3, 512), (50000, 2048), (4096 * 3 + 17, 4096), (100, 128),
                                      (2048 * 4, 128), (2048 * 3 + 128 * 5, 256), (2048 * 7 + 130, 1024)])
