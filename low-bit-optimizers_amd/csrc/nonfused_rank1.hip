@@ -31,137 +31,9 @@
 // of pass i at (i * comb + k) * pass_rows), so that at any time a group works on one contiguous
 // band of the tensor instead of on `comb` bands a tile apart.  Together 2130 -> 1990 us (first
 // pass) and 770 -> 705 us (second pass) per launch of 8.4e8 elements.
-#include "lpmm_search.hpp"
-#include "lpmm_update.hpp"
+#include "rank1_tiles.hpp"
 
 namespace lpmm {
-
-constexpr int kThreads = 256;
-constexpr int kEltsPerLane = 8;
-constexpr int kDppRows = kThreads / 16;  // 128-column groups a workgroup handles per pass
-constexpr int kR1Max = 32;               // tensors per launch
-// Tile policy: widest tile (lg of 128-column groups), tensor rows per workgroup (more where one pass
-// of a narrow tile covers more), workgroups taken to be resident together.
-#ifndef LPMM_R1_LG
-#define LPMM_R1_LG 1
-#endif
-#ifndef LPMM_R1_ROWS
-#define LPMM_R1_ROWS 64
-#endif
-#ifndef LPMM_R1_RESIDENT
-#define LPMM_R1_RESIDENT 256
-#endif
-constexpr int kPolicyLgWide = LPMM_R1_LG;
-constexpr uint32_t kPolicyRows = LPMM_R1_ROWS, kPolicyResident = LPMM_R1_RESIDENT;
-static_assert(LPMM_R1_LG >= 1 && LPMM_R1_LG <= 3, "a tile is 256 to 1024 columns wide at most");
-constexpr int kMaxLgWide = kPolicyLgWide;   // the LDS column arrays hold 128 << kMaxLgWide columns
-constexpr int kMaxWide = 1 << kMaxLgWide;
-// Per-column data of a tile lives in LDS, not in registers (occupancy): the current column
-// statistics in the unused bytes between the maps and the encode table, further arrays after
-// the table.
-constexpr uint32_t kColBytes = kMaxWide * kGroup * 4;
-constexpr uint32_t kColOld = kLdsQ1 + 64;
-static_assert(kColOld + kColBytes <= kEncLdsBegin, "column statistics overlap the encode table");
-constexpr uint32_t kColExtra = (kLdsBytes + 15) / 16 * 16;  // first byte after the table
-// Column maxima of the tile, one slot of 8 x 16 words (+16 words of skew, so that the DPP rows
-// of a wave hit different banks) per column group: word k * 16 + lane16 of a slot is element k
-// of lane lane16.
-constexpr uint32_t kRedSlotWords = kGroup + 16;
-
-// A workgroup covers tile_rows rows x (128 << lg_wide) columns: per pass, (16 >> lg_wide) rows of
-// (1 << lg_wide) adjacent groups each.
-struct TileShape {
-    uint32_t lg_wide : 8;
-    uint32_t tile_rows : 24;  // max(the policy's rows, rows of one pass)
-    uint32_t comb;            // row blocks whose passes interleave
-};
-
-struct TensorR1 {
-    float *p;
-    const float *g;
-    uint8_t *mc;  // fp32 first moment: the moment itself (float[rows * cols]), ms unused
-    float *ms;
-    float *ms_new;  // first-moment groups wider than 128 values: the scales of the new first moment
-    uint8_t *vc;
-    const float *row_old;
-    const float *col_old;
-    float *row_new;
-    float *col_new;
-    int64_t rows;
-    uint32_t col_blocks;  // columns / 128
-    float neg_step_size, bc2_sqrt, rbc2_sqrt;
-    uint32_t m_lg;  // the first moment's group holds 128 << m_lg values
-    uint32_t col_tail;  // columns in the last 128-column block (128 unless the column count is ragged)
-    TileShape tile;
-};
-
-// How the first moment is kept: 4-bit codes in groups of 128 values (re-quantised where it is
-// updated), fp32 (read and written as floats), or 4-bit codes in wider groups (256 .. 4096
-// values of the flattened tensor: a group spans several DPP rows, tiles and, where the column
-// count is not a multiple of the group size, tensor rows.  The update pass only merges the
-// groups' maxima into the next scales, the second pass recomputes the moment from g and the old
-// codes, bit-identically, and writes its codes -- what both passes do for the second moment).
-enum MomentMode { kMCodes128 = 0, kMFloat = 1, kMCodesWide = 2 };
-
-struct MultiR1 {
-    TensorR1 t[kR1Max];
-    uint32_t tile_start[kR1Max + 1];  // prefix sum of tiles per tensor; unused slots hold the total
-    int count;
-    float decay, w1, b2, w2, eps;
-};
-
-static_assert(sizeof(MultiR1) + 2 * sizeof(void *) <= 4096, "kernel arguments exceed 4 KB");
-static_assert(kR1Max <= kWave, "one tile_start entry per lane");
-
-// tensor of this workgroup (uniform): the number of later tensors whose first tile is not
-// after this one
-__device__ __forceinline__ int find_tensor(const MultiR1 &args)
-{
-    const int lane = threadIdx.x & (kWave - 1);
-    const bool started = lane + 1 < kR1Max && args.tile_start[lane + 1] <= blockIdx.x;
-    return __popcll(__ballot(started));
-}
-
-__device__ __forceinline__ void unpack8(const float4 &a, const float4 &b, float (&o)[kEltsPerLane])
-{
-    o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w;
-    o[4] = b.x; o[5] = b.y; o[6] = b.z; o[7] = b.w;
-}
-
-// Where a DPP row of this workgroup works: column group `cg` (fixed), rows row0, row0 + step, ...
-struct Geometry {
-    int64_t row0;
-    uint32_t cg, col_tile;
-    int step, passes, wide;
-};
-
-__device__ __forceinline__ Geometry geometry(const TensorR1 &t, uint32_t tile, int drow)
-{
-    Geometry q;
-    const TileShape &ts = t.tile;
-    q.wide = 1 << ts.lg_wide;
-    const uint32_t col_tiles = (t.col_blocks + q.wide - 1) >> ts.lg_wide;
-    const uint32_t rb = tile / col_tiles;
-    q.col_tile = tile - rb * col_tiles;
-    q.cg = q.col_tile * q.wide + (drow & (q.wide - 1));
-    const int pass_rows = kDppRows >> ts.lg_wide;
-    q.passes = (int)ts.tile_rows / pass_rows;
-    // block k of group grp: pass i covers the rows from (grp * passes * comb + i * comb + k) * pass_rows on
-    const uint32_t grp = rb / ts.comb, k = rb - grp * ts.comb;
-    q.row0 = (int64_t)grp * ts.tile_rows * ts.comb + (int64_t)k * pass_rows + (drow >> ts.lg_wide);
-    q.step = pass_rows * (int)ts.comb;
-    return q;
-}
-
-// Codes of a plain 0.0 into the padding [n, n_padded) of a packed array and 0 into the extra
-// last byte; one workgroup.  n and n_padded are multiples of 8, the array is 4-byte aligned.
-__device__ __forceinline__ void write_padding(uint8_t *codes, int64_t n, int64_t n_padded, uint32_t zero_word)
-{
-    for (int64_t i = n + (int64_t)threadIdx.x * kEltsPerLane; i < n_padded; i += kThreads * kEltsPerLane)
-        *reinterpret_cast<uint32_t *>(codes + (i >> 1)) = zero_word;
-    if (threadIdx.x == 0)
-        codes[n_padded / 2] = 0;
-}
 
 __global__ __launch_bounds__(kThreads) void rank1_clear_kernel(const MultiR1 args)
 {
@@ -495,489 +367,6 @@ __global__ __launch_bounds__(kThreads) void rank1_requant_kernel(const MultiR1 a
     }
 }
 
-// ---------------------------------------------------------------------------------------
-// The same two passes for code widths of 5 to 8 bits (lpmm/configs/default_{5,6,7,8}b.yml): one
-// code per byte (lpmm/cpp_extension/quantization_kernel.cu:516-533, :656-669), maps of 2^bits
-// entries in LDS, decoded by indexing and encoded by the reference's search (:397-427) as the
-// stand-alone quantisers of these widths do it.  Same tiles and statistics as above; a lane's
-// eight codes are two dwords.  21.06 bytes per parameter cross HBM (p 8, g 4 + 4, m codes 2,
-// v codes 1 + 2, scales).  LLaMA-7B-shaped set: 25.1 ms per step with 5 bits, 25.3 ms with 8
-// (the staged path 67.6 ms); the second moment's evenly spaced map takes the closed form of
-// lpmm_search.hpp, so only the first moment is searched.
-// ---------------------------------------------------------------------------------------
-__device__ __forceinline__ uint32_t byte_of(uint32_t w0, uint32_t w1, int k)
-{
-    return ((k < 4 ? w0 : w1) >> (8 * (k & 3))) & 0xFFu;
-}
-
-__device__ __forceinline__ uint32_t pack4(const uint32_t (&c)[kEltsPerLane], int h)
-{
-    return c[4 * h] | (c[4 * h + 1] << 8) | (c[4 * h + 2] << 16) | (c[4 * h + 3] << 24);
-}
-
-// Code `zero` into the padding [n, n_padded) of an array of one code per byte and 0 into the extra
-// last byte; one workgroup.  n and n_padded are multiples of 4, the array is 4-byte aligned.
-__device__ __forceinline__ void write_padding_bytes(uint8_t *codes, int64_t n, int64_t n_padded, uint32_t zero)
-{
-    for (int64_t i = n + (int64_t)threadIdx.x * 4; i < n_padded; i += kThreads * 4)
-        *reinterpret_cast<uint32_t *>(codes + i) = zero * 0x01010101u;
-    if (threadIdx.x == 0)
-        codes[n_padded] = 0;
-}
-
-__global__ __launch_bounds__(kThreads) void rank1_update_bits_kernel(const MultiR1 args, const float *__restrict__ qmap_m,
-                                                                    const float *__restrict__ qmap_v, int bits_m,
-                                                                    int bits_v)
-{
-    __shared__ float map_m[256], map_v[256];
-    __shared__ SearchLds search_m;
-    __shared__ __align__(16) float col_old[kMaxWide * kGroup];
-    __shared__ uint32_t colred[kMaxWide * kRedSlotWords];
-    const int lo = find_tensor(args);
-    const TensorR1 &t = args.t[lo];
-    const uint32_t tl = blockIdx.x - args.tile_start[lo];
-    const int lane16 = threadIdx.x & 15, drow = threadIdx.x >> 4;
-    const Geometry q = geometry(t, tl, drow);
-    const int64_t cols = (int64_t)t.col_blocks * kGroup;
-    const int64_t tile_c0 = (int64_t)q.col_tile * q.wide * kGroup;
-    fill_map(map_m, qmap_m, bits_m);
-    fill_map(map_v, qmap_v, bits_v);
-    fill_search(search_m, qmap_m, bits_m);
-    for (int j = threadIdx.x; j < kMaxWide * kGroup; j += kThreads)
-        col_old[j] = (j < q.wide * kGroup && tile_c0 + j < cols) ? t.col_old[tile_c0 + j] : 0.0f;
-    for (int j = threadIdx.x; j < kMaxWide * (int)kRedSlotWords; j += kThreads)
-        colred[j] = 0u;
-    NfHyper h;
-    h.decay = args.decay;
-    h.w1 = args.w1;
-    h.b2 = args.b2;
-    h.w2 = args.w2;
-    h.eps = args.eps;
-    h.neg_step_size = t.neg_step_size;
-    h.bc2_sqrt = t.bc2_sqrt;
-    h.rbc2_sqrt = t.rbc2_sqrt;
-    __syncthreads();
-    const bool map_even = map_is_even(search_m);
-
-    if (tl == 0) {
-        const int64_t n = t.rows * cols;
-        write_padding_bytes(t.mc, n, (n + LPMM_PACK_GROUP - 1) / LPMM_PACK_GROUP * LPMM_PACK_GROUP,
-                            search_code(search_m, bits_m, 0.0f));
-    }
-    const uint32_t mask_m = (1u << bits_m) - 1u, mask_v = (1u << bits_v) - 1u;
-    const int slot = drow & (q.wide - 1);
-    if (q.cg < t.col_blocks) {
-        const float *cop = col_old + slot * kGroup + lane16 * 4;
-        uint32_t *red = colred + slot * kRedSlotWords + lane16;
-        float co[kEltsPerLane];
-        unpack8(*reinterpret_cast<const float4 *>(cop), *reinterpret_cast<const float4 *>(cop + 64), co);
-#pragma unroll 1
-        for (int it = 0; it < q.passes; ++it) {
-            const int64_t r = q.row0 + it * q.step;
-            if (r >= t.rows)
-                break;
-            const int64_t grp = r * t.col_blocks + q.cg;
-            const int64_t gbase = grp * kGroup;
-            float *pp = t.p + gbase + lane16 * 4;
-            const float *gp = t.g + gbase + lane16 * 4;
-            uint32_t *mcp = reinterpret_cast<uint32_t *>(t.mc + gbase) + lane16;
-            const uint32_t *vcp = reinterpret_cast<const uint32_t *>(t.vc + gbase) + lane16;
-            const float4 a0 = load4(pp), a1 = load4(pp + 64), b0 = load4(gp), b1 = load4(gp + 64);
-            const uint32_t wm0 = load_u32(mcp), wm1 = load_u32(mcp + 16);
-            const uint32_t wv0 = load_u32(vcp), wv1 = load_u32(vcp + 16);
-            const float sm = t.ms[grp], ro = t.row_old[r];
-            float pv[kEltsPerLane], gv[kEltsPerLane], m[kEltsPerLane], v[kEltsPerLane];
-            unpack8(a0, a1, pv);
-            unpack8(b0, b1, gv);
-            float amax_m = 0.0f, vmax = 0.0f;
-#pragma unroll
-            for (int k = 0; k < kEltsPerLane; ++k) {
-                m[k] = map_m[byte_of(wm0, wm1, k) & mask_m] * sm;
-                v[k] = map_v[byte_of(wv0, wv1, k) & mask_v] * ((co[k] < ro) ? co[k] : ro);
-                nonfused_elt(pv[k], gv[k], m[k], v[k], h);
-                amax_m = fmaxf(amax_m, fabsf(m[k]));
-                vmax = fmaxf(vmax, v[k]);
-                atomicMax(red + k * 16, __float_as_uint(v[k]));
-            }
-            row16_max2(amax_m, vmax);
-            // |m| <= amax: with the correctly rounded reciprocal one multiply and two fmas give the
-            // correctly rounded quotient; maxima outside the reciprocal's exact range (0 included:
-            // 0/0 must give NaN) take the plain division
-            float xs[kEltsPerLane];
-            if (__all(rc_safe(amax_m))) {
-                const float rc = rcp_exact(amax_m);
-#pragma unroll
-                for (int k = 0; k < kEltsPerLane; ++k)
-                    xs[k] = div_by_rc(m[k], amax_m, rc);
-            } else {
-#pragma unroll
-                for (int k = 0; k < kEltsPerLane; ++k)
-                    xs[k] = m[k] / amax_m;
-            }
-            uint32_t c[kEltsPerLane];
-            search_codes8(search_m, bits_m, map_even, xs, c);
-            store4(pp, make_float4(pv[0], pv[1], pv[2], pv[3]));
-            store4(pp + 64, make_float4(pv[4], pv[5], pv[6], pv[7]));
-            store_u32(mcp, pack4(c, 0));
-            store_u32(mcp + 16, pack4(c, 1));
-            if (lane16 == 0) {
-                t.ms[grp] = amax_m;
-                atomic_max_nonneg(t.row_new + r, vmax);
-            }
-        }
-    }
-    __syncthreads();
-    // column j of the tile = element k of lane l of slot s
-    for (int j = threadIdx.x; j < q.wide * kGroup; j += kThreads) {
-        const int w = j & (kGroup - 1);
-        const int k = ((w >> 6) << 2) | (w & 3), l = (w >> 2) & 15;
-        if (tile_c0 + j < cols)
-            atomic_max_nonneg(t.col_new + tile_c0 + j, __uint_as_float(colred[(j >> 7) * kRedSlotWords + k * 16 + l]));
-    }
-}
-
-__global__ __launch_bounds__(kThreads) void rank1_requant_bits_kernel(const MultiR1 args, const float *__restrict__ qmap_v,
-                                                                     int bits_v)
-{
-    __shared__ float map_v[256];
-    __shared__ SearchLds search_v;
-    __shared__ __align__(16) float col_old[kMaxWide * kGroup], col_new[kMaxWide * kGroup];
-    const int lo = find_tensor(args);
-    const TensorR1 &t = args.t[lo];
-    const uint32_t tl = blockIdx.x - args.tile_start[lo];
-    const int lane16 = threadIdx.x & 15, drow = threadIdx.x >> 4;
-    const Geometry q = geometry(t, tl, drow);
-    const int64_t cols = (int64_t)t.col_blocks * kGroup;
-    const int64_t tile_c0 = (int64_t)q.col_tile * q.wide * kGroup;
-    fill_map(map_v, qmap_v, bits_v);
-    fill_search(search_v, qmap_v, bits_v);
-    for (int j = threadIdx.x; j < kMaxWide * kGroup; j += kThreads) {
-        const bool in = j < q.wide * kGroup && tile_c0 + j < cols;
-        col_old[j] = in ? t.col_old[tile_c0 + j] : 0.0f;
-        col_new[j] = in ? t.col_new[tile_c0 + j] : 0.0f;
-    }
-    NfHyper h;
-    h.b2 = args.b2;
-    h.w2 = args.w2;
-    __syncthreads();
-    const bool map_even = map_is_even(search_v);
-
-    if (tl == 0) {
-        const int64_t n = t.rows * cols;
-        write_padding_bytes(t.vc, n, (n + LPMM_PACK_GROUP - 1) / LPMM_PACK_GROUP * LPMM_PACK_GROUP,
-                            search_code(search_v, bits_v, 0.0f));
-    }
-    if (q.cg >= t.col_blocks)
-        return;
-    const uint32_t mask_v = (1u << bits_v) - 1u;
-    const int col_off = (drow & (q.wide - 1)) * kGroup + lane16 * 4;
-    float co[kEltsPerLane], cn[kEltsPerLane];
-    unpack8(*reinterpret_cast<const float4 *>(col_old + col_off), *reinterpret_cast<const float4 *>(col_old + col_off + 64), co);
-    unpack8(*reinterpret_cast<const float4 *>(col_new + col_off), *reinterpret_cast<const float4 *>(col_new + col_off + 64), cn);
-#pragma unroll 1
-    for (int it = 0; it < q.passes; ++it) {
-        const int64_t r = q.row0 + it * q.step;
-        if (r >= t.rows)
-            break;
-        const int64_t gbase = (r * t.col_blocks + q.cg) * kGroup;
-        const float *gp = t.g + gbase + lane16 * 4;
-        const float4 b0 = load4(gp), b1 = load4(gp + 64);
-        uint32_t *vcp = reinterpret_cast<uint32_t *>(t.vc + gbase) + lane16;
-        const uint32_t wv0 = load_u32(vcp), wv1 = load_u32(vcp + 16);
-        const float ro = t.row_old[r], rn = t.row_new[r];
-        float gv[kEltsPerLane], x[kEltsPerLane];
-        unpack8(b0, b1, gv);
-#pragma unroll
-        for (int k = 0; k < kEltsPerLane; ++k) {
-            float v = map_v[byte_of(wv0, wv1, k) & mask_v] * ((co[k] < ro) ? co[k] : ro);
-            nonfused_second_moment(v, gv[k], h);
-            x[k] = v / ((cn[k] < rn) ? cn[k] : rn);
-        }
-        uint32_t c[kEltsPerLane];
-        search_codes8(search_v, bits_v, map_even, x, c);
-        store_u32(vcp, pack4(c, 0));
-        store_u32(vcp + 16, pack4(c, 1));
-    }
-}
-
-// ---------------------------------------------------------------------------------------
-// The two passes for a column count that is no multiple of 128 (a multiple of 8: GPT-2-XL's
-// d = 1600, a 1000-class head).  The 128-value groups of the first moment are cut from the
-// flattened tensor (group_tensor, lpmm/functional.py:404-422), so here they straddle tensor rows
-// and the 128 columns a DPP row works on lie in up to two of them.  The first moment therefore
-// takes the route of the wide groups above: the update pass merges the maxima of the new first
-// moment into the next scales (one masked row maximum per group a DPP row touches) and the second
-// pass recomputes it and writes its codes; any group size from 128 to 4096 is served.  The last
-// 128-column block of a row is cut: its lanes beyond the row load nothing, store nothing and
-// contribute zeros to every maximum.  A lane's two runs of four values stay whole (the column
-// count is a multiple of 4), their codes are one 16-bit access each.
-// ---------------------------------------------------------------------------------------
-struct RaggedRow {
-    int64_t flat;  // index of the DPP row's first value in the flattened tensor
-    bool in0, in1;  // does the lane's first / second run of four lie inside the tensor row
-};
-
-__device__ __forceinline__ RaggedRow ragged_row(const TensorR1 &t, int64_t cols, uint32_t cg, int lane16, int64_t r)
-{
-    RaggedRow w;
-    const int64_t c0 = (int64_t)cg * kGroup;
-    w.flat = r * cols + c0;
-    w.in0 = c0 + lane16 * 4 < cols;
-    w.in1 = c0 + 64 + lane16 * 4 < cols;
-    return w;
-}
-
-__global__ __launch_bounds__(kThreads) void rank1_update_ragged_kernel(const MultiR1 args, const float *__restrict__ qmap_m,
-                                                                      const float *__restrict__ qmap_v)
-{
-    __shared__ __align__(16) uint32_t lds[(kColExtra + kMaxWide * kRedSlotWords * 4) / 4];
-    uint32_t *colred = lds + kColExtra / 4;
-    const int lo = find_tensor(args);
-    const TensorR1 &t = args.t[lo];
-    const uint32_t tl = blockIdx.x - args.tile_start[lo];
-    const int lane16 = threadIdx.x & 15, drow = threadIdx.x >> 4;
-    const Geometry q = geometry(t, tl, drow);
-    const int64_t cols = (int64_t)(t.col_blocks - 1) * kGroup + t.col_tail;
-    const int64_t tile_c0 = (int64_t)q.col_tile * q.wide * kGroup;
-    lds_fill(lds, qmap_m, qmap_v);
-    for (int j = threadIdx.x; j < kMaxWide * kGroup; j += kThreads)
-        lds[kColOld / 4 + j] = (j < q.wide * kGroup && tile_c0 + j < cols) ? __float_as_uint(t.col_old[tile_c0 + j]) : 0u;
-    for (int j = threadIdx.x; j < kMaxWide * (int)kRedSlotWords; j += kThreads)
-        colred[j] = 0u;
-    NfHyper h;
-    h.decay = args.decay;
-    h.w1 = args.w1;
-    h.b2 = args.b2;
-    h.w2 = args.w2;
-    h.eps = args.eps;
-    h.neg_step_size = t.neg_step_size;
-    h.bc2_sqrt = t.bc2_sqrt;
-    h.rbc2_sqrt = t.rbc2_sqrt;
-    __syncthreads();
-
-    const int slot = drow & (q.wide - 1);
-    const int lg_group = 7 + (int)t.m_lg;
-    if (q.cg < t.col_blocks) {
-        const uint32_t co_off = kColOld + (slot * kGroup + lane16 * 4) * 4;
-        uint32_t *red = colred + slot * kRedSlotWords + lane16;
-        float co[kEltsPerLane];
-        unpack8(lds_read<float4>(lds, co_off), lds_read<float4>(lds, co_off + 256), co);
-#pragma unroll 1
-        for (int it = 0; it < q.passes; ++it) {
-            const int64_t r = q.row0 + it * q.step;
-            if (r >= t.rows)
-                break;
-            const RaggedRow w = ragged_row(t, cols, q.cg, lane16, r);
-            const int64_t f0 = w.flat + lane16 * 4, f1 = f0 + 64;
-            const float4 zero4 = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-            const float4 a0 = w.in0 ? load4(t.p + f0) : zero4, a1 = w.in1 ? load4(t.p + f1) : zero4;
-            const float4 b0 = w.in0 ? load4(t.g + f0) : zero4, b1 = w.in1 ? load4(t.g + f1) : zero4;
-            const int64_t g0 = f0 >> lg_group, g1 = f1 >> lg_group;
-            uint32_t wm = 0, wv = 0;
-            float sm0 = 0.0f, sm1 = 0.0f;
-            if (w.in0) {
-                wm = load_u16(reinterpret_cast<const uint16_t *>(t.mc + (f0 >> 1)));
-                wv = load_u16(reinterpret_cast<const uint16_t *>(t.vc + (f0 >> 1)));
-                sm0 = t.ms[g0];
-            }
-            if (w.in1) {
-                wm |= (uint32_t)load_u16(reinterpret_cast<const uint16_t *>(t.mc + (f1 >> 1))) << 16;
-                wv |= (uint32_t)load_u16(reinterpret_cast<const uint16_t *>(t.vc + (f1 >> 1))) << 16;
-                sm1 = t.ms[g1];
-            }
-            const float ro = t.row_old[r];
-            float pv[kEltsPerLane], gv[kEltsPerLane], m[kEltsPerLane], v[kEltsPerLane];
-            unpack8(a0, a1, pv);
-            unpack8(b0, b1, gv);
-            const Nibbles nm = split_nibbles(wm), nv = split_nibbles(wv);
-            float max0 = 0.0f, max1 = 0.0f, vmax = 0.0f;
-#pragma unroll
-            for (int k = 0; k < kEltsPerLane; ++k) {
-                // outside the row: p = g = 0 and zero scales, so m = v = 0 and nothing below sees them
-                m[k] = decode_nibble(lds, kLdsQ0, nm, k) * (k < 4 ? sm0 : sm1);
-                const float sc = (co[k] < ro) ? co[k] : ro;
-                v[k] = decode_nibble(lds, kLdsQ1, nv, k) * ((k < 4 ? w.in0 : w.in1) ? sc : 0.0f);
-                nonfused_elt(pv[k], gv[k], m[k], v[k], h);
-                if (k < 4)
-                    max0 = fmaxf(max0, fabsf(m[k]));
-                else
-                    max1 = fmaxf(max1, fabsf(m[k]));
-                vmax = fmaxf(vmax, v[k]);
-                atomicMax(red + k * 16, __float_as_uint(v[k]));
-            }
-            // the DPP row's 128 values lie in the group of its first value or in the next one
-            const int64_t glo = w.flat >> lg_group;
-            float mlo = fmaxf(g0 == glo ? max0 : 0.0f, g1 == glo ? max1 : 0.0f);
-            float mhi = fmaxf(g0 == glo ? 0.0f : max0, g1 == glo ? 0.0f : max1);
-            row16_max2(mlo, mhi);
-            vmax = row16_max(vmax);
-            if (w.in0)
-                store4(t.p + f0, make_float4(pv[0], pv[1], pv[2], pv[3]));
-            if (w.in1)
-                store4(t.p + f1, make_float4(pv[4], pv[5], pv[6], pv[7]));
-            if (lane16 == 0) {
-                // a maximum of zero changes nothing (the next scales start at zero), and only then
-                // can the group lie past the end of the tensor
-                if (mlo != 0.0f)
-                    atomic_max_nonneg(t.ms_new + glo, mlo);
-                if (mhi != 0.0f)
-                    atomic_max_nonneg(t.ms_new + glo + 1, mhi);
-                atomic_max_nonneg(t.row_new + r, vmax);
-            }
-        }
-    }
-    __syncthreads();
-    // column j of the tile = element k of lane l of slot s
-    for (int j = threadIdx.x; j < q.wide * kGroup; j += kThreads) {
-        const int w = j & (kGroup - 1);
-        const int k = ((w >> 6) << 2) | (w & 3), l = (w >> 2) & 15;
-        if (tile_c0 + j < cols)
-            atomic_max_nonneg(t.col_new + tile_c0 + j, __uint_as_float(colred[(j >> 7) * kRedSlotWords + k * 16 + l]));
-    }
-}
-
-__global__ __launch_bounds__(kThreads) void rank1_requant_ragged_kernel(const MultiR1 args, const float *__restrict__ qmap_m,
-                                                                       const float *__restrict__ qmap_v)
-{
-    __shared__ __align__(16) uint32_t lds[(kColExtra + 2 * kColBytes) / 4];
-    constexpr uint32_t kColNew = kColExtra, kColRcp = kColExtra + kColBytes;
-    lds_fill(lds, qmap_m, qmap_v);
-    const int kind_m = classify_map(qmap_m), kind_v = classify_map(qmap_v);
-    const int lo = find_tensor(args);
-    const TensorR1 &t = args.t[lo];
-    const uint32_t tl = blockIdx.x - args.tile_start[lo];
-    const int lane16 = threadIdx.x & 15, drow = threadIdx.x >> 4;
-    const Geometry q = geometry(t, tl, drow);
-    const int64_t cols = (int64_t)(t.col_blocks - 1) * kGroup + t.col_tail;
-    const int64_t tile_c0 = (int64_t)q.col_tile * q.wide * kGroup;
-    for (int j = threadIdx.x; j < kMaxWide * kGroup; j += kThreads) {
-        const bool in = j < q.wide * kGroup && tile_c0 + j < cols;
-        // columns outside the tensor: statistics of 1, so that they do not keep a wave off the fast division
-        const float cn = in ? t.col_new[tile_c0 + j] : 1.0f;
-        lds[kColOld / 4 + j] = in ? __float_as_uint(t.col_old[tile_c0 + j]) : 0u;
-        lds[kColNew / 4 + j] = __float_as_uint(cn);
-        lds[kColRcp / 4 + j] = __float_as_uint(1.0f / cn);
-    }
-    NfHyper h;
-    h.b2 = args.b2;
-    h.w2 = args.w2;
-    h.w1 = args.w1;
-    __syncthreads();
-
-    const int lg_group = 7 + (int)t.m_lg;
-    if (tl == 0) {
-        // Padding.  Second moment: plain zeros from the end of the tensor to whole pack groups of 2048
-        // values.  First moment: the quantiser pads the flattened tensor with zeros to whole groups,
-        // which are divided by the last group's scale like its other values (0/0 -> NaN -> code 15
-        // when the group is all zero); the packing pads with plain zeros behind that.
-        const float z[kEltsPerLane] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
-        const int64_t n = t.rows * cols;
-        write_padding(t.vc, n, (n + LPMM_PACK_GROUP - 1) / LPMM_PACK_GROUP * LPMM_PACK_GROUP,
-                      encode8_plain(lds, kLdsQ1, kind_v, z));
-        const int64_t group = (int64_t)1 << lg_group;
-        const int64_t n_grp = (n + group - 1) / group * group;
-        const int64_t n_all = (n_grp + LPMM_PACK_GROUP - 1) / LPMM_PACK_GROUP * LPMM_PACK_GROUP;
-        const uint32_t zero_word = encode8_plain(lds, kLdsQ0, kind_m, z);
-        uint32_t last_word = zero_word;
-        if (n_grp > n) {
-            const float last = t.ms_new[(n - 1) >> lg_group];
-            const float zs[kEltsPerLane] = {0.0f / last, 0.0f / last, 0.0f / last, 0.0f / last,
-                                            0.0f / last, 0.0f / last, 0.0f / last, 0.0f / last};
-            last_word = encode8_plain(lds, kLdsQ0, kind_m, zs);
-        }
-        for (int64_t i = n + (int64_t)threadIdx.x * kEltsPerLane; i < n_all; i += kThreads * kEltsPerLane)
-            *reinterpret_cast<uint32_t *>(t.mc + (i >> 1)) = i < n_grp ? last_word : zero_word;
-        if (threadIdx.x == 0)
-            t.mc[n_all / 2] = 0;
-    }
-    if (q.cg >= t.col_blocks)
-        return;
-
-    const uint32_t col_off = ((drow & (q.wide - 1)) * kGroup + lane16 * 4) * 4;
-    float co[kEltsPerLane], cn[kEltsPerLane], rcn[kEltsPerLane];
-    unpack8(lds_read<float4>(lds, kColOld + col_off), lds_read<float4>(lds, kColOld + col_off + 256), co);
-    unpack8(lds_read<float4>(lds, kColNew + col_off), lds_read<float4>(lds, kColNew + col_off + 256), cn);
-    unpack8(lds_read<float4>(lds, kColRcp + col_off), lds_read<float4>(lds, kColRcp + col_off + 256), rcn);
-    bool cols_safe = true;
-#pragma unroll
-    for (int k = 0; k < kEltsPerLane; ++k)
-        cols_safe = cols_safe && rc_safe(cn[k]);
-#pragma unroll 1
-    for (int it = 0; it < q.passes; ++it) {
-        const int64_t r = q.row0 + it * q.step;
-        if (r >= t.rows)
-            break;
-        const RaggedRow w = ragged_row(t, cols, q.cg, lane16, r);
-        const int64_t f0 = w.flat + lane16 * 4, f1 = f0 + 64;
-        const float4 zero4 = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-        const float4 b0 = w.in0 ? load4(t.g + f0) : zero4, b1 = w.in1 ? load4(t.g + f1) : zero4;
-        uint16_t *mc0 = reinterpret_cast<uint16_t *>(t.mc + (f0 >> 1)), *mc1 = reinterpret_cast<uint16_t *>(t.mc + (f1 >> 1));
-        uint16_t *vc0 = reinterpret_cast<uint16_t *>(t.vc + (f0 >> 1)), *vc1 = reinterpret_cast<uint16_t *>(t.vc + (f1 >> 1));
-        uint32_t wm = 0, wv = 0;
-        float so0 = 0.0f, so1 = 0.0f, sn0 = 1.0f, sn1 = 1.0f;  // outside the row: 0 / 1
-        if (w.in0) {
-            wm = load_u16(mc0);
-            wv = load_u16(vc0);
-            so0 = t.ms[f0 >> lg_group];
-            sn0 = t.ms_new[f0 >> lg_group];
-        }
-        if (w.in1) {
-            wm |= (uint32_t)load_u16(mc1) << 16;
-            wv |= (uint32_t)load_u16(vc1) << 16;
-            so1 = t.ms[f1 >> lg_group];
-            sn1 = t.ms_new[f1 >> lg_group];
-        }
-        const float ro = t.row_old[r], rn = t.row_new[r];
-        float gv[kEltsPerLane], v[kEltsPerLane], m[kEltsPerLane], x[kEltsPerLane];
-        unpack8(b0, b1, gv);
-        const Nibbles nm = split_nibbles(wm), nv = split_nibbles(wv);
-#pragma unroll
-        for (int k = 0; k < kEltsPerLane; ++k) {
-            v[k] = decode_nibble(lds, kLdsQ1, nv, k) * ((co[k] < ro) ? co[k] : ro);
-            nonfused_second_moment(v[k], gv[k], h);
-            m[k] = lerp_w(decode_nibble(lds, kLdsQ0, nm, k) * (k < 4 ? so0 : so1), gv[k], h.w1);
-        }
-        // Every divisor is a maximum over the values it divides (|x| <= y): where all of a wave's
-        // divisors lie in the range in which the reciprocal is exact, the correctly rounded
-        // reciprocal, one multiply and two fmas give the correctly rounded quotient.
-        uint32_t cm, cv;
-        if (kind_m == kMapStdM && __all(rc_safe(sn0) && rc_safe(sn1))) {
-            const float rc0 = rcp_exact(sn0), rc1 = rcp_exact(sn1);
-#pragma unroll
-            for (int k = 0; k < kEltsPerLane; ++k)
-                x[k] = div_by_rc(m[k], k < 4 ? sn0 : sn1, k < 4 ? rc0 : rc1);
-            cm = encode8_std_m(lds, x);
-        } else {
-#pragma unroll
-            for (int k = 0; k < kEltsPerLane; ++k)
-                x[k] = m[k] / (k < 4 ? sn0 : sn1);
-            cm = encode8_plain(lds, kLdsQ0, kind_m, x);
-        }
-        if (kind_v == kMapStdV && __all(cols_safe && rc_safe(rn))) {
-            const float rcr = rcp_exact(rn);
-#pragma unroll
-            for (int k = 0; k < kEltsPerLane; ++k) {
-                const bool by_col = cn[k] < rn;
-                x[k] = div_by_rc(v[k], by_col ? cn[k] : rn, by_col ? rcn[k] : rcr);
-            }
-            cv = encode8_std_v(x);
-        } else {
-#pragma unroll
-            for (int k = 0; k < kEltsPerLane; ++k)
-                x[k] = v[k] / ((cn[k] < rn) ? cn[k] : rn);
-            cv = encode8_plain(lds, kLdsQ1, kind_v, x);
-        }
-        if (w.in0) {
-            store_u16(mc0, cm & 0xFFFFu);
-            store_u16(vc0, cv & 0xFFFFu);
-        }
-        if (w.in1) {
-            store_u16(mc1, cm >> 16);
-            store_u16(vc1, cv >> 16);
-        }
-    }
-}
-
 }  // namespace lpmm
 
 using namespace lpmm;
@@ -1153,15 +542,9 @@ static int rank1_step_multi(const Record *tensors, int64_t count, const float *q
         hipLaunchKernelGGL(rank1_clear_kernel, dim3((uint32_t)clear_blocks, (uint32_t)k), dim3(kThreads), 0,
                            (hipStream_t)stream, args);
         if (ragged || (MODE == kMCodesWide && m_lg == 0)) {
-            hipLaunchKernelGGL(rank1_update_ragged_kernel, dim3((uint32_t)tiles), dim3(kThreads), 0,
-                               (hipStream_t)stream, args, qmap_m, qmap_v);
-            hipLaunchKernelGGL(rank1_requant_ragged_kernel, dim3((uint32_t)tiles), dim3(kThreads), 0,
-                               (hipStream_t)stream, args, qmap_m, qmap_v);
+            launch_rank1_ragged(args, (uint32_t)tiles, qmap_m, qmap_v, (hipStream_t)stream);
         } else if (bits_m != 4) {
-            hipLaunchKernelGGL(rank1_update_bits_kernel, dim3((uint32_t)tiles), dim3(kThreads), 0, (hipStream_t)stream,
-                               args, qmap_m, qmap_v, bits_m, bits_v);
-            hipLaunchKernelGGL(rank1_requant_bits_kernel, dim3((uint32_t)tiles), dim3(kThreads), 0,
-                               (hipStream_t)stream, args, qmap_v, bits_v);
+            launch_rank1_bits(args, (uint32_t)tiles, qmap_m, qmap_v, bits_m, bits_v, (hipStream_t)stream);
         } else {
             hipLaunchKernelGGL(rank1_update_kernel<MODE>, dim3((uint32_t)tiles), dim3(kThreads), 0,
                                (hipStream_t)stream, args, qmap_m, qmap_v);

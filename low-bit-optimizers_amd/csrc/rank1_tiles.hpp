@@ -1,0 +1,142 @@
+// Shared by the two-pass rank-1 step kernels (nonfused_rank1.hip: 4-bit states, the tuned passes;
+// nonfused_rank1_bits.hip: 5-8-bit states; nonfused_rank1_ragged.hip: column counts that are no
+// multiple of 128): the tensor records of a launch, the tile geometry and small helpers.
+#pragma once
+#include "lpmm_update.hpp"
+
+namespace lpmm {
+
+constexpr int kThreads = 256;
+constexpr int kEltsPerLane = 8;
+constexpr int kDppRows = kThreads / 16;  // 128-column groups a workgroup handles per pass
+constexpr int kR1Max = 32;               // tensors per launch
+// Tile policy: widest tile (lg of 128-column groups), tensor rows per workgroup (more where one pass
+// of a narrow tile covers more), workgroups taken to be resident together.
+#ifndef LPMM_R1_LG
+#define LPMM_R1_LG 1
+#endif
+#ifndef LPMM_R1_ROWS
+#define LPMM_R1_ROWS 64
+#endif
+#ifndef LPMM_R1_RESIDENT
+#define LPMM_R1_RESIDENT 256
+#endif
+constexpr int kPolicyLgWide = LPMM_R1_LG;
+constexpr uint32_t kPolicyRows = LPMM_R1_ROWS, kPolicyResident = LPMM_R1_RESIDENT;
+static_assert(LPMM_R1_LG >= 1 && LPMM_R1_LG <= 3, "a tile is 256 to 1024 columns wide at most");
+constexpr int kMaxLgWide = kPolicyLgWide;   // the LDS column arrays hold 128 << kMaxLgWide columns
+constexpr int kMaxWide = 1 << kMaxLgWide;
+// Per-column data of a tile lives in LDS, not in registers (occupancy): the current column
+// statistics in the unused bytes between the maps and the encode table, further arrays after
+// the table.
+constexpr uint32_t kColBytes = kMaxWide * kGroup * 4;
+constexpr uint32_t kColOld = kLdsQ1 + 64;
+static_assert(kColOld + kColBytes <= kEncLdsBegin, "column statistics overlap the encode table");
+constexpr uint32_t kColExtra = (kLdsBytes + 15) / 16 * 16;  // first byte after the table
+// Column maxima of the tile, one slot of 8 x 16 words (+16 words of skew, so that the DPP rows
+// of a wave hit different banks) per column group: word k * 16 + lane16 of a slot is element k
+// of lane lane16.
+constexpr uint32_t kRedSlotWords = kGroup + 16;
+
+// A workgroup covers tile_rows rows x (128 << lg_wide) columns: per pass, (16 >> lg_wide) rows of
+// (1 << lg_wide) adjacent groups each.
+struct TileShape {
+    uint32_t lg_wide : 8;
+    uint32_t tile_rows : 24;  // max(the policy's rows, rows of one pass)
+    uint32_t comb;            // row blocks whose passes interleave
+};
+
+struct TensorR1 {
+    float *p;
+    const float *g;
+    uint8_t *mc;  // fp32 first moment: the moment itself (float[rows * cols]), ms unused
+    float *ms;
+    float *ms_new;  // first-moment groups wider than 128 values: the scales of the new first moment
+    uint8_t *vc;
+    const float *row_old;
+    const float *col_old;
+    float *row_new;
+    float *col_new;
+    int64_t rows;
+    uint32_t col_blocks;  // columns / 128
+    float neg_step_size, bc2_sqrt, rbc2_sqrt;
+    uint32_t m_lg;  // the first moment's group holds 128 << m_lg values
+    uint32_t col_tail;  // columns in the last 128-column block (128 unless the column count is ragged)
+    TileShape tile;
+};
+
+// How the first moment is kept: 4-bit codes in groups of 128 values (re-quantised where it is
+// updated), fp32 (read and written as floats), or 4-bit codes in wider groups (256 .. 4096
+// values of the flattened tensor: a group spans several DPP rows, tiles and, where the column
+// count is not a multiple of the group size, tensor rows.  The update pass only merges the
+// groups' maxima into the next scales, the second pass recomputes the moment from g and the old
+// codes, bit-identically, and writes its codes -- what both passes do for the second moment).
+enum MomentMode { kMCodes128 = 0, kMFloat = 1, kMCodesWide = 2 };
+
+struct MultiR1 {
+    TensorR1 t[kR1Max];
+    uint32_t tile_start[kR1Max + 1];  // prefix sum of tiles per tensor; unused slots hold the total
+    int count;
+    float decay, w1, b2, w2, eps;
+};
+
+static_assert(sizeof(MultiR1) + 2 * sizeof(void *) <= 4096, "kernel arguments exceed 4 KB");
+static_assert(kR1Max <= kWave, "one tile_start entry per lane");
+
+// tensor of this workgroup (uniform): the number of later tensors whose first tile is not
+// after this one
+__device__ __forceinline__ int find_tensor(const MultiR1 &args)
+{
+    const int lane = threadIdx.x & (kWave - 1);
+    const bool started = lane + 1 < kR1Max && args.tile_start[lane + 1] <= blockIdx.x;
+    return __popcll(__ballot(started));
+}
+
+__device__ __forceinline__ void unpack8(const float4 &a, const float4 &b, float (&o)[kEltsPerLane])
+{
+    o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w;
+    o[4] = b.x; o[5] = b.y; o[6] = b.z; o[7] = b.w;
+}
+
+// Where a DPP row of this workgroup works: column group `cg` (fixed), rows row0, row0 + step, ...
+struct Geometry {
+    int64_t row0;
+    uint32_t cg, col_tile;
+    int step, passes, wide;
+};
+
+__device__ __forceinline__ Geometry geometry(const TensorR1 &t, uint32_t tile, int drow)
+{
+    Geometry q;
+    const TileShape &ts = t.tile;
+    q.wide = 1 << ts.lg_wide;
+    const uint32_t col_tiles = (t.col_blocks + q.wide - 1) >> ts.lg_wide;
+    const uint32_t rb = tile / col_tiles;
+    q.col_tile = tile - rb * col_tiles;
+    q.cg = q.col_tile * q.wide + (drow & (q.wide - 1));
+    const int pass_rows = kDppRows >> ts.lg_wide;
+    q.passes = (int)ts.tile_rows / pass_rows;
+    // block k of group grp: pass i covers the rows from (grp * passes * comb + i * comb + k) * pass_rows on
+    const uint32_t grp = rb / ts.comb, k = rb - grp * ts.comb;
+    q.row0 = (int64_t)grp * ts.tile_rows * ts.comb + (int64_t)k * pass_rows + (drow >> ts.lg_wide);
+    q.step = pass_rows * (int)ts.comb;
+    return q;
+}
+
+// Codes of a plain 0.0 into the padding [n, n_padded) of a packed array and 0 into the extra
+// last byte; one workgroup.  n and n_padded are multiples of 8, the array is 4-byte aligned.
+__device__ __forceinline__ void write_padding(uint8_t *codes, int64_t n, int64_t n_padded, uint32_t zero_word)
+{
+    for (int64_t i = n + (int64_t)threadIdx.x * kEltsPerLane; i < n_padded; i += kThreads * kEltsPerLane)
+        *reinterpret_cast<uint32_t *>(codes + (i >> 1)) = zero_word;
+    if (threadIdx.x == 0)
+        codes[n_padded / 2] = 0;
+}
+
+// The launches of the other kernel families (defined next to their kernels); tiles = workgroups.
+void launch_rank1_bits(const MultiR1 &args, uint32_t tiles, const float *qmap_m, const float *qmap_v, int bits_m,
+                       int bits_v, hipStream_t stream);
+void launch_rank1_ragged(const MultiR1 &args, uint32_t tiles, const float *qmap_m, const float *qmap_v,
+                         hipStream_t stream);
+
+}  // namespace lpmm
