@@ -9,11 +9,12 @@ def check_cuda_tensor_float(t, name, *, fp32_only=True):
         raise RuntimeError(f"{name} must be a CUDA tensor!")
     if not t.is_contiguous():
         raise RuntimeError(f"{name} must be contiguous!")
-    if t.dtype not in (torch.float32, torch.float16):
-        raise RuntimeError(f"The type of {name} is not kFloat32 or kFloat16!")
+    if t.dtype not in (torch.float32, torch.float16, torch.float64):
+        raise RuntimeError(f"The type of {name} is not kFloat32, kFloat16 or kFloat64!")
     if fp32_only and t.dtype != torch.float32:
-        raise RuntimeError(f"The type of {name} is kFloat16: float32 is required here (half tensors are accepted "
-                           "where the reference can run them: adamw_single_tensor and the data of pack_nonlinear)")
+        raise RuntimeError(f"The type of {name} is {t.dtype}: float32 is required here (half tensors are accepted "
+                           "where the reference can run them: adamw_single_tensor and the data of pack_nonlinear; "
+                           "double tensors as the data of pack_nonlinear)")
 
 
 def check_cuda_tensor_dim_float(t, name, n_dim, *, fp32_only=True):

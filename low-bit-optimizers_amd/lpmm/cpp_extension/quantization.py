@@ -26,7 +26,7 @@ def _storage_bits(bits):
 
 
 def pack_nonlinear(data, qmap, bits, stochastic):
-    """data: float32 or float16 (num_groups, group_size), already normalised.  Returns int8 of
+    """data: float32, float16 or float64 (num_groups, group_size), already normalised.  Returns int8 of
     storage_bits*numel/8 + 1 bytes (lpmm/cpp_extension/quantization_kernel.cu:475-477, :549-550; storage_bits
     is `bits` for 1, 2 and 4 and 8 otherwise); the final byte,
     left uninitialised by the reference, is 0.
@@ -43,7 +43,9 @@ def pack_nonlinear(data, qmap, bits, stochastic):
     there too (qmap.data_ptr<float>())."""
     check_cuda_tensor_dim_float(data, "data", 2, fp32_only=False)
     check_cuda_tensor_dim_float(qmap, "qmap", 1)
-    if data.dtype is torch.float16:
+    if data.dtype is not torch.float32:
+        # half: exact widening; double: rounded to float, which is the kernel's `const float x = data[i]`
+        # (lpmm/cpp_extension/quantization_kernel.cu:450, dispatched for double as well, :492)
         data = data.float()
     _check_bits(bits, qmap)
     if data.size(1) % (4 * (8 // _storage_bits(bits))) != 0 or data.numel() % 8 != 0:

@@ -305,9 +305,9 @@ def vectorwise_quant(x, **kwargs):
     qmap = _select_qmap(kwargs)
     md = {"dtype": x.dtype, "stride": x.stride()}
     src = x.detach()
-    if src.dtype not in (torch.float32, torch.float16):
-        raise NotImplementedError(f"{src.dtype} states: the quantisers take float32 and float16")
-    # float16 states (half parameters on the non-fused path): the scaling runs as PyTorch device ops
+    if src.dtype not in (torch.float32, torch.float16, torch.float64):
+        raise NotImplementedError(f"{src.dtype} states: the quantisers take float32, float16 and float64")
+    # float16 and float64 states (half or double parameters on the non-fused path): the scaling runs as PyTorch device ops
     # of that type, one rounding per op, exactly the reference's chain (lpmm/functional.py:184-203);
     # the search and the packing widen each value to float, as the reference's half kernel does
     fp32 = src.dtype is torch.float32

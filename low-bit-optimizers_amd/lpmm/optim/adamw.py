@@ -273,9 +273,10 @@ class AdamW(LowBitOptimizer):
             _native.check(st, "fused fp16 AdamW step")
 
     @staticmethod
-    def _check_fp32_cuda(p, grad, why="the HIP kernels of this path compute in float32 (float16 parameters take "
-                         "the reference's own chain of PyTorch ops on the non-fused path, and the fp32-state "
-                         "operator under fused=True; the factored second moment and bfloat16 are float32 only)",
+    def _check_fp32_cuda(p, grad, why="the HIP kernels of this path compute in float32 (float16 and float64 parameters "
+                         "take the reference's own chain of PyTorch ops on the non-fused path, float16 also the "
+                         "fp32-state operator under fused=True; the factored second moment and bfloat16 are "
+                         "float32 only)",
                          strided_ok=False):
         if (p.dtype is torch.float32 and grad.dtype is torch.float32 and p.is_cuda and grad.is_cuda
                 and (strided_ok or (p.is_contiguous() and grad.is_contiguous()))):
@@ -407,7 +408,7 @@ class AdamW(LowBitOptimizer):
             if factored:
                 factored_work.append((p, grad, state, step))
                 continue
-            if p.dtype is torch.float16:
+            if p.dtype in (torch.float16, torch.float64):
                 self._half_step(group, p, grad, state, step, md_m, md_v)
                 continue
             dense, grad = self._dense_operands(p, grad, held)
@@ -527,15 +528,17 @@ class AdamW(LowBitOptimizer):
         self._write_back(held)
 
     def _half_step(self, group, p, grad, state, step, md_m, md_v):
-        """float16 parameters on the non-fused path.  The reference runs them through PyTorch's
-        float16 kernels, every op rounding to half once (lpmm/optim/adamw.py:367-369, :394-434), with
-        half states, half statistics and a scaling in half (lpmm/functional.py:184-203, :97-118).  The
-        same chain of PyTorch device ops runs here, so every rounding falls where it falls there;
-        the code search, packing and unpacking are the HIP operators."""
+        """float16 (and float64) parameters on the non-fused path.  The reference runs them through
+        PyTorch's kernels of that type, every op rounding to it once (lpmm/optim/adamw.py:367-369,
+        :394-434), with states, statistics and the scaling in that type (lpmm/functional.py:184-203,
+        :97-118); its pack kernel converts every normalised value to float before the search
+        (lpmm/cpp_extension/quantization_kernel.cu:450).  The same chain of PyTorch device ops runs
+        here, so every rounding falls where it falls there; the code search, packing and unpacking
+        are the HIP operators."""
         if not (p.is_cuda and grad.is_cuda):
             raise RuntimeError("p and g must be CUDA tensors!")
-        if grad.dtype is not torch.float16:
-            raise RuntimeError(f"The type of g is {grad.dtype}: half parameters need half gradients "
+        if grad.dtype is not p.dtype:
+            raise RuntimeError(f"The type of g is {grad.dtype}: {p.dtype} parameters need gradients of their type "
                                "(the reference's lerp_ raises for mixed types as well)")
         beta1, beta2 = group["betas"]
         lr, wd, eps = group["lr"], group["weight_decay"], group["eps"]

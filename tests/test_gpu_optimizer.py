@@ -732,3 +732,62 @@ def test_half_parameters_on_the_nonfused_path(v_scale):
         small = opt.state[params[2]]
         assert small["exp_avg"].dtype == torch.float16 and small["exp_avg_sq"].dtype == torch.float16
     assert all(torch.isfinite(p).all() for p in params)
+
+
+@pytest.mark.parametrize("v_scale", ["rank1", "group"])
+def test_double_parameters_on_the_nonfused_path(v_scale):
+    """float64 parameters with fused=False: the reference's chain of PyTorch ops in double
+    (lpmm/optim/adamw.py:394-434; its pack kernel rounds every normalised value to float before the
+    search, lpmm/cpp_extension/quantization_kernel.cu:450), here on the device with the HIP pack /
+    unpack operators, against the same chain run by PyTorch's CPU kernels with the C oracle's pack /
+    unpack.  Double arithmetic is correctly rounded on both sides; what can differ is an op that
+    one library fuses and the other does not, so values are compared to 1e-13 relative and codes
+    to a small budget, and every step starts from the device's own state."""
+    import lpmm
+    from oracle.nonfused_torch import TorchNonFusedAdamW
+
+    torch.manual_seed(6)
+    shapes = [(96, 160), (11008,), (2000,)]  # quantised 2-D, quantised 1-D, double states
+    hyper = dict(lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01)
+    host = [(torch.randn(s) * 0.02).double() for s in shapes]
+    params = [torch.nn.Parameter(h.cuda()) for h in host]
+    cfg = os.path.join(os.path.dirname(lpmm.config.__file__), "configs",
+                       "default.yml" if v_scale == "rank1" else "2nd_moment_group_128.yml")
+    opt = lpmm.optim.AdamW(params, fused=False, qconfig=cfg, **hyper)
+    ref = TorchNonFusedAdamW([h.clone() for h in host[:2]], v_scale_type=v_scale, **hyper)
+    for step in range(1, 4):
+        grads = [(torch.randn(s) * 1e-3).double() for s in shapes]
+        for p, g in zip(params, grads):
+            p.grad = g.cuda()
+        opt.step()
+        ref.step(grads[:2])
+        torch.cuda.synchronize()
+        for i in range(2):
+            st, rs = opt.state[params[i]], ref.state[i]
+            n = host[i].numel()
+            assert params[i].dtype == torch.float64 and st["exp_avg"].dtype == torch.int8
+            got_p, want_p = params[i].detach().cpu(), ref.params[i]
+            assert torch.all((got_p - want_p).abs() <= 1e-13 * want_p.abs().clamp_min(1e-6)), f"p {i} step {step}"
+            oh_m, oh_v = st["exp_avg_qstate"]["overhead"], st["exp_avg_sq_qstate"]["overhead"]
+            assert oh_m["max1"].dtype == torch.float64 and oh_m["dtype"] == torch.float64
+            gm1, wm1 = oh_m["max1"].cpu().reshape(-1), rs["m"][1].reshape(-1)
+            assert torch.all((gm1 - wm1).abs() <= 1e-14 * wm1.abs()), f"m scales {i} step {step}"
+            dm = np.mean(nibbles(to_np(st["exp_avg"]), n) != nibbles(rs["m"][0].numpy(), n))
+            dv = np.mean(nibbles(to_np(st["exp_avg_sq"]), n) != nibbles(rs["v"][0].numpy(), n))
+            assert dm < 1e-4 and dv < 1e-4, (i, step, dm, dv)
+            if v_scale == "rank1" and i == 0:
+                assert oh_v["dim"] == 2 and oh_v["max_dims"][0].dtype == torch.float64
+            # continue from the device's state
+            ref.params[i].copy_(params[i].detach().cpu())
+            rs["m"] = (st["exp_avg"].cpu().clone(), oh_m["max1"].cpu().clone())
+            if v_scale == "rank1" and i == 0:
+                rs["v"] = (st["exp_avg_sq"].cpu().clone(), [m.cpu().clone() for m in oh_v["max_dims"]])
+            else:
+                rs["v"] = (st["exp_avg_sq"].cpu().clone(), oh_v["max1"].cpu().clone())
+        small = opt.state[params[2]]
+        assert small["exp_avg"].dtype == torch.float64 and small["exp_avg_sq"].dtype == torch.float64
+    assert all(torch.isfinite(p).all() for p in params)
+    with pytest.raises(RuntimeError, match="float32 is required"):
+        bad = lpmm.optim.AdamW([torch.nn.Parameter(host[1].cuda())], fused=True, **hyper)
+        bad.param_groups[0]["params"][0].grad = host[1].cuda()
+        bad.step()
