@@ -12,7 +12,8 @@ def check_cuda_tensor_float(t, name, *, fp32_only=True):
     if t.dtype not in (torch.float32, torch.float16, torch.float64):
         raise RuntimeError(f"The type of {name} is not kFloat32, kFloat16 or kFloat64!")
     if fp32_only and t.dtype != torch.float32:
-        raise RuntimeError(f"The type of {name} is {t.dtype}: float32 is required here (half tensors are accepted "
+        kind = "kFloat16" if t.dtype is torch.float16 else "kFloat64"
+        raise RuntimeError(f"The type of {name} is {kind}: float32 is required here (half tensors are accepted "
                            "where the reference can run them: adamw_single_tensor and the data of pack_nonlinear; "
                            "double tensors as the data of pack_nonlinear)")
 

@@ -265,6 +265,13 @@ def test_shim_pack_unpack_signatures(oracle, qmaps):
         np.testing.assert_array_equal(to_np(got).view(np.uint8), want)
     with pytest.raises(RuntimeError, match="kFloat16"):
         ext.pack_nonlinear(to_dev(x), dq.half(), 4, False)  # the map must be float32 there as well
+    # double data is rounded to float before the search (the reference's kernel: `const float x = data[i]`)
+    xd = to_dev(x).double() * (1.0 + 2.0 ** -30)
+    got = ext.pack_nonlinear(xd, dq, 4, False)
+    want = oracle.pack_nonlinear_4bit(xd.float().cpu().numpy().reshape(-1), qmaps[1])
+    np.testing.assert_array_equal(to_np(got).view(np.uint8), want)
+    with pytest.raises(RuntimeError, match="kFloat64"):
+        ext.pack_nonlinear(to_dev(x), dq.double(), 4, False)
     with pytest.raises(RuntimeError):
         ext.pack_nonlinear(torch.from_numpy(x), dq, 4, False)  # CPU tensor
     with pytest.raises(RuntimeError):
