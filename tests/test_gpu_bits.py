@@ -50,14 +50,26 @@ def test_pack_unpack_bits(oracle, bits):
         np.testing.assert_array_equal(to_np(back), oracle.unpack_nonlinear(want, qmap, bits, n))
 
 
+@pytest.mark.parametrize("kind", ["even", "dynamic", "pow2_signed", "pow3_unsigned"])
 @pytest.mark.parametrize("bits", [1, 2, 3, 5, 6, 7, 8])
-def test_evenly_spaced_map_closed_form_on_a_dense_sample(oracle, bits):
-    """The evenly spaced map without zero takes a closed form instead of the search: every 251st
-    float bit pattern (negative values, infinities and NaNs included) and the 17 floats around
-    every midpoint and every entry of the map, against the oracle's search."""
+def test_code_assignment_on_a_dense_sample(oracle, bits, kind):
+    """The evenly spaced map without zero takes a closed form instead of the search, other maps
+    the descent through the map's entries: every 251st float bit pattern (negative values,
+    infinities and NaNs included) and the 17 floats around every midpoint and every entry of the
+    map, against the oracle's search."""
     lib = _lib()
-    qmap = oracle.create_pow_map(bits, False, 1)
-    assert np.array_equal(qmap, (np.arange(1, 2 ** bits + 1) / 2 ** bits).astype(np.float32))
+    if kind == "even":
+        qmap = oracle.create_pow_map(bits, False, 1)
+        assert np.array_equal(qmap, (np.arange(1, 2 ** bits + 1) / 2 ** bits).astype(np.float32))
+    elif kind == "dynamic":
+        if bits < 2:
+            pytest.skip("the dynamic-exponent map needs a sign bit and an exponent bit")
+        qmap = oracle.create_dynamic_map(True, bits - 1, bits)
+    elif kind == "pow2_signed":
+        qmap = oracle.create_pow_map(bits, True, 2)
+    else:
+        qmap = oracle.create_pow_map(bits, False, 3)
+    assert qmap.size == 2 ** bits
     mids = oracle.midpoints(qmap)
     sample = np.arange(0, 2 ** 32, 251, dtype=np.uint64).astype(np.uint32)
     near = (np.concatenate([mids, qmap]).view(np.uint32)[:, None].astype(np.int64) + np.arange(-8, 9)[None, :]).reshape(-1)
