@@ -28,18 +28,19 @@ namespace lpmm {
 constexpr int kThreads = 256;
 constexpr int kEltsPerLane = 8;
 constexpr int kTile = kThreads * kEltsPerLane;  // 2048 elements = 16 groups
+// tiles per run of xcd_run_order: 16 tiles x 8 KB of parameters = 128 KB
+constexpr int kRunLog2 = 4;
+static_assert((kTile * sizeof(float)) << kRunLog2 == kXcdRunBytes, "run length");
 
 // LDS per workgroup.  The tables need kLdsBytes; the allocation is larger on purpose: it caps
 // the workgroups resident on a CU (160 KB of LDS).  With the 7 that the registers would allow,
 // the waves that are not computing all sit in the memory queues, and the HBM system of MI355X
 // sustains less with deeper queues: streaming kernels with this kernel's access pattern and no
-// arithmetic (lpmm_stream_probe) peak at 4-5 resident workgroups per CU and lose 3 % at 8.
-// Measured optimum of the kernel itself: 4 per CU (40 KB) where every tensor of the launch is a
-// whole number of tiles (the straight-line variant; LLaMA-7B-shaped set 15.80 ms per step with 5,
-// 15.43 with 4, and only 5.05 TB/s with 3: too few waves to cover the arithmetic), 5 per CU
-// (30 KB) for the guarded variant (GPT-2-XL-shaped set 3.74 ms per step with 5, 3.81 with 4).
+// arithmetic peak at 3-5 resident workgroups per CU and lose 8 % at 8.  The kernel itself does
+// best with 5 per CU (32 KB; 4 per CU is within 0.3 %, 6 per CU loses 1 %, 3 per CU 20 %: too few
+// waves to cover the arithmetic).
 #ifndef LPMM_FUSED_LDS_KB_WHOLE
-#define LPMM_FUSED_LDS_KB_WHOLE 40
+#define LPMM_FUSED_LDS_KB_WHOLE 32
 #endif
 #ifndef LPMM_FUSED_LDS_KB_RAGGED
 #define LPMM_FUSED_LDS_KB_RAGGED 30
@@ -51,16 +52,20 @@ constexpr uint32_t fused_lds_bytes()
 }
 static_assert(fused_lds_bytes<true>() >= kLdsBytes && fused_lds_bytes<false>() >= kLdsBytes, "tables do not fit");
 static_assert(kThreads == kEncEntries, "lds_fill_load / lds_fill_store: one encode-table entry per thread");
-// Waves of the straight-line variant of the fused arithmetic pause this many units of 64 cycles before their first load.
-// The memory system has an optimum number of requests in flight that lies between what 4 and 5
-// resident workgroups per CU keep there; the pause trims the 4.  Measured on the LLaMA-7B-shaped
-// launches: 0 -> 6.36 TB/s, 4 -> 6.40, 6 -> 6.41, 8 -> 6.41, 10 -> 6.37, 20 -> 6.13; pauses that differ
-// between neighbouring workgroups lose 3-5 % (tiles next to each other should be in flight together).
+// Optional pause (units of 64 cycles) of every wave of the straight-line variant before its first load.
+// It paid 0.8 % while consecutive tiles went to different XCDs (6 units); with the tile order below it
+// gains nothing and is off.
 #ifndef LPMM_FUSED_START_DELAY
-#define LPMM_FUSED_START_DELAY 6
+#define LPMM_FUSED_START_DELAY 0
 #endif
 constexpr int kStartDelay = LPMM_FUSED_START_DELAY;
 
+// The parameter update of the 4-bit step uses adamw_param_folded (lpmm_update.hpp); building with
+// -DLPMM_FUSED_EXACT_P=1 keeps the reference's operation order with correctly rounded sqrt and divisions
+// (bit-identical parameters, 13 more vector instructions per element).
+#ifndef LPMM_FUSED_EXACT_P
+#define LPMM_FUSED_EXACT_P 0
+#endif
 
 struct Tensor4 {
     float *p;
@@ -70,10 +75,7 @@ struct Tensor4 {
     float *ms;
     float *vs;
     int64_t n;
-    float c1;    // 1 - beta1^step
-    float c2s;   // sqrt(1 - beta2^step)
-    float rc2s;  // 1 / c2s, correctly rounded (host division)
-    float pad;
+    float k[4];  // per-tensor scalars; which ones, the arithmetic says (FusedArith4, FusedArith, NonFusedArith)
 };
 
 constexpr int kStartSlots = LPMM_MULTI_MAX + 8;   // tile_start is read 8 entries at a time
@@ -88,8 +90,8 @@ struct Multi4 {
 };
 static_assert(LPMM_MULTI_MAX % 8 == 0, "coarse table");
 
-// The two arithmetics the kernel is instantiated with.  Both read the shared scalars from
-// Multi4::s and three per-tensor ones from Tensor4::{c1, c2s, rc2s}.
+// The arithmetics the kernels are instantiated with.  They read the shared scalars from
+// Multi4::s / MultiF::s and the per-tensor ones from Tensor4::k / TensorF::k.
 struct FusedArith {
     // code buffers hold exactly ceil(n/2) bytes; a last odd element leaves its high nibble 0
     static constexpr bool kPadded = false;
@@ -104,12 +106,56 @@ struct FusedArith {
         h.lr = a.s[4];
         h.wd = a.s[5];
         h.eps = a.s[6];
-        h.c1 = t.c1;
-        h.c2s = t.c2s;
-        h.rc2s = t.rc2s;
+        h.c1 = t.k[0];   // 1 - beta1^step
+        h.c2s = t.k[1];  // sqrt(1 - beta2^step)
+        h.rc2s = t.k[2]; // 1 / c2s, correctly rounded (host division)
     }
     __device__ __forceinline__ void elt(float &p, float g, float &m, float &v) const { p = adamw_elt(p, g, m, v, h); }
+    // per-tensor scalars of a tensor at step `step`, as the reference computes them per thread
+    static void per_tensor(float beta1, float beta2, float eps, float step, float (&k)[4])
+    {
+        bias_corrections(beta1, beta2, step, &k[0], &k[1]);
+        k[2] = 1.0f / k[1];
+        k[3] = 0.0f;
+    }
 };
+
+// The 4-bit step: the moments as FusedArith computes them, the parameter with the folded update.
+struct FusedArith4 {
+    static constexpr bool kPadded = false;
+    Hyper h;
+    float fa, fb;
+    template <class M, class T>
+    __device__ __forceinline__ FusedArith4(const M &a, const T &t)
+    {
+        h.beta1 = a.s[0];
+        h.beta2 = a.s[1];
+        h.omb1 = a.s[2];
+        h.omb2 = a.s[3];
+        h.lr = a.s[4];
+        h.wd = a.s[5];
+        fa = t.k[0];  // c1 / c2s
+        fb = t.k[1];  // eps * c1
+    }
+    __device__ __forceinline__ void elt(float &p, float g, float &m, float &v) const
+    {
+        adamw_moments(g, m, v, h);
+        p = adamw_param_folded(p, m, v, h.lr, h.wd, fa, fb);
+    }
+    static void per_tensor(float beta1, float beta2, float eps, float step, float (&k)[4])
+    {
+        float c1, c2s;
+        bias_corrections(beta1, beta2, step, &c1, &c2s);
+        k[0] = (float)((double)c1 / (double)c2s);
+        k[1] = (float)((double)eps * (double)c1);
+        k[2] = k[3] = 0.0f;
+    }
+};
+#if LPMM_FUSED_EXACT_P
+using FusedStep4 = FusedArith;
+#else
+using FusedStep4 = FusedArith4;
+#endif
 
 struct NonFusedArith {
     // code buffers are padded to whole tiles plus one byte, as the reference's packing
@@ -125,9 +171,9 @@ struct NonFusedArith {
         h.b2 = a.s[2];
         h.w2 = a.s[3];
         h.eps = a.s[4];
-        h.neg_step_size = t.c1;
-        h.bc2_sqrt = t.c2s;
-        h.rbc2_sqrt = t.rc2s;
+        h.neg_step_size = t.k[0];
+        h.bc2_sqrt = t.k[1];
+        h.rbc2_sqrt = t.k[2];
     }
     __device__ __forceinline__ void elt(float &p, float g, float &m, float &v) const { nonfused_elt(p, g, m, v, h); }
 };
@@ -328,7 +374,10 @@ __global__ __launch_bounds__(kThreads) void adamw4bit_kernel(const Multi4 args,
         lo += (args.tile_start[base + i] - 1u - bid) >> 31;
     const Tensor4 &t = args.t[lo];
     const int lane16 = threadIdx.x & 15;
-    const uint32_t tile_in_tensor = bid - args.tile_start[lo];
+    // which tile of the tensor: launch order rearranged so that an XCD streams 128 KB runs of the parameters
+    const uint32_t tiles_in_tensor = args.tile_start[lo + 1] - args.tile_start[lo];
+    const uint32_t tile_in_tensor = xcd_run_order<kRunLog2>(bid - args.tile_start[lo], tiles_in_tensor,
+                                                            run_phase<kRunLog2>(t.p, kTile * sizeof(float)));
     const int64_t grp = (int64_t)tile_in_tensor * (kTile / kGroup) + (threadIdx.x >> 4);
     const TileView view = tile_view(t, tile_in_tensor);
 
@@ -348,9 +397,9 @@ __global__ __launch_bounds__(kThreads) void adamw4bit_kernel(const Multi4 args,
     // the loaded words stay as they are until here, so that nothing above waits for them
     asm volatile("" : "+v"(regs.m0), "+v"(regs.m1), "+v"(regs.v0), "+v"(regs.v1));
 
-    if (Arith::kPadded && threadIdx.x == 0 && blockIdx.x + 1 == args.tile_start[lo + 1]) {
+    if (Arith::kPadded && threadIdx.x == 0 && tile_in_tensor + 1 == tiles_in_tensor) {
         // the tensor's last tile also owns the extra byte at the end of each code buffer
-        const int64_t end = (int64_t)(args.tile_start[lo + 1] - args.tile_start[lo]) * (kTile / 2);
+        const int64_t end = (int64_t)tiles_in_tensor * (kTile / 2);
         t.mc[end] = 0;
         t.vc[end] = 0;
     }
@@ -382,8 +431,7 @@ struct TensorF {
     float *m;
     float *v;
     int64_t n;
-    float c1, c2s, rc2s;  // per-tensor scalars, as in Tensor4
-    float pad;
+    float k[4];  // per-tensor scalars, as in Tensor4
 };
 
 constexpr int kMultiFMax = 64;
@@ -469,7 +517,7 @@ __global__ __launch_bounds__(kThreads) void adamw_fp16_kernel(const MultiF args)
 using namespace lpmm;
 
 // Validation, batching into launches of at most LPMM_MULTI_MAX tensors, and launch, shared
-// by the two arithmetics.  per_tensor(step, &c1, &c2s, &rc2s) fills the per-tensor scalars.
+// by the arithmetics.  per_tensor(step, k) fills the per-tensor scalars.
 template <class Arith, class PerTensor>
 static int step_multi4(const lpmm_adamw4bit_tensor *tensors, int64_t count, const float *qmap_m,
                        const float *qmap_v, const float (&scalars)[7], PerTensor per_tensor, void *stream)
@@ -533,8 +581,7 @@ static int step_multi4(const lpmm_adamw4bit_tensor *tensors, int64_t count, cons
             d.ms = t.m_scale;
             d.vs = t.v_scale;
             d.n = t.n;
-            per_tensor(t.step, &d.c1, &d.c2s, &d.rc2s);
-            d.pad = 0.0f;
+            per_tensor(t.step, d.k);
             tiles += nt;
             args.tile_start[++k] = (uint32_t)tiles;
             ++i;
@@ -570,11 +617,8 @@ extern "C" int lpmm_adamw4bit_step_multi(const lpmm_adamw4bit_tensor *tensors, i
 {
     // 1 - beta is formed in float, as the reference kernel does
     const float scalars[7] = {beta1, beta2, 1 - beta1, 1 - beta2, lr, weight_decay, eps};
-    return step_multi4<FusedArith>(tensors, count, qmap_m, qmap_v, scalars,
-                                   [=](float step, float *c1, float *c2s, float *rc2s) {
-                                       bias_corrections(beta1, beta2, step, c1, c2s);
-                                       *rc2s = 1.0f / *c2s;
-                                   },
+    return step_multi4<FusedStep4>(tensors, count, qmap_m, qmap_v, scalars,
+                                   [=](float step, float (&k)[4]) { FusedStep4::per_tensor(beta1, beta2, eps, step, k); },
                                    stream);
 }
 
@@ -586,11 +630,12 @@ extern "C" int lpmm_nonfused_adamw4bit_step_multi(const lpmm_adamw4bit_tensor *t
     const NfHyper c = make_nf_hyper(beta1, beta2, lr, weight_decay, eps, 1.0);
     const float scalars[7] = {c.decay, c.w1, c.b2, c.w2, c.eps, 0.0f, 0.0f};
     return step_multi4<NonFusedArith>(tensors, count, qmap_m, qmap_v, scalars,
-                                      [=](float step, float *nss, float *bc2s, float *rbc2s) {
+                                      [=](float step, float (&k)[4]) {
                                           const NfHyper h = make_nf_hyper(beta1, beta2, lr, weight_decay, eps, step);
-                                          *nss = h.neg_step_size;
-                                          *bc2s = h.bc2_sqrt;
-                                          *rbc2s = h.rbc2_sqrt;
+                                          k[0] = h.neg_step_size;
+                                          k[1] = h.bc2_sqrt;
+                                          k[2] = h.rbc2_sqrt;
+                                          k[3] = 0.0f;
                                       },
                                       stream);
 }
@@ -661,8 +706,7 @@ static int step_multi_fp32(const lpmm_adamw_fp32_tensor *tensors, int64_t count,
             d.m = t.m;
             d.v = t.v;
             d.n = t.n;
-            per_tensor(t.step, &d.c1, &d.c2s, &d.rc2s);
-            d.pad = 0.0f;
+            per_tensor(t.step, d.k);
             tiles += nt;
             args.tile_start[++k] = (uint32_t)tiles;
             ++i;
@@ -690,10 +734,7 @@ extern "C" int lpmm_adamw_fp32_step_multi(const lpmm_adamw_fp32_tensor *tensors,
 {
     const float scalars[7] = {beta1, beta2, 1 - beta1, 1 - beta2, lr, weight_decay, eps};
     return step_multi_fp32<FusedArith>(tensors, count, scalars,
-                                       [=](float step, float *c1, float *c2s, float *rc2s) {
-                                           bias_corrections(beta1, beta2, step, c1, c2s);
-                                           *rc2s = 1.0f / *c2s;
-                                       },
+                                       [=](float step, float (&k)[4]) { FusedArith::per_tensor(beta1, beta2, eps, step, k); },
                                        stream);
 }
 
@@ -702,10 +743,7 @@ extern "C" int lpmm_adamw_fp16_step_multi(const lpmm_adamw_fp32_tensor *tensors,
 {
     const float scalars[7] = {beta1, beta2, 1 - beta1, 1 - beta2, lr, weight_decay, eps};
     return step_multi_fp32<FusedArith, true>(tensors, count, scalars,
-                                             [=](float step, float *c1, float *c2s, float *rc2s) {
-                                                 bias_corrections(beta1, beta2, step, c1, c2s);
-                                                 *rc2s = 1.0f / *c2s;
-                                             },
+                                             [=](float step, float (&k)[4]) { FusedArith::per_tensor(beta1, beta2, eps, step, k); },
                                              stream);
 }
 
@@ -716,11 +754,12 @@ extern "C" int lpmm_nonfused_update_multi(const lpmm_adamw_fp32_tensor *tensors,
     const NfHyper c = make_nf_hyper(beta1, beta2, lr, weight_decay, eps, 1.0);
     const float scalars[7] = {c.decay, c.w1, c.b2, c.w2, c.eps, 0.0f, 0.0f};
     return step_multi_fp32<NonFusedArith>(tensors, count, scalars,
-                                          [=](float step, float *nss, float *bc2s, float *rbc2s) {
+                                          [=](float step, float (&k)[4]) {
                                               const NfHyper h = make_nf_hyper(beta1, beta2, lr, weight_decay, eps, step);
-                                              *nss = h.neg_step_size;
-                                              *bc2s = h.bc2_sqrt;
-                                              *rbc2s = h.rbc2_sqrt;
+                                              k[0] = h.neg_step_size;
+                                              k[1] = h.bc2_sqrt;
+                                              k[2] = h.rbc2_sqrt;
+                                              k[3] = 0.0f;
                                           },
                                           stream);
 }

@@ -34,6 +34,40 @@ inline int launch_status()
 }
 
 // ---------------------------------------------------------------------------------------
+// Tile order of the one-shot streaming kernels.  The hardware hands consecutive workgroup indices to
+// the 8 XCDs of an MI355X in turn, so with "workgroup i takes tile i" every XCD touches every
+// neighbouring tile of every operand.  The memory system gives 3-5 % more to a streaming kernel when
+// each XCD instead works through runs of 128 KB of address space whose position within the enclosing
+// 1 MB block is the same for all of its runs (measured on copies, in-place updates and the seven streams of the
+// fused step; 96, 160 or 256 KB runs, or 128 KB runs that start 64 KB off a 128 KB boundary, lose the
+// gain again; which XCD takes which of the eight positions does not matter).  xcd_run_order maps the index a
+// workgroup has within its tensor to the tile it works on: within every whole, 1 MB-aligned block of
+// tiles the 8 << LOG2 consecutive indices go to the 8 runs in turn, so the 8 XCDs advance through their
+// runs side by side and the tiles in flight still form one compact window.  Blocks cut by either end of
+// the tensor keep the plain order.  `phase` is the position of the tensor's first tile within its 1 MB
+// block of address space, in tiles (run_phase).
+// ---------------------------------------------------------------------------------------
+constexpr uint32_t kXcds = 8;
+constexpr uint32_t kXcdRunBytes = 128 * 1024;
+
+template <int LOG2>
+__device__ __forceinline__ uint32_t xcd_run_order(uint32_t index, uint32_t tiles, uint32_t phase)
+{
+    constexpr uint32_t kBlock = kXcds << LOG2, kMask = kBlock - 1u;
+    const uint32_t v = index + phase, block0 = v & ~kMask;
+    if (block0 < phase || block0 + kBlock > phase + tiles)
+        return index;
+    return (block0 | ((v & (kXcds - 1u)) << LOG2) | ((v >> 3) & ((1u << LOG2) - 1u))) - phase;
+}
+
+// tile_bytes: bytes of the dominant operand per tile (a power of two); 8 << LOG2 tiles make 1 MB
+template <int LOG2>
+__device__ __forceinline__ uint32_t run_phase(const void *base, uint32_t tile_bytes)
+{
+    return (uint32_t)(reinterpret_cast<uintptr_t>(base) / tile_bytes) & ((kXcds << LOG2) - 1u);
+}
+
+// ---------------------------------------------------------------------------------------
 // DPP lane exchange inside a 16-lane row.  The four steps quad xor 1, quad xor 2,
 // half-row mirror and row mirror leave the row-wide result in every lane.
 // ---------------------------------------------------------------------------------------

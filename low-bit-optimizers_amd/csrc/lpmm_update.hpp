@@ -19,11 +19,16 @@ struct Hyper {
 #define LPMM_P_MODE 1  // 0: IEEE sqrt/div, 1: approximation + residual correction, 2: approximation only
 #endif
 
-// AdamW on one element; returns the new parameter, updates m and v in place.
-__device__ __forceinline__ float adamw_elt(float p, float g, float &m, float &v, const Hyper &h)
+// The two moments of one element, operation by operation as the reference writes them.
+__device__ __forceinline__ void adamw_moments(float g, float &m, float &v, const Hyper &h)
 {
     m = h.beta1 * m + h.omb1 * g;
     v = h.beta2 * v + h.omb2 * g * g;
+}
+
+// The parameter of one element from the updated moments, in the reference's operation order.
+__device__ __forceinline__ float adamw_param(float p, float m, float v, const Hyper &h)
+{
 #if LPMM_P_MODE == 0
     const float denom = (sqrtf(v) / h.c2s + h.eps) * h.c1;
     const float update = (m / denom) + (h.wd * p);
@@ -35,6 +40,26 @@ __device__ __forceinline__ float adamw_elt(float p, float g, float &m, float &v,
     const float update = m * __builtin_amdgcn_rcpf(denom) + (h.wd * p);
 #endif
     return p - (h.lr * update);
+}
+
+// AdamW on one element; returns the new parameter, updates m and v in place.
+__device__ __forceinline__ float adamw_elt(float p, float g, float &m, float &v, const Hyper &h)
+{
+    adamw_moments(g, m, v, h);
+    return adamw_param(p, m, v, h);
+}
+
+// The same parameter update with the per-tensor constants folded on the host,
+//     denom = sqrt(v) * (c1 / c2s) + eps * c1,   p - lr * (m / denom + wd * p)  as two fmas,
+// and the hardware's square root and reciprocal (1 ulp each) without correction steps: 6 instructions
+// instead of 19.  The result differs from adamw_param's by the rounding of at most four operations of
+// the update term: |difference| <= 4e-7 * lr * |m / denom| + 1 ulp of p, far inside the 1e-6 relative
+// bound on updated parameters.  The moments, and with them every code and scale, do not depend on it.
+__device__ __forceinline__ float adamw_param_folded(float p, float m, float v, float lr, float wd, float fa, float fb)
+{
+    const float denom = __builtin_fmaf(__builtin_amdgcn_sqrtf(v), fa, fb);
+    const float update = __builtin_fmaf(wd, p, m * __builtin_amdgcn_rcpf(denom));
+    return __builtin_fmaf(-lr, update, p);
 }
 
 // bias corrections exactly as the reference computes them per thread

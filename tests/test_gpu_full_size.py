@@ -7,7 +7,7 @@ import numpy as np
 import pytest
 import torch
 
-from util import assert_codes, assert_rel, nibbles, to_dev, to_np
+from util import assert_codes, assert_params, assert_rel, nibbles, to_dev, to_np
 
 pytestmark = pytest.mark.gpu
 
@@ -46,9 +46,10 @@ def test_fused_step_llama_shapes(oracle, qmaps, shape):
         flips += assert_codes(to_np(vc), vc_ref, n, f"v codes step {step}")
         assert_rel(to_np(ms), ms_ref, "m scales")
         assert_rel(to_np(vs), vs_ref, "v scales")
-        assert_rel(to_np(p), p_ref, "p", scale=p_before)
+        assert_params(to_np(p), p_ref, p_before, f"p step {step}")
+        p.copy_(torch.from_numpy(p_ref))
         if flips:
-            for d, h in ((mc, mc_ref), (vc, vc_ref), (ms, ms_ref), (vs, vs_ref), (p, p_ref)):
+            for d, h in ((mc, mc_ref), (vc, vc_ref), (ms, ms_ref), (vs, vs_ref)):
                 d.copy_(torch.from_numpy(h))
     # property: the group maximum decodes to the scale (code 15 on the v map)
     cv = nibbles(to_np(vc), n).reshape(-1, 128)

@@ -4,7 +4,7 @@ import numpy as np
 import pytest
 import torch
 
-from util import assert_codes, assert_rel, to_dev, to_np
+from util import assert_codes, assert_params, assert_rel, to_dev, to_np
 
 pytestmark = pytest.mark.gpu
 
@@ -46,6 +46,7 @@ def _run_fused_steps(oracle, qmaps, n, steps, seed, grad_fn=None, p_scale=0.02, 
                                      HYPER["beta2"], HYPER["lr"], HYPER["wd"], HYPER["eps"], float(s),
                                      torch.cuda.current_stream().cuda_stream)
         assert st == 0, lib.lpmm_status_string(st)
+        p_before = p_ref.copy()
         oracle.adamw4bit_step(p_ref, g_np, mc_ref, vc_ref, ms_ref, vs_ref, qm, qv, HYPER["beta1"], HYPER["beta2"],
                               HYPER["lr"], HYPER["wd"], HYPER["eps"], float(s))
         torch.cuda.synchronize()
@@ -53,7 +54,9 @@ def _run_fused_steps(oracle, qmaps, n, steps, seed, grad_fn=None, p_scale=0.02, 
         flips += assert_codes(to_np(vc), vc_ref, n, f"v codes step {s}")
         assert_rel(to_np(ms), ms_ref, f"m scale step {s}")
         assert_rel(to_np(vs), vs_ref, f"v scale step {s}")
-        assert_rel(to_np(p), p_ref, f"p step {s}")
+        assert_params(to_np(p), p_ref, p_before, f"p step {s}")
+        # every step starts from identical inputs: the oracle's parameters go back to the GPU
+        p.copy_(torch.from_numpy(p_ref))
         if flips:
             # after a tie flip the two runs legitimately diverge: resynchronise the GPU state
             mc.copy_(torch.from_numpy(mc_ref)); vc.copy_(torch.from_numpy(vc_ref))
@@ -185,13 +188,14 @@ def test_multi_tensor_matches_single(oracle, qmaps):
     assert st == 0
     torch.cuda.synchronize()
     for h, d, n in zip(host, devs, sizes):
+        p_before = h["p"].copy()
         oracle.adamw4bit_step(h["p"], h["g"], h["mc"], h["vc"], h["ms"], h["vs"], qm, qv, 0.9, 0.999, 1e-3, 0.01,
                               1e-8, h["step"])
         assert_codes(to_np(d["mc"]), h["mc"], n, "m codes")
         assert_codes(to_np(d["vc"]), h["vc"], n, "v codes")
         assert_rel(to_np(d["ms"]), h["ms"], "m scale")
         assert_rel(to_np(d["vs"]), h["vs"], "v scale")
-        assert_rel(to_np(d["p"]), h["p"], "p")
+        assert_params(to_np(d["p"]), h["p"], p_before, "p")
 
 
 def test_multi_tensor_whole_tiles(oracle, qmaps):
@@ -221,13 +225,58 @@ def test_multi_tensor_whole_tiles(oracle, qmaps):
     assert st == 0
     torch.cuda.synchronize()
     for i, (h, d, n) in enumerate(zip(host, devs, sizes)):
+        p_before = h["p"].copy()
         oracle.adamw4bit_step(h["p"], h["g"], h["mc"], h["vc"], h["ms"], h["vs"], qm, qv, 0.9, 0.999, 1e-3, 0.01,
                               1e-8, h["step"])
         assert_codes(to_np(d["mc"]), h["mc"], n, f"m codes of tensor {i}")
         assert_codes(to_np(d["vc"]), h["vc"], n, f"v codes of tensor {i}")
         assert_rel(to_np(d["ms"]), h["ms"], f"m scale of tensor {i}")
         assert_rel(to_np(d["vs"]), h["vs"], f"v scale of tensor {i}")
-        assert_rel(to_np(d["p"]), h["p"], f"p of tensor {i}")
+        assert_params(to_np(d["p"]), h["p"], p_before, f"p of tensor {i}")
+
+
+def test_tile_order_with_offset_bases(oracle, qmaps):
+    """The kernel hands the tiles of a tensor to the workgroups in runs of 16 inside 1 MB-aligned blocks
+    of the parameter's address range.  Tensors of 300-700 tiles whose parameters start 0, 5, 77 and 130
+    tiles (and 1028 elements) past a 1 MB boundary, whole-tile and ragged, in one launch: every tile is
+    processed exactly once, whatever block it falls into."""
+    nat = _native()
+    lib = nat.lib()
+    qm, qv = qmaps
+    dqm, dqv = to_dev(qm), to_dev(qv)
+    rng = np.random.default_rng(123)
+    arena = torch.empty((1 << 20) // 4 + 2048 * 3200, dtype=torch.float32, device="cuda")
+    skip = (-arena.data_ptr() % (1 << 20)) // 4  # elements to the next 1 MB boundary
+    offsets = [0, 2048 * 5, 2048 * 77, 2048 * 130, 2048 * 7 + 1028]
+    sizes = [2048 * 400, 2048 * 300 + 700, 2048 * 512, 2048 * 700, 2048 * 333 + 64]
+    host, devs, recs, cursor = [], [], [], skip
+    for off, n in zip(offsets, sizes):
+        start = cursor + off
+        cursor = (start + n + (1 << 18) - 1) // (1 << 18) * (1 << 18) + skip % (1 << 18)  # next 1 MB boundary
+        h = dict(p=(rng.standard_normal(n) * 0.02).astype(np.float32), g=(rng.standard_normal(n) * 1e-3).astype(np.float32),
+                 mc=rng.integers(0, 256, (n + 1) // 2, dtype=np.uint8), vc=rng.integers(0, 256, (n + 1) // 2, dtype=np.uint8),
+                 ms=np.abs(rng.standard_normal((n + 127) // 128) * 1e-3).astype(np.float32),
+                 vs=np.abs(rng.standard_normal((n + 127) // 128) * 1e-6).astype(np.float32))
+        d = {k: to_dev(v) for k, v in h.items() if k != "p"}
+        d["p"] = arena[start:start + n]
+        d["p"].copy_(torch.from_numpy(h["p"]))
+        assert (d["p"].data_ptr() % (1 << 20)) // 8192 == (off // 2048) % 128
+        host.append(h); devs.append(d)
+        recs.append((d["p"].data_ptr(), d["g"].data_ptr(), d["mc"].data_ptr(), d["vc"].data_ptr(),
+                     d["ms"].data_ptr(), d["vs"].data_ptr(), n, 3.0, 0.0))
+    table = np.array(recs, dtype=nat.ADAMW4BIT_TENSOR)
+    st = lib.lpmm_adamw4bit_step_multi(table.ctypes.data, len(recs), dqm.data_ptr(), dqv.data_ptr(), 0.9, 0.999,
+                                       1e-3, 0.01, 1e-8, torch.cuda.current_stream().cuda_stream)
+    assert st == 0
+    torch.cuda.synchronize()
+    for i, (h, d, n) in enumerate(zip(host, devs, sizes)):
+        p_before = h["p"].copy()
+        oracle.adamw4bit_step(h["p"], h["g"], h["mc"], h["vc"], h["ms"], h["vs"], qm, qv, 0.9, 0.999, 1e-3, 0.01, 1e-8, 3.0)
+        assert assert_codes(to_np(d["mc"]), h["mc"], n, f"m codes of tensor {i}") == 0
+        assert assert_codes(to_np(d["vc"]), h["vc"], n, f"v codes of tensor {i}") == 0
+        np.testing.assert_array_equal(to_np(d["ms"]), h["ms"])
+        np.testing.assert_array_equal(to_np(d["vs"]), h["vs"])
+        assert_params(to_np(d["p"]), h["p"], p_before, f"p of tensor {i}")
 
 
 def test_fused_step_extreme_scales(oracle, qmaps):

@@ -7,7 +7,7 @@ import numpy as np
 import pytest
 import torch
 
-from util import assert_codes, assert_rel, nibbles, to_dev, to_np
+from util import assert_codes, assert_params, assert_rel, nibbles, to_dev, to_np
 
 pytestmark = pytest.mark.gpu
 
@@ -42,11 +42,15 @@ def test_fused_optimizer_matches_oracle_and_layout(oracle, qmaps):
         for p, g in zip(params, grads):
             p.grad = to_dev(g)
         opt.step()
-        for h, g, r in zip(host, grads, ref):
+        for p, h, g, r in zip(params, host, grads, ref):
+            before = h.copy()
             if "mc" in r:
                 oracle.adamw4bit_step(h.reshape(-1), g.reshape(-1), r["mc"], r["vc"], r["ms"], r["vs"], qm, qv, *HO, float(step))
             else:
                 oracle.adamw_fp32_step(h.reshape(-1), g.reshape(-1), r["m"], r["v"], *HO, float(step))
+            # one step from identical inputs; the next one starts from the oracle's parameters
+            assert_params(to_np(p), h, before, f"p step {step}")
+            p.data.copy_(to_dev(h))
     torch.cuda.synchronize()
     for p, h, r in zip(params, host, ref):
         st = opt.state[p]
@@ -296,7 +300,10 @@ def test_factored_optimizer_matches_oracle(oracle, qmaps, fused):
         mean_all = oracle.factored_ema(row2, col2, rm, cm, 0.999)
         oracle.factored_update(host[2], grads[2], m2, row2, col2, mean_all, 0.9, 0.999, H["lr"], H["weight_decay"], H["eps"], float(step))
         if fused:
+            before = host[3].copy()
             oracle.adamw4bit_step(host[3], grads[3], fz["mc"], fz["vc"], fz["ms"], fz["vs"], qm, qv, *HO, float(step))
+            assert_params(to_np(params[3]), host[3], before, f"p 1-D step {step}")
+            params[3].data.copy_(to_dev(host[3]))
         else:
             oracle.nonfused_step(host[3], grads[3], st1d, qm, qv, H["lr"], 0.9, 0.999, H["eps"], H["weight_decay"])
     torch.cuda.synchronize()
@@ -599,8 +606,11 @@ def test_param_groups_missing_grads_and_closure(oracle, qmaps, fused):
             steps_done[i] += 1
             b1, b2, lr, wd, eps = hyper[i]
             if fused:
+                before = h.copy()
                 oracle.adamw4bit_step(h.reshape(-1), g.reshape(-1), r["mc"], r["vc"], r["ms"], r["vs"], qm, qv,
                                       b1, b2, lr, wd, eps, float(steps_done[i]))
+                assert_params(to_np(params[i]), h, before, f"p of tensor {i}, call {it}")
+                params[i].data.copy_(to_dev(h))
             else:
                 n = h.size
                 m = np.zeros(n, np.float32) if r["m"] is None else oracle.dequant_group(r["m"][0], r["m"][1], qm, n)
