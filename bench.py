@@ -176,16 +176,23 @@ def cpu_baseline(torch, steps=100):
 
 PROBE_KINDS = {"read": (0, 4.0), "write": (1, 4.0), "copy": (2, 8.0), "update_2r1w": (3, 12.0),
                "fused_mix": (4, BYTES_PER_PARAM_4BIT), "fused_mix_dword_codes": (5, BYTES_PER_PARAM_4BIT)}
+# workgroup shapes of lpmm_stream_probe (LPMM_PROBE_SHAPE_*) and the flag for the fused step's tile order
+PROBE_SHAPES = {"256 threads, 1 tile": 0x000, "512 threads, 2 adjacent tiles": 0x100, "128 threads, half a tile": 0x200,
+                "256 threads, 2 tiles loaded up front": 0x300}
+PROBE_RUN_ORDER = 0x1000
 # dynamic LDS per workgroup -> workgroups resident per CU (160 KB of LDS per CU)
-PROBE_RESIDENCY = {8: 0, 6: 26 * 1024, 5: 30 * 1024, 4: 40 * 1024, 3: 53 * 1024, 2: 80 * 1024}
+PROBE_RESIDENCY = {16: 10 * 1024, 12: 13 * 1024, 8: 20 * 1024, 6: 26 * 1024, 5: 32 * 1024, 4: 40 * 1024, 3: 53 * 1024,
+                   2: 80 * 1024}
 
 
 def calibrate(torch, lib, n=1 << 29, iters=5, full=False):
     """What the memory system of this box gives to plain streaming kernels with the fused step's
-    access pattern (lpmm_stream_probe: same workgroup shape, tile, lane layout and nontemporal
-    accesses, no arithmetic): read, write, copy, the in-place 2-reads-1-write update, and the seven
-    streams of the fused step at several residencies.  GB/s over `iters` back-to-back launches on
-    2^29 elements of random data (events on the launch stream), after 2 warm-up launches."""
+    access pattern (lpmm_stream_probe: same lane layout and nontemporal accesses, no arithmetic):
+    read, write, copy, the in-place 2-reads-1-write update, and the seven streams of the fused step,
+    for four workgroup shapes at several residencies, with workgroup i on span i ("plain") and with
+    the fused step's tile order ("run_order": every XCD streams 128 KB runs).  GB/s over `iters`
+    back-to-back launches on 2^29 elements of random data (events on the launch stream), after 2
+    warm-up launches."""
     from lpmm import _native
 
     dev = torch.device("cuda:0")
@@ -198,12 +205,12 @@ def calibrate(torch, lib, n=1 << 29, iters=5, full=False):
     s1 = torch.ones(n // 128, device=dev)
     stream = _native.current_stream(dev)
 
-    def rate(kind, lds):
+    def rate(kind, lds, flags=0):
         code, bytes_per_elt = PROBE_KINDS[kind]
 
         def launch():
-            st = lib.lpmm_stream_probe(code, a.data_ptr(), b.data_ptr(), c0.data_ptr(), c1.data_ptr(), s0.data_ptr(),
-                                       s1.data_ptr(), n, lds, stream)
+            st = lib.lpmm_stream_probe(code | flags, a.data_ptr(), b.data_ptr(), c0.data_ptr(), c1.data_ptr(),
+                                       s0.data_ptr(), s1.data_ptr(), n, lds, stream)
             _native.check(st, "stream probe")
 
         launch()
@@ -217,18 +224,28 @@ def calibrate(torch, lib, n=1 << 29, iters=5, full=False):
         return n * bytes_per_elt * iters / (e0.elapsed_time(e1) * 1e-3) / 1e9
 
     out = {"elements": n, "unit": "GB/s", "data": "random"}
-    res_list = sorted(PROBE_RESIDENCY, reverse=True)
+    # residencies per shape: the same numbers of waves per CU
+    shape_res = {"256 threads, 1 tile": (5, 4, 8, 3, 2), "512 threads, 2 adjacent tiles": (3, 2, 4),
+                 "128 threads, half a tile": (8, 6, 16, 12), "256 threads, 2 tiles loaded up front": (3, 2, 4)}
     for kind in ("read", "write", "copy", "update_2r1w"):
-        if full:
-            out[kind] = {str(r): round(rate(kind, PROBE_RESIDENCY[r]), 1) for r in res_list}
-        else:
-            out[kind] = round(max(rate(kind, PROBE_RESIDENCY[r]) for r in (8, 4)), 1)
-    mix = {str(r): round(rate("fused_mix", PROBE_RESIDENCY[r]), 1) for r in res_list}
-    out["fused_mix_by_workgroups_per_cu"] = mix
-    out["fused_mix_best"] = max(mix.values())
+        for order, flag in (("plain", 0), ("run_order", PROBE_RUN_ORDER)):
+            key = kind if order == "plain" else kind + "_run_order"
+            if full:
+                out[key] = {str(r): round(rate(kind, PROBE_RESIDENCY[r], flag), 1) for r in (8, 5, 4, 3, 2)}
+            else:
+                out[key] = round(max(rate(kind, PROBE_RESIDENCY[r], flag) for r in (5, 3)), 1)
+    best = {}
+    for shape, sflag in PROBE_SHAPES.items():
+        for order, flag in (("plain", 0), ("run_order", PROBE_RUN_ORDER)):
+            res = shape_res[shape] if full else shape_res[shape][:2]
+            table = {str(r): round(rate("fused_mix", PROBE_RESIDENCY[r], sflag | flag), 1) for r in res}
+            out.setdefault("fused_mix_by_workgroups_per_cu", {})[f"{shape}, {order}"] = table
+            best[f"{shape}, {order}"] = max(table.values())
+    out["fused_mix_best_by_shape"] = best
+    out["fused_mix_best"] = max(best.values())
     if full:  # the same streams with one 4-byte code access per lane and state instead of two 2-byte ones
         out["fused_mix_dword_codes_by_workgroups_per_cu"] = {
-            str(r): round(rate("fused_mix_dword_codes", PROBE_RESIDENCY[r]), 1) for r in res_list}
+            str(r): round(rate("fused_mix_dword_codes", PROBE_RESIDENCY[r], PROBE_RUN_ORDER), 1) for r in (8, 5, 4, 3, 2)}
     del a, b, c0, c1, s0, s1
     return out
 
@@ -662,14 +679,15 @@ def main():
         "verified": verified,
         "verified_on": verified_on,
         "config": {"workload": desc, "tensors": len(params), "params": n_total, "quantized_params": n_quant,
-                   "launches_per_step": launches_per_step + 1},
+                   # the 4-bit kernel's launches plus the fp32-state kernel's (tensors of <= 4096 elements, 64 per launch)
+                   "launches_per_step": launches_per_step + math.ceil((len(params) - n_quant_tensors) / 64)},
         "effective_gbs": (n_quant * BYTES_PER_PARAM_4BIT + (n_total - n_quant) * BYTES_PER_PARAM_FP32)
         / (elapsed / args.steps) / 1e9,
         "roofline": {
             "bound": "hbm",
             # second template argument, chosen per launch: every tensor of the launch is a whole
             # number of 2048-element tiles
-            "kernel": "lpmm::adamw4bit_kernel<true, %s, lpmm::FusedArith>" % (
+            "kernel": "lpmm::adamw4bit_kernel<true, %s, lpmm::FusedArith4>" % (
                 "true" if all(p.numel() % 2048 == 0 for p in params if p.numel() > 4096) else "true|false"),
             "achieved": achieved,
             "peak": HBM_PEAK_GBS,

@@ -518,12 +518,22 @@ int lpmm_selftest_encoders(unsigned long long *counts, void *stream);
  *                         written                                 14.125 B/element
  *   LPMM_PROBE_FUSED_MIX_DWORD  the same with one 4-byte code access per lane and state
  *                         instead of two 2-byte ones              14.125 B/element
- * n: a multiple of 2048; a, b: fp32[n], 16-byte aligned; code arrays 4-byte aligned.  lds_bytes (0..163840) of dynamic LDS
+ * kind = pattern | workgroup shape | tile order:
+ *   LPMM_PROBE_SHAPE_256    256 threads on one 2048-element tile (the fused step's own shape; the default)
+ *   LPMM_PROBE_SHAPE_512    512 threads on two adjacent tiles
+ *   LPMM_PROBE_SHAPE_128    128 threads on half a tile
+ *   LPMM_PROBE_SHAPE_256X2  256 threads that load two adjacent tiles before they store either
+ *   LPMM_PROBE_RUN_ORDER    the workgroups take their spans so that every XCD streams 128 KB runs of a (the
+ *                           fused step's tile order); without it workgroup i takes span i
+ * n: a multiple of 4096; a, b: fp32[n], 16-byte aligned; code arrays 4-byte aligned.  lds_bytes (0..163840) of dynamic LDS
  * that the kernels never touch cap the workgroups resident per CU at floor(160 KB / lds_bytes)
- * (0: the hardware's own limit of 8).  Buffers a kind does not use may be NULL. */
+ * (0: the hardware's own limit).  Buffers a pattern does not use may be NULL. */
 enum {
     LPMM_PROBE_READ = 0, LPMM_PROBE_WRITE = 1, LPMM_PROBE_COPY = 2, LPMM_PROBE_UPDATE = 3, LPMM_PROBE_FUSED_MIX = 4,
-    LPMM_PROBE_FUSED_MIX_DWORD = 5
+    LPMM_PROBE_FUSED_MIX_DWORD = 5,
+    LPMM_PROBE_SHAPE_256 = 0x000, LPMM_PROBE_SHAPE_512 = 0x100, LPMM_PROBE_SHAPE_128 = 0x200,
+    LPMM_PROBE_SHAPE_256X2 = 0x300, LPMM_PROBE_SHAPE_MASK = 0x300,
+    LPMM_PROBE_RUN_ORDER = 0x1000
 };
 int lpmm_stream_probe(int kind, float *a, const float *b, uint8_t *codes0, uint8_t *codes1, float *scale0,
                       float *scale1, int64_t n, int64_t lds_bytes, void *stream);
