@@ -26,6 +26,7 @@ constexpr int kV4Elts = 8;
 constexpr int kV4Tile = kV4Threads * kV4Elts;  // 2048 = one pack group
 constexpr int kV4Max = 48;                     // tensors per launch
 static_assert(kV4Tile == LPMM_PACK_GROUP, "a tile is a pack group of the non-fused layout");
+static_assert((kV4Tile * sizeof(float)) << 4 == kXcdRunBytes, "16 tiles per run");
 
 struct TensorV4 {
     float *p;
@@ -61,7 +62,10 @@ __global__ __launch_bounds__(kV4Threads) void adamw_v4bit_kernel(const MultiV4 a
     const bool started = lane + 1 < kV4Max && args.tile_start[lane + 1] <= blockIdx.x;
     const int lo = __popcll(__ballot(started));
     const TensorV4 &t = args.t[lo];
-    const uint32_t tile = blockIdx.x - args.tile_start[lo];
+    // which tile of the tensor: launch order rearranged so that an XCD streams 128 KB runs of the parameters
+    const uint32_t tiles_in_tensor = args.tile_start[lo + 1] - args.tile_start[lo];
+    const uint32_t tile = xcd_run_order<4>(blockIdx.x - args.tile_start[lo], tiles_in_tensor,
+                                           run_phase<4>(t.p, kV4Tile * sizeof(float)));
     const int lane16 = threadIdx.x & 15;
     const int64_t n = t.n;
     const int64_t n_groups = (n + kGroup - 1) / kGroup;
@@ -103,9 +107,9 @@ __global__ __launch_bounds__(kV4Threads) void adamw_v4bit_kernel(const MultiV4 a
     const int kind = classify_map(qmap_v);
     lds_barrier();
 
-    if (threadIdx.x == 0 && blockIdx.x + 1 == args.tile_start[lo + 1]) {
+    if (threadIdx.x == 0 && tile + 1 == tiles_in_tensor) {
         // the tensor's last tile also owns the extra byte at the end of the code buffer
-        t.vc[(int64_t)(args.tile_start[lo + 1] - args.tile_start[lo]) * (kV4Tile / 2)] = 0;
+        t.vc[(int64_t)tiles_in_tensor * (kV4Tile / 2)] = 0;
     }
     if (!live) {
         // codes of a plain 0.0

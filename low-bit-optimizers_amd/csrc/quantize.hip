@@ -130,7 +130,12 @@ __global__ __launch_bounds__(THREADS) void quant_group_kernel(const float *__res
     constexpr int kTileElts = THREADS * kQElts;
     __shared__ __align__(16) uint32_t lds[kLdsBytes / 4];
     __shared__ float s_row[T][THREADS / 16];
-    const int64_t tile0 = (int64_t)blockIdx.x * T * kTileElts;
+    // the workgroup's span of T tiles, in the launch order that lets an XCD stream 128 KB runs of x
+    constexpr int kSpanLog2 = (T * kTileElts * sizeof(float) == 16384) ? 3 : ((T * kTileElts * sizeof(float) == 8192) ? 4 : -1);
+    uint32_t span = blockIdx.x;
+    if constexpr (kSpanLog2 > 0)
+        span = xcd_run_order<kSpanLog2>(span, gridDim.x, run_phase<kSpanLog2>(x, T * kTileElts * sizeof(float)));
+    const int64_t tile0 = (int64_t)span * T * kTileElts;
     const int lane16 = threadIdx.x & 15;
     const int wrow = threadIdx.x >> 4;
     const int64_t gp_sz = (int64_t)rows_per_group * kGroup;
@@ -265,7 +270,12 @@ __global__ __launch_bounds__(kQThreads) void dequant_group_rows_kernel(const uin
     __shared__ __align__(16) uint32_t lds[kDequantLdsWords];
     const int lane16 = threadIdx.x & 15;
     // T passes of 16 rows each; the loads of all passes first, the map afterwards
-    const int64_t row0 = (int64_t)blockIdx.x * T * (kQThreads / 16) + (threadIdx.x >> 4);
+    // the workgroup's span of T x 16 rows, in the launch order that lets an XCD stream 128 KB runs of the output
+    constexpr int kSpanLog2 = (T * 2048 * sizeof(float) == 16384) ? 3 : ((T * 2048 * sizeof(float) == 8192) ? 4 : -1);
+    uint32_t span = blockIdx.x;
+    if constexpr (kSpanLog2 > 0)
+        span = xcd_run_order<kSpanLog2>(span, gridDim.x, run_phase<kSpanLog2>(out, T * 2048 * sizeof(float)));
+    const int64_t row0 = (int64_t)span * T * (kQThreads / 16) + (threadIdx.x >> 4);
     uint32_t c0[T], c1[T];
     float s[T];
 #pragma unroll

@@ -29,6 +29,7 @@ constexpr int kSgdElts = 8;
 constexpr int kSgdTile = kSgdThreads * kSgdElts;  // 2048 = one pack group
 constexpr int kSgdMax = 64;                       // tensors per launch
 static_assert(kSgdTile == LPMM_PACK_GROUP, "a tile is a pack group of the non-fused layout");
+static_assert((kSgdTile * sizeof(float)) << 4 == kXcdRunBytes, "16 tiles per run");
 
 struct TensorSgd {
     float *p;
@@ -75,7 +76,10 @@ __global__ __launch_bounds__(kSgdThreads) void sgd4bit_kernel(const MultiSgd arg
     const bool started = lane + 1 < kSgdMax && args.tile_start[lane + 1] <= blockIdx.x;
     const int lo = __popcll(__ballot(started));
     const TensorSgd &t = args.t[lo];
-    const uint32_t tile = blockIdx.x - args.tile_start[lo];
+    // which tile of the tensor: launch order rearranged so that an XCD streams 128 KB runs of the parameters
+    const uint32_t tiles_in_tensor = args.tile_start[lo + 1] - args.tile_start[lo];
+    const uint32_t tile = xcd_run_order<4>(blockIdx.x - args.tile_start[lo], tiles_in_tensor,
+                                           run_phase<4>(t.p, kSgdTile * sizeof(float)));
     const int lane16 = threadIdx.x & 15;
     const int64_t n = t.n;
     const int64_t n_groups = (n + kGroup - 1) / kGroup;
@@ -116,9 +120,9 @@ __global__ __launch_bounds__(kSgdThreads) void sgd4bit_kernel(const MultiSgd arg
     const int kind = classify_map(qmap);
     lds_barrier();
 
-    if (threadIdx.x == 0 && blockIdx.x + 1 == args.tile_start[lo + 1]) {
+    if (threadIdx.x == 0 && tile + 1 == tiles_in_tensor) {
         // the tensor's last tile also owns the extra byte at the end of the code buffer
-        t.mc[(int64_t)(args.tile_start[lo + 1] - args.tile_start[lo]) * (kSgdTile / 2)] = 0;
+        t.mc[(int64_t)tiles_in_tensor * (kSgdTile / 2)] = 0;
     }
     if (!live) {
         // codes of a plain 0.0
