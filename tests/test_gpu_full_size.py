@@ -134,12 +134,14 @@ def test_quant_roundtrip_64m(oracle, qmaps):
     np.testing.assert_array_equal(to_np(back), oracle.dequant_rank1(want_codes, row, col, qmaps[1], 8192, 8192))
 
 
-def test_factored_step_llama_mlp_shape(oracle, qmaps):
+@pytest.mark.parametrize("shape", [(4096, 11008), (11008, 4096), (4096, 4096)])
+def test_factored_step_llama_shapes(oracle, qmaps, shape):
+    """The three matrix shapes of the factored configuration at full size, three steps each, against
+    the oracle (the tall 11008 x 4096 has the most row tiles, the wide 4096 x 11008 the most column tiles)."""
     import lpmm
 
     qm, qv = qmaps
-    shape = (4096, 11008)
-    rng = np.random.default_rng(9)
+    rng = np.random.default_rng(9 + shape[0])
     host = (rng.standard_normal(shape, dtype=np.float32) * 0.02).astype(np.float32)
     param = torch.nn.Parameter(to_dev(host))
     opt = lpmm.optim.AdamW([param], lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01,

@@ -207,3 +207,142 @@ def test_llama7b_whole_set_equals_single_tensor_calls(qmaps):
         _single_tensor_step(lib, copies, params, dqm, dqv, step)
         torch.cuda.synchronize()
         _assert_set_equal(opt, params, copies, step)
+
+
+# ---------------------------------------------------------------------------------------
+# The factored configuration as a whole set (lpmm/optim/adamw.py:579-627 for the matrices,
+# :332-436 / :439-561 for the vectors, which keep a 4-bit or fp32 second moment).
+# ---------------------------------------------------------------------------------------
+def factored_shapes():
+    shapes = []
+    for _ in range(32):
+        shapes += [(4096, 11008), (11008, 4096), (4096, 4096), (11008,), (4096,)]
+    return shapes
+
+
+def _factored_copies(params, fused, qm):
+    """Per tensor: a copy of the parameter and fresh states in the layouts the single-tensor entry points take."""
+    from lpmm import _native
+    from lpmm.functional import packed_nbytes
+    from lpmm.optim.adamw import _zero_byte
+
+    lib = _native.lib()
+    out = []
+    for p in params:
+        n, dev = p.numel(), p.device
+        c = dict(n=n, p=p.detach().clone())
+        if p.dim() == 2:
+            rows, cols = p.shape
+            c.update(kind="factored", mc=torch.empty(packed_nbytes(n), dtype=torch.int8, device=dev),
+                     ms=torch.empty(n // 128, device=dev), row=torch.zeros(rows, device=dev),
+                     col=torch.zeros(cols, device=dev), mean=torch.zeros(1, device=dev),
+                     work=torch.empty(lib.lpmm_factored_workspace_bytes(rows, cols), dtype=torch.uint8, device=dev))
+        elif n > 4096 and fused:
+            c.update(kind="fused4", mc=torch.zeros(n // 2, dtype=torch.int8, device=dev),
+                     vc=torch.zeros(n // 2, dtype=torch.int8, device=dev), ms=torch.zeros(n // 128, device=dev),
+                     vs=torch.zeros(n // 128, device=dev))
+        elif n > 4096:
+            zero = _zero_byte(qm)
+            c.update(kind="nonfused4", mc=torch.full((packed_nbytes(n),), zero, dtype=torch.int8, device=dev),
+                     vc=torch.full((packed_nbytes(n),), 0, dtype=torch.int8, device=dev),
+                     ms=torch.zeros(n // 128, device=dev), vs=torch.zeros(n // 128, device=dev))
+        else:
+            c.update(kind="fp32", m=torch.zeros(n, device=dev), v=torch.zeros(n, device=dev))
+        out.append(c)
+    return out
+
+
+def _factored_single_step(lib, nat, copies, params, dqm, dqv, step, fused):
+    stream = torch.cuda.current_stream().cuda_stream
+    b1, b2, lr, wd, eps = HO
+    for c, p in zip(copies, params):
+        g = p.grad
+        if c["kind"] == "factored":
+            rows, cols = p.shape
+            st = lib.lpmm_factored_stats(g.data_ptr(), rows, cols, c["row"].data_ptr(), c["col"].data_ptr(),
+                                         c["mean"].data_ptr(), b2, c["work"].data_ptr(), stream)
+            assert st == 0
+            st = lib.lpmm_factored_update(c["p"].data_ptr(), g.data_ptr(), c["mc"].data_ptr(), c["ms"].data_ptr(),
+                                          dqm.data_ptr(), c["row"].data_ptr(), c["col"].data_ptr(),
+                                          c["mean"].data_ptr(), rows, cols, b1, b2, lr, wd, eps, float(step),
+                                          1 if step == 1 else 0, stream)
+        elif c["kind"] == "fused4":
+            st = lib.lpmm_adamw4bit_step(c["p"].data_ptr(), g.data_ptr(), c["mc"].data_ptr(), c["vc"].data_ptr(),
+                                         c["ms"].data_ptr(), c["vs"].data_ptr(), dqm.data_ptr(), dqv.data_ptr(),
+                                         c["n"], *HO, float(step), stream)
+        elif c["kind"] == "nonfused4":
+            rec = np.array([(c["p"].data_ptr(), g.data_ptr(), c["mc"].data_ptr(), c["vc"].data_ptr(),
+                             c["ms"].data_ptr(), c["vs"].data_ptr(), c["n"], float(step), 0.0)],
+                           dtype=nat.ADAMW4BIT_TENSOR)
+            st = lib.lpmm_nonfused_adamw4bit_step_multi(rec.ctypes.data, 1, dqm.data_ptr(), dqv.data_ptr(), b1, b2,
+                                                        lr, wd, eps, stream)
+        elif fused:
+            st = lib.lpmm_adamw_fp32_step(c["p"].data_ptr(), g.data_ptr(), c["m"].data_ptr(), c["v"].data_ptr(),
+                                          c["n"], *HO, float(step), stream)
+        else:
+            st = lib.lpmm_nonfused_update(c["p"].data_ptr(), g.data_ptr(), c["m"].data_ptr(), c["v"].data_ptr(),
+                                          c["n"], b1, b2, lr, wd, eps, float(step), stream)
+        assert st == 0
+
+
+def _assert_factored_set_equal(opt, params, copies, step):
+    for i, (p, c) in enumerate(zip(params, copies)):
+        st = opt.state[p]
+        what = f"tensor {i} {tuple(p.shape)} step {step}"
+        assert float(st["step"]) == float(step)
+        assert torch.equal(p.detach().view(-1), c["p"].view(-1)), "p of " + what
+        if c["kind"] == "factored":
+            assert "exp_avg_sq" not in st
+            assert torch.equal(st["exp_avg_sq_row"].view(-1), c["row"]), "row statistics of " + what
+            assert torch.equal(st["exp_avg_sq_col"].view(-1), c["col"]), "column statistics of " + what
+            assert torch.equal(st["exp_avg"], c["mc"]), "m codes of " + what
+            assert torch.equal(st["exp_avg_qstate"]["overhead"]["max1"].view(-1), c["ms"]), "m scales of " + what
+        elif c["kind"] in ("fused4", "nonfused4"):
+            assert torch.equal(st["exp_avg"], c["mc"]), "m codes of " + what
+            assert torch.equal(st["exp_avg_sq"], c["vc"]), "v codes of " + what
+            assert torch.equal(st["exp_avg_qstate"]["overhead"]["max1"].view(-1), c["ms"]), "m scales of " + what
+            assert torch.equal(st["exp_avg_sq_qstate"]["overhead"]["max1"].view(-1), c["vs"]), "v scales of " + what
+        else:
+            assert torch.equal(st["exp_avg"].view(-1), c["m"]), "m of " + what
+            assert torch.equal(st["exp_avg_sq"].view(-1), c["v"]), "v of " + what
+
+
+@pytest.mark.parametrize("fused", [True, False])
+def test_factored_whole_set_equals_single_tensor_calls(qmaps, fused):
+    """The factored configuration as written: 32 x {4096 x 11008, 11008 x 4096, 4096 x 4096} with a factored
+    second moment, 32 vectors of 11008 values that keep 4-bit moments and 32 of 4096 values with fp32 moments
+    (3.4e9 parameters), gradients N(0, 1e-3) reseeded every step, 20 steps through
+    lpmm.optim.AdamW(factor_second_moment=True).  The optimizer's launches (96 matrices in groups of 24 with
+    four launches each and a workspace carved per tensor, the vectors in multi-tensor launches of their own)
+    must leave exactly the bytes that single-tensor calls leave on copies: lpmm_factored_stats +
+    lpmm_factored_update per matrix, the 4-bit and fp32 step entry points per vector."""
+    import lpmm
+    from lpmm import _native
+
+    lib = _native.lib()
+    dev = torch.device("cuda:0")
+    gen = torch.Generator(device=dev)
+    params = []
+    for i, shape in enumerate(factored_shapes()):
+        gen.manual_seed(10000 + i)
+        params.append(torch.nn.Parameter(torch.randn(shape, device=dev, generator=gen) * 0.02))
+    assert sum(p.numel() for p in params) == 32 * (2 * 4096 * 11008 + 4096 * 4096 + 11008 + 4096)
+    opt = lpmm.optim.AdamW(params, lr=HO[2], betas=(HO[0], HO[1]), eps=HO[4], weight_decay=HO[3], fused=fused,
+                           factor_second_moment=True)
+    dqm, dqv = to_dev(qmaps[0]), to_dev(qmaps[1])
+    copies = _factored_copies(params, fused, dqm)
+    for p in params:
+        p.grad = torch.empty_like(p)
+    for step in range(1, 21):
+        for i, p in enumerate(params):
+            gen.manual_seed(20000 + 1000 * step + i)
+            p.grad.normal_(0.0, 1e-3, generator=gen)
+        opt.step()
+        _factored_single_step(lib, _native, copies, params, dqm, dqv, step, fused)
+        if step in (1, 2, 20):
+            torch.cuda.synchronize()
+            _assert_factored_set_equal(opt, params, copies, step)
+    # the states really are the factored ones and have moved
+    st = opt.state[params[0]]
+    assert st["exp_avg_sq_row"].shape[0] == 4096 and st["exp_avg_sq_col"].shape[0] == 11008
+    assert float(st["exp_avg_sq_row"].min()) > 0.0 and int(st["exp_avg"].ne(0).sum()) > 0
