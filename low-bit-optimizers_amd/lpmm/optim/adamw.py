@@ -52,6 +52,22 @@ def _zero_byte(qmap):
     return hit[1]
 
 
+class _Batch(list):
+    """Records of one pending launch, plus what becomes true once that launch has been enqueued: states
+    whose statistics trade places with a second buffer point to the new buffer only after the kernels
+    that fill it are on the stream.  A check that raises before the launch, or a launch that returns an
+    error, leaves those states as they were (old codes with the statistics they are scaled by)."""
+
+    def __init__(self):
+        super().__init__()
+        self.commits = []
+
+    def launched(self):
+        for commit in self.commits:
+            commit()
+        self.commits.clear()
+
+
 class AdamW(LowBitOptimizer):
     def __init__(
         self,
@@ -368,6 +384,7 @@ class AdamW(LowBitOptimizer):
                                                                   beta1, beta2, lr, wd, eps,
                                                                   _native.current_stream(dev))
             _native.check(st, "non-fused 4-bit AdamW step (rank-1 second moment)")
+            records.launched()
 
         def launch_group_m32(key, records):
             dev, qv_ptr = key
@@ -384,6 +401,7 @@ class AdamW(LowBitOptimizer):
                 st = lib.lpmm_nonfused_adamw_v4bit_rank1_step_multi(table.ctypes.data, len(records), qv_ptr, beta1,
                                                                     beta2, lr, wd, eps, _native.current_stream(dev))
             _native.check(st, "non-fused AdamW step (fp32 first moment, rank-1 4-bit second moment)")
+            records.launched()
 
         def launch_rank1_mgroup(key, records):
             dev, qm_ptr, qv_ptr = key[:3]
@@ -393,6 +411,7 @@ class AdamW(LowBitOptimizer):
                     table.ctypes.data, len(records), qm_ptr, qv_ptr, md_m["gp_sz"], beta1, beta2, lr, wd, eps,
                     _native.current_stream(dev))
             _native.check(st, "non-fused 4-bit AdamW step (wide first-moment groups, rank-1 second moment)")
+            records.launched()
 
         def launch_rank1_bits(key, records):
             dev, qm_ptr, qv_ptr = key
@@ -402,6 +421,7 @@ class AdamW(LowBitOptimizer):
                     table.ctypes.data, len(records), qm_ptr, md_m["b"], qv_ptr, md_v["b"], beta1, beta2, lr, wd, eps,
                     _native.current_stream(dev))
             _native.check(st, "non-fused AdamW step (5-8-bit states, rank-1 second moment)")
+            records.launched()
 
         for p, grad, state, factored in work:
             step = self._next_step(state)
@@ -425,8 +445,8 @@ class AdamW(LowBitOptimizer):
                         pending.clear()
                     continue
                 if v_rank1 and p.dim() == 2 and p.shape[1] % 128 == 0:
-                    pending = batched_rank1.setdefault(key, [])
-                    pending.append(self._nonfused_rank1_record(p, dense, grad, state, step))
+                    pending = batched_rank1.setdefault(key, _Batch())
+                    pending.append(self._nonfused_rank1_record(p, dense, grad, state, step, pending))
                     if len(pending) == _native.RANK1_MULTI_MAX:
                         launch_rank1(key, pending)
                         pending.clear()
@@ -434,9 +454,9 @@ class AdamW(LowBitOptimizer):
             if bits_rank1 and en_m and en_v and p.dim() == 2 and p.shape[1] % 128 == 0:
                 key = (p.device, state["exp_avg_qstate"]["qmap"].data_ptr(),
                        state["exp_avg_sq_qstate"]["qmap"].data_ptr())
-                pending = batched_rank1_bits.setdefault(key, [])
+                pending = batched_rank1_bits.setdefault(key, _Batch())
                 mc, ms = self._group_state(p, state, "exp_avg", b=md_m["b"])
-                pending.append((dense.data_ptr(), grad.data_ptr(), mc, ms) + self._rank1_state(p, state, b=md_v["b"])
+                pending.append((dense.data_ptr(), grad.data_ptr(), mc, ms) + self._rank1_state(p, state, pending, b=md_v["b"])
                                + (p.shape[0], p.shape[1], step, 0.0))
                 if len(pending) == _native.RANK1_MULTI_MAX:
                     launch_rank1_bits(key, pending)
@@ -449,18 +469,22 @@ class AdamW(LowBitOptimizer):
                     and ((m_group_wide and p.shape[1] % 128 == 0) or ((m_group_wide or m_group128) and ragged))):
                 key = (p.device, state["exp_avg_qstate"]["qmap"].data_ptr(),
                        state["exp_avg_sq_qstate"]["qmap"].data_ptr(), ragged)
-                pending = batched_rank1_mgroup.setdefault(key, [])
+                pending = batched_rank1_mgroup.setdefault(key, _Batch())
                 mc, _ = self._group_state(p, state, "exp_avg", md_m["gp_sz"])
                 # the scales trade places with a second buffer, like the second moment's statistics
                 oh = state["exp_avg_qstate"]["overhead"]
                 cur = oh["max1"]
-                nxt = self._spare_scales.pop(p, None)
+                nxt = self._spare_scales.get(p)
                 if nxt is None or nxt.device != cur.device or nxt.shape != cur.shape:
                     nxt = torch.empty_like(cur)
-                self._spare_scales[p] = cur
-                oh["max1"] = nxt
+
+                def commit(p=p, oh=oh, cur=cur, nxt=nxt):
+                    self._spare_scales[p] = cur
+                    oh["max1"] = nxt
+
+                pending.commits.append(commit)
                 pending.append((dense.data_ptr(), grad.data_ptr(), mc, cur.data_ptr(), nxt.data_ptr())
-                               + self._rank1_state(p, state) + (p.shape[0], p.shape[1], step, 0.0))
+                               + self._rank1_state(p, state, pending) + (p.shape[0], p.shape[1], step, 0.0))
                 if len(pending) == _native.RANK1_MULTI_MAX:
                     launch_rank1_mgroup(key, pending)
                     pending.clear()
@@ -479,8 +503,8 @@ class AdamW(LowBitOptimizer):
                         pending.clear()
                     continue
                 if v_rank1 and p.dim() == 2 and p.shape[1] % 128 == 0 and m.data_ptr() % 16 == 0:
-                    pending = batched_rank1_m32.setdefault(key, [])
-                    pending.append((dense.data_ptr(), grad.data_ptr(), m.data_ptr()) + self._rank1_state(p, state)
+                    pending = batched_rank1_m32.setdefault(key, _Batch())
+                    pending.append((dense.data_ptr(), grad.data_ptr(), m.data_ptr()) + self._rank1_state(p, state, pending)
                                    + (p.shape[0], p.shape[1], step, 0.0))
                     if len(pending) == _native.RANK1_MULTI_MAX:
                         launch_rank1_m32(key, pending)
@@ -591,12 +615,12 @@ class AdamW(LowBitOptimizer):
                 oh["dim"] = 1
         return state[name].data_ptr(), qstate["overhead"]["max1"].data_ptr()
 
-    def _rank1_state(self, p, state, b=4):
+    def _rank1_state(self, p, state, batch, b=4):
         """Pointers to the codes of a rank-1 scaled second moment, the statistics they are scaled
         by and the pair of buffers that receives the next statistics; creates the state on first
         use.  The kernels leave the statistics of the new second moment in the second pair; the
-        pairs trade places here, so that the state's `max_dims` always are the statistics its
-        codes are scaled by."""
+        pairs trade places once the launch is enqueued (`batch.launched()`), so that the state's
+        `max_dims` always are the statistics its codes are scaled by, also after a step that raised."""
         rows, cols = p.shape
         dev = p.device
         qs_v = state["exp_avg_sq_qstate"]
@@ -610,11 +634,15 @@ class AdamW(LowBitOptimizer):
                                      "scaled_shape": p.shape})
         oh = qs_v["overhead"]
         cur = oh["max_dims"]
-        nxt = self._spare_stats.pop(p, None)
+        nxt = self._spare_stats.get(p)
         if nxt is None or nxt[0].device != dev:
             nxt = [torch.empty_like(cur[0]), torch.empty_like(cur[1])]
-        self._spare_stats[p] = cur
-        oh["max_dims"] = nxt
+
+        def commit():
+            self._spare_stats[p] = cur
+            oh["max_dims"] = nxt
+
+        batch.commits.append(commit)
         return (state["exp_avg_sq"].data_ptr(), cur[0].data_ptr(), cur[1].data_ptr(), nxt[0].data_ptr(),
                 nxt[1].data_ptr())
 
@@ -624,10 +652,10 @@ class AdamW(LowBitOptimizer):
         vc, vs = self._group_state(p, state, "exp_avg_sq", rank1_vector=rank1_vector)
         return (dense.data_ptr(), grad.data_ptr(), mc, vc, ms, vs, p.numel(), step, 0.0)
 
-    def _nonfused_rank1_record(self, p, dense, grad, state, step):
+    def _nonfused_rank1_record(self, p, dense, grad, state, step, batch):
         """The tensor's record for the two-pass step with a rank-1 second moment."""
         mc, ms = self._group_state(p, state, "exp_avg")
-        return (dense.data_ptr(), grad.data_ptr(), mc, ms) + self._rank1_state(p, state) + (
+        return (dense.data_ptr(), grad.data_ptr(), mc, ms) + self._rank1_state(p, state, batch) + (
             p.shape[0], p.shape[1], step, 0.0)
 
     @property

@@ -801,3 +801,64 @@ def test_double_parameters_on_the_nonfused_path(v_scale):
         bad = lpmm.optim.AdamW([torch.nn.Parameter(host[1].cuda())], fused=True, **hyper)
         bad.param_groups[0]["params"][0].grad = host[1].cuda()
         bad.step()
+
+
+@pytest.mark.parametrize("config", ["default.yml", "1st_moment_group_1024.yml"])
+def test_failed_launch_leaves_the_statistics_with_their_codes(config):
+    """The two-pass kernels write the next row/column statistics (and, with wide first-moment groups, the
+    next scales) into a second buffer that trades places with the state's.  A launch that returns an error
+    must leave the state pointing at the statistics its codes are scaled by: the step after the failure
+    continues exactly like a run that never failed."""
+    import lpmm
+    from lpmm import _native
+
+    cfg = os.path.join(os.path.dirname(lpmm.config.__file__), "configs", config)
+    entry = ("lpmm_nonfused_adamw4bit_rank1_step_multi" if config == "default.yml"
+             else "lpmm_nonfused_adamw4bit_rank1_mgroup_step_multi")
+    rng = np.random.default_rng(31)
+    shapes = [(64, 256), (96, 128)]
+    host, params = _params(shapes, rng)
+    _, twins = _params(shapes, np.random.default_rng(31))
+    opt = lpmm.optim.AdamW(params, fused=False, qconfig=cfg, **H)
+    ref = lpmm.optim.AdamW(twins, fused=False, qconfig=cfg, **H)
+    lib = _native.lib()
+
+    def step_both(which):
+        grads = [(rng.standard_normal(s) * 1e-3).astype(np.float32) for s in shapes]
+        for o, ps in which:
+            for p, g in zip(ps, grads):
+                p.grad = to_dev(g)
+            o.step()
+        return grads
+
+    step_both([(opt, params), (ref, twins)])
+    before = [(opt.state[p]["exp_avg_sq_qstate"]["overhead"]["max_dims"][0].data_ptr(),
+               opt.state[p]["exp_avg_qstate"]["overhead"]["max1"].data_ptr(),
+               to_np(opt.state[p]["exp_avg_sq_qstate"]["overhead"]["max_dims"][0]).copy()) for p in params]
+    real = getattr(lib, entry)
+    setattr(lib, entry, lambda *a: 5)  # any status but LPMM_OK
+    try:
+        for p in params:
+            p.grad = torch.zeros_like(p)
+        with pytest.raises(RuntimeError):
+            opt.step()
+    finally:
+        setattr(lib, entry, real)
+    torch.cuda.synchronize()
+    for p, (rows_ptr, max1_ptr, rows) in zip(params, before):
+        oh_v, oh_m = opt.state[p]["exp_avg_sq_qstate"]["overhead"], opt.state[p]["exp_avg_qstate"]["overhead"]
+        assert oh_v["max_dims"][0].data_ptr() == rows_ptr and oh_m["max1"].data_ptr() == max1_ptr
+        np.testing.assert_array_equal(to_np(oh_v["max_dims"][0]), rows)
+    # the failed call counted a step for every tensor; give the twin the same count, then both continue alike
+    for p, t in zip(params, twins):
+        ref.state[t]["step"] += 1
+        assert float(opt.state[p]["step"]) == float(ref.state[t]["step"])
+    step_both([(opt, params), (ref, twins)])
+    torch.cuda.synchronize()
+    for p, t in zip(params, twins):
+        assert torch.equal(p.detach(), t.detach())
+        assert torch.equal(opt.state[p]["exp_avg_sq"], ref.state[t]["exp_avg_sq"])
+        assert torch.equal(opt.state[p]["exp_avg"], ref.state[t]["exp_avg"])
+        for a, b in zip(opt.state[p]["exp_avg_sq_qstate"]["overhead"]["max_dims"],
+                        ref.state[t]["exp_avg_sq_qstate"]["overhead"]["max_dims"]):
+            assert torch.equal(a, b)
