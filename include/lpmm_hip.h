@@ -399,7 +399,11 @@ int lpmm_factored_stats(const float *g, int64_t rows, int64_t cols, float *row, 
  * the process ends; the call allocates and frees nothing.  Shapes whose
  * lpmm_factored_workspace_bytes(rows, cols) exceeds that size return LPMM_ERR_SIZE.  All calls
  * on one GPU share the array: calls that overlap on one GPU (different streams) race.  Same
- * results as lpmm_factored_stats. */
+ * results as lpmm_factored_stats.
+ * The first call on each GPU looks the array's address up (hipGetSymbolAddress, which may load the
+ * code object): make that call outside any stream capture, as a warm-up on a small input.  Every
+ * later call on that GPU only enqueues three kernels on `stream` and may be recorded into a HIP
+ * graph; replays use the same array. */
 #define LPMM_FACTORED_STATIC_BYTES (32u << 20)
 int lpmm_factored_stats_static(const float *g, int64_t rows, int64_t cols, float *row, float *col,
                                float *row_mean_all, double beta2, void *stream);

@@ -675,6 +675,8 @@ extern "C" int lpmm_factored_stats_static(const float *g, int64_t rows, int64_t 
     int dev = -1;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices)
         return LPMM_ERR_LAUNCH;
+    // The address is looked up on the first call on each GPU (callers make that call outside stream
+    // capture); afterwards this block only reads the cached pointer.
     void *ws = nullptr;
     {
         std::lock_guard<std::mutex> hold(g_scratch_lock);

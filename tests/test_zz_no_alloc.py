@@ -53,3 +53,42 @@ def test_static_scratch_rejects_what_does_not_fit():
     x = torch.zeros(16, device="cuda:0")
     st = lib.lpmm_factored_stats_static(x.data_ptr(), rows, cols, x.data_ptr(), x.data_ptr(), x.data_ptr(), BETA2, None)
     assert st == 3  # LPMM_ERR_SIZE, before anything touches the GPU
+
+
+def test_static_scratch_call_replayed_from_a_graph():
+    """After a warm-up call on the GPU (the first call looks up the array's address and must stay outside
+    capture), the allocation-free call records into a HIP graph.  Three replays on changing gradients, with
+    eager work and synchronisations in between, each against the workspace form issued eagerly."""
+    from lpmm import _native
+
+    lib = _native.lib()
+    dev = torch.device("cuda:0")
+    gen = torch.Generator(device=dev).manual_seed(12)
+    warm = torch.randn((64, 128), device=dev, generator=gen)
+    _run(lib, warm, torch.zeros(64, device=dev), torch.zeros(128, device=dev), static=True)
+
+    rows, cols = 515, 1400
+    g = torch.randn((rows, cols), device=dev, generator=gen) * 1e-3
+    row, col = torch.zeros(rows, device=dev), torch.zeros(cols, device=dev)
+    mean = torch.zeros(1, device=dev)
+    side = torch.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            st = lib.lpmm_factored_stats_static(g.data_ptr(), rows, cols, row.data_ptr(), col.data_ptr(),
+                                                mean.data_ptr(), BETA2, torch.cuda.current_stream().cuda_stream)
+            assert st == 0
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    assert float(row.abs().sum()) == 0.0  # capture records, it does not run
+    for replay in range(3):
+        g.copy_(torch.randn((rows, cols), device=dev, generator=gen) * (1e-3 * (replay + 1)))
+        row0, col0 = row.clone(), col.clone()
+        want = _run(lib, g, row0, col0, static=False)
+        graph.replay()
+        torch.cuda.synchronize()
+        # eager work between the replays, some of it through the same array
+        _run(lib, warm, torch.zeros(64, device=dev), torch.zeros(128, device=dev), static=True)
+        for a, b, what in zip((row.cpu().numpy(), col.cpu().numpy(), mean.cpu().numpy()), want, ("row", "col", "mean(row)")):
+            np.testing.assert_array_equal(a, b, err_msg=f"{what}, replay {replay}")
