@@ -340,6 +340,14 @@ __device__ __forceinline__ void update_rows128_body(
     // tile = kFaTileRows rows by 16 / kFaTileRows adjacent groups
     constexpr uint32_t kGPS = (kFTile / kGroup) / kFaTileRows;
     const uint32_t col_tiles = (col_blocks + kGPS - 1) / kGPS;
+#ifndef LPMM_FA_RUN_ORDER
+#define LPMM_FA_RUN_ORDER 1
+#endif
+    // Where 16 consecutive tiles (column tile fastest) are 128 KB of contiguous parameters -- 256, 512, ...
+    // 4096 columns -- the tiles are handed out in the order of xcd_run_order: an XCD streams whole runs.
+    if (LPMM_FA_RUN_ORDER && kFaTileRows == 8 && (16u % col_tiles) == 0u)
+        tile = xcd_run_order<4>(tile, (uint32_t)((R + kFaTileRows - 1) / kFaTileRows) * col_tiles,
+                                run_phase<4>(p, kFTile * sizeof(float)));
     const uint32_t rb = tile / col_tiles, ct = tile - rb * col_tiles;
     const uint32_t drow = threadIdx.x >> 4;
     const int64_t r = (int64_t)rb * kFaTileRows + drow / kGPS;
