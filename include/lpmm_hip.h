@@ -21,7 +21,7 @@
 extern "C" {
 #endif
 
-#define LPMM_HIP_ABI_VERSION 1
+#define LPMM_HIP_ABI_VERSION 2
 
 /* One quantisation group of the fused path = 128 elements = one scale
  * (lpmm/cpp_extension/fused_adamw_kernel.cu:216-219). */
@@ -208,6 +208,25 @@ int lpmm_dequant_group_bits(const uint8_t *codes, const float *max1, const float
                             int64_t n, int64_t gp_sz, float *out, void *stream);
 int lpmm_quant_rank1_bits(const float *x, int64_t rows, int64_t cols, const float *rowmax,
                           const float *colmax, const float *qmap, int bits, uint8_t *codes, void *stream);
+
+/* Code tables (no counterpart in the reference, whose kernels search the map for every value).
+ * For a map that qualifies -- strictly increasing, as create_dynamic_map gives
+ * (lpmm/functional.py:272-300) -- the code of the search of quantization_kernel.cu:397-427 is the
+ * number of midpoints below x, and one read of a table over the sign, the exponent and the
+ * leading bits - 2 mantissa bits of x finds it.  The table belongs to the map: build it once
+ * (one small launch) and pass it with the map to the _table entry points below, which otherwise
+ * equal the entry points without the suffix and give the same bytes; NULL, a table built for
+ * another width or one of a map that does not qualify means the search.  table:
+ * LPMM_CODE_TABLE_BYTES device bytes, 16-byte aligned, written in full; its last word says what
+ * the builder found (search / the evenly spaced map's closed form / table).  A table that was
+ * built from a different map of the same width gives wrong codes without an error. */
+#define LPMM_CODE_TABLE_BYTES 12288
+int lpmm_code_table_build(const float *qmap, int bits, void *table, void *stream);
+int lpmm_quant_group_bits_table(const float *x, int64_t n, int64_t gp_sz, const float *qmap, int bits,
+                                const void *table, uint8_t *codes, float *max1, void *stream);
+int lpmm_quant_rank1_bits_table(const float *x, int64_t rows, int64_t cols, const float *rowmax,
+                                const float *colmax, const float *qmap, int bits, const void *table,
+                                uint8_t *codes, void *stream);
 int lpmm_dequant_rank1_bits(const uint8_t *codes, const float *rowmax, const float *colmax,
                             const float *qmap, int bits, int64_t rows, int64_t cols, float *out,
                             void *stream);
@@ -377,6 +396,13 @@ int lpmm_nonfused_adamw_bits_rank1_step_multi(const lpmm_nonfused_rank1_tensor *
                                               const float *qmap_v, int bits_v, double beta1,
                                               double beta2, double lr, double weight_decay,
                                               double eps, void *stream);
+/* The same with the code tables of the two maps (lpmm_code_table_build; either may be NULL). */
+int lpmm_nonfused_adamw_bits_rank1_step_multi_table(const lpmm_nonfused_rank1_tensor *tensors,
+                                                    int64_t count, const float *qmap_m, int bits_m,
+                                                    const void *table_m, const float *qmap_v,
+                                                    int bits_v, const void *table_v, double beta1,
+                                                    double beta2, double lr, double weight_decay,
+                                                    double eps, void *stream);
 
 /* ---------------------------------------------------------------------------------------
  * (c) Factored second moment on a row-major R x C tensor.
@@ -508,6 +534,14 @@ int lpmm_selftest_arithmetic(unsigned long long *counts, uint32_t sqrt_stride, u
  *   within 128 floats of every midpoint * maximum and random), [7] wrong codes; [8], [9] the
  *   same with the second-moment map.  Every odd entry must stay 0. */
 int lpmm_selftest_encoders(unsigned long long *counts, void *stream);
+
+/* Diagnostic (no counterpart in the reference): builds the code table of a map as
+ * lpmm_code_table_build does and runs the one-read code assignment against the search of
+ * lpmm/cpp_extension/quantization_kernel.cu:397-427 as the library restates it, on the device, for
+ * all 2^32 bit patterns of x (NaNs included).  qmap: 2^bits floats, 3 <= bits <= 8.  counts: 3
+ * zero-initialised device uint64: [0] patterns tried, [1] codes that differ (must stay 0),
+ * [2] 1 if the map qualifies for a table; for a map that does not, nothing is tried. */
+int lpmm_selftest_bucket_encoder(const float *qmap, int bits, unsigned long long *counts, void *stream);
 
 /* Diagnostic (no counterpart in the reference): streaming-rate calibration.  Kernels that move
  * bytes the way the fused 4-bit step moves them (256-thread workgroups, 2048-element tiles, the

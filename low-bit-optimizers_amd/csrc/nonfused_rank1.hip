@@ -425,7 +425,8 @@ static float *next_scales(const lpmm_rank1_mgroup_tensor &t) { return t.m_max1_n
 template <int MODE, class Record>
 static int rank1_step_multi(const Record *tensors, int64_t count, const float *qmap_m, const float *qmap_v,
                             uint32_t m_lg, double beta1, double beta2, double lr, double weight_decay, double eps,
-                            void *stream, int bits_m = 4, int bits_v = 4)
+                            void *stream, int bits_m = 4, int bits_v = 4, const void *table_m = nullptr,
+                            const void *table_v = nullptr)
 {
     constexpr bool M32 = MODE == kMFloat;
     // column counts that are no multiple of 128 (wide-group records only): every tensor of the call
@@ -544,7 +545,9 @@ static int rank1_step_multi(const Record *tensors, int64_t count, const float *q
         if (ragged || (MODE == kMCodesWide && m_lg == 0)) {
             launch_rank1_ragged(args, (uint32_t)tiles, qmap_m, qmap_v, (hipStream_t)stream);
         } else if (bits_m != 4) {
-            launch_rank1_bits(args, (uint32_t)tiles, qmap_m, qmap_v, bits_m, bits_v, (hipStream_t)stream);
+            launch_rank1_bits(args, (uint32_t)tiles, qmap_m, qmap_v, bits_m, bits_v,
+                              static_cast<const uint32_t *>(table_m), static_cast<const uint32_t *>(table_v),
+                              (hipStream_t)stream);
         } else {
             hipLaunchKernelGGL(rank1_update_kernel<MODE>, dim3((uint32_t)tiles), dim3(kThreads), 0,
                                (hipStream_t)stream, args, qmap_m, qmap_v);
@@ -595,8 +598,22 @@ extern "C" int lpmm_nonfused_adamw_bits_rank1_step_multi(const lpmm_nonfused_ran
                                                          int bits_v, double beta1, double beta2, double lr,
                                                          double weight_decay, double eps, void *stream)
 {
+    return lpmm_nonfused_adamw_bits_rank1_step_multi_table(tensors, count, qmap_m, bits_m, nullptr, qmap_v, bits_v,
+                                                           nullptr, beta1, beta2, lr, weight_decay, eps, stream);
+}
+
+extern "C" int lpmm_nonfused_adamw_bits_rank1_step_multi_table(const lpmm_nonfused_rank1_tensor *tensors, int64_t count,
+                                                               const float *qmap_m, int bits_m, const void *table_m,
+                                                               const float *qmap_v, int bits_v, const void *table_v,
+                                                               double beta1, double beta2, double lr,
+                                                               double weight_decay, double eps, void *stream)
+{
     if (bits_m < 5 || bits_m > 8 || bits_v < 5 || bits_v > 8)
         return LPMM_ERR_ARG;  // the widths that store one code per byte
+    if (table_m != nullptr)
+        LPMM_REQUIRE_ALIGN(table_m, 16);
+    if (table_v != nullptr)
+        LPMM_REQUIRE_ALIGN(table_v, 16);
     return rank1_step_multi<kMCodes128>(tensors, count, qmap_m, qmap_v, 0, beta1, beta2, lr, weight_decay, eps, stream,
-                                        bits_m, bits_v);
+                                        bits_m, bits_v, table_m, table_v);
 }

@@ -37,10 +37,12 @@ __device__ __forceinline__ void write_padding_bytes(uint8_t *codes, int64_t n, i
 
 __global__ __launch_bounds__(kThreads) void rank1_update_bits_kernel(const MultiR1 args, const float *__restrict__ qmap_m,
                                                                     const float *__restrict__ qmap_v, int bits_m,
-                                                                    int bits_v)
+                                                                    int bits_v, const uint32_t *__restrict__ table_m)
 {
     __shared__ float map_m[256], map_v[256];
     __shared__ SearchLds search_m;
+    __shared__ BucketLds bucket_m;
+    const uint32_t mode = code_table_mode(code_table_tag(table_m), bits_m);
     __shared__ __align__(16) float col_old[kMaxWide * kGroup];
     __shared__ uint32_t colred[kMaxWide * kRedSlotWords];
     const int lo = find_tensor(args);
@@ -52,7 +54,10 @@ __global__ __launch_bounds__(kThreads) void rank1_update_bits_kernel(const Multi
     const int64_t tile_c0 = (int64_t)q.col_tile * q.wide * kGroup;
     fill_map(map_m, qmap_m, bits_m);
     fill_map(map_v, qmap_v, bits_v);
-    fill_search(search_m, qmap_m, bits_m);
+    if (mode == kCodeTable)
+        code_table_store(bucket_m, code_table_load(table_m));
+    else if (mode == kCodeSearch)
+        fill_search(search_m, qmap_m, bits_m);
     for (int j = threadIdx.x; j < kMaxWide * kGroup; j += kThreads)
         col_old[j] = (j < q.wide * kGroup && tile_c0 + j < cols) ? t.col_old[tile_c0 + j] : 0.0f;
     for (int j = threadIdx.x; j < kMaxWide * (int)kRedSlotWords; j += kThreads)
@@ -67,12 +72,12 @@ __global__ __launch_bounds__(kThreads) void rank1_update_bits_kernel(const Multi
     h.bc2_sqrt = t.bc2_sqrt;
     h.rbc2_sqrt = t.rbc2_sqrt;
     __syncthreads();
-    const bool map_even = map_is_even(search_m);
+    const bool map_even = mode == kCodeEven || (mode == kCodeSearch && map_is_even(search_m));
 
     if (tl == 0) {
         const int64_t n = t.rows * cols;
         write_padding_bytes(t.mc, n, (n + LPMM_PACK_GROUP - 1) / LPMM_PACK_GROUP * LPMM_PACK_GROUP,
-                            search_code(search_m, bits_m, 0.0f));
+                            code1_by_mode(mode, search_m, bucket_m, bits_m, 0.0f));
     }
     const uint32_t mask_m = (1u << bits_m) - 1u, mask_v = (1u << bits_v) - 1u;
     const int slot = drow & (q.wide - 1);
@@ -125,7 +130,7 @@ __global__ __launch_bounds__(kThreads) void rank1_update_bits_kernel(const Multi
                     xs[k] = m[k] / amax_m;
             }
             uint32_t c[kEltsPerLane];
-            search_codes8(search_m, bits_m, map_even, xs, c);
+            codes8_by_mode(mode, search_m, bucket_m, bits_m, map_even, xs, c);
             store4(pp, make_float4(pv[0], pv[1], pv[2], pv[3]));
             store4(pp + 64, make_float4(pv[4], pv[5], pv[6], pv[7]));
             store_u32(mcp, pack4(c, 0));
@@ -147,10 +152,12 @@ __global__ __launch_bounds__(kThreads) void rank1_update_bits_kernel(const Multi
 }
 
 __global__ __launch_bounds__(kThreads) void rank1_requant_bits_kernel(const MultiR1 args, const float *__restrict__ qmap_v,
-                                                                     int bits_v)
+                                                                     int bits_v, const uint32_t *__restrict__ table_v)
 {
     __shared__ float map_v[256];
     __shared__ SearchLds search_v;
+    __shared__ BucketLds bucket_v;
+    const uint32_t mode = code_table_mode(code_table_tag(table_v), bits_v);
     __shared__ __align__(16) float col_old[kMaxWide * kGroup], col_new[kMaxWide * kGroup];
     const int lo = find_tensor(args);
     const TensorR1 &t = args.t[lo];
@@ -160,7 +167,10 @@ __global__ __launch_bounds__(kThreads) void rank1_requant_bits_kernel(const Mult
     const int64_t cols = (int64_t)t.col_blocks * kGroup;
     const int64_t tile_c0 = (int64_t)q.col_tile * q.wide * kGroup;
     fill_map(map_v, qmap_v, bits_v);
-    fill_search(search_v, qmap_v, bits_v);
+    if (mode == kCodeTable)
+        code_table_store(bucket_v, code_table_load(table_v));
+    else if (mode == kCodeSearch)
+        fill_search(search_v, qmap_v, bits_v);
     for (int j = threadIdx.x; j < kMaxWide * kGroup; j += kThreads) {
         const bool in = j < q.wide * kGroup && tile_c0 + j < cols;
         col_old[j] = in ? t.col_old[tile_c0 + j] : 0.0f;
@@ -170,12 +180,12 @@ __global__ __launch_bounds__(kThreads) void rank1_requant_bits_kernel(const Mult
     h.b2 = args.b2;
     h.w2 = args.w2;
     __syncthreads();
-    const bool map_even = map_is_even(search_v);
+    const bool map_even = mode == kCodeEven || (mode == kCodeSearch && map_is_even(search_v));
 
     if (tl == 0) {
         const int64_t n = t.rows * cols;
         write_padding_bytes(t.vc, n, (n + LPMM_PACK_GROUP - 1) / LPMM_PACK_GROUP * LPMM_PACK_GROUP,
-                            search_code(search_v, bits_v, 0.0f));
+                            code1_by_mode(mode, search_v, bucket_v, bits_v, 0.0f));
     }
     if (q.cg >= t.col_blocks)
         return;
@@ -184,6 +194,14 @@ __global__ __launch_bounds__(kThreads) void rank1_requant_bits_kernel(const Mult
     float co[kEltsPerLane], cn[kEltsPerLane];
     unpack8(*reinterpret_cast<const float4 *>(col_old + col_off), *reinterpret_cast<const float4 *>(col_old + col_off + 64), co);
     unpack8(*reinterpret_cast<const float4 *>(col_new + col_off), *reinterpret_cast<const float4 *>(col_new + col_off + 64), cn);
+    // the lane's columns through all passes: the correctly rounded reciprocals of their statistics once
+    float rcn[kEltsPerLane];
+    bool cols_safe = true;
+#pragma unroll
+    for (int k = 0; k < kEltsPerLane; ++k) {
+        rcn[k] = rcp_exact(cn[k]);
+        cols_safe = cols_safe && rc_safe(cn[k]);
+    }
 #pragma unroll 1
     for (int it = 0; it < q.passes; ++it) {
         const int64_t r = q.row0 + it * q.step;
@@ -195,27 +213,41 @@ __global__ __launch_bounds__(kThreads) void rank1_requant_bits_kernel(const Mult
         uint32_t *vcp = reinterpret_cast<uint32_t *>(t.vc + gbase) + lane16;
         const uint32_t wv0 = load_u32(vcp), wv1 = load_u32(vcp + 16);
         const float ro = t.row_old[r], rn = t.row_new[r];
-        float gv[kEltsPerLane], x[kEltsPerLane];
+        float gv[kEltsPerLane], v[kEltsPerLane], x[kEltsPerLane];
         unpack8(b0, b1, gv);
 #pragma unroll
         for (int k = 0; k < kEltsPerLane; ++k) {
-            float v = map_v[byte_of(wv0, wv1, k) & mask_v] * ((co[k] < ro) ? co[k] : ro);
-            nonfused_second_moment(v, gv[k], h);
-            x[k] = v / ((cn[k] < rn) ? cn[k] : rn);
+            v[k] = map_v[byte_of(wv0, wv1, k) & mask_v] * ((co[k] < ro) ? co[k] : ro);
+            nonfused_second_moment(v[k], gv[k], h);
+        }
+        // every scale is a maximum over the values it divides (v <= scale): where all of the wave's
+        // scales lie in the range in which the reciprocal is exact, the correctly rounded reciprocal,
+        // one multiply and two fmas give the correctly rounded quotient
+        if (__all(cols_safe && rc_safe(rn))) {
+            const float rcr = rcp_exact(rn);
+#pragma unroll
+            for (int k = 0; k < kEltsPerLane; ++k) {
+                const bool by_col = cn[k] < rn;
+                x[k] = div_by_rc(v[k], by_col ? cn[k] : rn, by_col ? rcn[k] : rcr);
+            }
+        } else {
+#pragma unroll
+            for (int k = 0; k < kEltsPerLane; ++k)
+                x[k] = v[k] / ((cn[k] < rn) ? cn[k] : rn);
         }
         uint32_t c[kEltsPerLane];
-        search_codes8(search_v, bits_v, map_even, x, c);
+        codes8_by_mode(mode, search_v, bucket_v, bits_v, map_even, x, c);
         store_u32(vcp, pack4(c, 0));
         store_u32(vcp + 16, pack4(c, 1));
     }
 }
 
 void launch_rank1_bits(const MultiR1 &args, uint32_t tiles, const float *qmap_m, const float *qmap_v, int bits_m,
-                       int bits_v, hipStream_t stream)
+                       int bits_v, const uint32_t *table_m, const uint32_t *table_v, hipStream_t stream)
 {
     hipLaunchKernelGGL(rank1_update_bits_kernel, dim3(tiles), dim3(kThreads), 0, stream, args, qmap_m, qmap_v, bits_m,
-                       bits_v);
-    hipLaunchKernelGGL(rank1_requant_bits_kernel, dim3(tiles), dim3(kThreads), 0, stream, args, qmap_v, bits_v);
+                       bits_v, table_m);
+    hipLaunchKernelGGL(rank1_requant_bits_kernel, dim3(tiles), dim3(kThreads), 0, stream, args, qmap_v, bits_v, table_v);
 }
 
 }  // namespace lpmm

@@ -415,7 +415,10 @@ __global__ __launch_bounds__(kBThreads) void dequant_rank1_bits_kernel(const uin
 // tensor that consists of whole 2048-value tiles (whole 128-value groups for the dequantiser);
 // the flat kernels above take the rest and every packed width.
 // ---------------------------------------------------------------------------------------
-constexpr int kBRowsT = 2;       // tiles (passes of 16 groups) per workgroup: loads first, map afterwards
+#ifndef LPMM_BROWS_T
+#define LPMM_BROWS_T 2
+#endif
+constexpr int kBRowsT = LPMM_BROWS_T;       // tiles (passes of 16 groups) per workgroup: loads first, map afterwards
 constexpr int kBRank1Rows = 4;   // rows of one 2048-column chunk per workgroup of the rank-1 kernels
 
 __device__ __forceinline__ uint32_t bytes4(uint32_t a, uint32_t b, uint32_t c, uint32_t d)
@@ -439,19 +442,51 @@ __device__ __forceinline__ void decode_bytes(uint32_t w0, uint32_t w1, uint32_t 
     }
 }
 
+// Builds the code table of a map (lpmm_search.hpp): one workgroup of 256 threads.
+__global__ __launch_bounds__(256) void code_table_kernel(const float *__restrict__ qmap, int bits,
+                                                         uint32_t *__restrict__ table)
+{
+    __shared__ SearchLds tree;
+    __shared__ BucketLds bucket;
+    const SearchFill fill = fill_search_load(qmap, bits);
+    fill_search_store(tree, fill, bits);
+    uint32_t mode = kCodeSearch, total = 0;
+    if (bucket_bits_ok(bits)) {  // uniform
+        const BucketFill bucket_fill = fill_buckets_init(bucket, fill, bits);
+        __syncthreads();
+        fill_buckets_scatter(bucket, bucket_fill);
+        __syncthreads();
+        fill_buckets_counts(bucket, bucket_fill, bits);
+        __syncthreads();
+        total = 2u * bucket_shape(bits).side;
+        mode = buckets_ok(bucket) ? kCodeTable : kCodeSearch;
+    } else {
+        __syncthreads();
+    }
+    if (map_is_even(tree))
+        mode = kCodeEven;
+    for (uint32_t i = threadIdx.x; i < (uint32_t)kBucketEntries; i += blockDim.x)
+        table[i] = i == (uint32_t)kCodeTableTag ? ((uint32_t)bits << 8) | mode : (mode == kCodeTable && i < total ? bucket.entry[i] : 0u);
+}
+
 template <int T>
 __global__ __launch_bounds__(kBThreads) void quant_group_bits_rows_kernel(const float *__restrict__ x,
                                                                           int64_t full_tiles, int rows_per_group,
                                                                           const float *__restrict__ qmap, int bits,
+                                                                          const uint32_t *__restrict__ table,
                                                                           uint8_t *__restrict__ codes,
                                                                           float *__restrict__ max1, int64_t trailing)
 {
     __shared__ SearchLds lds_map;
+    __shared__ BucketLds lds_bucket;
     __shared__ float s_row[T][kBThreads / 16];
     const int lane16 = threadIdx.x & 15, wrow = threadIdx.x >> 4;
     const int64_t tile0 = (int64_t)blockIdx.x * T;
     // the small loads that feed LDS first (they return first), then the tiles' loads
-    const SearchFill fill = fill_search_load(qmap, bits);
+    const uint32_t tag = code_table_tag(table);
+    SearchFill fill;
+    if (table == nullptr)
+        fill = fill_search_load(qmap, bits);
     float v[T][kBElts];
 #pragma unroll
     for (int t = 0; t < T; ++t) {
@@ -463,7 +498,14 @@ __global__ __launch_bounds__(kBThreads) void quant_group_bits_rows_kernel(const 
         }
         unpack8(a, b, v[t]);
     }
-    fill_search_store(lds_map, fill, bits);
+    const uint32_t mode = code_table_mode(tag, bits);
+    if (mode == kCodeTable) {
+        code_table_store(lds_bucket, code_table_load(table));
+    } else if (mode == kCodeSearch) {
+        if (table != nullptr)  // a table that says "search"
+            fill = fill_search_load(qmap, bits);
+        fill_search_store(lds_map, fill, bits);
+    }
     if (blockIdx.x == 0 && threadIdx.x == 0)
         codes[trailing] = 0;
     float amax[T];
@@ -478,7 +520,7 @@ __global__ __launch_bounds__(kBThreads) void quant_group_bits_rows_kernel(const 
             s_row[t][wrow] = amax[t];
     }
     lds_barrier();
-    const bool map_even = map_is_even(lds_map);
+    const bool map_even = mode == kCodeEven || (mode == kCodeSearch && map_is_even(lds_map));
     const int first = wrow & ~(rows_per_group - 1);
     const int64_t gp_sz = (int64_t)rows_per_group * kGroup;
 #pragma unroll
@@ -505,7 +547,7 @@ __global__ __launch_bounds__(kBThreads) void quant_group_bits_rows_kernel(const 
                 xs[k] = v[t][k] / amax[t];
         }
         uint32_t c[kBElts];
-        search_codes8(lds_map, bits, map_even, xs, c);
+        codes8_by_mode(mode, lds_map, lds_bucket, bits, map_even, xs, c);
         uint32_t *cp = reinterpret_cast<uint32_t *>(codes + base) + lane16;
         store_u32(cp, bytes4(c[0], c[1], c[2], c[3]));
         store_u32(cp + 16, bytes4(c[4], c[5], c[6], c[7]));
@@ -562,18 +604,23 @@ __global__ __launch_bounds__(kBThreads) void quant_rank1_bits_rows128_kernel(con
                                                                              const float *__restrict__ rowmax,
                                                                              const float *__restrict__ colmax,
                                                                              const float *__restrict__ qmap, int bits,
+                                                                             const uint32_t *__restrict__ table,
                                                                              uint8_t *__restrict__ codes,
                                                                              int64_t n_padded)
 {
     constexpr int T = kBRank1Rows;
     __shared__ SearchLds lds_map;
+    __shared__ BucketLds lds_bucket;
+    const uint32_t tag = code_table_tag(table);
     const int64_t n = R * C;
     const int lane16 = threadIdx.x & 15;
     const int64_t r0 = (int64_t)blockIdx.y * T;
     const int64_t c0 = (int64_t)blockIdx.x * kBTile + (int64_t)(threadIdx.x >> 4) * kGroup;
     const bool live = c0 < C;  // uniform over the 16 lanes of a group
     // the small loads that feed LDS first (they return first), then the rows' loads
-    const SearchFill fill = fill_search_load(qmap, bits);
+    SearchFill fill;
+    if (table == nullptr)
+        fill = fill_search_load(qmap, bits);
     float4 a[T], b[T], ca, cb;
     float rm[T];
     if (live) {
@@ -590,12 +637,19 @@ __global__ __launch_bounds__(kBThreads) void quant_rank1_bits_rows128_kernel(con
             }
         }
     }
-    fill_search_store(lds_map, fill, bits);
+    const uint32_t mode = code_table_mode(tag, bits);
+    if (mode == kCodeTable) {
+        code_table_store(lds_bucket, code_table_load(table));
+    } else if (mode == kCodeSearch) {
+        if (table != nullptr)  // a table that says "search"
+            fill = fill_search_load(qmap, bits);
+        fill_search_store(lds_map, fill, bits);
+    }
     lds_barrier();
-    const bool map_even = map_is_even(lds_map);
+    const bool map_even = mode == kCodeEven || (mode == kCodeSearch && map_is_even(lds_map));
     if (blockIdx.x == 0 && blockIdx.y == 0) {
         // the padding added by the re-grouping to 2048: plain zeros, not divided by anything
-        const uint32_t z = search_code(lds_map, bits, 0.0f);
+        const uint32_t z = code1_by_mode(mode, lds_map, lds_bucket, bits, 0.0f);
         const uint32_t wz = bytes4(z, z, z, z);
         for (int64_t i = n + (int64_t)threadIdx.x * 4; i < n_padded; i += kBThreads * 4)
             *reinterpret_cast<uint32_t *>(codes + i) = wz;
@@ -631,7 +685,7 @@ __global__ __launch_bounds__(kBThreads) void quant_rank1_bits_rows128_kernel(con
                 xs[k] = v[k] / ((cmx[k] < rm[t]) ? cmx[k] : rm[t]);
         }
         uint32_t c[kBElts];
-        search_codes8(lds_map, bits, map_even, xs, c);
+        codes8_by_mode(mode, lds_map, lds_bucket, bits, map_even, xs, c);
         uint32_t *cp = reinterpret_cast<uint32_t *>(codes + (r0 + t) * C + c0) + lane16;
         store_u32(cp, bytes4(c[0], c[1], c[2], c[3]));
         store_u32(cp + 16, bytes4(c[4], c[5], c[6], c[7]));
@@ -772,11 +826,33 @@ extern "C" int lpmm_unpack_nonlinear(const uint8_t *codes, const float *qmap, in
     return launch_status();
 }
 
+extern "C" int lpmm_code_table_build(const float *qmap, int bits, void *table, void *stream)
+{
+    if (!bits_ok(bits))
+        return LPMM_ERR_SIZE;
+    LPMM_REQUIRE_PTR(qmap);
+    LPMM_REQUIRE_PTR(table);
+    LPMM_REQUIRE_ALIGN(qmap, 4);
+    LPMM_REQUIRE_ALIGN(table, 16);
+    static_assert(LPMM_CODE_TABLE_BYTES == kBucketEntries * 4, "the header's size of a code table");
+    hipLaunchKernelGGL(code_table_kernel, dim3(1), dim3(256), 0, (hipStream_t)stream, qmap, bits,
+                       static_cast<uint32_t *>(table));
+    return launch_status();
+}
+
 extern "C" int lpmm_quant_group_bits(const float *x, int64_t n, int64_t gp_sz, const float *qmap, int bits,
                                      uint8_t *codes, float *max1, void *stream)
 {
+    return lpmm_quant_group_bits_table(x, n, gp_sz, qmap, bits, nullptr, codes, max1, stream);
+}
+
+extern "C" int lpmm_quant_group_bits_table(const float *x, int64_t n, int64_t gp_sz, const float *qmap, int bits,
+                                           const void *table, uint8_t *codes, float *max1, void *stream)
+{
     if (!bits_ok(bits) || n <= 0)
         return LPMM_ERR_SIZE;
+    if (table != nullptr)
+        LPMM_REQUIRE_ALIGN(table, 16);
     if (gp_sz < kGroup || gp_sz > 2 * kBTile || (gp_sz & (gp_sz - 1)) != 0)
         return LPMM_ERR_SIZE;
     LPMM_REQUIRE_PTR(x);
@@ -798,7 +874,8 @@ extern "C" int lpmm_quant_group_bits(const float *x, int64_t n, int64_t gp_sz, c
         // whole tiles in the row layout, the ragged end and the padding by the flat kernel
         const uint32_t wgs = (uint32_t)((full_tiles + kBRowsT - 1) / kBRowsT);
         hipLaunchKernelGGL(quant_group_bits_rows_kernel<kBRowsT>, dim3(wgs), dim3(kBThreads), 0, s, x, full_tiles,
-                           (int)(gp_sz / kGroup), qmap, bits, codes, max1, n_padded);
+                           (int)(gp_sz / kGroup), qmap, bits, static_cast<const uint32_t *>(table), codes, max1,
+                           n_padded);
         const int64_t done = full_tiles * kBTile;
         if (done < n_padded)
             hipLaunchKernelGGL(quant_group_bits_kernel<kBThreads>, dim3((uint32_t)((n_padded - done) / kBTile)),
@@ -854,8 +931,17 @@ extern "C" int lpmm_quant_rank1_bits(const float *x, int64_t rows, int64_t cols,
                                      const float *colmax, const float *qmap, int bits, uint8_t *codes,
                                      void *stream)
 {
+    return lpmm_quant_rank1_bits_table(x, rows, cols, rowmax, colmax, qmap, bits, nullptr, codes, stream);
+}
+
+extern "C" int lpmm_quant_rank1_bits_table(const float *x, int64_t rows, int64_t cols, const float *rowmax,
+                                           const float *colmax, const float *qmap, int bits, const void *table,
+                                           uint8_t *codes, void *stream)
+{
     if (!bits_ok(bits) || rows <= 0 || cols <= 0 || rows > INT64_MAX / cols)
         return LPMM_ERR_SIZE;
+    if (table != nullptr)
+        LPMM_REQUIRE_ALIGN(table, 16);
     LPMM_REQUIRE_PTR(x);
     LPMM_REQUIRE_PTR(rowmax);
     LPMM_REQUIRE_PTR(colmax);
@@ -873,7 +959,8 @@ extern "C" int lpmm_quant_rank1_bits(const float *x, int64_t rows, int64_t cols,
     if (rank1_bits_rows_ok(bits, x, colmax, codes, rows, cols)) {
         const dim3 grid((uint32_t)((cols + kBTile - 1) / kBTile), (uint32_t)((rows + kBRank1Rows - 1) / kBRank1Rows));
         hipLaunchKernelGGL(quant_rank1_bits_rows128_kernel, grid, dim3(kBThreads), 0, (hipStream_t)stream, x, rows, cols,
-                           rowmax, colmax, qmap, bits, codes, (int64_t)tiles * kBTile);
+                           rowmax, colmax, qmap, bits, static_cast<const uint32_t *>(table), codes,
+                           (int64_t)tiles * kBTile);
         return launch_status();
     }
     hipLaunchKernelGGL(quant_rank1_bits_kernel, dim3(tiles), dim3(kBThreads), 0, (hipStream_t)stream, x, n, cols,

@@ -80,7 +80,7 @@ struct MultiR1 {
     float decay, w1, b2, w2, eps;
 };
 
-static_assert(sizeof(MultiR1) + 2 * sizeof(void *) <= 4096, "kernel arguments exceed 4 KB");
+static_assert(sizeof(MultiR1) + 3 * sizeof(void *) + 2 * sizeof(int) <= 4096, "kernel arguments exceed 4 KB");
 static_assert(kR1Max <= kWave, "one tile_start entry per lane");
 
 // tensor of this workgroup (uniform): the number of later tensors whose first tile is not
@@ -135,7 +135,7 @@ __device__ __forceinline__ void write_padding(uint8_t *codes, int64_t n, int64_t
 
 // The launches of the other kernel families (defined next to their kernels); tiles = workgroups.
 void launch_rank1_bits(const MultiR1 &args, uint32_t tiles, const float *qmap_m, const float *qmap_v, int bits_m,
-                       int bits_v, hipStream_t stream);
+                       int bits_v, const uint32_t *table_m, const uint32_t *table_v, hipStream_t stream);
 void launch_rank1_ragged(const MultiR1 &args, uint32_t tiles, const float *qmap_m, const float *qmap_v,
                          hipStream_t stream);
 

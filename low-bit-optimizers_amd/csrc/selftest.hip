@@ -1,6 +1,6 @@
 // Device self-test of the near-exact arithmetic in lpmm_codec.hpp against the compiler's
 // correctly rounded sqrt and division.  Diagnostic only: no counterpart in the reference.
-#include "lpmm_codec.hpp"
+#include "lpmm_search.hpp"
 
 namespace lpmm {
 
@@ -201,7 +201,55 @@ __global__ __launch_bounds__(256) void encoder_scaled_kernel(unsigned long long 
             atomicAdd(counts + 6 + k, c[k]);
 }
 
+// counts[0] bit patterns tried, [1] codes of the table that differ from the search's,
+// [2] 1 if the map qualifies for the table (otherwise nothing is tried).  The table is built in
+// LDS by the steps of the builder kernel and read back through the kernels' own look-up.
+__global__ __launch_bounds__(256) void bucket_sweep_kernel(const float *__restrict__ qmap, int bits,
+                                                           unsigned long long *counts)
+{
+    __shared__ SearchLds tree;
+    __shared__ BucketLds bucket;
+    const SearchFill fill = fill_search_load(qmap, bits);
+    fill_search_store(tree, fill, bits);
+    const BucketFill bucket_fill = fill_buckets_init(bucket, fill, bits);
+    __syncthreads();
+    fill_buckets_scatter(bucket, bucket_fill);
+    __syncthreads();
+    fill_buckets_counts(bucket, bucket_fill, bits);
+    __syncthreads();
+    const bool ok = buckets_ok(bucket);
+    if (blockIdx.x == 0 && threadIdx.x == 0)
+        counts[2] = ok ? 1ull : 0ull;
+    if (!ok)
+        return;
+    const BucketShape s = bucket_shape(bits);
+    const uint32_t nan_code = codes_per_byte(bits) == 1 ? 255u : (1u << bits) - 1u;
+    unsigned long long tried = 0, wrong = 0;
+    const uint64_t tid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const uint64_t nthreads = (uint64_t)gridDim.x * blockDim.x;
+    for (uint64_t i = tid; i < (1ull << 32); i += nthreads) {
+        const float x = __uint_as_float((uint32_t)i);
+        wrong += bucket_code(bucket, s, nan_code, x) != search_code(tree, bits, x);
+        ++tried;
+    }
+    atomicAdd(counts, tried);
+    if (wrong)
+        atomicAdd(counts + 1, wrong);
+}
+
 }  // namespace lpmm
+
+extern "C" int lpmm_selftest_bucket_encoder(const float *qmap, int bits, unsigned long long *counts, void *stream)
+{
+    LPMM_REQUIRE_PTR(qmap);
+    LPMM_REQUIRE_PTR(counts);
+    LPMM_REQUIRE_ALIGN(qmap, 4);
+    LPMM_REQUIRE_ALIGN(counts, 8);
+    if (!lpmm::bucket_bits_ok(bits))
+        return LPMM_ERR_SIZE;
+    hipLaunchKernelGGL(lpmm::bucket_sweep_kernel, dim3(8192), dim3(256), 0, (hipStream_t)stream, qmap, bits, counts);
+    return lpmm::launch_status();
+}
 
 extern "C" int lpmm_selftest_encoders(unsigned long long *counts, void *stream)
 {

@@ -13,7 +13,8 @@ MULTI_MAX = 48  # tensors per launch of the fused step (LPMM_MULTI_MAX in includ
 RANK1_MULTI_MAX = 32  # tensors per launch of the two-pass rank-1 step (kR1Max in csrc/nonfused_rank1.hip)
 SGD_MULTI_MAX = 64  # tensors per launch of the one-pass SGD step (kSgdMax in csrc/sgd.hip)
 V4BIT_MULTI_MAX = 48  # tensors per launch of the one-pass step with an fp32 first moment (kV4Max in csrc/nonfused_m32.hip)
-ABI_VERSION = 1
+ABI_VERSION = 2
+CODE_TABLE_BYTES = 12288  # LPMM_CODE_TABLE_BYTES
 
 _vp = ctypes.c_void_p
 _i64 = ctypes.c_int64
@@ -45,6 +46,9 @@ PROTOTYPES = {
     "lpmm_quant_group_bits": (_int, [_vp, _i64, _i64, _vp, _int, _vp, _vp, _vp]),
     "lpmm_dequant_group_bits": (_int, [_vp, _vp, _vp, _int, _i64, _i64, _vp, _vp]),
     "lpmm_quant_rank1_bits": (_int, [_vp, _i64, _i64, _vp, _vp, _vp, _int, _vp, _vp]),
+    "lpmm_code_table_build": (_int, [_vp, _int, _vp, _vp]),
+    "lpmm_quant_group_bits_table": (_int, [_vp, _i64, _i64, _vp, _int, _vp, _vp, _vp, _vp]),
+    "lpmm_quant_rank1_bits_table": (_int, [_vp, _i64, _i64, _vp, _vp, _vp, _int, _vp, _vp, _vp]),
     "lpmm_dequant_rank1_bits": (_int, [_vp, _vp, _vp, _vp, _int, _i64, _i64, _vp, _vp]),
     "lpmm_nonfused_update": (_int, [_vp] * 4 + [_i64] + [_d] * 6 + [_vp]),
     "lpmm_nonfused_update_multi": (_int, [_vp, _i64] + [_d] * 5 + [_vp]),
@@ -54,6 +58,7 @@ PROTOTYPES = {
     "lpmm_nonfused_adamw_v4bit_rank1_step_multi": (_int, [_vp, _i64, _vp] + [_d] * 5 + [_vp]),
     "lpmm_nonfused_adamw4bit_rank1_mgroup_step_multi": (_int, [_vp, _i64, _vp, _vp, _i64] + [_d] * 5 + [_vp]),
     "lpmm_nonfused_adamw_bits_rank1_step_multi": (_int, [_vp, _i64, _vp, _int, _vp, _int] + [_d] * 5 + [_vp]),
+    "lpmm_nonfused_adamw_bits_rank1_step_multi_table": (_int, [_vp, _i64, _vp, _int, _vp, _vp, _int, _vp] + [_d] * 5 + [_vp]),
     "lpmm_factored_workspace_bytes": (_i64, [_i64, _i64]),
     "lpmm_factored_stats": (_int, [_vp, _i64, _i64, _vp, _vp, _vp, _d, _vp, _vp]),
     "lpmm_factored_stats_static": (_int, [_vp, _i64, _i64, _vp, _vp, _vp, _d, _vp]),
@@ -63,6 +68,7 @@ PROTOTYPES = {
     "lpmm_sgd4bit_step_multi": (_int, [_vp, _i64, _vp] + [_d] * 4 + [_int, _int, _vp]),
     "lpmm_stream_probe": (_int, [_int] + [_vp] * 6 + [_i64, _i64, _vp]),
     "lpmm_selftest_encoders": (_int, [_vp, _vp]),
+    "lpmm_selftest_bucket_encoder": (_int, [_vp, _int, _vp, _vp]),
     "lpmm_selftest_arithmetic": (_int, [_vp, ctypes.c_uint32, ctypes.c_uint64, ctypes.c_uint32, _vp]),
 }
 

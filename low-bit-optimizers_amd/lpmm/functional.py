@@ -246,6 +246,34 @@ def packed_nbytes(numel_scaled, b=4):
     return (numel_scaled + PACK_GROUP - 1) // PACK_GROUP * (PACK_GROUP * storage_bits(b) // 8) + 1
 
 
+_CODE_TABLES = {}
+_CODE_TABLES_MAX = 64
+
+
+def code_table(qmap, b):
+    """The code table of a device map for the quantisers and step kernels of widths other than 4
+    (lpmm_code_table_build): built by one small launch the first time a map tensor is seen and kept
+    with that tensor, so that the kernels find a code with one table read instead of the
+    reference's search (lpmm/cpp_extension/quantization_kernel.cu:397-427; same codes).  The entry
+    holds the map tensor itself: its memory cannot be handed to another map while the table lives,
+    and a map that was modified in place (tensor version) gets a new table."""
+    key = (qmap.data_ptr(), qmap._version, int(b))
+    hit = _CODE_TABLES.get(key)
+    if hit is not None:
+        return hit[1]
+    if qmap.dtype != torch.float32 or not qmap.is_cuda or not qmap.is_contiguous() or qmap.numel() != 2 ** b:
+        raise ValueError("lpmm: code_table needs a contiguous float32 CUDA map of 2^b entries")
+    table = torch.empty(_native.CODE_TABLE_BYTES // 4, dtype=torch.int32, device=qmap.device)
+    with torch.cuda.device(qmap.device):
+        st = _native.lib().lpmm_code_table_build(qmap.data_ptr(), int(b), table.data_ptr(),
+                                                 _native.current_stream(qmap.device))
+    _native.check(st, "code_table_build")
+    if len(_CODE_TABLES) >= _CODE_TABLES_MAX:
+        _CODE_TABLES.pop(next(iter(_CODE_TABLES)))
+    _CODE_TABLES[key] = (qmap, table)
+    return table
+
+
 def _group_gp_sz_ok(gp_sz):
     return gp_sz in (128, 256, 512, 1024, 2048, 4096)
 
@@ -266,8 +294,9 @@ def quant_group_(x, qmap, gp_sz, codes=None, max1=None, b=4):
             st = lib.lpmm_quant_group(x.data_ptr(), n, gp_sz, qmap.data_ptr(), codes.data_ptr(), max1.data_ptr(),
                                       stream)
         else:
-            st = lib.lpmm_quant_group_bits(x.data_ptr(), n, gp_sz, qmap.data_ptr(), b, codes.data_ptr(),
-                                           max1.data_ptr(), stream)
+            st = lib.lpmm_quant_group_bits_table(x.data_ptr(), n, gp_sz, qmap.data_ptr(), b,
+                                                 code_table(qmap, b).data_ptr(), codes.data_ptr(), max1.data_ptr(),
+                                                 stream)
     _native.check(st, "quant_group")
     return codes, max1
 
@@ -292,8 +321,9 @@ def quant_rank1_(x, qmap, codes=None, b=4):
             st = lib.lpmm_quant_rank1(x.data_ptr(), rows, cols, rowmax.data_ptr(), colmax.data_ptr(),
                                       qmap.data_ptr(), codes.data_ptr(), stream)
         else:
-            st = lib.lpmm_quant_rank1_bits(x.data_ptr(), rows, cols, rowmax.data_ptr(), colmax.data_ptr(),
-                                           qmap.data_ptr(), b, codes.data_ptr(), stream)
+            st = lib.lpmm_quant_rank1_bits_table(x.data_ptr(), rows, cols, rowmax.data_ptr(), colmax.data_ptr(),
+                                                 qmap.data_ptr(), b, code_table(qmap, b).data_ptr(),
+                                                 codes.data_ptr(), stream)
     _native.check(st, "quant_rank1")
     return codes, max_dims
 

@@ -23,7 +23,7 @@ import numpy as np
 import torch
 
 from .. import _native
-from ..functional import packed_nbytes, vectorwise_dequant, vectorwise_quant
+from ..functional import code_table, packed_nbytes, vectorwise_dequant, vectorwise_quant
 from .optimizer import LowBitOptimizer
 
 __all__ = ["AdamW"]
@@ -414,12 +414,12 @@ class AdamW(LowBitOptimizer):
             records.launched()
 
         def launch_rank1_bits(key, records):
-            dev, qm_ptr, qv_ptr = key
+            dev, qm_ptr, qv_ptr, tm_ptr, tv_ptr = key
             table = np.array(records, dtype=_native.NONFUSED_RANK1_TENSOR)
             with torch.cuda.device(dev):
-                st = lib.lpmm_nonfused_adamw_bits_rank1_step_multi(
-                    table.ctypes.data, len(records), qm_ptr, md_m["b"], qv_ptr, md_v["b"], beta1, beta2, lr, wd, eps,
-                    _native.current_stream(dev))
+                st = lib.lpmm_nonfused_adamw_bits_rank1_step_multi_table(
+                    table.ctypes.data, len(records), qm_ptr, md_m["b"], tm_ptr, qv_ptr, md_v["b"], tv_ptr, beta1, beta2,
+                    lr, wd, eps, _native.current_stream(dev))
             _native.check(st, "non-fused AdamW step (5-8-bit states, rank-1 second moment)")
             records.launched()
 
@@ -452,8 +452,9 @@ class AdamW(LowBitOptimizer):
                         pending.clear()
                     continue
             if bits_rank1 and en_m and en_v and p.dim() == 2 and p.shape[1] % 128 == 0:
-                key = (p.device, state["exp_avg_qstate"]["qmap"].data_ptr(),
-                       state["exp_avg_sq_qstate"]["qmap"].data_ptr())
+                qm, qv = state["exp_avg_qstate"]["qmap"], state["exp_avg_sq_qstate"]["qmap"]
+                key = (p.device, qm.data_ptr(), qv.data_ptr(), code_table(qm, md_m["b"]).data_ptr(),
+                       code_table(qv, md_v["b"]).data_ptr())
                 pending = batched_rank1_bits.setdefault(key, _Batch())
                 mc, ms = self._group_state(p, state, "exp_avg", b=md_m["b"])
                 pending.append((dense.data_ptr(), grad.data_ptr(), mc, ms) + self._rank1_state(p, state, pending, b=md_v["b"])

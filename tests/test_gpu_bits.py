@@ -116,6 +116,118 @@ def test_quant_dequant_group_bits(oracle, bits, n, gp_sz):
         np.testing.assert_array_equal(to_np(out), oracle.dequant_group_bits(want_codes, want_max1, qmap, bits, n, gp_sz))
 
 
+@pytest.mark.parametrize("bits", [3, 5, 6, 7, 8])
+def test_bucket_table_equals_the_search_on_all_floats(oracle, bits):
+    """Maps that qualify are encoded with one table read (sign, exponent and leading mantissa bits
+    pick a bucket that holds at most one midpoint) instead of the search: both on the device over
+    all 2^32 bit patterns.  The reference's signed dynamic-exponent maps must qualify; a map with a
+    repeated entry must not (the search's answer for it depends on more than the midpoints)."""
+    lib = _lib()
+    dynamic = oracle.create_dynamic_map(True, bits - 1, bits)
+    repeated = dynamic.copy()
+    repeated[3] = repeated[2]
+    cases = [(dynamic, True), (oracle.create_pow_map(bits, True, 2), None), (oracle.create_pow_map(bits, False, 3), None),
+             (oracle.create_pow_map(bits, False, 1), None), (repeated, False)]
+    for qmap, qualifies in cases:
+        assert qmap.size == 2 ** bits
+        counts = torch.zeros(3, dtype=torch.int64, device="cuda")
+        assert lib.lpmm_selftest_bucket_encoder(to_dev(qmap).data_ptr(), bits, counts.data_ptr(), _stream()) == 0
+        torch.cuda.synchronize()
+        tried, wrong, ok = counts.tolist()
+        if qualifies is not None:
+            assert bool(ok) == qualifies
+        assert (tried, wrong) == ((2 ** 32, 0) if ok else (0, 0))
+
+
+def _code_table(dq, bits):
+    from lpmm import _native
+
+    table = torch.full((_native.CODE_TABLE_BYTES // 4,), 0x5A5A5A5A, dtype=torch.int32, device="cuda")
+    assert _lib().lpmm_code_table_build(dq.data_ptr(), bits, table.data_ptr(), _stream()) == 0
+    return table
+
+
+@pytest.mark.parametrize("bits", BITS)
+def test_code_table_says_what_the_map_allows(oracle, bits):
+    """Last word of a table: bits << 8 | 0 (search), 1 (the evenly spaced map's closed form), 2 (table)."""
+    even = oracle.create_pow_map(bits, False, 1)
+    cases = [(even, 1)]
+    if bits >= 2:
+        dynamic = oracle.create_dynamic_map(True, bits - 1, bits)
+        repeated = dynamic.copy()
+        repeated[1] = repeated[0]
+        cases += [(dynamic, 2 if bits >= 3 else 0), (repeated, 0)]
+    for qmap, mode in cases:
+        table = _code_table(to_dev(qmap), bits)
+        torch.cuda.synchronize()
+        assert int(table[-1]) == (bits << 8 | mode), (bits, mode, hex(int(table[-1])))
+    lib = _lib()
+    assert lib.lpmm_code_table_build(to_dev(even).data_ptr(), 9, table.data_ptr(), _stream()) != 0
+    assert lib.lpmm_code_table_build(to_dev(even).data_ptr(), bits, table.data_ptr() + 4, _stream()) != 0
+
+
+@pytest.mark.parametrize("with_table", [False, True])
+@pytest.mark.parametrize("bits", [5, 6, 7, 8])
+@pytest.mark.parametrize("gp_sz", [128, 512])
+def test_quant_group_bits_with_the_dynamic_map(oracle, bits, gp_sz, with_table):
+    """Whole tiles through the row-layout kernel with the map of configs/default_{5,6,7,8}b.yml:
+    groups whose maximum is 1 hold every entry of the map, every midpoint and the floats next to
+    them, so that their quotients are those values exactly; random groups follow."""
+    lib = _lib()
+    rng = np.random.default_rng(bits * 7 + gp_sz)
+    qmap = oracle.create_dynamic_map(True, bits - 1, bits)
+    mids = oracle.midpoints(qmap)
+    two = np.float32(2)
+    special = np.concatenate([qmap, mids, np.nextafter(mids, two), np.nextafter(mids, -two), np.nextafter(qmap, two),
+                              np.nextafter(qmap, -two), [0.0, -0.0, 1e-30, -1e-30, 2.0 ** -24, -2.0 ** -24]]).astype(np.float32)
+    special = special[np.abs(special) <= 1.0]
+    per = gp_sz - 1
+    groups = -(-special.size // per)
+    head = np.zeros((groups, gp_sz), np.float32)
+    head[:, 0] = 1.0
+    head[:, 1:].reshape(-1)[:special.size] = special
+    n = 2048 * 24 + 136
+    x = (rng.standard_t(3, n) * 1e-3).astype(np.float32)
+    x[:head.size] = head.reshape(-1)
+    assert head.size < n - 4096
+    want_codes, want_max1 = oracle.quant_group_bits(x, qmap, bits, gp_sz)
+    codes = torch.full((want_codes.size,), 0x5A, dtype=torch.uint8, device="cuda")
+    max1 = torch.empty(want_max1.size, dtype=torch.float32, device="cuda")
+    dq = to_dev(qmap)
+    if with_table:
+        table = _code_table(dq, bits)
+        assert int(table[-1]) == (bits << 8 | 2)
+        st = lib.lpmm_quant_group_bits_table(to_dev(x).data_ptr(), n, gp_sz, dq.data_ptr(), bits, table.data_ptr(),
+                                             codes.data_ptr(), max1.data_ptr(), _stream())
+    else:
+        st = lib.lpmm_quant_group_bits(to_dev(x).data_ptr(), n, gp_sz, dq.data_ptr(), bits, codes.data_ptr(),
+                                       max1.data_ptr(), _stream())
+    assert st == 0
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(to_np(max1), want_max1)
+    np.testing.assert_array_equal(to_np(codes), want_codes)
+
+
+def test_a_table_of_another_width_or_of_a_map_that_does_not_qualify_means_the_search(oracle):
+    lib = _lib()
+    rng = np.random.default_rng(5)
+    n = 2048 * 6
+    x = (rng.standard_t(3, n) * 1e-3).astype(np.float32)
+    dx = to_dev(x)
+    dynamic8 = oracle.create_dynamic_map(True, 7, 8)
+    repeated = oracle.create_dynamic_map(True, 5, 6)
+    repeated[5] = repeated[4]
+    for qmap, bits, table_map, table_bits in [(oracle.create_dynamic_map(True, 5, 6), 6, dynamic8, 8), (repeated, 6, repeated, 6)]:
+        want_codes, want_max1 = oracle.quant_group_bits(x, qmap, bits, 128)
+        table = _code_table(to_dev(table_map), table_bits)
+        codes = torch.full((want_codes.size,), 0x5A, dtype=torch.uint8, device="cuda")
+        max1 = torch.empty(want_max1.size, dtype=torch.float32, device="cuda")
+        assert lib.lpmm_quant_group_bits_table(dx.data_ptr(), n, 128, to_dev(qmap).data_ptr(), bits, table.data_ptr(),
+                                               codes.data_ptr(), max1.data_ptr(), _stream()) == 0
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(to_np(codes), want_codes)
+
+
 def test_width_4_generic_kernels_equal_the_fast_path(oracle, qmaps):
     """The any-width kernels at width 4 and the 4-bit kernels give the same bytes."""
     lib = _lib()
@@ -139,12 +251,25 @@ def test_width_4_generic_kernels_equal_the_fast_path(oracle, qmaps):
 @pytest.mark.parametrize("bits", [2, 3, 5, 8])
 @pytest.mark.parametrize("shape", [(64, 80), (33, 1000), (257, 1029), (70, 256), (5, 2176), (130, 128)])
 def test_rank1_bits(oracle, bits, shape):
+    _rank1_bits_case(oracle, bits, shape, oracle.create_pow_map(bits, False, 1), False)
+
+
+@pytest.mark.parametrize("with_table", [False, True])
+@pytest.mark.parametrize("bits", [5, 8])
+@pytest.mark.parametrize("shape", [(70, 256), (5, 2176), (130, 128), (33, 1000)])
+def test_rank1_bits_with_the_dynamic_map(oracle, bits, shape, with_table):
+    """A signed map under the rank-1 scaling (values of both signs), with and without its code table."""
+    _rank1_bits_case(oracle, bits, shape, oracle.create_dynamic_map(True, bits - 1, bits), with_table, signed=True)
+
+
+def _rank1_bits_case(oracle, bits, shape, qmap, with_table, signed=False):
     lib = _lib()
     r, c = shape
     rng = np.random.default_rng(r + bits)
-    qmap = oracle.create_pow_map(bits, False, 1)
     x = ((rng.standard_normal(shape) * np.exp(rng.standard_normal((r, 1))) * np.exp(rng.standard_normal((1, c)))) ** 2
          ).astype(np.float32)
+    if signed:
+        x *= rng.choice([-1.0, 1.0], shape).astype(np.float32)
     x[3, :] = 0.0
     x[:, 7] = 0.0
     x[4, :] *= 1e-25  # a row whose scales lie below the range of the reciprocal-based division
@@ -152,8 +277,13 @@ def test_rank1_bits(oracle, bits, shape):
     want = oracle.quant_rank1_bits(x, rowmax, colmax, qmap, bits)
     dx, dq, dr, dc = to_dev(x), to_dev(qmap), to_dev(rowmax), to_dev(colmax)
     codes = torch.full((want.size,), 0x5A, dtype=torch.uint8, device="cuda")
-    st = lib.lpmm_quant_rank1_bits(dx.data_ptr(), r, c, dr.data_ptr(), dc.data_ptr(), dq.data_ptr(), bits,
-                                   codes.data_ptr(), _stream())
+    if with_table:
+        table = _code_table(dq, bits)
+        st = lib.lpmm_quant_rank1_bits_table(dx.data_ptr(), r, c, dr.data_ptr(), dc.data_ptr(), dq.data_ptr(), bits,
+                                             table.data_ptr(), codes.data_ptr(), _stream())
+    else:
+        st = lib.lpmm_quant_rank1_bits(dx.data_ptr(), r, c, dr.data_ptr(), dc.data_ptr(), dq.data_ptr(), bits,
+                                       codes.data_ptr(), _stream())
     assert st == 0
     torch.cuda.synchronize()
     np.testing.assert_array_equal(to_np(codes), want)

@@ -80,13 +80,32 @@ class _Tensor:
         self.p.copy_(torch.from_numpy(self.host_p))
 
 
-def _step_all(oracle, tensors, grads, bits, qm, qv, dqm, dqv, step):
+def _code_table(dq, bits):
+    nat = _native()
+    table = torch.empty(nat.CODE_TABLE_BYTES // 4, dtype=torch.int32, device="cuda")
+    assert nat.lib().lpmm_code_table_build(dq.data_ptr(), bits, table.data_ptr(),
+                                           torch.cuda.current_stream().cuda_stream) == 0
+    return table
+
+
+def _step_all(oracle, tensors, grads, bits, qm, qv, dqm, dqv, step, with_tables=False):
+    """with_tables: the code tables of the two maps (one table read per value instead of the search;
+    the dynamic-exponent map of the first moment qualifies, the second moment's evenly spaced map
+    takes its closed form either way)."""
     nat = _native()
     lib = nat.lib()
     table = np.array([t.record(g, step) for t, g in zip(tensors, grads)], dtype=nat.NONFUSED_RANK1_TENSOR)
-    st = lib.lpmm_nonfused_adamw_bits_rank1_step_multi(table.ctypes.data, len(tensors), dqm.data_ptr(), bits,
-                                                       dqv.data_ptr(), bits, H["beta1"], H["beta2"], H["lr"],
-                                                       H["wd"], H["eps"], torch.cuda.current_stream().cuda_stream)
+    stream = torch.cuda.current_stream().cuda_stream
+    if with_tables:
+        tm, tv = _code_table(dqm, bits), _code_table(dqv, bits)
+        assert int(tm[-1]) == (bits << 8 | 2) and int(tv[-1]) == (bits << 8 | 1)
+        st = lib.lpmm_nonfused_adamw_bits_rank1_step_multi_table(
+            table.ctypes.data, len(tensors), dqm.data_ptr(), bits, tm.data_ptr(), dqv.data_ptr(), bits, tv.data_ptr(),
+            H["beta1"], H["beta2"], H["lr"], H["wd"], H["eps"], stream)
+    else:
+        st = lib.lpmm_nonfused_adamw_bits_rank1_step_multi(table.ctypes.data, len(tensors), dqm.data_ptr(), bits,
+                                                           dqv.data_ptr(), bits, H["beta1"], H["beta2"], H["lr"],
+                                                           H["wd"], H["eps"], stream)
     assert st == 0, lib.lpmm_status_string(st)
     for t, g in zip(tensors, grads):
         t.oracle_step(oracle, g, qm, qv, step)
@@ -103,8 +122,9 @@ def _grad(rng, t, zero_rows=0):
     return g
 
 
+@pytest.mark.parametrize("with_tables", [False, True])
 @pytest.mark.parametrize("bits", [5, 6, 7, 8])
-def test_bits_two_pass_matches_staged_oracle(oracle, bits):
+def test_bits_two_pass_matches_staged_oracle(oracle, bits, with_tables):
     qm, qv = _maps(oracle, bits)
     dqm, dqv = to_dev(qm), to_dev(qv)
     rng = np.random.default_rng(70 + bits)
@@ -114,13 +134,14 @@ def test_bits_two_pass_matches_staged_oracle(oracle, bits):
     tensors = [_Tensor(r, c, bits, rng) for r, c in shapes]
     for step in range(1, 4):
         grads = [_grad(rng, t) for t in tensors]
-        _step_all(oracle, tensors, grads, bits, qm, qv, dqm, dqv, step)
+        _step_all(oracle, tensors, grads, bits, qm, qv, dqm, dqv, step, with_tables)
         for t in tensors:
             t.check(f"{bits} bits, {t.rows}x{t.cols} step {step}")
 
 
+@pytest.mark.parametrize("with_tables", [False, True])
 @pytest.mark.parametrize("bits", [5, 8])
-def test_bits_all_zero_rows(oracle, bits):
+def test_bits_all_zero_rows(oracle, bits, with_tables):
     """Rows whose gradient stays zero: scale 0, 0/0 -> NaN -> the byte 255."""
     qm, qv = _maps(oracle, bits)
     dqm, dqv = to_dev(qm), to_dev(qv)
@@ -128,7 +149,7 @@ def test_bits_all_zero_rows(oracle, bits):
     tensors = [_Tensor(r, c, bits, rng) for r, c in [(40, 384), (70, 128)]]
     for step in (1, 2):
         grads = [_grad(rng, t, z) for t, z in zip(tensors, (34, 3))]
-        _step_all(oracle, tensors, grads, bits, qm, qv, dqm, dqv, step)
+        _step_all(oracle, tensors, grads, bits, qm, qv, dqm, dqv, step, with_tables)
         for t in tensors:
             t.check(f"{bits} bits, {t.rows}x{t.cols} step {step}")
 
