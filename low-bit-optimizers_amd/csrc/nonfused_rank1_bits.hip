@@ -8,12 +8,15 @@ namespace lpmm {
 // ---------------------------------------------------------------------------------------
 // The same two passes for code widths of 5 to 8 bits (lpmm/configs/default_{5,6,7,8}b.yml): one
 // code per byte (lpmm/cpp_extension/quantization_kernel.cu:516-533, :656-669), maps of 2^bits
-// entries in LDS, decoded by indexing and encoded by the reference's search (:397-427) as the
-// stand-alone quantisers of these widths do it.  Same tiles and statistics as above; a lane's
-// eight codes are two dwords.  21.06 bytes per parameter cross HBM (p 8, g 4 + 4, m codes 2,
-// v codes 1 + 2, scales).  LLaMA-7B-shaped set: 25.1 ms per step with 5 bits, 25.3 ms with 8
-// (the staged path 67.6 ms); the second moment's evenly spaced map takes the closed form of
-// lpmm_search.hpp, so only the first moment is searched.
+// entries in LDS, decoded by indexing and encoded as the stand-alone quantisers of these widths
+// do it: by the reference's search (:397-427), by one read of the map's code table where the
+// caller passes one, or by the closed form of the evenly spaced map (the second moment's in every
+// shipped configuration; lpmm_search.hpp).  Same tiles and statistics as above; a lane's eight
+// codes are two dwords.  21.06 bytes per parameter cross HBM (p 8, g 4 + 4, m codes 2, v codes
+// 1 + 2, scales).  LLaMA-7B-shaped set: 25.0 ms per step with 5 bits, 25.3 ms with 8 (the staged
+// path 67.6 ms).  Both passes run within 5 % of the rate of their 4-bit counterparts per byte:
+// with the arithmetic taken out, with the table instead of the search and with 8-byte instead of
+// 4-byte code accesses they take the same time -- the tile structure sets it, not the codes.
 // ---------------------------------------------------------------------------------------
 __device__ __forceinline__ uint32_t byte_of(uint32_t w0, uint32_t w1, int k)
 {
