@@ -59,13 +59,13 @@ struct PassRegs {
     float4 a0, a1, b0, b1;
     float4 c0, c1;  // fp32 first moment only
     uint32_t m0, m1, v0, v1;
-    float sm, ro;
+    float sm, ro, ro1;  // ro1: the second half's row statistic (folded rows; otherwise ro)
 };
 
-template <int MODE>
-__device__ __forceinline__ void pass_fetch(const TensorR1 &t, uint32_t cg, int lane16, int64_t r, PassRegs &x)
+template <int MODE, bool FOLD>
+__device__ __forceinline__ void pass_fetch(const TensorR1 &t, const Fold &f, uint32_t cg, int lane16, int64_t r, PassRegs &x)
 {
-    const int64_t grp = r * t.col_blocks + cg;
+    const int64_t grp = r * f.col_blocks + cg;
     const int64_t gbase = grp * kGroup;
     const float *pp = t.p + gbase + lane16 * 4;
     const float *gp = t.g + gbase + lane16 * 4;
@@ -86,7 +86,14 @@ __device__ __forceinline__ void pass_fetch(const TensorR1 &t, uint32_t cg, int l
     }
     x.v0 = load_u16(vcp);
     x.v1 = load_u16(vcp + 16);
-    x.ro = t.row_old[r];
+    if (FOLD) {
+        int64_t r0, r1;
+        fold_rows(f, r, cg, r0, r1);
+        x.ro = t.row_old[r0];
+        x.ro1 = t.row_old[r1];
+    } else {
+        x.ro = x.ro1 = t.row_old[r];
+    }
 }
 
 #ifndef LPMM_R1_WAVES
@@ -94,7 +101,7 @@ __device__ __forceinline__ void pass_fetch(const TensorR1 &t, uint32_t cg, int l
 #endif
 // 4 waves per SIMD, up to 128 registers: the first pass's operands stay live across the prologue and
 // the lane's column statistics across the passes (with 5 or 6 the compiler spills or re-reads)
-template <int MODE>
+template <int MODE, bool FOLD>
 __global__ __launch_bounds__(kThreads, LPMM_R1_WAVES) void rank1_update_kernel(const MultiR1 args, const float *__restrict__ qmap_m,
                                                                 const float *__restrict__ qmap_v)
 {
@@ -104,8 +111,9 @@ __global__ __launch_bounds__(kThreads, LPMM_R1_WAVES) void rank1_update_kernel(c
     const TensorR1 &t = args.t[lo];
     const uint32_t tl = blockIdx.x - args.tile_start[lo];
     const int lane16 = threadIdx.x & 15, drow = threadIdx.x >> 4;
-    const Geometry q = geometry(t, tl, drow);
-    const int64_t cols = (int64_t)t.col_blocks * kGroup;
+    const Fold f = fold_of<FOLD>(t);
+    const Geometry q = geometry(t.tile, f.col_blocks, tl, drow);
+    const int64_t cols = (int64_t)f.col_blocks * kGroup;
     const int64_t tile_c0 = (int64_t)q.col_tile * q.wide * kGroup;
 
     // Order of the prologue: the small loads that feed LDS (maps, encode table, the tile's current
@@ -118,12 +126,14 @@ __global__ __launch_bounds__(kThreads, LPMM_R1_WAVES) void rank1_update_kernel(c
 #pragma unroll
     for (int i = 0; i < kColPerThread; ++i) {
         const int j = threadIdx.x + i * kThreads;
-        co_in[i] = (j < q.wide * kGroup && tile_c0 + j < cols) ? __float_as_uint(t.col_old[tile_c0 + j]) : 0u;
+        co_in[i] = (j < q.wide * kGroup && tile_c0 + j < cols)
+                       ? __float_as_uint(t.col_old[FOLD ? fold_col(f, (uint32_t)(tile_c0 + j)) : tile_c0 + j])
+                       : 0u;
     }
-    const bool row_live = q.cg < t.col_blocks;  // the whole DPP row
+    const bool row_live = q.cg < f.col_blocks;  // the whole DPP row
     PassRegs x;
-    if (row_live && q.row0 < t.rows)
-        pass_fetch<MODE>(t, q.cg, lane16, q.row0, x);
+    if (row_live && q.row0 < f.rows)
+        pass_fetch<MODE, FOLD>(t, f, q.cg, lane16, q.row0, x);
     lds_fill_store(lds, fill);
     for (int j = threadIdx.x; j < kMaxWide * (int)kRedSlotWords; j += kThreads)
         colred[j] = 0u;
@@ -144,7 +154,7 @@ __global__ __launch_bounds__(kThreads, LPMM_R1_WAVES) void rank1_update_kernel(c
 
     if (MODE == kMCodes128 && tl == 0) {
         const float z[kEltsPerLane] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
-        const int64_t n = t.rows * cols;
+        const int64_t n = f.rows * cols;
         write_padding(t.mc, n, (n + LPMM_PACK_GROUP - 1) / LPMM_PACK_GROUP * LPMM_PACK_GROUP,
                       encode8_plain(lds, kLdsQ0, kind_m, z));
     }
@@ -159,15 +169,15 @@ __global__ __launch_bounds__(kThreads, LPMM_R1_WAVES) void rank1_update_kernel(c
 #pragma unroll 1
         for (int it = 0; it < q.passes; ++it) {
             const int64_t r = q.row0 + it * q.step;
-            if (r >= t.rows)
+            if (r >= f.rows)
                 break;
             if (it > 0)
-                pass_fetch<MODE>(t, q.cg, lane16, r, x);
-            const int64_t grp = r * t.col_blocks + q.cg;
+                pass_fetch<MODE, FOLD>(t, f, q.cg, lane16, r, x);
+            const int64_t grp = r * f.col_blocks + q.cg;
             const int64_t gbase = grp * kGroup;
             float *pp = t.p + gbase + lane16 * 4;
             const uint32_t wv = x.v0 | (x.v1 << 16);
-            const float ro = x.ro;
+            const float ro = x.ro, ro1 = FOLD ? x.ro1 : x.ro;
             float pv[kEltsPerLane], gv[kEltsPerLane], m[kEltsPerLane], v[kEltsPerLane];
             unpack8(x.a0, x.a1, pv);
             unpack8(x.b0, x.b1, gv);
@@ -178,15 +188,19 @@ __global__ __launch_bounds__(kThreads, LPMM_R1_WAVES) void rank1_update_kernel(c
                 unpack8(x.c0, x.c1, m);
 
             const Nibbles nv = split_nibbles(wv);
-            float amax_m = 0.0f, vmax = 0.0f;
+            float amax_m = 0.0f, vmax = 0.0f, vmax1 = 0.0f;  // vmax1: the second half's (folded rows)
 #pragma unroll
             for (int k = 0; k < kEltsPerLane; ++k) {
                 if (!M32)
                     m[k] = decode_nibble(lds, kLdsQ0, nm, k) * sm;
-                v[k] = decode_nibble(lds, kLdsQ1, nv, k) * ((co[k] < ro) ? co[k] : ro);
+                const float rk = (FOLD && k >= 4) ? ro1 : ro;
+                v[k] = decode_nibble(lds, kLdsQ1, nv, k) * ((co[k] < rk) ? co[k] : rk);
                 nonfused_elt(pv[k], gv[k], m[k], v[k], h);
                 amax_m = fmaxf(amax_m, fabsf(m[k]));
-                vmax = fmaxf(vmax, v[k]);
+                if (FOLD && k >= 4)
+                    vmax1 = fmaxf(vmax1, v[k]);
+                else
+                    vmax = fmaxf(vmax, v[k]);
                 atomicMax(red + k * 16, __float_as_uint(v[k]));
             }
             uint32_t cm = 0;
@@ -197,6 +211,8 @@ __global__ __launch_bounds__(kThreads, LPMM_R1_WAVES) void rank1_update_kernel(c
                 if (MODE == kMCodes128)
                     cm = encode8_scaled(lds, kLdsQ0, kind_m, m, amax_m);
             }
+            if (FOLD)
+                vmax1 = row16_max(vmax1);
 
             store4(pp, make_float4(pv[0], pv[1], pv[2], pv[3]));
             store4(pp + 64, make_float4(pv[4], pv[5], pv[6], pv[7]));
@@ -213,8 +229,16 @@ __global__ __launch_bounds__(kThreads, LPMM_R1_WAVES) void rank1_update_kernel(c
             } else if (lane16 == 0) {
                 atomic_max_nonneg(t.ms_new + (grp >> t.m_lg), amax_m);
             }
-            if (lane16 == 0)
-                atomic_max_nonneg(t.row_new + r, vmax);
+            if (lane16 == 0) {
+                if (FOLD) {
+                    int64_t r0, r1;
+                    fold_rows(f, r, q.cg, r0, r1);
+                    atomic_max_nonneg(t.row_new + r0, vmax);
+                    atomic_max_nonneg(t.row_new + r1, vmax1);
+                } else {
+                    atomic_max_nonneg(t.row_new + r, vmax);
+                }
+            }
         }
     }
     // the column maxima meet in LDS: nothing below depends on the global stores still in flight
@@ -224,12 +248,13 @@ __global__ __launch_bounds__(kThreads, LPMM_R1_WAVES) void rank1_update_kernel(c
         const int w = j & (kGroup - 1);
         const int k = ((w >> 6) << 2) | (w & 3), l = (w >> 2) & 15;
         if (tile_c0 + j < cols)
-            atomic_max_nonneg(t.col_new + tile_c0 + j, __uint_as_float(colred[(j >> 7) * kRedSlotWords + k * 16 + l]));
+            atomic_max_nonneg(t.col_new + (FOLD ? fold_col(f, (uint32_t)(tile_c0 + j)) : tile_c0 + j),
+                              __uint_as_float(colred[(j >> 7) * kRedSlotWords + k * 16 + l]));
     }
 }
 
 // MWIDE: the first moment's groups are wider than 128 values; its codes are written here too.
-template <bool MWIDE>
+template <bool MWIDE, bool FOLD>
 __global__ __launch_bounds__(kThreads) void rank1_requant_kernel(const MultiR1 args, const float *__restrict__ qmap_m,
                                                                  const float *__restrict__ qmap_v)
 {
@@ -246,13 +271,15 @@ __global__ __launch_bounds__(kThreads) void rank1_requant_kernel(const MultiR1 a
     const TensorR1 &t = args.t[lo];
     const uint32_t tl = blockIdx.x - args.tile_start[lo];
     const int lane16 = threadIdx.x & 15, drow = threadIdx.x >> 4;
-    const Geometry q = geometry(t, tl, drow);
-    const int64_t cols = (int64_t)t.col_blocks * kGroup;
+    const Fold f = fold_of<FOLD>(t);
+    const Geometry q = geometry(t.tile, f.col_blocks, tl, drow);
+    const int64_t cols = (int64_t)f.col_blocks * kGroup;
     const int64_t tile_c0 = (int64_t)q.col_tile * q.wide * kGroup;
     for (int j = threadIdx.x; j < q.wide * kGroup; j += kThreads) {
         const bool in = tile_c0 + j < cols;
-        const float cn = in ? t.col_new[tile_c0 + j] : 0.0f;
-        lds[kColOld / 4 + j] = in ? __float_as_uint(t.col_old[tile_c0 + j]) : 0u;
+        const int64_t c = FOLD ? fold_col(f, (uint32_t)(tile_c0 + j)) : tile_c0 + j;
+        const float cn = in ? t.col_new[c] : 0.0f;
+        lds[kColOld / 4 + j] = in ? __float_as_uint(t.col_old[c]) : 0u;
         lds[kColNew / 4 + j] = __float_as_uint(cn);
         lds[kColRcp / 4 + j] = __float_as_uint(1.0f / cn);
     }
@@ -264,7 +291,7 @@ __global__ __launch_bounds__(kThreads) void rank1_requant_kernel(const MultiR1 a
 
     if (tl == 0) {
         const float z[kEltsPerLane] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
-        const int64_t n = t.rows * cols;
+        const int64_t n = f.rows * cols;
         const int64_t n_pack = (n + LPMM_PACK_GROUP - 1) / LPMM_PACK_GROUP * LPMM_PACK_GROUP;
         write_padding(t.vc, n, n_pack, encode8_plain(lds, kVMap, kind, z));
         if (MWIDE) {
@@ -289,7 +316,7 @@ __global__ __launch_bounds__(kThreads) void rank1_requant_kernel(const MultiR1 a
                 t.mc[n_all / 2] = 0;
         }
     }
-    if (q.cg >= t.col_blocks)
+    if (q.cg >= f.col_blocks)
         return;
 
     // a lane keeps its eight columns through all passes: their old and new statistics and the
@@ -309,9 +336,9 @@ __global__ __launch_bounds__(kThreads) void rank1_requant_kernel(const MultiR1 a
 #pragma unroll 1
     for (int it = 0; it < q.passes; ++it) {
         const int64_t r = q.row0 + it * q.step;
-        if (r >= t.rows)
+        if (r >= f.rows)
             break;
-        const int64_t gbase = (r * t.col_blocks + q.cg) * kGroup;
+        const int64_t gbase = (r * f.col_blocks + q.cg) * kGroup;
         const float *gp = t.g + gbase + lane16 * 4;
         const float4 b0 = load4(gp), b1 = load4(gp + 64);
         uint32_t *vcp = reinterpret_cast<uint32_t *>(t.vc + (gbase >> 1)) + code_dword;
@@ -326,13 +353,18 @@ __global__ __launch_bounds__(kThreads) void rank1_requant_kernel(const MultiR1 a
             ms_old = t.ms[mg];
             ms_new = t.ms_new[mg];
         }
-        const float ro = t.row_old[r], rn = t.row_new[r];
+        int64_t r0 = r, r1 = r;  // the tensor rows of the DPP row's two halves
+        if (FOLD)
+            fold_rows(f, r, q.cg, r0, r1);
+        const float ro = t.row_old[r0], rn = t.row_new[r0];
+        const float ro1 = FOLD ? t.row_old[r1] : ro, rn1 = FOLD ? t.row_new[r1] : rn;
         float gv[kEltsPerLane], v[kEltsPerLane], x[kEltsPerLane];
         unpack8(b0, b1, gv);
         const Nibbles nv = split_nibbles(wv);
 #pragma unroll
         for (int k = 0; k < kEltsPerLane; ++k) {
-            v[k] = decode_nibble(lds, kVMap, nv, k) * ((co[k] < ro) ? co[k] : ro);
+            const float rk = (FOLD && k >= 4) ? ro1 : ro;
+            v[k] = decode_nibble(lds, kVMap, nv, k) * ((co[k] < rk) ? co[k] : rk);
             nonfused_second_moment(v[k], gv[k], h);
         }
         if (MWIDE) {
@@ -347,20 +379,23 @@ __global__ __launch_bounds__(kThreads) void rank1_requant_kernel(const MultiR1 a
         uint32_t w;
         // every scale the wave divides by is a column or the row statistic: all in the range in
         // which the reciprocal is exact?
-        if (kind == kMapStdV && __all(cols_safe && rc_safe(rn))) {
+        if (kind == kMapStdV && __all(cols_safe && rc_safe(rn) && rc_safe(rn1))) {
             // the correctly rounded reciprocal of whichever statistic is the scale, then one
             // multiply and two fmas: the correctly rounded quotient (v <= scale by construction)
-            const float rcr = rcp_exact(rn);
+            const float rcr = rcp_exact(rn), rcr1 = FOLD ? rcp_exact(rn1) : rcr;
 #pragma unroll
             for (int k = 0; k < kEltsPerLane; ++k) {
-                const bool by_col = cn[k] < rn;
-                x[k] = div_by_rc(v[k], by_col ? cn[k] : rn, by_col ? rcn[k] : rcr);
+                const float rnk = (FOLD && k >= 4) ? rn1 : rn, rck = (FOLD && k >= 4) ? rcr1 : rcr;
+                const bool by_col = cn[k] < rnk;
+                x[k] = div_by_rc(v[k], by_col ? cn[k] : rnk, by_col ? rcn[k] : rck);
             }
             w = encode8_std_v(x);
         } else {
 #pragma unroll
-            for (int k = 0; k < kEltsPerLane; ++k)
-                x[k] = v[k] / ((cn[k] < rn) ? cn[k] : rn);
+            for (int k = 0; k < kEltsPerLane; ++k) {
+                const float rnk = (FOLD && k >= 4) ? rn1 : rn;
+                x[k] = v[k] / ((cn[k] < rnk) ? cn[k] : rnk);
+            }
             w = encode8_plain(lds, kVMap, kind, x);
         }
         store_u32(vcp, swap_code_halves(w, code_sel));
@@ -420,6 +455,9 @@ static float *next_scales(const lpmm_nonfused_rank1_tensor &) { return nullptr; 
 static float *next_scales(const lpmm_rank1_v4bit_tensor &) { return nullptr; }
 static float *next_scales(const lpmm_rank1_mgroup_tensor &t) { return t.m_max1_next; }
 
+// a tensor that the kernels take as double rows
+static bool folds(int64_t rows, int64_t cols) { return cols % kGroup == 64 && rows % 2 == 0; }
+
 // Validation, batching into launches of at most kR1Max tensors, and the three launches.
 // m_lg: the first moment's group holds 128 << m_lg values (MODE kMCodesWide only).
 template <int MODE, class Record>
@@ -429,6 +467,9 @@ static int rank1_step_multi(const Record *tensors, int64_t count, const float *q
                             const void *table_v = nullptr)
 {
     constexpr bool M32 = MODE == kMFloat;
+    // 4-bit codes in 128-value groups: a column count of 64 modulo 128 with an even row count is
+    // served as double rows (rank1_tiles.hpp)
+    const bool can_fold = MODE == kMCodes128 && bits_m == 4;
     // column counts that are no multiple of 128 (wide-group records only): every tensor of the call
     // then takes the kernels for ragged rows
     bool ragged = false;
@@ -443,9 +484,11 @@ static int rank1_step_multi(const Record *tensors, int64_t count, const float *q
     LPMM_REQUIRE_ALIGN(qmap_v, 4);
     for (int64_t i = 0; i < count; ++i) {
         const Record &t = tensors[i];
-        if (t.rows < 0 || t.cols < 0 || t.cols % (MODE == kMCodesWide ? 8 : kGroup) != 0)
+        if (t.rows < 0 || t.cols < 0)
             return LPMM_ERR_SIZE;
-        ragged = ragged || t.cols % kGroup != 0;
+        if (t.cols % (MODE == kMCodesWide ? 8 : kGroup) != 0 && !(can_fold && folds(t.rows, t.cols)))
+            return LPMM_ERR_SIZE;
+        ragged = ragged || (MODE == kMCodesWide && t.cols % kGroup != 0);
         if (t.rows == 0 || t.cols == 0)
             continue;
         const int64_t col_blocks = (t.cols + kGroup - 1) / kGroup;
@@ -495,6 +538,7 @@ static int rank1_step_multi(const Record *tensors, int64_t count, const float *q
         int k = 0;
         uint64_t tiles = 0;
         int64_t longest = 0;
+        bool folded = false;  // does a tensor of this launch have folded rows
         args.tile_start[0] = 0;
         while (i < count && k < kR1Max) {
             const Record &t = tensors[i];
@@ -504,7 +548,9 @@ static int rank1_step_multi(const Record *tensors, int64_t count, const float *q
             }
             const uint32_t col_blocks = (uint32_t)((t.cols + kGroup - 1) / kGroup);
             TensorR1 &d = args.t[k];
-            const uint64_t nt = shape_tiles(t.rows, col_blocks, d.tile);
+            const bool fold = t.cols % kGroup != 0 && can_fold;  // validated above: 64 modulo 128, even rows
+            const uint64_t nt = fold ? shape_tiles(t.rows / 2, 2 * col_blocks - 1, d.tile)
+                                     : shape_tiles(t.rows, col_blocks, d.tile);
             if (tiles + nt > 0x7fffffffULL)
                 break;
             d.p = t.p;
@@ -527,6 +573,7 @@ static int rank1_step_multi(const Record *tensors, int64_t count, const float *q
             d.rbc2_sqrt = h.rbc2_sqrt;
             longest = t.rows + t.cols > longest ? t.rows + t.cols : longest;
             tiles += nt;
+            folded = folded || fold;
             args.tile_start[++k] = (uint32_t)tiles;
             ++i;
         }
@@ -538,21 +585,27 @@ static int rank1_step_multi(const Record *tensors, int64_t count, const float *q
         args.count = k;
         for (int j = k + 1; j <= kR1Max; ++j)
             args.tile_start[j] = (uint32_t)tiles;
+        hipStream_t s = (hipStream_t)stream;
         int64_t clear_blocks = (longest + kThreads - 1) / kThreads;
         clear_blocks = clear_blocks > 64 ? 64 : clear_blocks;
         hipLaunchKernelGGL(rank1_clear_kernel, dim3((uint32_t)clear_blocks, (uint32_t)k), dim3(kThreads), 0,
-                           (hipStream_t)stream, args);
+                           s, args);
         if (ragged || (MODE == kMCodesWide && m_lg == 0)) {
-            launch_rank1_ragged(args, (uint32_t)tiles, qmap_m, qmap_v, (hipStream_t)stream);
+            launch_rank1_ragged(args, (uint32_t)tiles, qmap_m, qmap_v, s);
         } else if (bits_m != 4) {
             launch_rank1_bits(args, (uint32_t)tiles, qmap_m, qmap_v, bits_m, bits_v,
                               static_cast<const uint32_t *>(table_m), static_cast<const uint32_t *>(table_v),
-                              (hipStream_t)stream);
+                              s);
+        } else if (MODE == kMCodes128 && folded) {
+            hipLaunchKernelGGL((rank1_update_kernel<kMCodes128, true>), dim3((uint32_t)tiles), dim3(kThreads), 0,
+                               s, args, qmap_m, qmap_v);
+            hipLaunchKernelGGL((rank1_requant_kernel<false, true>), dim3((uint32_t)tiles), dim3(kThreads), 0,
+                               s, args, qmap_m, qmap_v);
         } else {
-            hipLaunchKernelGGL(rank1_update_kernel<MODE>, dim3((uint32_t)tiles), dim3(kThreads), 0,
-                               (hipStream_t)stream, args, qmap_m, qmap_v);
-            hipLaunchKernelGGL(rank1_requant_kernel<MODE == kMCodesWide>, dim3((uint32_t)tiles), dim3(kThreads), 0,
-                               (hipStream_t)stream, args, qmap_m, qmap_v);
+            hipLaunchKernelGGL((rank1_update_kernel<MODE, false>), dim3((uint32_t)tiles), dim3(kThreads), 0,
+                               s, args, qmap_m, qmap_v);
+            hipLaunchKernelGGL((rank1_requant_kernel<MODE == kMCodesWide, false>), dim3((uint32_t)tiles), dim3(kThreads),
+                               0, s, args, qmap_m, qmap_v);
         }
         const int st = launch_status();
         if (st != LPMM_OK)

@@ -105,12 +105,11 @@ struct Geometry {
     int step, passes, wide;
 };
 
-__device__ __forceinline__ Geometry geometry(const TensorR1 &t, uint32_t tile, int drow)
+__device__ __forceinline__ Geometry geometry(const TileShape &ts, uint32_t col_blocks, uint32_t tile, int drow)
 {
     Geometry q;
-    const TileShape &ts = t.tile;
     q.wide = 1 << ts.lg_wide;
-    const uint32_t col_tiles = (t.col_blocks + q.wide - 1) >> ts.lg_wide;
+    const uint32_t col_tiles = (col_blocks + q.wide - 1) >> ts.lg_wide;
     const uint32_t rb = tile / col_tiles;
     q.col_tile = tile - rb * col_tiles;
     q.cg = q.col_tile * q.wide + (drow & (q.wide - 1));
@@ -121,6 +120,51 @@ __device__ __forceinline__ Geometry geometry(const TensorR1 &t, uint32_t tile, i
     q.row0 = (int64_t)grp * ts.tile_rows * ts.comb + (int64_t)k * pass_rows + (drow >> ts.lg_wide);
     q.step = pass_rows * (int)ts.comb;
     return q;
+}
+
+__device__ __forceinline__ Geometry geometry(const TensorR1 &t, uint32_t tile, int drow)
+{
+    return geometry(t.tile, t.col_blocks, tile, drow);
+}
+
+// Folded rows.  A tensor of R x C values with C = 64 modulo 128 and R even is the same memory as
+// the row-major matrix of R / 2 double rows of 2 C values, and 2 C is a multiple of 128: the
+// 128-value groups of the first moment, cut from the flattened tensor (lpmm/functional.py:404-422),
+// never straddle a double row, so the kernels for whole column blocks apply to that matrix (GPT-2-XL's
+// d = 1600 and 3 d = 4800).  What changes is where a value's statistics sit: a DPP row's 128 values
+// are two halves of 64 (a lane's first and second run of four), half h of column block cg of double
+// row r lies in tensor row 2 r + (128 cg + 64 h >= C) at column (128 cg + 64 h) mod C.  The record
+// keeps the tensor's own shape (col_blocks = ceil(C / 128), col_tail = 64); kernels instantiated
+// with FOLD read it this way, tensors with whole column blocks in the same launch as before.
+struct Fold {
+    bool on;
+    uint32_t real_cols, col_blocks;  // columns of the tensor; column blocks of the matrix the kernel works on
+    int64_t rows;                    // rows of that matrix
+};
+
+template <bool FOLD>
+__device__ __forceinline__ Fold fold_of(const TensorR1 &t)
+{
+    Fold f;
+    f.on = FOLD && t.col_tail != (uint32_t)kGroup;
+    f.real_cols = (t.col_blocks - 1) * kGroup + t.col_tail;
+    f.col_blocks = f.on ? 2 * t.col_blocks - 1 : t.col_blocks;
+    f.rows = f.on ? t.rows >> 1 : t.rows;
+    return f;
+}
+
+// column of the tensor for column c of the matrix (c < 2 C)
+__device__ __forceinline__ uint32_t fold_col(const Fold &f, uint32_t c) { return c >= f.real_cols ? c - f.real_cols : c; }
+
+// tensor rows of the two halves of column block cg in row r of the matrix
+__device__ __forceinline__ void fold_rows(const Fold &f, int64_t r, uint32_t cg, int64_t &r0, int64_t &r1)
+{
+    if (f.on) {
+        r0 = 2 * r + (cg * kGroup >= f.real_cols ? 1 : 0);
+        r1 = 2 * r + (cg * kGroup + 64 >= f.real_cols ? 1 : 0);
+    } else {
+        r0 = r1 = r;
+    }
 }
 
 // Codes of a plain 0.0 into the padding [n, n_padded) of a packed array and 0 into the extra

@@ -444,7 +444,10 @@ class AdamW(LowBitOptimizer):
                         launch_group(key, pending)
                         pending.clear()
                     continue
-                if v_rank1 and p.dim() == 2 and p.shape[1] % 128 == 0:
+                # whole 128-column blocks, or half a block left over with an even row count (taken
+                # as double rows: GPT-2-XL's 1600 and 4800 columns)
+                if v_rank1 and p.dim() == 2 and (p.shape[1] % 128 == 0
+                                                 or (p.shape[1] % 128 == 64 and p.shape[0] % 2 == 0)):
                     pending = batched_rank1.setdefault(key, _Batch())
                     pending.append(self._nonfused_rank1_record(p, dense, grad, state, step, pending))
                     if len(pending) == _native.RANK1_MULTI_MAX:

@@ -108,6 +108,28 @@ def test_rank1_two_pass_matches_staged_oracle(oracle, qmaps):
             t.check(f"{t.rows}x{t.cols} step {step}")
 
 
+def test_rank1_folded_rows(oracle, qmaps):
+    """Column counts of 64 modulo 128 with an even row count (GPT-2-XL's 1600 and 4800): the kernels take
+    two tensor rows as one row of whole column blocks; the statistics of a value sit at its own row and
+    column.  Fewer double rows than one pass, more than one tile, one and several column tiles, tensors
+    with whole column blocks in the same launch."""
+    qm, qv = qmaps
+    dqm, dqv = to_dev(qm), to_dev(qv)
+    rng = np.random.default_rng(29)
+    shapes = [(2, 64), (2, 192), (6, 1600), (65, 384), (64, 192), (130, 320), (66, 4800), (258, 1600), (16, 256),
+              (1024, 1600), (200, 6464)]
+    tensors = [_Tensor(r, c, rng) for r, c in shapes]
+    for step in range(1, 4):
+        grads = [_grad(rng, t) for t in tensors]
+        if step == 2:
+            grads[5][7, :] = 0.0  # a row and a column of zeros, one of each half of a double row
+            grads[5][:, 300] = 0.0
+            grads[7][100:102, :] = 0.0
+        _step_all(oracle, tensors, grads, qm, qv, dqm, dqv, step)
+        for t in tensors:
+            t.check(f"{t.rows}x{t.cols} step {step}")
+
+
 def test_rank1_interleaved_row_blocks_with_ragged_last_group(oracle, qmaps):
     """Tensors with more row blocks than interleave in one group: several groups, the last one
     short of blocks and ending in a ragged block (2500 = 39 * 64 + 4 rows over 16 column tiles,
@@ -192,7 +214,8 @@ def test_rank1_argument_checks(qmaps):
     ptr = buf.data_ptr()
     ok = (ptr, ptr, ptr, ptr, ptr, ptr, ptr, ptr + 2048, ptr + 4096, 4, 128, 1.0, 0.0)
     bad_cols = ok[:10] + (100,) + ok[11:]
+    odd_rows_of_half_blocks = ok[:9] + (3, 192) + ok[11:]  # 64 modulo 128 columns need an even row count
     aliased = ok[:7] + (ptr, ptr) + ok[9:]
-    for rec in (bad_cols, aliased):
+    for rec in (bad_cols, odd_rows_of_half_blocks, aliased):
         table = np.array([rec], dtype=nat.NONFUSED_RANK1_TENSOR)
         assert call(table.ctypes.data, 1, *tail) != 0
