@@ -105,8 +105,9 @@ template <int MODE, bool FOLD>
 __global__ __launch_bounds__(kThreads, LPMM_R1_WAVES) void rank1_update_kernel(const MultiR1 args, const float *__restrict__ qmap_m,
                                                                 const float *__restrict__ qmap_v)
 {
-    __shared__ __align__(16) uint32_t lds[(kColExtra + kMaxWide * kRedSlotWords * 4) / 4];
+    __shared__ __align__(16) uint32_t lds[(kColExtra + kMaxWide * kRedSlotWords * 4) / 4 + kRowSlots];
     uint32_t *colred = lds + kColExtra / 4;
+    uint32_t *rowred = colred + kMaxWide * kRedSlotWords;
     const int lo = find_tensor(args);
     const TensorR1 &t = args.t[lo];
     const uint32_t tl = blockIdx.x - args.tile_start[lo];
@@ -137,6 +138,8 @@ __global__ __launch_bounds__(kThreads, LPMM_R1_WAVES) void rank1_update_kernel(c
     lds_fill_store(lds, fill);
     for (int j = threadIdx.x; j < kMaxWide * (int)kRedSlotWords; j += kThreads)
         colred[j] = 0u;
+    if (threadIdx.x < kRowSlots)
+        rowred[threadIdx.x] = 0u;
 #pragma unroll
     for (int i = 0; i < kColPerThread; ++i)
         lds[kColOld / 4 + threadIdx.x + i * kThreads] = co_in[i];
@@ -230,26 +233,31 @@ __global__ __launch_bounds__(kThreads, LPMM_R1_WAVES) void rank1_update_kernel(c
                 atomic_max_nonneg(t.ms_new + (grp >> t.m_lg), amax_m);
             }
             if (lane16 == 0) {
+                // the maxima of a tensor row meet in LDS (rank1_tiles.hpp); folded rows: a half goes to the
+                // tensor row it lies in
+                uint32_t *slot = rowred + row_slot(t.tile, it, drow);
                 if (FOLD) {
-                    int64_t r0, r1;
-                    fold_rows(f, r, q.cg, r0, r1);
-                    atomic_max_nonneg(t.row_new + r0, vmax);
-                    atomic_max_nonneg(t.row_new + r1, vmax1);
+                    const bool h0 = f.on && q.cg * kGroup >= f.real_cols, h1 = f.on && q.cg * kGroup + 64 >= f.real_cols;
+                    atomicMax(slot + (h0 ? 1 : 0), __float_as_uint(vmax));
+                    atomicMax(slot + (h1 ? 1 : 0), __float_as_uint(vmax1));
                 } else {
-                    atomic_max_nonneg(t.row_new + r, vmax);
+                    atomicMax(slot, __float_as_uint(vmax));
                 }
             }
         }
     }
     // the column maxima meet in LDS: nothing below depends on the global stores still in flight
     lds_barrier();
+    flush_row_maxima(rowred, t.tile, q, drow, f.rows, FOLD && f.on, t.row_new);
     // column j of the tile = element k of lane l of slot s
     for (int j = threadIdx.x; j < q.wide * kGroup; j += kThreads) {
         const int w = j & (kGroup - 1);
         const int k = ((w >> 6) << 2) | (w & 3), l = (w >> 2) & 15;
-        if (tile_c0 + j < cols)
-            atomic_max_nonneg(t.col_new + (FOLD ? fold_col(f, (uint32_t)(tile_c0 + j)) : tile_c0 + j),
-                              __uint_as_float(colred[(j >> 7) * kRedSlotWords + k * 16 + l]));
+        if (tile_c0 + j < cols) {
+            float *dst = t.col_new + (FOLD ? fold_col(f, (uint32_t)(tile_c0 + j)) : tile_c0 + j);
+            const uint32_t mine = colred[(j >> 7) * kRedSlotWords + k * 16 + l];
+            atomic_max_nonneg(dst, __uint_as_float(mine));
+        }
     }
 }
 

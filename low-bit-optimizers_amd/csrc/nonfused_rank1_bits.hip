@@ -48,6 +48,7 @@ __global__ __launch_bounds__(kThreads) void rank1_update_bits_kernel(const Multi
     const uint32_t mode = code_table_mode(code_table_tag(table_m), bits_m);
     __shared__ __align__(16) float col_old[kMaxWide * kGroup];
     __shared__ uint32_t colred[kMaxWide * kRedSlotWords];
+    __shared__ uint32_t rowred[kRowSlots];
     const int lo = find_tensor(args);
     const TensorR1 &t = args.t[lo];
     const uint32_t tl = blockIdx.x - args.tile_start[lo];
@@ -65,6 +66,8 @@ __global__ __launch_bounds__(kThreads) void rank1_update_bits_kernel(const Multi
         col_old[j] = (j < q.wide * kGroup && tile_c0 + j < cols) ? t.col_old[tile_c0 + j] : 0.0f;
     for (int j = threadIdx.x; j < kMaxWide * (int)kRedSlotWords; j += kThreads)
         colred[j] = 0u;
+    if (threadIdx.x < kRowSlots)
+        rowred[threadIdx.x] = 0u;
     NfHyper h;
     h.decay = args.decay;
     h.w1 = args.w1;
@@ -140,11 +143,12 @@ __global__ __launch_bounds__(kThreads) void rank1_update_bits_kernel(const Multi
             store_u32(mcp + 16, pack4(c, 1));
             if (lane16 == 0) {
                 t.ms[grp] = amax_m;
-                atomic_max_nonneg(t.row_new + r, vmax);
+                atomicMax(rowred + row_slot(t.tile, it, drow), __float_as_uint(vmax));  // rank1_tiles.hpp
             }
         }
     }
     __syncthreads();
+    flush_row_maxima(rowred, t.tile, q, drow, t.rows, false, t.row_new);
     // column j of the tile = element k of lane l of slot s
     for (int j = threadIdx.x; j < q.wide * kGroup; j += kThreads) {
         const int w = j & (kGroup - 1);

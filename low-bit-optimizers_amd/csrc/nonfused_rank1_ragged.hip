@@ -34,8 +34,9 @@ __device__ __forceinline__ RaggedRow ragged_row(const TensorR1 &t, int64_t cols,
 __global__ __launch_bounds__(kThreads) void rank1_update_ragged_kernel(const MultiR1 args, const float *__restrict__ qmap_m,
                                                                       const float *__restrict__ qmap_v)
 {
-    __shared__ __align__(16) uint32_t lds[(kColExtra + kMaxWide * kRedSlotWords * 4) / 4];
+    __shared__ __align__(16) uint32_t lds[(kColExtra + kMaxWide * kRedSlotWords * 4) / 4 + kRowSlots];
     uint32_t *colred = lds + kColExtra / 4;
+    uint32_t *rowred = colred + kMaxWide * kRedSlotWords;
     const int lo = find_tensor(args);
     const TensorR1 &t = args.t[lo];
     const uint32_t tl = blockIdx.x - args.tile_start[lo];
@@ -48,6 +49,8 @@ __global__ __launch_bounds__(kThreads) void rank1_update_ragged_kernel(const Mul
         lds[kColOld / 4 + j] = (j < q.wide * kGroup && tile_c0 + j < cols) ? __float_as_uint(t.col_old[tile_c0 + j]) : 0u;
     for (int j = threadIdx.x; j < kMaxWide * (int)kRedSlotWords; j += kThreads)
         colred[j] = 0u;
+    if (threadIdx.x < kRowSlots)
+        rowred[threadIdx.x] = 0u;
     NfHyper h;
     h.decay = args.decay;
     h.w1 = args.w1;
@@ -126,11 +129,12 @@ __global__ __launch_bounds__(kThreads) void rank1_update_ragged_kernel(const Mul
                     atomic_max_nonneg(t.ms_new + glo, mlo);
                 if (mhi != 0.0f)
                     atomic_max_nonneg(t.ms_new + glo + 1, mhi);
-                atomic_max_nonneg(t.row_new + r, vmax);
+                atomicMax(rowred + row_slot(t.tile, it, drow), __float_as_uint(vmax));  // rank1_tiles.hpp
             }
         }
     }
     __syncthreads();
+    flush_row_maxima(rowred, t.tile, q, drow, t.rows, false, t.row_new);
     // column j of the tile = element k of lane l of slot s
     for (int j = threadIdx.x; j < q.wide * kGroup; j += kThreads) {
         const int w = j & (kGroup - 1);

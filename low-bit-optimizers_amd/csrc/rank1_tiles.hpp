@@ -167,6 +167,37 @@ __device__ __forceinline__ void fold_rows(const Fold &f, int64_t r, uint32_t cg,
     }
 }
 
+// Row maxima of a tile.  An atomic maximum on global memory goes out to the fabric (the L2s of
+// the XCDs are not coherent with each other), and the passes of a tile produce one per tensor row,
+// column group and pass: 0.008 per element, a tenth of the first pass's DRAM transactions together
+// with its partial writes.  So the maxima of a tile's rows meet in LDS first -- slot 2 * (row of
+// the tile) + (tensor row of a double row: folded rows only) -- and one global atomic per row and
+// tile follows the passes, issued by neighbouring threads for neighbouring rows (LLaMA-7B-shaped
+// set 21.23 -> 20.85 ms per step, GPT-2-XL-shaped set 6.30 -> 5.71 ms).
+constexpr int kRowSlots = 2 * (int)kPolicyRows;
+static_assert(kRowSlots <= kThreads, "one thread per row slot");
+static_assert(kPolicyRows >= (uint32_t)kDppRows, "a tile holds the policy's rows: one slot pair per row");
+
+__device__ __forceinline__ int row_slot(const TileShape &ts, int pass, int drow)
+{
+    return 2 * (pass * (kDppRows >> ts.lg_wide) + (drow >> ts.lg_wide));
+}
+
+// after the passes and a barrier: rows = rows of the matrix the tile works on; fold: its rows are double rows
+__device__ __forceinline__ void flush_row_maxima(const uint32_t *rowred, const TileShape &ts, const Geometry &q, int drow,
+                                                 int64_t rows, bool fold, float *__restrict__ row_new)
+{
+    if (threadIdx.x >= (uint32_t)kRowSlots)
+        return;
+    const int pr = kDppRows >> ts.lg_wide;
+    const int local = threadIdx.x >> 1, half = threadIdx.x & 1;
+    const int pass = local / pr, in_pass = local - pass * pr;
+    // the first row of the tile's first pass: row0 of this thread's DPP row less its place in the pass
+    const int64_t r = (q.row0 - (drow >> ts.lg_wide)) + (int64_t)pass * q.step + in_pass;
+    if (pass < q.passes && r < rows && (half == 0 || fold))
+        atomic_max_nonneg(row_new + (fold ? 2 * r + half : r), __uint_as_float(rowred[threadIdx.x]));
+}
+
 // Codes of a plain 0.0 into the padding [n, n_padded) of a packed array and 0 into the extra
 // last byte; one workgroup.  n and n_padded are multiples of 8, the array is 4-byte aligned.
 __device__ __forceinline__ void write_padding(uint8_t *codes, int64_t n, int64_t n_padded, uint32_t zero_word)
