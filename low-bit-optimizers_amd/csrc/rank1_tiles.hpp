@@ -23,6 +23,7 @@ constexpr int kR1Max = 32;               // tensors per launch
 #endif
 constexpr int kPolicyLgWide = LPMM_R1_LG;
 constexpr uint32_t kPolicyRows = LPMM_R1_ROWS, kPolicyResident = LPMM_R1_RESIDENT;
+constexpr uint32_t kPolicyRowsM32 = LPMM_R1_ROWS / 2;  // fp32 first moment
 static_assert(LPMM_R1_LG >= 1 && LPMM_R1_LG <= 3, "a tile is 256 to 1024 columns wide at most");
 constexpr int kMaxLgWide = kPolicyLgWide;   // the LDS column arrays hold 128 << kMaxLgWide columns
 constexpr int kMaxWide = 1 << kMaxLgWide;
