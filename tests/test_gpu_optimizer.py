@@ -144,6 +144,38 @@ def test_nonfused_optimizer_matches_oracle(oracle, qmaps, v_scale):
     assert_rel(to_np(params[2]), host[2], 'p small', scale=host[2])
 
 
+def test_nonfused_optimizer_routes_every_column_count(oracle, qmaps):
+    """fused=False under the default configuration with the column counts that take different kernels:
+    whole 128-column blocks, 64 modulo 128 with an even row count (taken as double rows), the same
+    with an odd row count and 32 modulo 128 (ragged rows) -- all in one optimizer, against the oracle."""
+    import lpmm
+
+    qm, qv = qmaps
+    rng = np.random.default_rng(11)
+    shapes = [(48, 256), (64, 192), (40, 320), (33, 192), (96, 160), (130, 1600)]
+    host, params = _params(shapes, rng)
+    cfg = os.path.join(os.path.dirname(lpmm.config.__file__), "configs", "default.yml")
+    opt = lpmm.optim.AdamW(params, fused=False, qconfig=cfg, **H)
+    states = [oracle.NonFusedState(s, v_scale_type="rank1") for s in shapes]
+    for step in range(1, 5):
+        grads = [(rng.standard_normal(s) * 1e-3 * np.exp(rng.standard_normal((s[0], 1)))).astype(np.float32) for s in shapes]
+        for p, g in zip(params, grads):
+            p.grad = to_dev(g)
+        opt.step()
+        for h, g, st in zip(host, grads, states):
+            oracle.nonfused_step(h, g, st, qm, qv, H["lr"], 0.9, 0.999, H["eps"], H["weight_decay"])
+    torch.cuda.synchronize()
+    for i, shape in enumerate(shapes):
+        s = opt.state[params[i]]
+        np.testing.assert_array_equal(to_np(s["exp_avg"]).view(np.uint8), states[i].m[0], err_msg=str(shape))
+        np.testing.assert_array_equal(to_np(s["exp_avg_qstate"]["overhead"]["max1"]).reshape(-1), states[i].m[1])
+        oh = s["exp_avg_sq_qstate"]["overhead"]
+        np.testing.assert_array_equal(to_np(s["exp_avg_sq"]).view(np.uint8), states[i].v[0], err_msg=str(shape))
+        np.testing.assert_array_equal(to_np(oh["max_dims"][0]).reshape(-1), states[i].v[1], err_msg=str(shape))
+        np.testing.assert_array_equal(to_np(oh["max_dims"][1]).reshape(-1), states[i].v[2], err_msg=str(shape))
+        assert_rel(to_np(params[i]), host[i], f"p {shape}", scale=host[i])
+
+
 def test_nonfused_rank1_on_tensors_of_more_than_two_dimensions(oracle, qmaps):
     """Default configuration (rank-1 second moment) on 3-D and 4-D parameters: statistics,
     quantiser and dequantiser run in HIP (N-D statistics kernels plus the 2-D kernels on the
