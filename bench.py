@@ -82,6 +82,17 @@ def gpt2xl_shapes():
     return shapes
 
 
+def conv_shapes():
+    """The convolution weights of a ResNet-152 at twice the width (bottleneck blocks: 1x1, 3x3, 1x1), 2.3e8
+    parameters in 4-D tensors, plus the stem and the classifier."""
+    shapes = [(128, 3, 7, 7)]
+    for w, blocks in ((512, 3), (1024, 8), (2048, 36), (4096, 3)):
+        for _ in range(blocks):
+            shapes += [(w // 4, w, 1, 1), (w // 4, w // 4, 3, 3), (w, w // 4, 1, 1), (w,)]
+    shapes += [(1000, 4096), (1000,)]
+    return shapes
+
+
 def tiny_shapes():
     return [(4096, 1024), (1024, 4096), (4096,), (8192,), (1000, 1000)] * 4
 
@@ -480,7 +491,7 @@ def run_nonfused(torch, args, v_scale, m32=False, mgroup=False):
     import lpmm
 
     dev = torch.device("cuda:0")
-    shapes = gpt2xl_shapes() if args.shapes == "gpt2xl" else llama7b_shapes()
+    shapes = {"gpt2xl": gpt2xl_shapes, "conv": conv_shapes, "llama7b": llama7b_shapes}[args.shapes]()
     params = make_params(torch, shapes, dev, heavy_tailed=True)
     bits = args.bits if (v_scale == "rank1" and not m32 and not mgroup) else 4
     if bits != 4:
@@ -516,19 +527,24 @@ def run_nonfused(torch, args, v_scale, m32=False, mgroup=False):
     if bits != 4:  # one code per byte: p 8, g 4 + 4, m codes 2, v codes 1 + 2, scales 8/128
         bytes_per_param = 21.0625
     if args.shapes != "llama7b":
-        # a mix of paths: per tensor, what its path moves (rank-1: matrices with a multiple of 128 columns
-        # as above, other multiples of 8 through the kernels for ragged rows 19.0625, quantised vectors one
+        # a mix of paths: per tensor, what its path moves (rank-1: tensors whose shape[0] x rest view has
+        # whole 128-column blocks, or half a block left over with an even row count, as above; other
+        # multiples of 8 through the kernels for ragged rows 19.0625; what is left takes the staged path
+        # (dequantise, update on fp32 temporaries, statistics, quantise: about 50); quantised vectors one
         # pass 14.125; fp32 states 28)
         total = 0.0
         for p in params:
+            rows, cols = p.shape[0], p.numel() // p.shape[0]
             if p.numel() <= 4096:
                 total += 28.0 * p.numel()
             elif v_scale == "group" or p.dim() == 1:
                 total += BYTES_PER_PARAM_4BIT * p.numel()
-            elif p.shape[1] % 128 == 0:
+            elif cols % 128 == 0 or (cols % 128 == 64 and rows % 2 == 0):
                 total += 18.5625 * p.numel()
-            else:
+            elif p.dim() == 2 and cols % 8 == 0:
                 total += 19.0625 * p.numel()
+            else:
+                total += 50.0 * p.numel()
         bytes_per_param = total / n_total
     achieved = n_total * bytes_per_param / dt / 1e9
     print(json.dumps({
@@ -536,7 +552,7 @@ def run_nonfused(torch, args, v_scale, m32=False, mgroup=False):
         "unit": "params/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": dt * 1e3,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": f"fused=False, {'fp32 first moment, ' if m32 else ''}{'first-moment groups of 1024, ' if mgroup else ''}second moment '{v_scale}' scaling, "
-                               f"{'GPT-2-XL' if args.shapes == 'gpt2xl' else 'LLaMA-7B'}-shaped fp32 set", "qconfig": name,
+                               f"{ {'gpt2xl': 'GPT-2-XL-shaped', 'conv': 'wide-ResNet-152 convolution', 'llama7b': 'LLaMA-7B-shaped'}[args.shapes]} fp32 set", "qconfig": name,
                    "tensors": len(params), "params": n_total},
         "roofline": {"bound": "hbm", "kernel": "whole step", "achieved": achieved, "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None,
@@ -551,7 +567,7 @@ def main():
     ap.add_argument("--workload", default="llama7b", choices=sorted(WORKLOADS) + ["quant64m", "factored", "nonfused_group", "nonfused_rank1", "nonfused_group_m32", "nonfused_rank1_m32", "nonfused_rank1_mgroup", "sgd", "calibrate"])
     ap.add_argument("--bits", type=int, default=4, choices=range(1, 9),
                     help="code width of --workload quant64m (1-8) and nonfused_rank1 (4-8)")
-    ap.add_argument("--shapes", default="llama7b", choices=["llama7b", "gpt2xl"],
+    ap.add_argument("--shapes", default="llama7b", choices=["llama7b", "gpt2xl", "conv"],
                     help="parameter set of the nonfused_* workloads")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--interleaved-grads", action="store_true",

@@ -180,6 +180,25 @@ int lpmm_rank1_stats_nd(const float *x, int ndim, const int64_t *shape, float *c
 int lpmm_rank1_row_scale_nd(const float *const *stats, int ndim, const int64_t *shape, float *row_scale,
                             void *stream);
 
+/* Statistics and scale of short vectors, many per call (no counterpart in the reference).  For
+ * each record: stats[i][j] = max |x| over the elements of the vector x (row-major, shape[0..ndim))
+ * whose i-th index is j, written in full, and scale[e] = the minimum of element e's statistics (NaN
+ * if any of them is).  That is lpmm_rank1_stats_nd followed by lpmm_rank1_row_scale_nd over all of the
+ * vector's dimensions, in one launch for up to 32 vectors -- what lies between the two passes of
+ * lpmm_nonfused_adamw4bit_rank1_pass_multi for tensors of more than two dimensions, whose trailing
+ * dimensions are the vector's.  ndim 1..7, at most 8192 statistics entries per vector (the sum of
+ * its dimensions), fewer than 2^31 elements; records live in host memory and are consumed during
+ * the call. */
+typedef struct lpmm_rank1_small_vector {
+    const float *x;
+    float *scale;
+    float *stats[LPMM_RANK1_ND_MAX - 1];
+    int64_t shape[LPMM_RANK1_ND_MAX - 1];
+    int32_t ndim;
+    int32_t reserved;
+} lpmm_rank1_small_vector;
+int lpmm_rank1_small_fold_scale_multi(const lpmm_rank1_small_vector *vectors, int64_t count, void *stream);
+
 /* ---------------------------------------------------------------------------------------
  * The same six operations for any code width 1..8(lpmm/configs/default_{5,6,7,8}b.yml use
  * 5..8).  Storage follows lpmm/cpp_extension/quantization_kernel.cu:592-601, :695-705:
@@ -297,6 +316,23 @@ int lpmm_nonfused_adamw4bit_rank1_step_multi(const lpmm_nonfused_rank1_tensor *t
                                              const float *qmap_m, const float *qmap_v, double beta1,
                                              double beta2, double lr, double weight_decay, double eps,
                                              void *stream);
+
+/* One pass of lpmm_nonfused_adamw4bit_rank1_step_multi at a time (no counterpart in the
+ * reference, which has no passes): pass 1 clears the next statistics, updates p, re-quantises m and
+ * leaves the row and column maxima of the new second moment in v_rowmax_next / v_colmax_next;
+ * pass 2 recomputes the new second moment from g and the old codes and statistics and quantises
+ * it with whatever v_rowmax_next / v_colmax_next hold then.  Between the two a caller may replace
+ * the maxima by scales derived from them: a tensor of more than two dimensions, viewed as
+ * shape[0] x (numel / shape[0]), has the reference's scale min over all dimensions
+ * (lpmm/functional.py:503-531) when its column scale is the minimum over the trailing dimensions'
+ * statistics -- lpmm_rank1_row_scale_nd on shape[1:] gives it before pass 1 (as v_colmax) and,
+ * from the statistics that lpmm_rank1_stats_nd folds out of pass 1's column maxima, before
+ * pass 2 (as v_colmax_next; see lpmm/optim/adamw.py::_rank1_nd_steps).  Both calls take the same
+ * records, apart from the pointers the caller redirects. */
+int lpmm_nonfused_adamw4bit_rank1_pass_multi(const lpmm_nonfused_rank1_tensor *tensors, int64_t count,
+                                             const float *qmap_m, const float *qmap_v, double beta1,
+                                             double beta2, double lr, double weight_decay, double eps,
+                                             int pass, void *stream);
 
 /* The non-fused step with an fp32 first moment and a 4-bit second moment: the configurations
  * that quantise the second moment only (QUANT.M.ENABLE False: lpmm/configs/

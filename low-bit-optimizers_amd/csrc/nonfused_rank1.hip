@@ -472,8 +472,12 @@ template <int MODE, class Record>
 static int rank1_step_multi(const Record *tensors, int64_t count, const float *qmap_m, const float *qmap_v,
                             uint32_t m_lg, double beta1, double beta2, double lr, double weight_decay, double eps,
                             void *stream, int bits_m = 4, int bits_v = 4, const void *table_m = nullptr,
-                            const void *table_v = nullptr)
+                            const void *table_v = nullptr, int passes = 3)
 {
+    // passes: 1 = the first pass alone (with the clearing of the next statistics), 2 = the second alone,
+    // 3 = both; one at a time only where the launches below are this file's own
+    if (passes < 1 || passes > 3 || (passes != 3 && (MODE != kMCodes128 || bits_m != 4)))
+        return LPMM_ERR_ARG;
     constexpr bool M32 = MODE == kMFloat;
     // 4-bit codes in 128-value groups: a column count of 64 modulo 128 with an even row count is
     // served as double rows (rank1_tiles.hpp)
@@ -599,8 +603,9 @@ static int rank1_step_multi(const Record *tensors, int64_t count, const float *q
         hipStream_t s = (hipStream_t)stream;
         int64_t clear_blocks = (longest + kThreads - 1) / kThreads;
         clear_blocks = clear_blocks > 64 ? 64 : clear_blocks;
-        hipLaunchKernelGGL(rank1_clear_kernel, dim3((uint32_t)clear_blocks, (uint32_t)k), dim3(kThreads), 0,
-                           s, args);
+        if (passes & 1)
+            hipLaunchKernelGGL(rank1_clear_kernel, dim3((uint32_t)clear_blocks, (uint32_t)k), dim3(kThreads), 0,
+                               s, args);
         if (ragged || (MODE == kMCodesWide && m_lg == 0)) {
             launch_rank1_ragged(args, (uint32_t)tiles, qmap_m, qmap_v, s);
         } else if (bits_m != 4) {
@@ -608,15 +613,19 @@ static int rank1_step_multi(const Record *tensors, int64_t count, const float *q
                               static_cast<const uint32_t *>(table_m), static_cast<const uint32_t *>(table_v),
                               s);
         } else if (MODE == kMCodes128 && folded) {
-            hipLaunchKernelGGL((rank1_update_kernel<kMCodes128, true>), dim3((uint32_t)tiles), dim3(kThreads), 0,
-                               s, args, qmap_m, qmap_v);
-            hipLaunchKernelGGL((rank1_requant_kernel<false, true>), dim3((uint32_t)tiles), dim3(kThreads), 0,
-                               s, args, qmap_m, qmap_v);
+            if (passes & 1)
+                hipLaunchKernelGGL((rank1_update_kernel<kMCodes128, true>), dim3((uint32_t)tiles), dim3(kThreads), 0,
+                                   s, args, qmap_m, qmap_v);
+            if (passes & 2)
+                hipLaunchKernelGGL((rank1_requant_kernel<false, true>), dim3((uint32_t)tiles), dim3(kThreads), 0,
+                                   s, args, qmap_m, qmap_v);
         } else {
-            hipLaunchKernelGGL((rank1_update_kernel<MODE, false>), dim3((uint32_t)tiles), dim3(kThreads), 0,
-                               s, args, qmap_m, qmap_v);
-            hipLaunchKernelGGL((rank1_requant_kernel<MODE == kMCodesWide, false>), dim3((uint32_t)tiles), dim3(kThreads),
-                               0, s, args, qmap_m, qmap_v);
+            if (passes & 1)
+                hipLaunchKernelGGL((rank1_update_kernel<MODE, false>), dim3((uint32_t)tiles), dim3(kThreads), 0,
+                                   s, args, qmap_m, qmap_v);
+            if (passes & 2)
+                hipLaunchKernelGGL((rank1_requant_kernel<MODE == kMCodesWide, false>), dim3((uint32_t)tiles),
+                                   dim3(kThreads), 0, s, args, qmap_m, qmap_v);
         }
         const int st = launch_status();
         if (st != LPMM_OK)
@@ -631,6 +640,17 @@ extern "C" int lpmm_nonfused_adamw4bit_rank1_step_multi(const lpmm_nonfused_rank
                                                         double eps, void *stream)
 {
     return rank1_step_multi<kMCodes128>(tensors, count, qmap_m, qmap_v, 0, beta1, beta2, lr, weight_decay, eps, stream);
+}
+
+extern "C" int lpmm_nonfused_adamw4bit_rank1_pass_multi(const lpmm_nonfused_rank1_tensor *tensors, int64_t count,
+                                                        const float *qmap_m, const float *qmap_v, double beta1,
+                                                        double beta2, double lr, double weight_decay,
+                                                        double eps, int pass, void *stream)
+{
+    if (pass != 1 && pass != 2)
+        return LPMM_ERR_ARG;
+    return rank1_step_multi<kMCodes128>(tensors, count, qmap_m, qmap_v, 0, beta1, beta2, lr, weight_decay, eps, stream,
+                                        4, 4, nullptr, nullptr, pass);
 }
 
 extern "C" int lpmm_nonfused_adamw_v4bit_rank1_step_multi(const lpmm_rank1_v4bit_tensor *tensors, int64_t count,

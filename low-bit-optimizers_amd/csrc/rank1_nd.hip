@@ -197,6 +197,71 @@ __global__ __launch_bounds__(256) void rank1_row_scale_nd_kernel(NdDims lead, fl
     out[row] = scale;
 }
 
+// ---------------------------------------------------------------------------------------
+// Statistics and scale of a short vector, many vectors per launch.  Between the two passes of the
+// optimizer step on a tensor of more than two dimensions (viewed as shape[0] x rest) the column
+// maxima of the new second moment -- a vector of `rest` values with the tensor's trailing
+// dimensions -- are folded into those dimensions' statistics, and the vector of their minima is
+// what the second pass divides by.  For a convolution weight that vector has a few thousand
+// entries and the statistics a few hundred: one workgroup per tensor keeps the statistics in LDS
+// (maxima by LDS atomics on the bit patterns), writes them out and derives the scale from the LDS
+// copy, in one launch for up to 32 tensors instead of three launches per tensor.
+// ---------------------------------------------------------------------------------------
+constexpr int kNdSmallMax = 32;      // vectors per launch
+constexpr int kNdSmallSlots = 8192;  // statistics entries of one vector (sum of its dimensions)
+
+struct NdSmall {
+    const float *x;   // the vector: product of dim[] values
+    float *scale;     // out: min over the dimensions' statistics, per element of the vector
+    float *stat[kNdMax - 1];
+    uint32_t dim[kNdMax - 1];
+    uint32_t ndim;
+    uint32_t n;
+};
+
+struct NdSmallArgs {
+    NdSmall t[kNdSmallMax];
+};
+static_assert(sizeof(NdSmallArgs) <= 4096, "kernel arguments exceed 4 KB");
+
+__global__ __launch_bounds__(256) void rank1_small_fold_scale_kernel(const NdSmallArgs args)
+{
+    __shared__ uint32_t slots[kNdSmallSlots];
+    const NdSmall &t = args.t[blockIdx.x];
+    uint32_t base[kNdMax - 1], total = 0;
+    for (uint32_t i = 0; i < t.ndim; ++i) {
+        base[i] = total;
+        total += t.dim[i];
+    }
+    for (uint32_t j = threadIdx.x; j < total; j += blockDim.x)
+        slots[j] = 0u;
+    __syncthreads();
+    for (uint32_t e = threadIdx.x; e < t.n; e += blockDim.x) {
+        const uint32_t v = abs_bits(t.x[e]);
+        uint32_t rem = e;
+        for (int i = (int)t.ndim - 1; i >= 0; --i) {
+            const uint32_t q = rem / t.dim[i];
+            atomicMax(slots + base[i] + (rem - q * t.dim[i]), v);
+            rem = q;
+        }
+    }
+    __syncthreads();
+    for (uint32_t i = 0; i < t.ndim; ++i)
+        for (uint32_t j = threadIdx.x; j < t.dim[i]; j += blockDim.x)
+            t.stat[i][j] = __uint_as_float(slots[base[i] + j]);
+    for (uint32_t e = threadIdx.x; e < t.n; e += blockDim.x) {
+        uint32_t rem = e;
+        float scale = 0.0f;
+        for (int i = (int)t.ndim - 1; i >= 0; --i) {
+            const uint32_t q = rem / t.dim[i];
+            const float s = __uint_as_float(slots[base[i] + (rem - q * t.dim[i])]);
+            rem = q;
+            scale = (i == (int)t.ndim - 1) ? s : min_nan(scale, s);
+        }
+        t.scale[e] = scale;
+    }
+}
+
 // shape -> NdDims for the first `ndim` dimensions; false when a size is not positive, the element
 // count overflows or the tile count does not fit a grid
 static bool nd_dims(int ndim, const int64_t *shape, float *const *stats, NdDims *out)
@@ -306,4 +371,56 @@ extern "C" int lpmm_rank1_row_scale_nd(const float *const *stats, int ndim, cons
     hipLaunchKernelGGL(rank1_row_scale_nd_kernel, dim3((uint32_t)((lead.n + 255) / 256)), dim3(256), 0,
                        (hipStream_t)stream, lead, row_scale);
     return launch_status();
+}
+
+extern "C" int lpmm_rank1_small_fold_scale_multi(const lpmm_rank1_small_vector *vectors, int64_t count, void *stream)
+{
+    if (count < 0)
+        return LPMM_ERR_SIZE;
+    if (count == 0)
+        return LPMM_OK;
+    LPMM_REQUIRE_PTR(vectors);
+    for (int64_t i = 0; i < count; ++i) {
+        const lpmm_rank1_small_vector &v = vectors[i];
+        if (v.ndim < 1 || v.ndim > kNdMax - 1)
+            return LPMM_ERR_ARG;
+        LPMM_REQUIRE_PTR(v.x);
+        LPMM_REQUIRE_PTR(v.scale);
+        LPMM_REQUIRE_ALIGN(v.x, 4);
+        LPMM_REQUIRE_ALIGN(v.scale, 4);
+        int64_t n = 1, slots = 0;
+        for (int k = 0; k < v.ndim; ++k) {
+            LPMM_REQUIRE_PTR(v.stats[k]);
+            LPMM_REQUIRE_ALIGN(v.stats[k], 4);
+            if (v.shape[k] <= 0 || v.shape[k] > kNdSmallSlots || n > (int64_t)0x7fffffff / v.shape[k])
+                return LPMM_ERR_SIZE;
+            n *= v.shape[k];
+            slots += v.shape[k];
+        }
+        if (slots > kNdSmallSlots)
+            return LPMM_ERR_SIZE;
+    }
+    for (int64_t i = 0; i < count; i += kNdSmallMax) {
+        NdSmallArgs args;
+        const int k = (int)(count - i < kNdSmallMax ? count - i : kNdSmallMax);
+        for (int j = 0; j < k; ++j) {
+            const lpmm_rank1_small_vector &v = vectors[i + j];
+            NdSmall &t = args.t[j];
+            t.x = v.x;
+            t.scale = v.scale;
+            t.ndim = (uint32_t)v.ndim;
+            uint32_t n = 1;
+            for (int a = 0; a < kNdMax - 1; ++a) {
+                t.stat[a] = a < v.ndim ? v.stats[a] : nullptr;
+                t.dim[a] = a < v.ndim ? (uint32_t)v.shape[a] : 1u;
+                n *= t.dim[a];
+            }
+            t.n = n;
+        }
+        hipLaunchKernelGGL(rank1_small_fold_scale_kernel, dim3((uint32_t)k), dim3(256), 0, (hipStream_t)stream, args);
+        const int st = launch_status();
+        if (st != LPMM_OK)
+            return st;
+    }
+    return LPMM_OK;
 }

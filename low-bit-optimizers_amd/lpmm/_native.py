@@ -10,6 +10,7 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "liblpmm_hip.so")
 MULTI_MAX = 48  # tensors per launch of the fused step (LPMM_MULTI_MAX in include/lpmm_hip.h)
+RANK1_SMALL_SLOTS = 8192  # statistics entries of a vector lpmm_rank1_small_fold_scale_multi takes (kNdSmallSlots)
 RANK1_MULTI_MAX = 32  # tensors per launch of the two-pass rank-1 step (kR1Max in csrc/nonfused_rank1.hip)
 SGD_MULTI_MAX = 64  # tensors per launch of the one-pass SGD step (kSgdMax in csrc/sgd.hip)
 V4BIT_MULTI_MAX = 48  # tensors per launch of the one-pass step with an fp32 first moment (kV4Max in csrc/nonfused_m32.hip)
@@ -54,6 +55,8 @@ PROTOTYPES = {
     "lpmm_nonfused_update_multi": (_int, [_vp, _i64] + [_d] * 5 + [_vp]),
     "lpmm_nonfused_adamw4bit_step_multi": (_int, [_vp, _i64, _vp, _vp] + [_d] * 5 + [_vp]),
     "lpmm_nonfused_adamw4bit_rank1_step_multi": (_int, [_vp, _i64, _vp, _vp] + [_d] * 5 + [_vp]),
+    "lpmm_rank1_small_fold_scale_multi": (_int, [_vp, _i64, _vp]),
+    "lpmm_nonfused_adamw4bit_rank1_pass_multi": (_int, [_vp, _i64, _vp, _vp] + [_d] * 5 + [_int, _vp]),
     "lpmm_nonfused_adamw_v4bit_step_multi": (_int, [_vp, _i64, _vp] + [_d] * 5 + [_vp]),
     "lpmm_nonfused_adamw_v4bit_rank1_step_multi": (_int, [_vp, _i64, _vp] + [_d] * 5 + [_vp]),
     "lpmm_nonfused_adamw4bit_rank1_mgroup_step_multi": (_int, [_vp, _i64, _vp, _vp, _i64] + [_d] * 5 + [_vp]),
@@ -80,6 +83,8 @@ NONFUSED_RANK1_TENSOR = np.dtype([("p", "<u8"), ("g", "<u8"), ("m_codes", "<u8")
                                   ("v_codes", "<u8"), ("v_rowmax", "<u8"), ("v_colmax", "<u8"),
                                   ("v_rowmax_next", "<u8"), ("v_colmax_next", "<u8"), ("rows", "<i8"),
                                   ("cols", "<i8"), ("step", "<f4"), ("reserved", "<f4")])
+RANK1_SMALL_VECTOR = np.dtype([("x", "<u8"), ("scale", "<u8"), ("stats", "<u8", (7,)), ("shape", "<i8", (7,)),
+                               ("ndim", "<i4"), ("reserved", "<i4")])
 ADAMW_V4BIT_TENSOR = np.dtype([("p", "<u8"), ("g", "<u8"), ("m", "<u8"), ("v_codes", "<u8"), ("v_max1", "<u8"),
                                ("n", "<i8"), ("step", "<f4"), ("reserved", "<f4")])
 RANK1_V4BIT_TENSOR = np.dtype([("p", "<u8"), ("g", "<u8"), ("m", "<u8"), ("v_codes", "<u8"), ("v_rowmax", "<u8"),

@@ -23,10 +23,16 @@ import numpy as np
 import torch
 
 from .. import _native
-from ..functional import code_table, packed_nbytes, vectorwise_dequant, vectorwise_quant
+from ..functional import RANK1_ND_MAX, _ptr_array, _shape_array, code_table, packed_nbytes, vectorwise_dequant, vectorwise_quant
 from .optimizer import LowBitOptimizer
 
 __all__ = ["AdamW"]
+
+
+def _two_pass_columns(rows, cols):
+    """Column counts the two-pass kernels take on a rows x cols matrix: whole 128-column blocks, or
+    half a block left over with an even row count (taken as double rows)."""
+    return cols % 128 == 0 or (cols % 128 == 64 and rows % 2 == 0)
 
 
 def _is_placeholder(t):
@@ -366,6 +372,7 @@ class AdamW(LowBitOptimizer):
                       and wide_codes(md_v) and md_v["scale_type"] == "rank1")
         batched_rank1_bits = {}
         factored_work = []
+        nd_work = {}  # tensors of more than two dimensions that take the two passes (per device and maps)
         held = []  # contiguous copies of strided operands
 
         def launch_group(key, records):
@@ -443,6 +450,10 @@ class AdamW(LowBitOptimizer):
                     if len(pending) == _native.MULTI_MAX:  # one launch's worth: enqueue it now
                         launch_group(key, pending)
                         pending.clear()
+                    continue
+                if v_rank1 and 2 < p.dim() <= RANK1_ND_MAX and _two_pass_columns(p.shape[0], p.numel() // p.shape[0]):
+                    # a convolution weight and its like, viewed as shape[0] x the rest
+                    nd_work.setdefault(key, []).append((p, dense, grad, state, step))
                     continue
                 # whole 128-column blocks, or half a block left over with an even row count (taken
                 # as double rows: GPT-2-XL's 1600 and 4800 columns)
@@ -529,6 +540,8 @@ class AdamW(LowBitOptimizer):
             if en_v:
                 self._requantise(p, state, "exp_avg_sq", v, md_v)
         self._factored_steps(group, factored_work)
+        for key, items in nd_work.items():
+            self._rank1_nd_steps(group, key, items)
         for dev, records in plain.items():
             table = np.array(records, dtype=_native.ADAMW_FP32_TENSOR)
             with torch.cuda.device(dev):
@@ -661,6 +674,127 @@ class AdamW(LowBitOptimizer):
         mc, ms = self._group_state(p, state, "exp_avg")
         return (dense.data_ptr(), grad.data_ptr(), mc, ms) + self._rank1_state(p, state, batch) + (
             p.shape[0], p.shape[1], step, 0.0)
+
+    def _rank1_nd_steps(self, group, key, items):
+        """The two-pass step on tensors of 3 to 8 dimensions (default configuration: first moment in
+        groups of 128 values, rank-1 second moment).  The reference's scale of such a tensor is the
+        minimum over all its dimensions' statistics (lpmm/functional.py:503-531).  Viewed as
+        shape[0] x (numel / shape[0]) that is min(statistic of row, column scale) with the column
+        scale the minimum over the trailing dimensions' statistics, so the kernels for matrices apply,
+        one pass at a time: the column scale of the current statistics goes in as the column
+        statistics of pass 1; what pass 1 leaves as column maxima of the new second moment is folded
+        into the next statistics of the trailing dimensions (lpmm_rank1_stats_nd on a vector of
+        shape[1:]), and their column scale is what pass 2 divides by.  The statistics of dimension 0
+        are the row statistics of the passes as they are."""
+        dev, qm_ptr, qv_ptr = key
+        lib = _native.lib()
+        beta1, beta2 = group["betas"]
+        lr, wd, eps = group["lr"], group["weight_decay"], group["eps"]
+        batch = _Batch()
+        first, second, between = [], [], []
+        with torch.cuda.device(dev):
+            stream = _native.current_stream(dev)
+            for p, dense, grad, state, step in items:
+                rows, cols = p.shape[0], p.numel() // p.shape[0]
+                trailing = tuple(p.shape[1:]) + (1,)  # lpmm_rank1_row_scale_nd leaves the last dimension out
+                mc, ms = self._group_state(p, state, "exp_avg")
+                vc, cur, nxt = self._rank1_nd_state(p, state, batch)
+                scratch = self._nd_scratch.get(p)
+                if scratch is None or scratch["work"].device != p.device:
+                    scratch = self._nd_scratch[p] = {
+                        "work": torch.empty((3, cols), dtype=torch.float32, device=p.device), "scale_of": None, "row": 0}
+                work = scratch["work"]
+                # rows of `work`: the column scale of the current statistics, the column maxima of the new
+                # second moment, the column scale of the next statistics.  The last step's third row is this
+                # step's first as long as the state still holds the statistics that step left
+                if scratch["scale_of"] is cur:
+                    old_row = scratch["row"]
+                else:
+                    old_row = 0
+                    st = lib.lpmm_rank1_row_scale_nd(_ptr_array(cur[1:] + [cur[0]]), len(trailing),
+                                                     _shape_array(trailing), work[0].data_ptr(), stream)
+                    _native.check(st, "rank1_row_scale_nd")
+                raw_row, new_row = [r for r in range(3) if r != old_row]
+                head = (dense.data_ptr(), grad.data_ptr(), mc, ms, vc, cur[0].data_ptr(), work[old_row].data_ptr(),
+                        nxt[0].data_ptr())
+                tail = (rows, cols, step, 0.0)
+                first.append(head + (work[raw_row].data_ptr(),) + tail)
+                second.append(head + (work[new_row].data_ptr(),) + tail)
+                between.append((p, nxt, work[raw_row], work[new_row], trailing))
+
+                def remember(scratch=scratch, nxt=nxt, new_row=new_row):
+                    scratch["scale_of"], scratch["row"] = nxt, new_row
+
+                batch.commits.append(remember)
+            for pass_no, records in ((1, first), (2, second)):
+                for i in range(0, len(records), _native.RANK1_MULTI_MAX):
+                    chunk = np.array(records[i:i + _native.RANK1_MULTI_MAX], dtype=_native.NONFUSED_RANK1_TENSOR)
+                    st = lib.lpmm_nonfused_adamw4bit_rank1_pass_multi(chunk.ctypes.data, len(chunk), qm_ptr, qv_ptr, beta1,
+                                                                      beta2, lr, wd, eps, pass_no, stream)
+                    _native.check(st, f"non-fused 4-bit AdamW step on tensors of more than two dimensions, pass {pass_no}")
+                if pass_no == 1:
+                    # the column maxima of the new second moment -> next statistics of the trailing dimensions
+                    # -> their column scale: one launch for all tensors whose statistics fit a workgroup's LDS
+                    # (every convolution weight), two calls per tensor otherwise
+                    small = []
+                    for p, nxt, raw, scale, trailing in between:
+                        dims = tuple(p.shape[1:])
+                        if sum(dims) <= _native.RANK1_SMALL_SLOTS:
+                            pad = 7 - len(dims)
+                            small.append((raw.data_ptr(), scale.data_ptr(), tuple(t.data_ptr() for t in nxt[1:]) + (0,) * pad,
+                                          dims + (1,) * pad, len(dims), 0))
+                            continue
+                        st = lib.lpmm_rank1_stats_nd(raw.data_ptr(), p.dim() - 1, _shape_array(dims),
+                                                     _ptr_array(nxt[1:]), None, stream)
+                        _native.check(st, "rank1_stats_nd")
+                        st = lib.lpmm_rank1_row_scale_nd(_ptr_array(nxt[1:] + [nxt[0]]), len(trailing),
+                                                         _shape_array(trailing), scale.data_ptr(), stream)
+                        _native.check(st, "rank1_row_scale_nd")
+                    if small:
+                        vectors = np.array(small, dtype=_native.RANK1_SMALL_VECTOR)
+                        st = lib.lpmm_rank1_small_fold_scale_multi(vectors.ctypes.data, len(small), stream)
+                        _native.check(st, "rank1_small_fold_scale_multi")
+        batch.launched()
+
+    def _rank1_nd_state(self, p, state, batch):
+        """_rank1_state for a tensor of more than two dimensions: one statistic per dimension, in the
+        shapes get_sm3_statistics gives them (lpmm/functional.py:512-531)."""
+        dev = p.device
+        qs_v = state["exp_avg_sq_qstate"]
+        if _is_placeholder(state["exp_avg_sq"]):
+            state["exp_avg_sq"] = torch.full((packed_nbytes(p.numel(), 4),), _zero_byte(qs_v["qmap"]), dtype=torch.int8,
+                                             device=dev)
+            stats = []
+            for i, n in enumerate(p.shape):
+                keep = [1] * p.dim()
+                keep[i] = n
+                stats.append(torch.zeros(keep, dtype=torch.float32, device=dev))
+            qs_v["overhead"].clear()
+            qs_v["overhead"].update({"dtype": p.dtype, "stride": self._state_stride(p), "dim": p.dim(), "max1": None,
+                                     "max_dims": stats, "scaled_shape": p.shape})
+        oh = qs_v["overhead"]
+        cur = oh["max_dims"]
+        nxt = self._spare_stats.get(p)
+        if nxt is None or len(nxt) != len(cur) or nxt[0].device != dev:
+            nxt = [torch.empty_like(t) for t in cur]
+
+        def commit():
+            self._spare_stats[p] = cur
+            oh["max_dims"] = nxt
+
+        batch.commits.append(commit)
+        return state["exp_avg_sq"].data_ptr(), cur, nxt
+
+    @property
+    def _nd_scratch(self):
+        # three vectors of numel / shape[0] floats per tensor of more than two dimensions (the column
+        # scale of the current statistics, the column maxima of the new second moment, the column
+        # scale of the next statistics) and which statistics the kept scale belongs to; not part of
+        # the optimizer state
+        d = self.__dict__.get("_nd_scratch_by_param")
+        if d is None:
+            d = self.__dict__["_nd_scratch_by_param"] = {}
+        return d
 
     @property
     def _spare_stats(self):

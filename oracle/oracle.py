@@ -318,13 +318,14 @@ def rank1_stats_nd(x):
 
 def rank1_scale_nd(stats, shape):
     """_compute_sm3_scale_tensor (lpmm/functional.py:503-509): the statistics broadcast to the
-    tensor's shape and folded with an elementwise minimum, dimension 0 first."""
+    tensor's shape and folded with an elementwise minimum, dimension 0 first; torch.min returns NaN
+    where either operand is NaN, as numpy.minimum does."""
     scale = None
     for i, st in enumerate(stats):
         keep = [1] * len(shape)
         keep[i] = shape[i]
         other = np.broadcast_to(_c(st, np.float32).reshape(keep), shape)
-        scale = other if scale is None else np.where(other < scale, other, scale)
+        scale = other if scale is None else np.minimum(scale, other)
     return np.ascontiguousarray(scale, dtype=np.float32)
 
 

@@ -130,6 +130,32 @@ def test_rank1_folded_rows(oracle, qmaps):
             t.check(f"{t.rows}x{t.cols} step {step}")
 
 
+def test_rank1_one_pass_at_a_time(oracle, qmaps):
+    """lpmm_nonfused_adamw4bit_rank1_pass_multi: pass 1 and pass 2 as separate calls give what the
+    two-pass call gives (here with nothing done in between)."""
+    nat = _native()
+    lib = nat.lib()
+    qm, qv = qmaps
+    dqm, dqv = to_dev(qm), to_dev(qv)
+    rng = np.random.default_rng(31)
+    tensors = [_Tensor(r, c, rng) for r, c in [(65, 384), (64, 192), (130, 128)]]
+    s = torch.cuda.current_stream().cuda_stream
+    for step in (1, 2, 3):
+        grads = [_grad(rng, t) for t in tensors]
+        table = np.array([t.record(g, step) for t, g in zip(tensors, grads)], dtype=nat.NONFUSED_RANK1_TENSOR)
+        for pass_no in (1, 2):
+            st = lib.lpmm_nonfused_adamw4bit_rank1_pass_multi(table.ctypes.data, len(tensors), dqm.data_ptr(), dqv.data_ptr(),
+                                                              H["beta1"], H["beta2"], H["lr"], H["wd"], H["eps"], pass_no, s)
+            assert st == 0, lib.lpmm_status_string(st)
+        for t, g in zip(tensors, grads):
+            t.oracle_step(oracle, g, qm, qv, step)
+        torch.cuda.synchronize()
+        for t in tensors:
+            t.check(f"{t.rows}x{t.cols} step {step}")
+    assert lib.lpmm_nonfused_adamw4bit_rank1_pass_multi(table.ctypes.data, len(tensors), dqm.data_ptr(), dqv.data_ptr(),
+                                                        H["beta1"], H["beta2"], H["lr"], H["wd"], H["eps"], 3, s) == 5
+
+
 def test_rank1_interleaved_row_blocks_with_ragged_last_group(oracle, qmaps):
     """Tensors with more row blocks than interleave in one group: several groups, the last one
     short of blocks and ending in a ragged block (2500 = 39 * 64 + 4 rows over 16 column tiles,

@@ -184,13 +184,23 @@ def test_nonfused_rank1_on_tensors_of_more_than_two_dimensions(oracle, qmaps):
 
     qm, qv = qmaps
     rng = np.random.default_rng(21)
-    shapes = [(6, 40, 64), (32, 16, 3, 3), (4, 24, 130)]
+    # the first five take the two passes on their shape[0] x rest view (rest a multiple of 128, or 64 modulo
+    # 128 with an even shape[0]: double rows), the last two the staged path
+    shapes = [(6, 40, 64), (64, 64, 3, 3), (16, 4, 8, 32), (12, 3, 128), (6, 2, 4, 4, 32), (32, 16, 3, 3), (4, 24, 130)]
     host, params = _params(shapes, rng)
     cfg = os.path.join(os.path.dirname(lpmm.config.__file__), "configs", "default.yml")
     opt = lpmm.optim.AdamW(params, fused=False, qconfig=cfg, **H)
     states = [oracle.NonFusedState(s, v_scale_type="rank1") for s in shapes]
     for step in range(1, 4):
-        grads = [(rng.standard_normal(s) * 1e-3).astype(np.float32) for s in shapes]
+        # structure along every dimension, so that each statistic decides the scale somewhere
+        grads = []
+        for s in shapes:
+            g = rng.standard_normal(s) * 1e-3
+            for d_ in range(len(s)):
+                keep = [1] * len(s)
+                keep[d_] = s[d_]
+                g = g * np.exp(0.7 * rng.standard_normal(keep))
+            grads.append(g.astype(np.float32))
         for p, g in zip(params, grads):
             p.grad = to_dev(g)
         opt.step()

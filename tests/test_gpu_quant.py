@@ -164,6 +164,46 @@ def test_rank1_nd(oracle, qmaps, shape, with_work):
         np.testing.assert_array_equal(to_np(out), oracle.dequant_rank1_nd_bits(want_codes, want_stats, qmap, bits, shape))
 
 
+def test_rank1_small_fold_scale_multi(oracle):
+    """Statistics of every dimension and the scale (their minimum per element) of short vectors, more
+    vectors than one launch holds, against the N-D oracle; signed values and NaN included (|x|, and a
+    NaN statistic makes the scale NaN as torch.min does)."""
+    from lpmm import _native
+
+    lib = _lib()
+    rng = np.random.default_rng(77)
+    shapes = [(64, 3, 3), (16, 1, 1), (7,), (5, 4, 3, 2, 2), (4096, 3, 3), (2, 2, 2, 2, 2, 2, 2), (640,)] * 6
+    shapes = shapes[:40]
+    xs, outs, records = [], [], []
+    for i, shape in enumerate(shapes):
+        x = (rng.standard_normal(shape) * np.exp(rng.standard_normal(shape))).astype(np.float32)
+        x[(0,) * len(shape)] = 0.0
+        if i == 3:
+            x[(1,) * len(shape)] = np.nan
+        dx = to_dev(x)
+        stats = [torch.full((d,), -1.0, dtype=torch.float32, device="cuda") for d in shape]
+        scale = torch.full((x.size,), -1.0, dtype=torch.float32, device="cuda")
+        pad = 7 - len(shape)
+        records.append((dx.data_ptr(), scale.data_ptr(), tuple(t.data_ptr() for t in stats) + (0,) * pad,
+                        tuple(shape) + (1,) * pad, len(shape), 0))
+        xs.append((x, dx))
+        outs.append((stats, scale))
+    table = np.array(records, dtype=_native.RANK1_SMALL_VECTOR)
+    assert lib.lpmm_rank1_small_fold_scale_multi(table.ctypes.data, len(records), _stream()) == 0
+    torch.cuda.synchronize()
+    for (x, _), (stats, scale), shape in zip(xs, outs, shapes):
+        want = oracle.rank1_stats_nd(x)
+        for i, (got, w) in enumerate(zip(stats, want)):
+            np.testing.assert_array_equal(to_np(got), w, err_msg=f"{shape}: statistics of dimension {i}")
+        np.testing.assert_array_equal(to_np(scale), oracle.rank1_scale_nd(want, shape).reshape(-1), err_msg=str(shape))
+    # arguments: no dimensions, more statistics than a workgroup keeps, a missing pointer
+    ok = records[0]
+    for bad, status in ((ok[:4] + (0, 0), 5), (ok[:3] + ((8190, 2, 1, 1, 1, 1, 1),) + ok[4:], 3), ((0,) + ok[1:], 1)):
+        table = np.array([bad], dtype=_native.RANK1_SMALL_VECTOR)
+        assert lib.lpmm_rank1_small_fold_scale_multi(table.ctypes.data, 1, _stream()) == status
+    assert lib.lpmm_rank1_small_fold_scale_multi(None, 0, _stream()) == 0
+
+
 def test_rank1_nd_rejects_bad_arguments():
     import ctypes
 

@@ -267,6 +267,22 @@ def test_rank1_nd_reduces_to_2d_and_to_library_ops(oracle, qmaps):
     stats = oracle.rank1_stats_nd(y)
     assert np.array_equal(stats[0], a) and np.array_equal(stats[1], b) and np.array_equal(stats[2], c)
     assert nibbles(oracle.quant_rank1_nd_bits(y, stats, qv, 4), y.size).reshape(y.shape)[2, 0, 3] == 15
+    # a NaN: max and min of PyTorch's CPU kernels both hand it on, so every slice through it gets a NaN scale
+    z = (rng.standard_normal((4, 3, 5)) ** 2).astype(f32)
+    z[1, 2, 3] = np.nan
+    stats = oracle.rank1_stats_nd(z)
+    t = torch.from_numpy(z).abs()
+    ts = None
+    for i in range(3):
+        red = t
+        for d in range(3):
+            if d != i:
+                red = red.max(dim=d, keepdim=True).values
+        assert np.array_equal(stats[i], red.numpy().reshape(-1), equal_nan=True)
+        ts = red.clone() if ts is None else torch.min(ts, red)
+    scale = oracle.rank1_scale_nd(stats, z.shape)
+    assert np.array_equal(scale, ts.numpy(), equal_nan=True)
+    assert np.isnan(scale).sum() == 4 * 3 * 5 - 3 * 2 * 4
 
 
 def test_nonfused_c_update_follows_torch_cpu_ops(oracle, qmaps):
