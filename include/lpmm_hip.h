@@ -334,6 +334,66 @@ int lpmm_nonfused_adamw4bit_rank1_pass_multi(const lpmm_nonfused_rank1_tensor *t
                                              double beta2, double lr, double weight_decay, double eps,
                                              int pass, void *stream);
 
+/* The non-fused step on float16 parameters (4-bit states, first moment 'group' gp_sz 128).  With
+ * fused=False the reference's op sequence runs PyTorch's half kernels: every op computes in float
+ * and rounds its result to half once, Python scalars enter as floats
+ *   (lpmm/optim/adamw.py:367-369, :394-434);
+ * states, scales and statistics are half tensors, the normalised values are rounded to half by the
+ * division and widened to float for the search
+ *   (lpmm/functional.py:184-203, lpmm/cpp_extension/quantization_kernel.cu:450),
+ * and a dequantised value is the float product of the map entry and the half scale, rounded to
+ * half (lpmm/functional.py:97-118, :150).  These two entry points are that chain in one and in two
+ * passes over HBM; p, g, the scales and the statistics are IEEE binary16 arrays, the code arrays
+ * have the layout of the float entry points above, the first-step convention is theirs too.
+ *
+ * lpmm_nonfused_adamw4bit_f16_step_multi: second moment 'group' gp_sz 128 (also a vector under
+ * 'rank1'); one pass; any n; up to 48 tensors per launch.
+ * lpmm_nonfused_adamw4bit_rank1_f16_step_multi: second moment 'rank1' on row-major R x C tensors
+ * whose column count is a multiple of 128; two passes.  v_rowmax / v_colmax (R / C halfs) are the
+ * statistics the v codes are scaled by, v_rowmax_next / v_colmax_next receive those of the new
+ * second moment (must not alias the current ones: the caller swaps the pairs); `work` is scratch
+ * of ((R + 3) / 4 * 4 + C) floats, 16-byte aligned, whose contents do not matter before and
+ * after the call.  p and g 16-byte aligned. */
+typedef struct lpmm_adamw4bit_f16_tensor {
+    void *p;
+    const void *g;
+    uint8_t *m_codes;
+    uint8_t *v_codes;
+    void *m_max1;
+    void *v_max1;
+    int64_t n;
+    float step;
+    float reserved;
+} lpmm_adamw4bit_f16_tensor;
+
+int lpmm_nonfused_adamw4bit_f16_step_multi(const lpmm_adamw4bit_f16_tensor *tensors, int64_t count,
+                                           const float *qmap_m, const float *qmap_v, double beta1,
+                                           double beta2, double lr, double weight_decay, double eps,
+                                           void *stream);
+
+typedef struct lpmm_nonfused_rank1_f16_tensor {
+    void *p;
+    const void *g;
+    uint8_t *m_codes;
+    void *m_max1;
+    uint8_t *v_codes;
+    const void *v_rowmax;
+    const void *v_colmax;
+    void *v_rowmax_next;
+    void *v_colmax_next;
+    float *work;
+    int64_t rows;
+    int64_t cols;
+    float step;
+    float reserved;
+} lpmm_nonfused_rank1_f16_tensor;
+
+int lpmm_nonfused_adamw4bit_rank1_f16_step_multi(const lpmm_nonfused_rank1_f16_tensor *tensors,
+                                                 int64_t count, const float *qmap_m,
+                                                 const float *qmap_v, double beta1, double beta2,
+                                                 double lr, double weight_decay, double eps,
+                                                 void *stream);
+
 /* The non-fused step with an fp32 first moment and a 4-bit second moment: the configurations
  * that quantise the second moment only (QUANT.M.ENABLE False: lpmm/configs/
  * 2nd_moment_only_group_128.yml and 2nd_moment_only_default.yml).  In _single_tensor_adamw4bit

@@ -472,16 +472,16 @@ template <int MODE, class Record>
 static int rank1_step_multi(const Record *tensors, int64_t count, const float *qmap_m, const float *qmap_v,
                             uint32_t m_lg, double beta1, double beta2, double lr, double weight_decay, double eps,
                             void *stream, int bits_m = 4, int bits_v = 4, const void *table_m = nullptr,
-                            const void *table_v = nullptr, int passes = 3)
+                            const void *table_v = nullptr, int passes = 3, bool half_io = false)
 {
     // passes: 1 = the first pass alone (with the clearing of the next statistics), 2 = the second alone,
     // 3 = both; one at a time only where the launches below are this file's own
-    if (passes < 1 || passes > 3 || (passes != 3 && (MODE != kMCodes128 || bits_m != 4)))
+    if (passes < 1 || passes > 3 || (passes != 3 && (MODE != kMCodes128 || bits_m != 4 || half_io)))
         return LPMM_ERR_ARG;
     constexpr bool M32 = MODE == kMFloat;
     // 4-bit codes in 128-value groups: a column count of 64 modulo 128 with an even row count is
     // served as double rows (rank1_tiles.hpp)
-    const bool can_fold = MODE == kMCodes128 && bits_m == 4;
+    const bool can_fold = MODE == kMCodes128 && bits_m == 4 && !half_io;
     // rows per tile: with an fp32 first moment a pass moves 24.5 instead of 13.5 bytes per element, and
     // tiles of half the rows do better (LLaMA-7B-shaped set 29.3 -> 28.6 ms per step)
     const uint32_t policy_rows = M32 ? kPolicyRowsM32 : kPolicyRows;
@@ -606,7 +606,9 @@ static int rank1_step_multi(const Record *tensors, int64_t count, const float *q
         if (passes & 1)
             hipLaunchKernelGGL(rank1_clear_kernel, dim3((uint32_t)clear_blocks, (uint32_t)k), dim3(kThreads), 0,
                                s, args);
-        if (ragged || (MODE == kMCodesWide && m_lg == 0)) {
+        if (half_io) {
+            launch_rank1_half(args, (uint32_t)tiles, qmap_m, qmap_v, s);
+        } else if (ragged || (MODE == kMCodesWide && m_lg == 0)) {
             launch_rank1_ragged(args, (uint32_t)tiles, qmap_m, qmap_v, s);
         } else if (bits_m != 4) {
             launch_rank1_bits(args, (uint32_t)tiles, qmap_m, qmap_v, bits_m, bits_v,
@@ -640,6 +642,14 @@ extern "C" int lpmm_nonfused_adamw4bit_rank1_step_multi(const lpmm_nonfused_rank
                                                         double eps, void *stream)
 {
     return rank1_step_multi<kMCodes128>(tensors, count, qmap_m, qmap_v, 0, beta1, beta2, lr, weight_decay, eps, stream);
+}
+
+int lpmm::rank1_step_multi_half(const lpmm_nonfused_rank1_tensor *tensors, int64_t count, const float *qmap_m,
+                                const float *qmap_v, double beta1, double beta2, double lr, double weight_decay,
+                                double eps, void *stream)
+{
+    return rank1_step_multi<kMCodes128>(tensors, count, qmap_m, qmap_v, 0, beta1, beta2, lr, weight_decay, eps, stream,
+                                        4, 4, nullptr, nullptr, 3, true);
 }
 
 extern "C" int lpmm_nonfused_adamw4bit_rank1_pass_multi(const lpmm_nonfused_rank1_tensor *tensors, int64_t count,

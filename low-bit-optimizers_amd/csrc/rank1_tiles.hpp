@@ -214,5 +214,11 @@ void launch_rank1_bits(const MultiR1 &args, uint32_t tiles, const float *qmap_m,
                        int bits_v, const uint32_t *table_m, const uint32_t *table_v, hipStream_t stream);
 void launch_rank1_ragged(const MultiR1 &args, uint32_t tiles, const float *qmap_m, const float *qmap_v,
                          hipStream_t stream);
+// float16 parameters (nonfused_half.hip): p, g, the first moment's scales and the current statistics
+// of the records point at halfs, the next statistics at float work arrays
+void launch_rank1_half(const MultiR1 &args, uint32_t tiles, const float *qmap_m, const float *qmap_v, hipStream_t stream);
+int rank1_step_multi_half(const lpmm_nonfused_rank1_tensor *tensors, int64_t count, const float *qmap_m,
+                          const float *qmap_v, double beta1, double beta2, double lr, double weight_decay, double eps,
+                          void *stream);
 
 }  // namespace lpmm

@@ -56,6 +56,8 @@ PROTOTYPES = {
     "lpmm_nonfused_adamw4bit_step_multi": (_int, [_vp, _i64, _vp, _vp] + [_d] * 5 + [_vp]),
     "lpmm_nonfused_adamw4bit_rank1_step_multi": (_int, [_vp, _i64, _vp, _vp] + [_d] * 5 + [_vp]),
     "lpmm_rank1_small_fold_scale_multi": (_int, [_vp, _i64, _vp]),
+    "lpmm_nonfused_adamw4bit_f16_step_multi": (_int, [_vp, _i64, _vp, _vp] + [_d] * 5 + [_vp]),
+    "lpmm_nonfused_adamw4bit_rank1_f16_step_multi": (_int, [_vp, _i64, _vp, _vp] + [_d] * 5 + [_vp]),
     "lpmm_nonfused_adamw4bit_rank1_pass_multi": (_int, [_vp, _i64, _vp, _vp] + [_d] * 5 + [_int, _vp]),
     "lpmm_nonfused_adamw_v4bit_step_multi": (_int, [_vp, _i64, _vp] + [_d] * 5 + [_vp]),
     "lpmm_nonfused_adamw_v4bit_rank1_step_multi": (_int, [_vp, _i64, _vp] + [_d] * 5 + [_vp]),
@@ -83,6 +85,11 @@ NONFUSED_RANK1_TENSOR = np.dtype([("p", "<u8"), ("g", "<u8"), ("m_codes", "<u8")
                                   ("v_codes", "<u8"), ("v_rowmax", "<u8"), ("v_colmax", "<u8"),
                                   ("v_rowmax_next", "<u8"), ("v_colmax_next", "<u8"), ("rows", "<i8"),
                                   ("cols", "<i8"), ("step", "<f4"), ("reserved", "<f4")])
+# float16 parameters: the one-pass record is ADAMW4BIT_TENSOR with half p, g and scales
+NONFUSED_RANK1_F16_TENSOR = np.dtype([("p", "<u8"), ("g", "<u8"), ("m_codes", "<u8"), ("m_max1", "<u8"),
+                                      ("v_codes", "<u8"), ("v_rowmax", "<u8"), ("v_colmax", "<u8"),
+                                      ("v_rowmax_next", "<u8"), ("v_colmax_next", "<u8"), ("work", "<u8"),
+                                      ("rows", "<i8"), ("cols", "<i8"), ("step", "<f4"), ("reserved", "<f4")])
 RANK1_SMALL_VECTOR = np.dtype([("x", "<u8"), ("scale", "<u8"), ("stats", "<u8", (7,)), ("shape", "<i8", (7,)),
                                ("ndim", "<i4"), ("reserved", "<i4")])
 ADAMW_V4BIT_TENSOR = np.dtype([("p", "<u8"), ("g", "<u8"), ("m", "<u8"), ("v_codes", "<u8"), ("v_max1", "<u8"),

@@ -28,6 +28,9 @@
  *   nonfused_step       PyTorch CPU op sequence (library ops) of the reference's
  *                       _single_tensor_adamw4bit, to 1e-6 relative.
  *   factored_step       closed form v = row*col/mean(row) (Adafactor); rank-one g^2 case.
+ *   nonfused_update_f16 PyTorch CPU op sequence on float16 tensors, bit for bit; the two
+ *                       conversions against numpy.float16 on all 65536 halfs and on floats
+ *                       around every rounding boundary.
  *   sgd_update          PyTorch CPU op sequence (library ops) of the reference's
  *                       _single_tensor_sgd4bit, bit for bit.
  *   philox / SR pack    Random123's known-answer vectors for philox4x32-10; torch.randint on
@@ -503,6 +506,103 @@ void lpmm_oracle_nonfused_update(float *p, const float *g, float *m, float *v, i
         p[i] = pi;
         m[i] = mi;
         v[i] = vi;
+    }
+}
+
+/* ------------------------------------------------------------------------------------ */
+/* The same elementwise part on float16 tensors (float16 parameters with fused=False:   */
+/* the reference's op sequence then runs PyTorch's half kernels, lpmm/optim/adamw.py     */
+/* :367-369, :412-422).  Every op of PyTorch on half tensors converts its operands to    */
+/* float, computes as the float kernel does and rounds the result to half once, so the   */
+/* chain below is the float chain above with a rounding to half after each op; Python    */
+/* scalars enter as floats, never as halfs.  Conversions: IEEE binary16, round to        */
+/* nearest even, subnormals kept (c10::Half, numpy.float16).                             */
+/* ------------------------------------------------------------------------------------ */
+static inline float h2f(uint16_t h)
+{
+    const uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+    const uint32_t exp = (h >> 10) & 0x1Fu, man = h & 0x3FFu;
+    uint32_t bits;
+    if (exp == 0x1Fu) {
+        bits = sign | 0x7F800000u | (man << 13);
+    } else if (exp != 0) {
+        bits = sign | ((exp + 112u) << 23) | (man << 13);
+    } else {
+        /* zero or subnormal: man * 2^-24, exact in float */
+        float f = (float)man * 0x1p-24f;
+        memcpy(&bits, &f, 4);
+        bits |= sign;
+    }
+    float out;
+    memcpy(&out, &bits, 4);
+    return out;
+}
+
+static inline uint16_t f2h(float f)
+{
+    uint32_t bits;
+    memcpy(&bits, &f, 4);
+    const uint16_t sign = (uint16_t)((bits >> 16) & 0x8000u);
+    const uint32_t a = bits & 0x7FFFFFFFu;
+    if (a > 0x7F800000u)
+        return (uint16_t)(sign | 0x7E00u | ((a >> 13) & 0x3FFu)); /* NaN stays NaN (quiet) */
+    if (a >= 0x47800000u)                                          /* |f| >= 65536: infinity (65520 rounds there below) */
+        return (uint16_t)(sign | 0x7C00u);
+    if (a < 0x38800000u) {
+        /* below the smallest normal half (2^-14): the result is round(|f| * 2^24) units of 2^-24; */
+        /* adding 0.5f places those units at the last place of the float sum, which rounds to nearest even */
+        float af;
+        memcpy(&af, &a, 4);
+        const float t = af + 0.5f;
+        uint32_t tb;
+        memcpy(&tb, &t, 4);
+        return (uint16_t)(sign | (tb - 0x3F000000u));
+    }
+    /* normal: drop 13 mantissa bits with round to nearest even; a carry runs into the exponent */
+    const uint32_t r = a + 0xFFFu + ((a >> 13) & 1u);
+    return (uint16_t)(sign | ((r - 0x38000000u) >> 13));
+}
+
+void lpmm_oracle_f16_to_f32(const uint16_t *h, float *f, int64_t n)
+{
+    for (int64_t i = 0; i < n; ++i)
+        f[i] = h2f(h[i]);
+}
+
+void lpmm_oracle_f32_to_f16(const float *f, uint16_t *h, int64_t n)
+{
+    for (int64_t i = 0; i < n; ++i)
+        h[i] = f2h(f[i]);
+}
+
+static inline float rh(float x) { return h2f(f2h(x)); }
+
+void lpmm_oracle_nonfused_update_f16(uint16_t *p, const uint16_t *g, uint16_t *m, uint16_t *v, int64_t n,
+                                     double beta1, double beta2, double lr, double weight_decay,
+                                     double eps, double step)
+{
+    const float decay = (float)(1.0 - lr * weight_decay);
+    const float w1 = (float)(1.0 - beta1);
+    const float b2 = (float)beta2;
+    const float w2 = (float)(1.0 - beta2);
+    const double bc1 = 1.0 - pow(beta1, step);
+    const double bc2 = 1.0 - pow(beta2, step);
+    const float neg_step_size = (float)(-(lr / bc1));
+    const float bc2_sqrt = (float)sqrt(bc2);
+    const float epsf = (float)eps;
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < n; ++i) {
+        const float gi = h2f(g[i]);
+        const float pi = rh(h2f(p[i]) * decay);            /* param.mul_(1 - lr * weight_decay) */
+        const float mi = rh(lerp_small_w(h2f(m[i]), gi, w1)); /* exp_avg.lerp_(grad, 1 - beta1) */
+        float vi = rh(h2f(v[i]) * b2);                      /* exp_avg_sq.mul_(beta2) */
+        vi = rh(vi + (w2 * gi) * gi);                       /* .addcmul_(grad, grad, value=1 - beta2) */
+        float denom = rh(sqrtf(vi));                        /* exp_avg_sq.sqrt() */
+        denom = rh(denom / bc2_sqrt);                       /* / bias_correction2_sqrt */
+        denom = rh(denom + epsf);                           /* .add_(eps) */
+        p[i] = f2h(pi + (neg_step_size * mi) / denom);      /* param.addcdiv_(exp_avg, denom, value=-step_size) */
+        m[i] = f2h(mi);
+        v[i] = f2h(vi);
     }
 }
 

@@ -11,6 +11,9 @@ Functions restated here in numpy rather than in C, and what pins them (tests/tes
                       float16 round trip of it operation by operation (moments re-read after rounding).
   rank1_*_nd          on a 2-D tensor the 2-D C functions bit for bit; on 3-D/4-D tensors the
                       reference's op sequence run by PyTorch's CPU kernels and a loop over all indices.
+  *_f16               float16 scaling around the C search: each op in float with one rounding to half
+                      (numpy.float16 arithmetic), against the same ops of PyTorch's CPU half kernels
+                      bit for bit (codes, scales, statistics and three whole steps).
   map construction    the bit patterns the reference's recipe gives when PyTorch's ops run it
                       (tests/golden/qmaps.json).
 """
@@ -82,6 +85,11 @@ _dequant_rank1 = _sig("lpmm_oracle_dequant_rank1", None, _u8p, _f32p, _f32p, _f3
                       _f32p)
 _nonfused_update = _sig("lpmm_oracle_nonfused_update", None, _f32p, _f32p, _f32p, _f32p, _i64,
                         _d, _d, _d, _d, _d, _d)
+_u16p = np.ctypeslib.ndpointer(dtype=np.uint16, flags="C_CONTIGUOUS")
+_nonfused_update_f16 = _sig("lpmm_oracle_nonfused_update_f16", None, _u16p, _u16p, _u16p, _u16p, _i64,
+                            _d, _d, _d, _d, _d, _d)
+_f16_to_f32 = _sig("lpmm_oracle_f16_to_f32", None, _u16p, _f32p, _i64)
+_f32_to_f16 = _sig("lpmm_oracle_f32_to_f16", None, _f32p, _u16p, _i64)
 _sgd_update = _sig("lpmm_oracle_sgd_update", None, _f32p, _f32p, _f32p, _i64, _d, _d, _d, _d, ctypes.c_int,
                    ctypes.c_int, ctypes.c_int)
 _factored_stats = _sig("lpmm_oracle_factored_stats", None, _f32p, _i64, _i64, _f32p, _f32p)
@@ -273,7 +281,7 @@ def unpack_nonlinear(codes, qmap, bits, n):
 
 def _pad_to(x, multiple):
     rem = (-x.size) % multiple
-    return np.concatenate([x, np.zeros(rem, np.float32)]) if rem else x
+    return np.concatenate([x, np.zeros(rem, x.dtype)]) if rem else x
 
 
 def quant_group_bits(x, qmap, bits, gp_sz=GROUP):
@@ -544,3 +552,111 @@ def _factored_step(p, g, state, qm, lr, beta1, beta2, eps, wd):
                     eps, float(state.step))
     state.m = quant_group(m, qm)
     return m, None
+
+
+# --------------------------------------------------------------------------------------
+# float16 parameters on the non-fused path: the reference's chain runs PyTorch's half kernels
+# (lpmm/optim/adamw.py:394-434, lpmm/functional.py:184-203, :97-118).  Every op converts to float,
+# computes and rounds to half once; states, scales and statistics are float16; the pack kernel
+# widens each normalised (half) value to float before the search
+# (lpmm/cpp_extension/quantization_kernel.cu:450); the unpacked map values are float32, their
+# product with the float16 scale is float32 (type promotion) and takes the state's type last
+# (lpmm/functional.py:150).
+# --------------------------------------------------------------------------------------
+f16 = np.float16
+
+
+def f16_to_f32(h):
+    h = _c(h, np.float16).reshape(-1)
+    out = np.empty(h.size, np.float32)
+    _f16_to_f32(h.view(np.uint16), out, h.size)
+    return out
+
+
+def f32_to_f16(x):
+    x = _c(x, np.float32).reshape(-1)
+    out = np.empty(x.size, np.uint16)
+    _f32_to_f16(x, out, x.size)
+    return out.view(np.float16)
+
+
+def nonfused_update_f16(p, g, m, v, beta1, beta2, lr, wd, eps, step):
+    """Elementwise part of the step on float16 arrays, in place."""
+    for a in (p, g, m, v):
+        assert a.dtype == np.float16 and a.flags.c_contiguous
+    _nonfused_update_f16(p.reshape(-1).view(np.uint16), g.reshape(-1).view(np.uint16), m.reshape(-1).view(np.uint16),
+                         v.reshape(-1).view(np.uint16), p.size, beta1, beta2, lr, wd, eps, step)
+
+
+def _pack_padded(normed16, qmap):
+    """functional.py:361-363 on half values: widen, zero-pad to whole pack groups, search, pack."""
+    return pack_nonlinear_4bit(_pad_to(normed16.astype(np.float32).reshape(-1), PACK_GROUP), qmap)
+
+
+def quant_group_f16(x, qmap, gp_sz=GROUP):
+    """functional.py:184-189 then :359-369 on a float16 tensor: (codes, float16 max1 of G values)."""
+    grouped = _pad_to(_c(x, np.float16).reshape(-1), gp_sz).reshape(-1, gp_sz)
+    max1 = np.abs(grouped).max(axis=1)
+    with np.errstate(invalid="ignore", divide="ignore"):
+        normed = (grouped.astype(np.float32) / max1.astype(np.float32)[:, None]).astype(np.float16)
+    return _pack_padded(normed, qmap), max1
+
+
+def dequant_group_f16(codes, max1, qmap, n, gp_sz=GROUP):
+    """functional.py:393-400, :115-118, :150: float32 map value times float16 scale, in float, then to half."""
+    g = max1.size
+    vals = unpack_nonlinear_4bit(codes, qmap, g * gp_sz).reshape(g, gp_sz)
+    return (vals * _c(max1, np.float16).reshape(-1, 1).astype(np.float32)).astype(np.float16).reshape(-1)[:n]
+
+
+def rank1_stats_f16(x):
+    a = np.abs(_c(x, np.float16))
+    return a.max(axis=1), a.max(axis=0)
+
+
+def _rank1_scale_f16(rowmax, colmax):
+    r, c = rowmax.astype(np.float32), colmax.astype(np.float32)
+    return np.where(c[None, :] < r[:, None], c[None, :], r[:, None])
+
+
+def quant_rank1_f16(x, rowmax, colmax, qmap):
+    """functional.py:190-203 on a float16 matrix."""
+    x = _c(x, np.float16)
+    with np.errstate(invalid="ignore", divide="ignore"):
+        normed = (x.astype(np.float32) / _rank1_scale_f16(rowmax, colmax)).astype(np.float16)
+    return _pack_padded(normed, qmap)
+
+
+def dequant_rank1_f16(codes, rowmax, colmax, qmap, r, c):
+    vals = unpack_nonlinear_4bit(codes, qmap, (r * c + 7) // 8 * 8)[: r * c].reshape(r, c)
+    return (vals * _rank1_scale_f16(rowmax, colmax)).astype(np.float16)
+
+
+def nonfused_step_f16(p, g, state, qm, qv, lr, beta1, beta2, eps, wd):
+    """One step of _single_tensor_adamw4bit on one quantised float16 tensor (4-bit states, first
+    moment 'group' 128, second 'group' 128 or 'rank1' on a matrix).  p (float16) is updated in place;
+    state is a NonFusedState whose scales and statistics are float16 arrays."""
+    assert p.dtype == np.float16 and g.dtype == np.float16 and state.bits == 4 and not state.factored
+    state.step += 1
+    n = state.n
+    rank1 = _v_is_rank1(state)
+    assert not rank1 or len(state.shape) == 2
+    m = np.zeros(n, np.float16) if state.m is None else dequant_group_f16(state.m[0], state.m[1], qm, n)
+    if state.v is None:
+        v = np.zeros(n, np.float16)
+    elif rank1:
+        r, c = state.shape
+        v = np.ascontiguousarray(dequant_rank1_f16(state.v[0], state.v[1], state.v[2], qv, r, c)).reshape(-1)
+    else:
+        v = dequant_group_f16(state.v[0], state.v[1], qv, n)
+    m, v = np.ascontiguousarray(m), np.ascontiguousarray(v)
+    nonfused_update_f16(p.reshape(-1), np.ascontiguousarray(g).reshape(-1), m, v, beta1, beta2, lr, wd, eps,
+                        float(state.step))
+    state.m = quant_group_f16(m, qm)
+    if rank1:
+        v2 = v.reshape(state.shape)
+        rowmax, colmax = rank1_stats_f16(v2)
+        state.v = (quant_rank1_f16(v2, rowmax, colmax, qv), rowmax, colmax)
+    else:
+        state.v = quant_group_f16(v, qv)
+    return m, v

@@ -1,0 +1,216 @@
+"""GPU parity of the non-fused AdamW step on float16 parameters (4-bit states; second moment block-wise
+in one pass, rank-1 in two) against the CPU oracle's float16 restatement of the reference's op chain
+(oracle.nonfused_step_f16: every op in float with one rounding to half, half scales and statistics),
+called through the C ABI on torch device memory.  Parameters, scales, statistics and the packed
+buffers are compared bit for bit, the buffers in full (padding codes and the extra last byte
+included); a NaN equals a NaN."""
+import numpy as np
+import pytest
+import torch
+
+from util import to_dev, to_np
+
+pytestmark = pytest.mark.gpu
+
+f16 = np.float16
+
+
+def _native():
+    from lpmm import _native
+
+    return _native
+
+
+def _nbytes(n):
+    return (n + 2047) // 2048 * 1024 + 1
+
+
+def _same_halfs(got, want, what):
+    got, want = np.ascontiguousarray(got).reshape(-1), np.ascontiguousarray(want).reshape(-1)
+    assert got.dtype == want.dtype == f16, what
+    ok = (got.view(np.uint16) == want.view(np.uint16)) | (np.isnan(got) & np.isnan(want))
+    assert ok.all(), (what, int((~ok).sum()), got[~ok][:5], want[~ok][:5])
+
+
+def _dev_halfs(a, offset=0):
+    buf = torch.empty(a.size + offset, dtype=torch.float16, device="cuda")
+    view = buf[offset:]
+    view.copy_(torch.from_numpy(np.ascontiguousarray(a).reshape(-1)))
+    return view
+
+
+def _codes(n, zero_byte):
+    c = np.full(_nbytes(n), 0xA5, np.uint8)  # a pattern the kernels have to overwrite
+    c[: (n + 1) // 2] = zero_byte
+    return to_dev(c)
+
+
+class _Flat:
+    """A tensor of n halfs, both moments block-wise over 128 values."""
+
+    def __init__(self, oracle, n, rng, offset=0):
+        self.n, self.offset = n, offset
+        self.host_p = (rng.standard_normal(n) * 0.5).astype(f16)
+        self.state = oracle.NonFusedState((n,), "group")
+        self.p = _dev_halfs(self.host_p, offset)
+        self.mc, self.vc = _codes(n, 0x77), _codes(n, 0x00)
+        groups = (n + 127) // 128
+        self.ms = torch.zeros(groups, dtype=torch.float16, device="cuda")
+        self.vs = torch.zeros(groups, dtype=torch.float16, device="cuda")
+        self.g = None
+
+    def record(self, g, step):
+        self.g = _dev_halfs(g, self.offset)
+        return (self.p.data_ptr(), self.g.data_ptr(), self.mc.data_ptr(), self.vc.data_ptr(), self.ms.data_ptr(),
+                self.vs.data_ptr(), self.n, float(step), 0.0)
+
+    def check(self, what):
+        st = self.state
+        _same_halfs(to_np(self.ms), st.m[1], f"{what}: m max1")
+        _same_halfs(to_np(self.vs), st.v[1], f"{what}: v max1")
+        np.testing.assert_array_equal(to_np(self.mc), st.m[0], err_msg=f"{what}: m codes")
+        np.testing.assert_array_equal(to_np(self.vc), st.v[0], err_msg=f"{what}: v codes")
+        _same_halfs(to_np(self.p), self.host_p, f"{what}: p")
+
+
+@pytest.mark.parametrize("eps", [1e-3, 1e-8])
+def test_one_pass_half_step(oracle, qmaps, eps):
+    """Whole tiles, a ragged end, fewer values than a group, pointers that allow no 8-byte accesses;
+    four steps with shrinking gradients, so that second moments underflow to zero in half.  With the
+    default eps (zero as a half) such elements divide by zero: the infinities and NaNs are compared too."""
+    nat = _native()
+    lib = nat.lib()
+    qm, qv = qmaps
+    dqm, dqv = to_dev(qm), to_dev(qv)
+    rng = np.random.default_rng(21)
+    hyper = dict(lr=1e-2, beta1=0.9, beta2=0.999, wd=0.01)
+    tensors = [_Flat(oracle, 2048 * 3, rng), _Flat(oracle, 5000, rng), _Flat(oracle, 100, rng),
+               _Flat(oracle, 11008, rng, offset=1), _Flat(oracle, 2048 * 2 + 128, rng, offset=3)]
+    for step in range(1, 5):
+        grads = [(rng.standard_normal(t.n) * 0.3 * 10.0 ** -step).astype(f16) for t in tensors]
+        records = [t.record(g, step) for t, g in zip(tensors, grads)]
+        table = np.array(records, dtype=nat.ADAMW4BIT_TENSOR)
+        st = lib.lpmm_nonfused_adamw4bit_f16_step_multi(table.ctypes.data, len(records), dqm.data_ptr(), dqv.data_ptr(),
+                                                        hyper["beta1"], hyper["beta2"], hyper["lr"], hyper["wd"], eps,
+                                                        nat.current_stream(torch.device("cuda:0")))
+        assert st == 0
+        torch.cuda.synchronize()
+        for i, (t, g) in enumerate(zip(tensors, grads)):
+            oracle.nonfused_step_f16(t.host_p, g, t.state, qm, qv, hyper["lr"], hyper["beta1"], hyper["beta2"], eps,
+                                     hyper["wd"])
+            t.check(f"step {step} tensor {i} (n = {t.n})")
+    if eps == 1e-3:
+        assert all(np.isfinite(t.host_p).all() for t in tensors)
+    else:
+        assert any(not np.isfinite(t.host_p).all() for t in tensors)
+
+
+class _Matrix:
+    """A matrix of halfs: first moment block-wise, second moment rank-1."""
+
+    def __init__(self, oracle, rows, cols, rng):
+        self.rows, self.cols, self.n = rows, cols, rows * cols
+        self.host_p = (rng.standard_normal((rows, cols)) * 0.5).astype(f16)
+        self.state = oracle.NonFusedState((rows, cols), "rank1")
+        self.p = _dev_halfs(self.host_p)
+        self.mc, self.vc = _codes(self.n, 0x77), _codes(self.n, 0x00)
+        self.ms = torch.zeros(self.n // 128, dtype=torch.float16, device="cuda")
+        self.stats = [torch.zeros(rows, dtype=torch.float16, device="cuda"),
+                      torch.zeros(cols, dtype=torch.float16, device="cuda")]
+        self.next = [torch.full((rows,), 7.0, dtype=torch.float16, device="cuda"),
+                     torch.full((cols,), 7.0, dtype=torch.float16, device="cuda")]
+        self.work = torch.full(((rows + 3) // 4 * 4 + cols,), 3.0, dtype=torch.float32, device="cuda")
+        self.g = None
+
+    def record(self, g, step):
+        self.g = _dev_halfs(g)
+        return (self.p.data_ptr(), self.g.data_ptr(), self.mc.data_ptr(), self.ms.data_ptr(), self.vc.data_ptr(),
+                self.stats[0].data_ptr(), self.stats[1].data_ptr(), self.next[0].data_ptr(), self.next[1].data_ptr(),
+                self.work.data_ptr(), self.rows, self.cols, float(step), 0.0)
+
+    def launched(self):
+        self.stats, self.next = self.next, self.stats
+
+    def check(self, what):
+        st = self.state
+        _same_halfs(to_np(self.ms), st.m[1], f"{what}: m max1")
+        np.testing.assert_array_equal(to_np(self.mc), st.m[0], err_msg=f"{what}: m codes")
+        _same_halfs(to_np(self.stats[0]), st.v[1], f"{what}: row statistics")
+        _same_halfs(to_np(self.stats[1]), st.v[2], f"{what}: column statistics")
+        np.testing.assert_array_equal(to_np(self.vc), st.v[0], err_msg=f"{what}: v codes")
+        _same_halfs(to_np(self.p), self.host_p, f"{what}: p")
+
+
+@pytest.mark.parametrize("eps", [1e-3, 1e-8])
+def test_two_pass_half_step(oracle, qmaps, eps):
+    """Matrices with one column block, with more blocks than a tile is wide, with fewer rows than a
+    tile, with a row count that is no multiple of the rows of a pass; 34 tensors (two launch groups),
+    four steps with shrinking gradients, a row and a column of zero gradients."""
+    nat = _native()
+    lib = nat.lib()
+    qm, qv = qmaps
+    dqm, dqv = to_dev(qm), to_dev(qv)
+    rng = np.random.default_rng(22)
+    hyper = dict(lr=1e-2, beta1=0.9, beta2=0.999, wd=0.01)
+    shapes = [(96, 256), (33, 128), (200, 384), (64, 1024), (7, 640), (130, 128)] + [(20, 128)] * 28
+    tensors = [_Matrix(oracle, r, c, rng) for r, c in shapes]
+    for step in range(1, 5):
+        grads = [(rng.standard_normal((t.rows, t.cols)) * 0.3 * 10.0 ** -step).astype(f16) for t in tensors]
+        grads[0][5, :] = 0
+        grads[0][:, 9] = 0
+        records = [t.record(g, step) for t, g in zip(tensors, grads)]
+        table = np.array(records, dtype=nat.NONFUSED_RANK1_F16_TENSOR)
+        st = lib.lpmm_nonfused_adamw4bit_rank1_f16_step_multi(
+            table.ctypes.data, len(records), dqm.data_ptr(), dqv.data_ptr(), hyper["beta1"], hyper["beta2"],
+            hyper["lr"], hyper["wd"], eps, nat.current_stream(torch.device("cuda:0")))
+        assert st == 0
+        torch.cuda.synchronize()
+        for i, (t, g) in enumerate(zip(tensors, grads)):
+            t.launched()
+            oracle.nonfused_step_f16(t.host_p, g, t.state, qm, qv, hyper["lr"], hyper["beta1"], hyper["beta2"], eps,
+                                     hyper["wd"])
+            if i < 8 or step == 4:
+                t.check(f"step {step} tensor {i} {t.rows} x {t.cols}")
+
+
+def test_half_steps_reject_bad_arguments(qmaps):
+    nat = _native()
+    lib = nat.lib()
+    dqm, dqv = to_dev(qmaps[0]), to_dev(qmaps[1])
+    s = nat.current_stream(torch.device("cuda:0"))
+    h = (0.9, 0.999, 1e-3, 0.01, 1e-8)
+    p = torch.zeros(256, dtype=torch.float16, device="cuda")
+    codes = torch.zeros(1025, dtype=torch.uint8, device="cuda")
+    sc = torch.zeros(2, dtype=torch.float16, device="cuda")
+    ok = (p.data_ptr(), p.data_ptr(), codes.data_ptr(), codes.data_ptr(), sc.data_ptr(), sc.data_ptr(), 256, 1.0, 0.0)
+
+    def flat(rec, count=1, qm=dqm.data_ptr()):
+        table = np.array([rec], dtype=nat.ADAMW4BIT_TENSOR)
+        return lib.lpmm_nonfused_adamw4bit_f16_step_multi(table.ctypes.data, count, qm, dqv.data_ptr(), *h, s)
+
+    assert flat(ok, count=0) == 0
+    assert flat(ok, count=-1) == 3
+    assert flat(ok, qm=None) == 1
+    assert flat((0,) + ok[1:]) == 1
+    assert flat(ok[:6] + (-1,) + ok[7:]) == 3
+    assert flat((p.data_ptr() + 1,) + ok[1:]) == 2
+    assert flat(ok[:6] + (0,) + ok[7:]) == 0  # an empty tensor is skipped
+
+    stats = [torch.zeros(2, dtype=torch.float16, device="cuda") for _ in range(2)]
+    cs = [torch.zeros(128, dtype=torch.float16, device="cuda") for _ in range(2)]
+    work = torch.zeros(4 + 128, dtype=torch.float32, device="cuda")
+    okr = (p.data_ptr(), p.data_ptr(), codes.data_ptr(), sc.data_ptr(), codes.data_ptr(), stats[0].data_ptr(),
+           cs[0].data_ptr(), stats[1].data_ptr(), cs[1].data_ptr(), work.data_ptr(), 2, 128, 1.0, 0.0)
+
+    def matrix(rec, count=1):
+        table = np.array([rec], dtype=nat.NONFUSED_RANK1_F16_TENSOR)
+        return lib.lpmm_nonfused_adamw4bit_rank1_f16_step_multi(table.ctypes.data, count, dqm.data_ptr(), dqv.data_ptr(),
+                                                                *h, s)
+
+    assert matrix(okr, count=0) == 0
+    assert matrix(okr[:11] + (64,) + okr[12:]) == 3  # the column count must be a multiple of 128
+    assert matrix(okr[:9] + (0,) + okr[10:]) == 1  # no work array
+    assert matrix(okr[:9] + (work.data_ptr() + 4,) + okr[10:]) == 2
+    assert matrix(okr[:7] + (stats[0].data_ptr(),) + okr[8:]) == 5  # the next statistics alias the current ones
+    assert matrix((0,) + okr[1:]) == 1
+    torch.cuda.synchronize()

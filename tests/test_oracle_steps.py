@@ -477,3 +477,65 @@ def test_fp16_step_reads_the_rounded_moments(oracle):
     from_rounded = update(mh.astype(f), vh.astype(f))
     assert np.mean(from_rounded == ph) > 0.999  # the C library's powf and ** may differ in the last place
     assert np.any(update(m32, v32) != from_rounded)
+
+
+def test_half_conversions_are_numpy_float16(oracle):
+    """The oracle's binary16 <-> binary32 conversions against numpy.float16: every half, and floats at and next to
+    every half, every midpoint between neighbouring halfs, the overflow threshold and random values."""
+    h = np.arange(65536, dtype=np.uint16).view(np.float16)
+    f = oracle.f16_to_f32(h)
+    assert np.array_equal(f.view(np.uint32), h.astype(f32).view(np.uint32))
+    rng = np.random.default_rng(0)
+    fs = np.sort(f[np.isfinite(f)])
+    mid = ((fs[:-1].astype(np.float64) + fs[1:].astype(np.float64)) / 2).astype(f32)
+    up, down = f32(np.inf), f32(-np.inf)
+    with np.errstate(invalid="ignore"):
+        x = np.concatenate([
+            rng.standard_normal(1 << 18).astype(f32) * np.exp(rng.standard_normal(1 << 18) * 6).astype(f32),
+            f, np.nextafter(f, up), np.nextafter(f, down), mid, np.nextafter(mid, up), np.nextafter(mid, down),
+            np.array([65519.99, 65520, 65520.01, 1e9, -1e9, np.inf, -np.inf, 0.0, -0.0, 2.0 ** -25, 2.0 ** -24], f32)])
+    with np.errstate(over="ignore"):
+        got, want = oracle.f32_to_f16(x), x.astype(np.float16)
+    assert np.all((got.view(np.uint16) == want.view(np.uint16)) | (np.isnan(got) & np.isnan(want)))
+
+
+@pytest.mark.parametrize("v_scale", ["rank1", "group"])
+@pytest.mark.parametrize("eps", [1e-3, 1e-8])
+def test_nonfused_half_step_is_the_torch_cpu_half_chain(oracle, qmaps, v_scale, eps):
+    """nonfused_step_f16 (C update with a rounding to half after every op, numpy float16 scaling, the C search)
+    against the reference's op sequence run by PyTorch's CPU half kernels: parameters, both moments, codes,
+    scales and statistics bit for bit over four steps with shrinking gradients.  With eps = 1e-8 (the default,
+    which float16 rounds to zero) elements whose second moment is zero divide by zero; both sides agree on the
+    infinities and NaNs as well."""
+    from oracle.nonfused_torch import TorchNonFusedAdamW
+
+    qm, qv = qmaps
+    torch.manual_seed(5)
+    shapes = [(96, 160), (11008,), (33, 256), (5000,), (45, 100)]  # the last two end in a partial group
+    hyper = dict(lr=1e-2, betas=(0.9, 0.999), eps=eps, weight_decay=0.01)
+    host = [(torch.randn(s) * 0.5).half() for s in shapes]
+    ref = TorchNonFusedAdamW([h.clone() for h in host], v_scale_type=v_scale, **hyper)
+    ps = [h.numpy().copy() for h in host]
+    states = [oracle.NonFusedState(s, v_scale) for s in shapes]
+
+    def same(a, b):
+        a, b = np.ascontiguousarray(a).reshape(-1), np.ascontiguousarray(b).reshape(-1)
+        assert a.dtype == b.dtype == np.float16
+        return np.all((a.view(np.uint16) == b.view(np.uint16)) | (np.isnan(a) & np.isnan(b)))
+
+    for step in range(1, 5):
+        grads = [(torch.randn(s) * 0.3 * 10.0 ** -step).half() for s in shapes]
+        ref.step(grads)
+        for i, s in enumerate(shapes):
+            m, v = oracle.nonfused_step_f16(ps[i], grads[i].numpy(), states[i], qm, qv, hyper["lr"], 0.9, 0.999, eps, 0.01)
+            rs = ref.state[i]
+            assert same(ps[i], ref.params[i].numpy()), (step, s)
+            assert same(m, rs["m_fp32"].numpy()) and same(v, rs["v_fp32"].numpy()), (step, s)
+            assert np.array_equal(states[i].m[0], rs["m"][0].numpy()) and same(states[i].m[1], rs["m"][1].numpy())
+            assert np.array_equal(states[i].v[0], rs["v"][0].numpy()), (step, s)
+            if v_scale == "rank1" and len(s) == 2:
+                assert same(states[i].v[1], rs["v"][1][0].numpy()) and same(states[i].v[2], rs["v"][1][1].numpy())
+            else:
+                assert same(states[i].v[1], rs["v"][1].numpy())
+        if eps == 1e-3:
+            assert all(np.isfinite(p).all() for p in ps)
