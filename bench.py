@@ -493,6 +493,18 @@ def run_nonfused(torch, args, v_scale, m32=False, mgroup=False):
     dev = torch.device("cuda:0")
     shapes = {"gpt2xl": gpt2xl_shapes, "conv": conv_shapes, "llama7b": llama7b_shapes}[args.shapes]()
     params = make_params(torch, shapes, dev, heavy_tailed=True)
+    half = args.half
+    if half:
+        if m32 or mgroup or args.bits != 4 or args.shapes != "llama7b":
+            sys.exit("bench.py: --half goes with --workload nonfused_group|nonfused_rank1 on the LLaMA-7B-shaped set")
+        # float16 parameters and gradients (gradients of 1e-3 scale: most squares underflow in half, as they
+        # do in a real float16 run without loss scaling); eps 1e-3, since float16 rounds 1e-8 to zero
+        halves = []
+        for q in params:
+            h = torch.nn.Parameter(q.detach().half())
+            h.grad = q.grad.half()
+            halves.append(h)
+        params = halves
     bits = args.bits if (v_scale == "rank1" and not m32 and not mgroup) else 4
     if bits != 4:
         if bits < 5:
@@ -505,8 +517,8 @@ def run_nonfused(torch, args, v_scale, m32=False, mgroup=False):
     else:
         name = "2nd_moment_group_128.yml" if v_scale == "group" else "default.yml"
     cfg = os.path.join(os.path.dirname(lpmm.config.__file__), "configs", name)
-    opt = lpmm.optim.AdamW(params, lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01, fused=False,
-                           qconfig=cfg)
+    opt = lpmm.optim.AdamW(params, lr=1e-3, betas=(0.9, 0.999), eps=1e-3 if half else 1e-8, weight_decay=0.01,
+                           fused=False, qconfig=cfg)
     n_total = sum(p.numel() for p in params)
     with _gc_paused():
         for _ in range(args.warmup):
@@ -526,6 +538,8 @@ def run_nonfused(torch, args, v_scale, m32=False, mgroup=False):
         bytes_per_param = 19.0 + 12.0 / 1024
     if bits != 4:  # one code per byte: p 8, g 4 + 4, m codes 2, v codes 1 + 2, scales 8/128
         bytes_per_param = 21.0625
+    if half:  # p 2 + 2, g 2 (+ 2 in the second pass), codes and half scales as above
+        bytes_per_param = 8.0625 if v_scale == "group" else 7.53125 + 3.0
     if args.shapes != "llama7b":
         # a mix of paths: per tensor, what its path moves (rank-1: tensors whose shape[0] x rest view has
         # whole 128-column blocks, or half a block left over with an even row count, as above; other
@@ -551,8 +565,8 @@ def run_nonfused(torch, args, v_scale, m32=False, mgroup=False):
         "metric": "non-fused 4-bit AdamW step: params/sec, 1 MI355X", "value": n_total / dt,
         "unit": "params/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": dt * 1e3,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": f"fused=False, {'fp32 first moment, ' if m32 else ''}{'first-moment groups of 1024, ' if mgroup else ''}second moment '{v_scale}' scaling, "
-                               f"{ {'gpt2xl': 'GPT-2-XL-shaped', 'conv': 'wide-ResNet-152 convolution', 'llama7b': 'LLaMA-7B-shaped'}[args.shapes]} fp32 set", "qconfig": name,
+        "config": {"workload": f"fused=False, {'float16 parameters, ' if half else ''}{'fp32 first moment, ' if m32 else ''}{'first-moment groups of 1024, ' if mgroup else ''}second moment '{v_scale}' scaling, "
+                               f"{ {'gpt2xl': 'GPT-2-XL-shaped', 'conv': 'wide-ResNet-152 convolution', 'llama7b': 'LLaMA-7B-shaped'}[args.shapes]} {'fp16' if half else 'fp32'} set", "qconfig": name,
                    "tensors": len(params), "params": n_total},
         "roofline": {"bound": "hbm", "kernel": "whole step", "achieved": achieved, "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None,
@@ -565,6 +579,8 @@ def main():
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="llama7b", choices=sorted(WORKLOADS) + ["quant64m", "factored", "nonfused_group", "nonfused_rank1", "nonfused_group_m32", "nonfused_rank1_m32", "nonfused_rank1_mgroup", "sgd", "calibrate"])
+    ap.add_argument("--half", action="store_true",
+                    help="float16 parameters and gradients for --workload nonfused_group|nonfused_rank1")
     ap.add_argument("--bits", type=int, default=4, choices=range(1, 9),
                     help="code width of --workload quant64m (1-8) and nonfused_rank1 (4-8)")
     ap.add_argument("--shapes", default="llama7b", choices=["llama7b", "gpt2xl", "conv"],

@@ -393,6 +393,26 @@ class AdamW(LowBitOptimizer):
             _native.check(st, "non-fused 4-bit AdamW step (rank-1 second moment)")
             records.launched()
 
+        half_flat, half_rank1 = {}, {}  # float16 parameters
+
+        def launch_half_flat(key, records):
+            dev, qm_ptr, qv_ptr = key
+            table = np.array(records, dtype=_native.ADAMW4BIT_TENSOR)
+            with torch.cuda.device(dev):
+                st = lib.lpmm_nonfused_adamw4bit_f16_step_multi(table.ctypes.data, len(records), qm_ptr, qv_ptr, beta1,
+                                                                beta2, lr, wd, eps, _native.current_stream(dev))
+            _native.check(st, "non-fused 4-bit AdamW step on float16 parameters")
+
+        def launch_half_rank1(key, records):
+            dev, qm_ptr, qv_ptr = key
+            table = np.array(records, dtype=_native.NONFUSED_RANK1_F16_TENSOR)
+            with torch.cuda.device(dev):
+                st = lib.lpmm_nonfused_adamw4bit_rank1_f16_step_multi(table.ctypes.data, len(records), qm_ptr, qv_ptr,
+                                                                      beta1, beta2, lr, wd, eps,
+                                                                      _native.current_stream(dev))
+            _native.check(st, "non-fused 4-bit AdamW step on float16 parameters (rank-1 second moment)")
+            records.launched()
+
         def launch_group_m32(key, records):
             dev, qv_ptr = key
             table = np.array(records, dtype=_native.ADAMW_V4BIT_TENSOR)
@@ -436,7 +456,27 @@ class AdamW(LowBitOptimizer):
                 factored_work.append((p, grad, state, step))
                 continue
             if p.dtype in (torch.float16, torch.float64):
-                self._half_step(group, p, grad, state, step, md_m, md_v)
+                # float16 with the default kinds of states: the chain of half ops as one or two HIP passes
+                kind = self._half_kernel_kind(p, grad, state, m_group128, v_group128, v_rank1)
+                if kind is None:
+                    self._half_step(group, p, grad, state, step, md_m, md_v)
+                    continue
+                key = (p.device, state["exp_avg_qstate"]["qmap"].data_ptr(),
+                       state["exp_avg_sq_qstate"]["qmap"].data_ptr())
+                if kind == "flat":
+                    pending = half_flat.setdefault(key, [])
+                    pending.append(self._nonfused_record(p, p, grad, state, step, v_rank1))
+                    if len(pending) == _native.MULTI_MAX:
+                        launch_half_flat(key, pending)
+                        pending.clear()
+                else:
+                    pending = half_rank1.setdefault(key, _Batch())
+                    mc, ms = self._group_state(p, state, "exp_avg")
+                    pending.append((p.data_ptr(), grad.data_ptr(), mc, ms) + self._rank1_state_f16(p, state, pending)
+                                   + (p.shape[0], p.shape[1], step, 0.0))
+                    if len(pending) == _native.RANK1_MULTI_MAX:
+                        launch_half_rank1(key, pending)
+                        pending.clear()
                 continue
             dense, grad = self._dense_operands(p, grad, held)
             en_m, en_v = self._enabled(p, state, "exp_avg"), self._enabled(p, state, "exp_avg_sq")
@@ -554,6 +594,12 @@ class AdamW(LowBitOptimizer):
         for key, records in batched_rank1.items():
             if records:
                 launch_rank1(key, records)
+        for key, records in half_flat.items():
+            if records:
+                launch_half_flat(key, records)
+        for key, records in half_rank1.items():
+            if records:
+                launch_half_rank1(key, records)
         for key, records in batched_rank1_mgroup.items():
             if records:
                 launch_rank1_mgroup(key, records)
@@ -567,6 +613,59 @@ class AdamW(LowBitOptimizer):
             if records:
                 launch_rank1_m32(key, records)
         self._write_back(held)
+
+    def _half_kernel_kind(self, p, grad, state, m_group128, v_group128, v_rank1):
+        """Which HIP step takes a float16 parameter on the non-fused path: "flat" (one pass: both moments
+        block-wise over 128 values, a vector under 'rank1' included), "rank1" (two passes: a matrix with
+        a multiple of 128 columns), or None for the chain of PyTorch ops (float64, strided operands,
+        unquantised or differently scaled states, states whose scales are not halfs)."""
+        if p.dtype is not torch.float16 or grad.dtype is not torch.float16 or not (p.is_cuda and grad.is_cuda):
+            return None
+        if not (p.is_contiguous() and grad.is_contiguous() and m_group128):
+            return None
+        if not (self._enabled(p, state, "exp_avg") and self._enabled(p, state, "exp_avg_sq")):
+            return None
+        for name in ("exp_avg", "exp_avg_sq"):
+            if not _is_placeholder(state[name]):
+                oh = state[f"{name}_qstate"]["overhead"]
+                scales = [oh["max1"]] if oh.get("max1") is not None else list(oh.get("max_dims", ()))
+                if oh.get("dtype") is not torch.float16 or any(t.dtype is not torch.float16 for t in scales):
+                    return None
+        if v_group128 or (v_rank1 and p.dim() == 1):
+            return "flat"
+        if (v_rank1 and p.dim() == 2 and p.shape[1] % 128 == 0 and p.shape[0] > 0
+                and p.data_ptr() % 16 == 0 and grad.data_ptr() % 16 == 0):
+            return "rank1"
+        return None
+
+    def _rank1_state_f16(self, p, state, batch):
+        """_rank1_state for float16 parameters: half statistics, and a float work array in which the
+        kernels take the maxima of the new second moment (kept until the launch is enqueued)."""
+        rows, cols = p.shape
+        dev = p.device
+        qs_v = state["exp_avg_sq_qstate"]
+        if _is_placeholder(state["exp_avg_sq"]):
+            state["exp_avg_sq"] = torch.full((packed_nbytes(p.numel(), 4),), _zero_byte(qs_v["qmap"]),
+                                             dtype=torch.int8, device=dev)
+            qs_v["overhead"].clear()
+            qs_v["overhead"].update({"dtype": p.dtype, "stride": self._state_stride(p), "dim": 2, "max1": None,
+                                     "max_dims": [torch.zeros((rows, 1), dtype=torch.float16, device=dev),
+                                                  torch.zeros((1, cols), dtype=torch.float16, device=dev)],
+                                     "scaled_shape": p.shape})
+        oh = qs_v["overhead"]
+        cur = oh["max_dims"]
+        nxt = self._spare_stats.get(p)
+        if nxt is None or nxt[0].device != dev or nxt[0].dtype is not torch.float16:
+            nxt = [torch.empty_like(cur[0]), torch.empty_like(cur[1])]
+        work = torch.empty(((rows + 3) // 4 * 4 + cols,), dtype=torch.float32, device=dev)
+
+        def commit(work=work):  # holds the work array until the kernels are on the stream
+            self._spare_stats[p] = cur
+            oh["max_dims"] = nxt
+
+        batch.commits.append(commit)
+        return (state["exp_avg_sq"].data_ptr(), cur[0].data_ptr(), cur[1].data_ptr(), nxt[0].data_ptr(),
+                nxt[1].data_ptr(), work.data_ptr())
 
     def _half_step(self, group, p, grad, state, step, md_m, md_v):
         """float16 (and float64) parameters on the non-fused path.  The reference runs them through
@@ -626,7 +725,9 @@ class AdamW(LowBitOptimizer):
             oh = qstate["overhead"]
             oh.clear()
             oh.update({"dtype": p.dtype, "stride": self._state_stride(p),
-                       "max1": torch.zeros((groups, 1), dtype=torch.float32, device=p.device),
+                       # scales take the state's type (lpmm/functional.py:187: a maximum of the tensor's values)
+                       "max1": torch.zeros((groups, 1), device=p.device,
+                                           dtype=torch.float16 if p.dtype is torch.float16 else torch.float32),
                        "scaled_shape": torch.Size((groups, gp_sz))})
             if rank1_vector:  # the 'rank1' branch records the dimension count (lpmm/functional.py:191)
                 oh["dim"] = 1

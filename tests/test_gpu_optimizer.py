@@ -787,6 +787,68 @@ def test_half_parameters_on_the_nonfused_path(v_scale):
 
 
 @pytest.mark.parametrize("v_scale", ["rank1", "group"])
+def test_half_parameters_take_the_hip_step_kernels(oracle, qmaps, v_scale):
+    """float16 parameters with fused=False whose states have the default kinds (first moment block-wise
+    over 128 values, second moment block-wise or rank-1 on a matrix with a multiple of 128 columns) go
+    through the one- and two-pass HIP kernels: parameters, codes, half scales and half statistics bit
+    for bit against the oracle's float16 restatement of the reference's chain
+    (lpmm/optim/adamw.py:394-434), four steps, one optimizer holding matrices, a vector, a matrix that
+    stays with the chain of PyTorch ops (160 columns under 'rank1') and a tensor with half states."""
+    import lpmm
+
+    qm, qv = qmaps
+    rng = np.random.default_rng(31)
+    shapes = [(96, 256), (40, 1024), (11008,), (64, 160), (2000,)]
+    hyper = dict(lr=1e-2, betas=(0.9, 0.999), eps=1e-3, weight_decay=0.01)
+    host = [(rng.standard_normal(s) * 0.5).astype(np.float16) for s in shapes]
+    params = [torch.nn.Parameter(to_dev(h.copy())) for h in host]
+    cfg = os.path.join(os.path.dirname(lpmm.config.__file__), "configs",
+                       "default.yml" if v_scale == "rank1" else "2nd_moment_group_128.yml")
+    opt = lpmm.optim.AdamW(params, fused=False, qconfig=cfg, **hyper)
+    states = [oracle.NonFusedState(s, v_scale) for s in shapes[:4]]
+    exact = [0, 1, 2] if v_scale == "rank1" else [0, 1, 2, 3]  # tensors on the kernels
+
+    def same(got, want, what):
+        got, want = np.ascontiguousarray(got).reshape(-1), np.ascontiguousarray(want).reshape(-1)
+        assert got.dtype == want.dtype == np.float16, what
+        assert np.array_equal(got.view(np.uint16), want.view(np.uint16)), what
+
+    for step in range(1, 5):
+        grads = [(rng.standard_normal(s) * 0.3 * 10.0 ** (1 - step)).astype(np.float16) for s in shapes]
+        for p, g in zip(params, grads):
+            p.grad = to_dev(g)
+        opt.step()
+        torch.cuda.synchronize()
+        for i in exact:
+            oracle.nonfused_step_f16(host[i], grads[i], states[i], qm, qv, hyper["lr"], 0.9, 0.999, hyper["eps"], 0.01)
+            st = opt.state[params[i]]
+            what = f"step {step} tensor {i}"
+            same(to_np(params[i].detach()), host[i], what + ": p")
+            oh_m, oh_v = st["exp_avg_qstate"]["overhead"], st["exp_avg_sq_qstate"]["overhead"]
+            assert oh_m["dtype"] is torch.float16 and oh_v["dtype"] is torch.float16
+            same(to_np(oh_m["max1"]), states[i].m[1], what + ": m max1")
+            np.testing.assert_array_equal(to_np(st["exp_avg"]).view(np.uint8), states[i].m[0], err_msg=what + ": m codes")
+            np.testing.assert_array_equal(to_np(st["exp_avg_sq"]).view(np.uint8), states[i].v[0], err_msg=what + ": v codes")
+            if v_scale == "rank1" and len(shapes[i]) == 2:
+                assert oh_v["max1"] is None and oh_v["dim"] == 2
+                assert oh_v["max_dims"][0].shape == (shapes[i][0], 1) and oh_v["max_dims"][1].shape == (1, shapes[i][1])
+                same(to_np(oh_v["max_dims"][0]), states[i].v[1], what + ": row statistics")
+                same(to_np(oh_v["max_dims"][1]), states[i].v[2], what + ": column statistics")
+            else:
+                same(to_np(oh_v["max1"]), states[i].v[1], what + ": v max1")
+    assert all(torch.isfinite(p).all() for p in params)
+    # the states read back as the reference's metadata describes them: half tensors of the parameter's shape
+    from lpmm.functional import vectorwise_dequant
+
+    st = opt.state[params[0]]
+    kw = dict(st["exp_avg_qstate"]["overhead"])
+    kw.update(opt.get_qmetadata_by_state_name("exp_avg"))
+    m = vectorwise_dequant(st["exp_avg"], qmap=st["exp_avg_qstate"]["qmap"], shape=params[0].shape, **kw)
+    assert m.dtype is torch.float16 and m.shape == params[0].shape
+    same(to_np(m), oracle.dequant_group_f16(states[0].m[0], states[0].m[1], qm, host[0].size), "dequantised m")
+
+
+@pytest.mark.parametrize("v_scale", ["rank1", "group"])
 def test_double_parameters_on_the_nonfused_path(v_scale):
     """float64 parameters with fused=False: the reference's chain of PyTorch ops in double
     (lpmm/optim/adamw.py:394-434; its pack kernel rounds every normalised value to float before the
