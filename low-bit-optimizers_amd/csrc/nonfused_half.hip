@@ -56,9 +56,20 @@ __device__ __forceinline__ void half_second_moment(float &v, float g, const NfHy
     v = rh(v + (h.w2 * g) * g);
 }
 
-// One element of the chain; p, m and v (halfs held as floats) are updated in place.  The last division
-// is the IEEE one: float16 rounds the default eps of 1e-8 to zero, so the denominator of an element
-// whose second moment is zero is zero and the parameter becomes infinite or NaN, as in the reference.
+// x / d for a denominator that may be zero: float16 rounds the default eps of 1e-8 to zero, so the
+// denominator of an element whose second moment is zero is zero and the parameter becomes infinite or
+// NaN, as in the reference.  The quotient of the approximate reciprocal is already the IEEE result then
+// (x * inf); elsewhere the residual correction makes it the correctly rounded quotient (div_fast).
+__device__ __forceinline__ float div_maybe_zero(float x, float d)
+{
+    const float rc = __builtin_amdgcn_rcpf(d);
+    const float q = x * rc;
+    const float r = __builtin_fmaf(-q, d, x);
+    const float c = __builtin_fmaf(r, rc, q);
+    return d == 0.0f ? q : c;
+}
+
+// One element of the chain; p, m and v (halfs held as floats) are updated in place.
 __device__ __forceinline__ void half_elt(float &p, float g, float &m, float &v, const NfHyper &h)
 {
     const float pi = rh(p * h.decay);
@@ -67,7 +78,7 @@ __device__ __forceinline__ void half_elt(float &p, float g, float &m, float &v, 
     float d = rh(sqrt_fast(v));
     d = rh(div_by_rc(d, h.bc2_sqrt, h.rbc2_sqrt));
     d = rh(d + h.eps);
-    p = rh(pi + (h.neg_step_size * m) / d);
+    p = rh(pi + div_maybe_zero(h.neg_step_size * m, d));
 }
 
 // Codes of rh(v[k] / scale) for a lane's 8 values; |v[k]| <= scale wherever the scale is finite and
@@ -76,16 +87,17 @@ __device__ __forceinline__ uint32_t encode8_scaled_h(const uint32_t *lds, uint32
                                                      const float (&v)[kEltsPerLane], float scale)
 {
     float x[kEltsPerLane];
-    if (rc_safe(scale)) {
+    if (kind != kMapGeneric && rc_safe(scale)) {
+        // quotients in [-1, 1], no NaN: the closed forms of the standard maps apply as they are
         const float rc = rcp_exact(scale);
 #pragma unroll
         for (int k = 0; k < kEltsPerLane; ++k)
             x[k] = rh(div_by_rc(v[k], scale, rc));
-    } else {
-#pragma unroll
-        for (int k = 0; k < kEltsPerLane; ++k)
-            x[k] = rh(v[k] / scale);
+        return kind == kMapStdM ? encode8_std_m(lds, x) : encode8_std_v(x);
     }
+#pragma unroll
+    for (int k = 0; k < kEltsPerLane; ++k)
+        x[k] = rh(v[k] / scale);
     return encode8_plain(lds, lds_map, kind, x);
 }
 
@@ -401,6 +413,7 @@ __global__ __launch_bounds__(kThreads) void rank1_requant_half_kernel(const Mult
         }
         // every scale is a maximum over the values it divides: where all of the wave's scales lie in the
         // range in which the reciprocal is exact, one multiply and two fmas give the correctly rounded quotient
+        uint32_t ov;
         if (__all(cols_safe && rc_safe(rn))) {
             const float rcr = rcp_exact(rn);
 #pragma unroll
@@ -408,12 +421,14 @@ __global__ __launch_bounds__(kThreads) void rank1_requant_half_kernel(const Mult
                 const bool by_col = cn[k] < rn;
                 x[k] = rh(div_by_rc(v[k], by_col ? cn[k] : rn, by_col ? rcn[k] : rcr));
             }
+            // quotients in [0, 1]: the closed form of the standard map applies as it is
+            ov = kind_v == kMapStdV ? encode8_std_v(x) : encode8_plain(lds, kLdsQ1, kind_v, x);
         } else {
 #pragma unroll
             for (int k = 0; k < kEltsPerLane; ++k)
                 x[k] = rh(v[k] / ((cn[k] < rn) ? cn[k] : rn));
+            ov = encode8_plain(lds, kLdsQ1, kind_v, x);
         }
-        const uint32_t ov = encode8_plain(lds, kLdsQ1, kind_v, x);
         store_u16(vcp, ov & 0xFFFFu);
         store_u16(vcp + 16, ov >> 16);
     }
