@@ -60,6 +60,20 @@ int lpmm_adamw4bit_step(float *p, const float *g, uint8_t *m_codes, uint8_t *v_c
                         const float *qmap_v, int64_t n, float beta1, float beta2, float lr,
                         float weight_decay, float eps, float step, void *stream);
 
+/* The same operator on float16 tensors: the reference dispatches its 4-bit kernel on at::Half as
+ * well (fused_adamw_kernel.cu:222-230), with p, g and both scale arrays of that type and the
+ * maps float32 (fused_adamw.cc:60-65).  The instantiation rounds a map entry to half before it
+ * meets the scale ((T)qmap[idx] * scale, a product of halfs), rounds the moments and the
+ * parameter to half where they are assigned to T and computes everything else in float, the
+ * normalised values included (fused_adamw_kernel.cu:119-128, :148-167).
+ *   p, g            float16[n]
+ *   m_scale,v_scale float16[ceil(n/128)]
+ * Codes, maps and step as above.  p and g need 2-byte alignment, the code arrays too. */
+int lpmm_adamw4bit_f16_step(void *p, const void *g, uint8_t *m_codes, uint8_t *v_codes,
+                            void *m_scale, void *v_scale, const float *qmap_m,
+                            const float *qmap_v, int64_t n, float beta1, float beta2, float lr,
+                            float weight_decay, float eps, float step, void *stream);
+
 /* One record of a multi-tensor launch; the array of records is HOST memory. */
 typedef struct lpmm_adamw4bit_tensor {
     float *p;

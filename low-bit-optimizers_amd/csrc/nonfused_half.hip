@@ -123,10 +123,44 @@ struct MultiH {
     uint32_t tile_start[kHMax + 1];
     float decay, w1, b2, w2, eps;
 };
-static_assert(sizeof(MultiH) + 2 * sizeof(void *) <= 4096, "kernel arguments exceed 4 KB");
+static_assert(sizeof(MultiH) + sizeof(Hyper) + 2 * sizeof(void *) <= 4096, "kernel arguments exceed 4 KB");
 static_assert(kHMax <= kWave, "one tile_start entry per lane");
 
-__global__ __launch_bounds__(kThreads) void adamw4bit_half_kernel(const MultiH args, const float *__restrict__ qmap_m,
+// The lane's four code bytes of a group that the end of the tensor cuts, in the layout without padding
+// (bytes whose first element lies past the end do not exist): byte j = elements 2 (j & 1) + 64 (j >> 1)
+// + 4 lane16 and the one after it.
+__device__ __forceinline__ uint32_t load_codes_guarded(const uint8_t *codes, int64_t gbase, int lane16, int64_t n)
+{
+    uint32_t w = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int64_t e = gbase + lane16 * 4 + (j & 1) * 2 + (j >> 1) * 64;
+        if (e < n)
+            w |= (uint32_t)codes[e >> 1] << (8 * j);
+    }
+    return w;
+}
+
+__device__ __forceinline__ void store_codes_guarded(uint8_t *codes, int64_t gbase, int lane16, int64_t n, uint32_t w)
+{
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int64_t e = gbase + lane16 * 4 + (j & 1) * 2 + (j >> 1) * 64;
+        // an element past the end leaves its nibble 0 (lpmm/cpp_extension/fused_adamw_kernel.cu:148-167)
+        const uint32_t byte = (w >> (8 * j)) & (e + 1 < n ? 0xFFu : 0x0Fu);
+        if (e < n)
+            codes[e >> 1] = (uint8_t)byte;
+    }
+}
+
+// FUSED: the half instantiation of the reference's fused 4-bit operator
+// (lpmm/cpp_extension/fused_adamw_kernel.cu:80-174 with T = at::Half) instead of the chain of PyTorch
+// ops: codes and scales without padding, the map entry rounded to half before it meets the scale
+// ((T)qmap[idx] * scale, a product of halfs), moments and parameter rounded to half where the kernel
+// assigns them to T, everything else in float -- the normalised values included.
+template <bool FUSED>
+__global__ __launch_bounds__(kThreads) void adamw4bit_half_kernel(const MultiH args, const Hyper fh,
+                                                                 const float *__restrict__ qmap_m,
                                                                  const float *__restrict__ qmap_v)
 {
     __shared__ __align__(16) uint32_t lds[kLdsBytes / 4];
@@ -167,9 +201,14 @@ __global__ __launch_bounds__(kThreads) void adamw4bit_half_kernel(const MultiH a
         }
     }
     if (live) {
-        // the code buffers are padded to whole pack groups: always inside
-        wm = load_u16(mcp) | (load_u16(mcp + 16) << 16);
-        wv = load_u16(vcp) | (load_u16(vcp + 16) << 16);
+        if (!FUSED || full) {
+            // padded to whole pack groups (the chain's layout), or a whole group: always inside
+            wm = load_u16(mcp) | (load_u16(mcp + 16) << 16);
+            wv = load_u16(vcp) | (load_u16(vcp + 16) << 16);
+        } else {
+            wm = load_codes_guarded(t.mc, gbase, lane16, n);
+            wv = load_codes_guarded(t.vc, gbase, lane16, n);
+        }
         sm = (float)t.ms[grp];
         sv = (float)t.vs[grp];
     }
@@ -177,11 +216,13 @@ __global__ __launch_bounds__(kThreads) void adamw4bit_half_kernel(const MultiH a
     const int kind_m = classify_map(qmap_m), kind_v = classify_map(qmap_v);
     lds_barrier();
 
-    if (threadIdx.x == 0 && tile + 1 == tiles_in_tensor) {
+    if (!FUSED && threadIdx.x == 0 && tile + 1 == tiles_in_tensor) {
         // the tensor's last tile also owns the extra byte at the end of the code buffers
         t.mc[(int64_t)tiles_in_tensor * (kHTile / 2)] = 0;
         t.vc[(int64_t)tiles_in_tensor * (kHTile / 2)] = 0;
     }
+    if (FUSED && !live)
+        return;
     if (!live) {
         const float z[kEltsPerLane] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
         const uint32_t zm = encode8_plain(lds, kLdsQ0, kind_m, z), zv = encode8_plain(lds, kLdsQ1, kind_v, z);
@@ -206,18 +247,29 @@ __global__ __launch_bounds__(kThreads) void adamw4bit_half_kernel(const MultiH a
     float amax_m = 0.0f, amax_v = 0.0f;
 #pragma unroll
     for (int k = 0; k < kEltsPerLane; ++k) {
-        m[k] = rh(decode_nibble(lds, kLdsQ0, nm, k) * sm);
-        v[k] = rh(decode_nibble(lds, kLdsQ1, nv, k) * sv);
-        half_elt(pv[k], gv[k], m[k], v[k], h);
-        // elements past the end of the tensor are the zero padding of the quantiser
+        if (FUSED) {
+            m[k] = rh(rh(decode_nibble(lds, kLdsQ0, nm, k)) * sm);
+            v[k] = rh(rh(decode_nibble(lds, kLdsQ1, nv, k)) * sv);
+            adamw_moments(gv[k], m[k], v[k], fh);
+            m[k] = rh(m[k]);
+            v[k] = rh(v[k]);
+            pv[k] = rh(adamw_param(pv[k], m[k], v[k], fh));
+        } else {
+            m[k] = rh(decode_nibble(lds, kLdsQ0, nm, k) * sm);
+            v[k] = rh(decode_nibble(lds, kLdsQ1, nv, k) * sv);
+            half_elt(pv[k], gv[k], m[k], v[k], h);
+        }
+        // elements past the end of the tensor: the zero padding of the chain's quantiser; threads that
+        // the fused operator does not have
         if (!full && gbase + elt_offset(lane16, k) >= n)
             m[k] = v[k] = 0.0f;
         amax_m = fmaxf(amax_m, fabsf(m[k]));
         amax_v = fmaxf(amax_v, fabsf(v[k]));
     }
     row16_max2(amax_m, amax_v);
-    const uint32_t om = encode8_scaled_h(lds, kLdsQ0, kind_m, m, amax_m);
-    const uint32_t ov = encode8_scaled_h(lds, kLdsQ1, kind_v, v, amax_v);
+    // the chain normalises in half (x.div(max1) on half tensors), the fused operator in float
+    const uint32_t om = FUSED ? encode8_scaled(lds, kLdsQ0, kind_m, m, amax_m) : encode8_scaled_h(lds, kLdsQ0, kind_m, m, amax_m);
+    const uint32_t ov = FUSED ? encode8_scaled(lds, kLdsQ1, kind_v, v, amax_v) : encode8_scaled_h(lds, kLdsQ1, kind_v, v, amax_v);
     if (full) {
         store_h4(pp, narrow4(pv, 0));
         store_h4(pp + 64, narrow4(pv, 1));
@@ -229,10 +281,15 @@ __global__ __launch_bounds__(kThreads) void adamw4bit_half_kernel(const MultiH a
                 t.p[i] = (h16)pv[k];
         }
     }
-    store_u16(mcp, om & 0xFFFFu);
-    store_u16(mcp + 16, om >> 16);
-    store_u16(vcp, ov & 0xFFFFu);
-    store_u16(vcp + 16, ov >> 16);
+    if (!FUSED || full) {
+        store_u16(mcp, om & 0xFFFFu);
+        store_u16(mcp + 16, om >> 16);
+        store_u16(vcp, ov & 0xFFFFu);
+        store_u16(vcp + 16, ov >> 16);
+    } else {
+        store_codes_guarded(t.mc, gbase, lane16, n, om);
+        store_codes_guarded(t.vc, gbase, lane16, n, ov);
+    }
     if (lane16 == 0) {
         t.ms[grp] = (h16)amax_m;
         t.vs[grp] = (h16)amax_v;
@@ -463,11 +520,14 @@ __global__ __launch_bounds__(kThreads) void narrow_stats_kernel(const NarrowArgs
 
 using namespace lpmm;
 
-extern "C" int lpmm_nonfused_adamw4bit_f16_step_multi(const lpmm_adamw4bit_f16_tensor *tensors, int64_t count,
-                                                      const float *qmap_m, const float *qmap_v, double beta1,
-                                                      double beta2, double lr, double weight_decay, double eps,
-                                                      void *stream)
+// FUSED: the operator's arithmetic and layout on one tensor (float hyperparameters, as its signature has them)
+template <bool FUSED>
+static int half_step_multi(const lpmm_adamw4bit_f16_tensor *tensors, int64_t count, const float *qmap_m,
+                           const float *qmap_v, double beta1, double beta2, double lr, double weight_decay, double eps,
+                           void *stream)
 {
+    if (FUSED && count != 1)
+        return LPMM_ERR_ARG;
     if (count < 0)
         return LPMM_ERR_SIZE;
     if (count == 0)
@@ -503,6 +563,17 @@ extern "C" int lpmm_nonfused_adamw4bit_f16_step_multi(const lpmm_adamw4bit_f16_t
     args.b2 = c.b2;
     args.w2 = c.w2;
     args.eps = c.eps;
+    Hyper fh;
+    fh.beta1 = (float)beta1;
+    fh.beta2 = (float)beta2;
+    fh.omb1 = 1 - fh.beta1;  // formed in float, as the operator does
+    fh.omb2 = 1 - fh.beta2;
+    fh.lr = (float)lr;
+    fh.wd = (float)weight_decay;
+    fh.eps = (float)eps;
+    // bias corrections as the operator computes them per thread, in float
+    bias_corrections(fh.beta1, fh.beta2, FUSED ? tensors[0].step : 1.0f, &fh.c1, &fh.c2s);
+    fh.rc2s = 1.0f / fh.c2s;
     int64_t i = 0;
     while (i < count) {
         int k = 0;
@@ -538,13 +609,38 @@ extern "C" int lpmm_nonfused_adamw4bit_f16_step_multi(const lpmm_adamw4bit_f16_t
             continue;
         for (int j = k + 1; j <= kHMax; ++j)
             args.tile_start[j] = (uint32_t)tiles;
-        hipLaunchKernelGGL(adamw4bit_half_kernel, dim3((uint32_t)tiles), dim3(kThreads), 0, (hipStream_t)stream, args,
-                           qmap_m, qmap_v);
+        hipLaunchKernelGGL(adamw4bit_half_kernel<FUSED>, dim3((uint32_t)tiles), dim3(kThreads), 0, (hipStream_t)stream,
+                           args, fh, qmap_m, qmap_v);
         const int st = launch_status();
         if (st != LPMM_OK)
             return st;
     }
     return LPMM_OK;
+}
+
+extern "C" int lpmm_nonfused_adamw4bit_f16_step_multi(const lpmm_adamw4bit_f16_tensor *tensors, int64_t count,
+                                                      const float *qmap_m, const float *qmap_v, double beta1,
+                                                      double beta2, double lr, double weight_decay, double eps,
+                                                      void *stream)
+{
+    return half_step_multi<false>(tensors, count, qmap_m, qmap_v, beta1, beta2, lr, weight_decay, eps, stream);
+}
+
+extern "C" int lpmm_adamw4bit_f16_step(void *p, const void *g, uint8_t *m_codes, uint8_t *v_codes, void *m_scale,
+                                       void *v_scale, const float *qmap_m, const float *qmap_v, int64_t n, float beta1,
+                                       float beta2, float lr, float weight_decay, float eps, float step, void *stream)
+{
+    lpmm_adamw4bit_f16_tensor t;
+    t.p = p;
+    t.g = g;
+    t.m_codes = m_codes;
+    t.v_codes = v_codes;
+    t.m_max1 = m_scale;
+    t.v_max1 = v_scale;
+    t.n = n;
+    t.step = step;
+    t.reserved = 0.0f;
+    return half_step_multi<true>(&t, 1, qmap_m, qmap_v, beta1, beta2, lr, weight_decay, eps, stream);
 }
 
 extern "C" int lpmm_nonfused_adamw4bit_rank1_f16_step_multi(const lpmm_nonfused_rank1_f16_tensor *tensors, int64_t count,

@@ -28,6 +28,7 @@ PROTOTYPES = {
     "lpmm_status_string": (ctypes.c_char_p, [_int]),
     "lpmm_abi_version": (_int, []),
     "lpmm_adamw4bit_step": (_int, [_vp] * 8 + [_i64] + [_f] * 6 + [_vp]),
+    "lpmm_adamw4bit_f16_step": (_int, [_vp] * 8 + [_i64] + [_f] * 6 + [_vp]),
     "lpmm_adamw4bit_step_multi": (_int, [_vp, _i64, _vp, _vp] + [_f] * 5 + [_vp]),
     "lpmm_adamw_fp32_step": (_int, [_vp] * 4 + [_i64] + [_f] * 6 + [_vp]),
     "lpmm_adamw_fp32_step_multi": (_int, [_vp, _i64] + [_f] * 5 + [_vp]),

@@ -48,10 +48,14 @@ def adamw4bit_single_tensor(p, g, exp_avg, exp_avg_sq, exp_avg_scale, exp_avg_sq
     the reference's own check (fused_adamw.cc:68-71; a tensor with an odd number of elements
     therefore fails here exactly as it does there).  The scales must have one entry per 128
     elements (lpmm/cpp_extension/fused_adamw_kernel.cu:218-219)."""
-    check_cuda_tensor_float(p, "p")
-    check_cuda_tensor_float(g, "g")
-    check_cuda_tensor_float(exp_avg_scale, "exp_avg_scale")
-    check_cuda_tensor_float(exp_avg_sq_scale, "exp_avg_sq_scale")
+    # float32, or float16 as the reference's dispatch also instantiates (fused_adamw_kernel.cu:222): p, g and
+    # the scales then share that type (data_ptr<scalar_t>(), :224-230), the maps stay float32 (:231-232)
+    half = p.dtype is torch.float16
+    check_cuda_tensor_float(p, "p", fp32_only=not half)
+    for t, name in ((g, "g"), (exp_avg_scale, "exp_avg_scale"), (exp_avg_sq_scale, "exp_avg_sq_scale")):
+        check_cuda_tensor_float(t, name, fp32_only=not half)
+        if t.dtype != p.dtype:
+            raise RuntimeError(f"expected scalar type {p.dtype} but found {t.dtype} for {name}")
     check_cuda_tensor_float(exp_avg_qmap, "exp_avg_qmap")
     check_cuda_tensor_float(exp_avg_sq_qmap, "exp_avg_sq_qmap")
     n = p.numel()
@@ -74,7 +78,8 @@ def adamw4bit_single_tensor(p, g, exp_avg, exp_avg_sq, exp_avg_scale, exp_avg_sq
     dev = same_device(p, g, exp_avg, exp_avg_sq, exp_avg_scale, exp_avg_sq_scale, exp_avg_qmap,
                       exp_avg_sq_qmap)
     with torch.cuda.device(dev):
-        st = _native.lib().lpmm_adamw4bit_step(
+        step_fn = _native.lib().lpmm_adamw4bit_f16_step if half else _native.lib().lpmm_adamw4bit_step
+        st = step_fn(
             p.data_ptr(), g.data_ptr(), exp_avg.data_ptr(), exp_avg_sq.data_ptr(),
             exp_avg_scale.data_ptr(), exp_avg_sq_scale.data_ptr(), exp_avg_qmap.data_ptr(),
             exp_avg_sq_qmap.data_ptr(), n, beta1, beta2, lr, weight_decay, eps, step,

@@ -31,6 +31,10 @@
  *   nonfused_update_f16 PyTorch CPU op sequence on float16 tensors, bit for bit; the two
  *                       conversions against numpy.float16 on all 65536 halfs and on floats
  *                       around every rounding boundary.
+ *   adamw4bit_step_f16  equals adamw4bit_step with the map rounded to half on inputs whose
+ *                       later roundings vanish (states and gradients on a coarse binary grid,
+ *                       betas 0.5 and 0.75); a numpy.float16 restatement operation by operation.
+ *                       Against a real CUDA build of the half instantiation: parity unpinned.
  *   sgd_update          PyTorch CPU op sequence (library ops) of the reference's
  *                       _single_tensor_sgd4bit, bit for bit.
  *   philox / SR pack    Random123's known-answer vectors for philox4x32-10; torch.randint on
@@ -603,6 +607,71 @@ void lpmm_oracle_nonfused_update_f16(uint16_t *p, const uint16_t *g, uint16_t *m
         p[i] = f2h(pi + (neg_step_size * mi) / denom);      /* param.addcdiv_(exp_avg, denom, value=-step_size) */
         m[i] = f2h(mi);
         v[i] = f2h(vi);
+    }
+}
+
+/* ------------------------------------------------------------------------------------ */
+/* The fused 4-bit step instantiated on at::Half                                         */
+/* (lpmm/cpp_extension/fused_adamw_kernel.cu:80-174 with T = at::Half, dispatch :222).   */
+/* c10::Half arithmetic converts to float and back: Half * Half is the float product     */
+/* rounded to half, float * Half and Half / float are float; an assignment to T rounds.  */
+/*   T m = (T)qmap[idx] * scale[b];            map entry to half, product to half  (:119) */
+/*   m = beta1 * m + (1 - beta1) * g[i];       float, rounded on assignment        (:120) */
+/*   T v = (T)qmap[idx] * scale[b]; v = beta2 * v + (1 - beta2) * g[i] * g[i];   (:121-123) */
+/*   denom, update in float; p[i] = p[i] - lr * update rounded on the store      (:125-127) */
+/*   maxima and the normalised values (float)m / absmax in float                 (:148-157) */
+/*   scale[b] = (T)absmax: exact, a maximum of halfs                             (:169-170) */
+/* Layout as lpmm_oracle_adamw4bit_step; p, g and the scales are binary16 bit patterns.  */
+/* ------------------------------------------------------------------------------------ */
+void lpmm_oracle_adamw4bit_step_f16(uint16_t *p, const uint16_t *g, uint8_t *m_codes, uint8_t *v_codes,
+                                    uint16_t *m_scale, uint16_t *v_scale, const float *qmap_m,
+                                    const float *qmap_v, int64_t n, float beta1, float beta2,
+                                    float lr, float weight_decay, float eps, float step)
+{
+    const float correction1 = 1.0f - powf(beta1, step);
+    const float correction2_sqrt = sqrtf(1.0f - powf(beta2, step));
+    const int64_t blocks = (n + LPMM_GROUP - 1) / LPMM_GROUP;
+
+#pragma omp parallel for schedule(static)
+    for (int64_t b = 0; b < blocks; ++b) {
+        const int64_t base = b * LPMM_GROUP;
+        const int cnt = (int)((n - base) < LPMM_GROUP ? (n - base) : LPMM_GROUP);
+        float mm[LPMM_GROUP], vv[LPMM_GROUP];
+        float absmax_m = 0.0f, absmax_v = 0.0f;
+        const float sm = h2f(m_scale[b]), sv = h2f(v_scale[b]);
+
+        for (int k = 0; k < cnt; ++k) {
+            const int64_t i = base + k;
+            const uint8_t byte_m = m_codes[i >> 1], byte_v = v_codes[i >> 1];
+            const int sh = (int)(i & 1) * 4;
+            const float gi = h2f(g[i]), pi = h2f(p[i]);
+            float ea = rh(rh(qmap_m[(byte_m >> sh) & 0xF]) * sm);
+            ea = rh(beta1 * ea + (1 - beta1) * gi);
+            float es = rh(rh(qmap_v[(byte_v >> sh) & 0xF]) * sv);
+            es = rh(beta2 * es + (1 - beta2) * gi * gi);
+
+            float denom = (sqrtf(es) / correction2_sqrt + eps) * correction1;
+            float update = (ea / denom) + (weight_decay * pi);
+            p[i] = f2h(pi - (lr * update));
+
+            mm[k] = ea;
+            vv[k] = es;
+            absmax_m = fmaxf(absmax_m, fabsf(ea));
+            absmax_v = fmaxf(absmax_v, es);
+        }
+        for (int k = 0; k < cnt; k += 2) {
+            const int64_t i = base + k;
+            uint8_t bm = code4(qmap_m, mm[k] / absmax_m);
+            uint8_t bv = code4(qmap_v, vv[k] / absmax_v);
+            if (k + 1 < cnt) {
+                bm |= (uint8_t)(code4(qmap_m, mm[k + 1] / absmax_m) << 4);
+                bv |= (uint8_t)(code4(qmap_v, vv[k + 1] / absmax_v) << 4);
+            }
+            m_codes[i >> 1] = bm;
+            v_codes[i >> 1] = bv;
+        }
+        m_scale[b] = f2h(absmax_m);
+        v_scale[b] = f2h(absmax_v);
     }
 }
 

@@ -88,6 +88,8 @@ _nonfused_update = _sig("lpmm_oracle_nonfused_update", None, _f32p, _f32p, _f32p
 _u16p = np.ctypeslib.ndpointer(dtype=np.uint16, flags="C_CONTIGUOUS")
 _nonfused_update_f16 = _sig("lpmm_oracle_nonfused_update_f16", None, _u16p, _u16p, _u16p, _u16p, _i64,
                             _d, _d, _d, _d, _d, _d)
+_adamw4bit_f16 = _sig("lpmm_oracle_adamw4bit_step_f16", None, _u16p, _u16p, _u8p, _u8p, _u16p, _u16p,
+                      _f32p, _f32p, _i64, _f, _f, _f, _f, _f, _f)
 _f16_to_f32 = _sig("lpmm_oracle_f16_to_f32", None, _u16p, _f32p, _i64)
 _f32_to_f16 = _sig("lpmm_oracle_f32_to_f16", None, _f32p, _u16p, _i64)
 _sgd_update = _sig("lpmm_oracle_sgd_update", None, _f32p, _f32p, _f32p, _i64, _d, _d, _d, _d, ctypes.c_int,
@@ -660,3 +662,13 @@ def nonfused_step_f16(p, g, state, qm, qv, lr, beta1, beta2, eps, wd):
     else:
         state.v = quant_group_f16(v, qv)
     return m, v
+
+
+def adamw4bit_step_f16(p, g, m_codes, v_codes, m_scale, v_scale, qm, qv, beta1, beta2, lr, wd, eps, step):
+    """The fused 4-bit operator instantiated on half (lpmm/cpp_extension/fused_adamw_kernel.cu:80-174,
+    T = at::Half): p, g and the scales are float16 arrays, updated in place like the codes."""
+    for a in (p, g, m_scale, v_scale):
+        assert a.dtype == np.float16 and a.flags.c_contiguous
+    _adamw4bit_f16(p.reshape(-1).view(np.uint16), g.reshape(-1).view(np.uint16), m_codes, v_codes,
+                   m_scale.reshape(-1).view(np.uint16), v_scale.reshape(-1).view(np.uint16), _c(qm, np.float32),
+                   _c(qv, np.float32), p.size, beta1, beta2, lr, wd, eps, step)

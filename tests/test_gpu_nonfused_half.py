@@ -3,7 +3,8 @@ in one pass, rank-1 in two) against the CPU oracle's float16 restatement of the 
 (oracle.nonfused_step_f16: every op in float with one rounding to half, half scales and statistics),
 called through the C ABI on torch device memory.  Parameters, scales, statistics and the packed
 buffers are compared bit for bit, the buffers in full (padding codes and the extra last byte
-included); a NaN equals a NaN."""
+included); a NaN equals a NaN.  Last, the fused 4-bit operator's instantiation on half tensors against
+the oracle's restatement of it."""
 import numpy as np
 import pytest
 import torch
@@ -214,3 +215,45 @@ def test_half_steps_reject_bad_arguments(qmaps):
     assert matrix(okr[:7] + (stats[0].data_ptr(),) + okr[8:]) == 5  # the next statistics alias the current ones
     assert matrix((0,) + okr[1:]) == 1
     torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("n", [2048 * 3, 128 * 21 + 38, 100, 2])
+def test_fused_operator_on_half_tensors(oracle, qmaps, n):
+    """The reference-named operator on float16 p, g and scales (the at::Half instantiation of the fused
+    4-bit kernel, lpmm/cpp_extension/fused_adamw_kernel.cu:80-174, :222-230) against the oracle's
+    restatement of that instantiation: codes, half scales and parameters bit for bit over three steps;
+    whole tiles, a group that the end of the tensor cuts, fewer values than a group, one byte."""
+    from lpmm.cpp_extension import fused_adamw
+
+    qm, qv = qmaps
+    dqm, dqv = to_dev(qm), to_dev(qv)
+    rng = np.random.default_rng(51 + n)
+    nb, ng = n // 2, (n + 127) // 128
+    hp = (rng.standard_normal(n) * 0.1).astype(f16)
+    hmc, hvc = np.zeros(nb, np.uint8), np.zeros(nb, np.uint8)
+    hms, hvs = np.zeros(ng, f16), np.zeros(ng, f16)
+    p = to_dev(hp.copy())
+    mc, vc = to_dev(hmc.copy()), to_dev(hvc.copy())
+    ms, vs = to_dev(hms.copy()), to_dev(hvs.copy())
+    guard = to_dev(np.full(64, 0x5A, np.uint8))  # a small allocation made right after the codes: must stay as it is
+    hyper = (0.9, 0.999, 1e-3, 0.01, 1e-8)
+    for step in range(1, 4):
+        hg = (rng.standard_normal(n) * 0.05).astype(f16)
+        g = to_dev(hg)
+        fused_adamw.adamw4bit_single_tensor(p, g, mc, vc, ms, vs, dqm, dqv, *hyper, float(step))
+        torch.cuda.synchronize()
+        oracle.adamw4bit_step_f16(hp, hg, hmc, hvc, hms, hvs, qm, qv, *hyper, float(step))
+        what = f"n = {n}, step {step}"
+        np.testing.assert_array_equal(to_np(mc), hmc, err_msg=what + ": m codes")
+        np.testing.assert_array_equal(to_np(vc), hvc, err_msg=what + ": v codes")
+        _same_halfs(to_np(ms), hms, what + ": m scales")
+        _same_halfs(to_np(vs), hvs, what + ": v scales")
+        _same_halfs(to_np(p), hp, what + ": p")
+    assert np.all(to_np(guard) == 0x5A)
+    # types: the gradient and the scales share the parameter's type, the maps stay float32
+    with pytest.raises(RuntimeError, match="expected scalar type"):
+        fused_adamw.adamw4bit_single_tensor(p, g.float(), mc, vc, ms, vs, dqm, dqv, *hyper, 4.0)
+    with pytest.raises(RuntimeError, match="expected scalar type"):
+        fused_adamw.adamw4bit_single_tensor(p, g, mc, vc, ms.float(), vs, dqm, dqv, *hyper, 4.0)
+    with pytest.raises(RuntimeError, match="float32 is required"):
+        fused_adamw.adamw4bit_single_tensor(p, g, mc, vc, ms, vs, dqm.half(), dqv, *hyper, 4.0)

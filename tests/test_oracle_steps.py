@@ -539,3 +539,74 @@ def test_nonfused_half_step_is_the_torch_cpu_half_chain(oracle, qmaps, v_scale, 
                 assert same(states[i].v[1], rs["v"][1].numpy())
         if eps == 1e-3:
             assert all(np.isfinite(p).all() for p in ps)
+
+
+def test_fused_half_step_reduces_to_the_float_step(oracle):
+    """adamw4bit_step_f16 (the operator's at::Half instantiation) against the pinned float step.  With
+    maps, scales, states and gradients on a coarse binary grid and betas of 0.5 and 0.75 every moment
+    is exactly representable in half, so the roundings at the assignments change nothing: codes and
+    scales equal the float step's, and the parameter is the float step's rounded to half once.  A wrong
+    operand, bias correction, nibble or rounding point in the half restatement fails it."""
+    rng = np.random.default_rng(41)
+    qm = (np.arange(16) / 8 - 1).astype(f32)  # -1 ... 0.875, three fractional bits
+    qv = ((np.arange(16) + 1) / 16).astype(f32)
+    for n in (128 * 6, 128 * 3 + 70, 50):
+        nb, ng = (n + 1) // 2, (n + 127) // 128
+        mc = rng.integers(0, 256, nb, dtype=np.uint8)
+        vc = rng.integers(0, 256, nb, dtype=np.uint8)
+        ms, vs = np.full(ng, 0.25, f32), np.full(ng, 0.25, f32)
+        p = (rng.integers(-512, 512, n) / 1024).astype(f32)
+        g = (rng.integers(-16, 16, n) / 16).astype(f32)
+        ph, gh = p.astype(np.float16), g.astype(np.float16)
+        mch, vch, msh, vsh = mc.copy(), vc.copy(), ms.astype(np.float16), vs.astype(np.float16)
+        hyper = (0.5, 0.75, 1e-2, 0.0625, 1e-3, 3.0)
+        oracle.adamw4bit_step(p, g, mc, vc, ms, vs, qm, qv, *hyper)
+        oracle.adamw4bit_step_f16(ph, gh, mch, vch, msh, vsh, qm, qv, *hyper)
+        assert np.array_equal(mch, mc) and np.array_equal(vch, vc), n
+        assert np.array_equal(msh.astype(f32), ms) and np.array_equal(vsh.astype(f32), vs), n
+        assert np.array_equal(ph.view(np.uint16), p.astype(np.float16).view(np.uint16)), n
+
+
+def test_fused_half_step_against_numpy_half_arithmetic(oracle, qmaps):
+    """The same function on random states and gradients against numpy.float16 arithmetic, operation by
+    operation as c10::Half defines it (Half * Half: float product rounded to half; float * Half, Half /
+    float: float; assignment to T: one rounding): the map entries are rounded to half before the
+    product, the normalised values are not rounded, elements past the end leave their nibble 0."""
+    qm, qv = qmaps
+    rng = np.random.default_rng(42)
+    h16 = np.float16
+    b1, b2, lr, wd, eps, step = f32(0.9), f32(0.999), f32(1e-3), f32(0.01), f32(1e-8), f32(2.0)
+    for n in (128 * 5, 128 * 2 + 38):
+        nb, ng = (n + 1) // 2, (n + 127) // 128
+        mc, vc = rng.integers(0, 256, nb, dtype=np.uint8), rng.integers(0, 256, nb, dtype=np.uint8)
+        ms = np.abs(rng.standard_normal(ng) * 1e-2).astype(h16)
+        vs = np.abs(rng.standard_normal(ng) * 1e-3).astype(h16)
+        p = (rng.standard_normal(n) * 0.1).astype(h16)
+        g = (rng.standard_normal(n) * 0.05).astype(h16)
+        # numpy restatement
+        cm, cv = nibbles(mc, n), nibbles(vc, n)
+        grp = np.arange(n) // 128
+        m0 = (qm[cm].astype(h16) * ms[grp])  # half * half -> half
+        v0 = (qv[cv].astype(h16) * vs[grp])
+        gf = g.astype(f32)
+        m = (b1 * m0.astype(f32) + (f32(1) - b1) * gf).astype(h16)
+        v = (b2 * v0.astype(f32) + (f32(1) - b2) * gf * gf).astype(h16)
+        c1 = f32(1) - f32(np.float32(b1) ** step)
+        c2s = np.sqrt(f32(1) - f32(np.float32(b2) ** step), dtype=f32)
+        denom = (np.sqrt(v.astype(f32)) / c2s + eps) * c1
+        update = m.astype(f32) / denom + wd * p.astype(f32)
+        want_p = (p.astype(f32) - lr * update).astype(h16)
+        pad = np.zeros(ng * 128, f32)
+        pad[:n] = np.abs(m.astype(f32))
+        want_ms = pad.reshape(ng, 128).max(1)
+        pad[:n] = v.astype(f32)
+        want_vs = pad.reshape(ng, 128).max(1)
+        with np.errstate(invalid="ignore", divide="ignore"):
+            want_cm = oracle.qmapping(qm, m.astype(f32) / want_ms[grp])
+            want_cv = oracle.qmapping(qv, v.astype(f32) / want_vs[grp])
+        oracle.adamw4bit_step_f16(p, g, mc, vc, ms, vs, qm, qv, float(b1), float(b2), float(lr), float(wd), float(eps), float(step))
+        assert np.array_equal(p.view(np.uint16), want_p.view(np.uint16)), n
+        assert np.array_equal(ms.astype(f32), want_ms) and np.array_equal(vs.astype(f32), want_vs), n
+        assert np.array_equal(nibbles(mc, n), want_cm) and np.array_equal(nibbles(vc, n), want_cv), n
+        if n % 2:
+            assert mc[-1] >> 4 == 0 and vc[-1] >> 4 == 0
