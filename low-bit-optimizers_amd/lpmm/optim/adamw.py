@@ -626,6 +626,8 @@ class AdamW(LowBitOptimizer):
         if not (self._enabled(p, state, "exp_avg") and self._enabled(p, state, "exp_avg_sq")):
             return None
         for name in ("exp_avg", "exp_avg_sq"):
+            if state[f"{name}_qstate"]["qmap"].dtype is not torch.float32:
+                return None
             if not _is_placeholder(state[name]):
                 oh = state[f"{name}_qstate"]["overhead"]
                 scales = [oh["max1"]] if oh.get("max1") is not None else list(oh.get("max_dims", ()))

@@ -82,8 +82,8 @@ class LowBitOptimizer(torch.optim.Optimizer):
 
     def load_state_dict(self, state_dict):
         """Restore a state_dict().  Tensors move to their parameter's device; floating-point
-        state follows the parameter's dtype, except `step` and the packed int8 code tensors,
-        which are kept as they are (lpmm/optim/optimizer.py:73-136)."""
+        state follows the parameter's dtype, except `step`, the packed int8 code tensors and the
+        quantisation maps, which are kept as they are (lpmm/optim/optimizer.py:73-136)."""
         # any mapping with the reference's keys: the plain dict written by state_dict() above, a
         # config node of this package, or a yacs CfgNode (a dict subclass) from a reference checkpoint
         self.qconfig = config_from_mapping(state_dict["qconfig"])
@@ -101,6 +101,12 @@ class LowBitOptimizer(torch.optim.Optimizer):
             if isinstance(value, torch.Tensor):
                 if key == "step":
                     return value
+                if key == "qmap":
+                    # the maps stay float32 whatever the parameter's type: the kernels (here and in the
+                    # reference, lpmm/cpp_extension/quantization_kernel.cu:496, :648: data_ptr<float>()) read them as floats,
+                    # and a map rounded to half would decode the saved codes to other values.  The reference
+                    # casts them with the rest (:107-108) and cannot step float16 parameters after a load.
+                    return value.to(param.device)
                 if param.is_floating_point() and value.dtype != torch.int8:
                     value = value.to(param.dtype)
                 return value.to(param.device)

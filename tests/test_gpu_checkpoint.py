@@ -36,6 +36,9 @@ MODES = {
     "nonfused_group_fp32_m": dict(fused=False, qconfig="2nd_moment_only_group_128.yml"),
     "nonfused_rank1_m_group_512": dict(fused=False, qconfig="1st_moment_group_512.yml"),
     "nonfused_rank1_6bit": dict(fused=False, qconfig="default_6b.yml"),
+    # float16 parameters: the half step kernels (and, for the ragged and 3-D tensors, the chain of PyTorch ops)
+    "nonfused_rank1_half": dict(fused=False, qconfig="default.yml", half=True),
+    "nonfused_group_half": dict(fused=False, qconfig="2nd_moment_group_128.yml", half=True),
     "factored": dict(fused=False, factor_second_moment=True),
     "factored_fused": dict(fused=True, factor_second_moment=True),
 }
@@ -50,7 +53,10 @@ def _make(mode, params):
     kw = dict(MODES[mode])
     if "qconfig" in kw:
         kw["qconfig"] = _config(kw["qconfig"])
-    return lpmm.optim.AdamW(params, **H, **kw)
+    hyper = dict(H)
+    if kw.pop("half", False):
+        hyper["eps"] = 1e-3  # float16 rounds 1e-8 to zero
+    return lpmm.optim.AdamW(params, **hyper, **kw)
 
 
 def _flat_state(opt, params):
@@ -80,8 +86,10 @@ def test_resume_through_a_file_equals_uninterrupted_run(mode, map_location, tmp_
     else:
         shapes = SHAPES
     rng = np.random.default_rng(12)
-    start = [(rng.standard_normal(s) * 0.02).astype(np.float32) for s in shapes]
-    grads = [[(rng.standard_normal(s) * 1e-3).astype(np.float32) for s in shapes] for _ in range(6)]
+    dtype = np.float16 if MODES[mode].get("half") else np.float32
+    start = [(rng.standard_normal(s) * 0.02).astype(dtype) for s in shapes]
+    grads = [[(rng.standard_normal(s) * (3e-2 if dtype is np.float16 else 1e-3)).astype(dtype) for s in shapes]
+             for _ in range(6)]
 
     def run(opt, params, steps):
         for k in steps:

@@ -38,6 +38,8 @@ def test_record_layouts_match_header():
     assert _native.ADAMW4BIT_TENSOR.itemsize == 64 and _native.ADAMW_FP32_TENSOR.itemsize == 48
     assert _native.ADAMW4BIT_TENSOR.fields["n"][1] == 48 and _native.ADAMW4BIT_TENSOR.fields["step"][1] == 56
     assert _native.ADAMW_FP32_TENSOR.fields["n"][1] == 32 and _native.ADAMW_FP32_TENSOR.fields["step"][1] == 40
+    assert _native.NONFUSED_RANK1_F16_TENSOR.itemsize == 104 and _native.NONFUSED_RANK1_F16_TENSOR.fields["work"][1] == 72
+    assert _native.NONFUSED_RANK1_F16_TENSOR.fields["rows"][1] == 80 and _native.NONFUSED_RANK1_F16_TENSOR.fields["step"][1] == 96
     header = open(os.path.join(ROOT, "include", "lpmm_hip.h")).read()
     assert int(re.search(r"#define LPMM_MULTI_MAX (\d+)", header).group(1)) == _native.MULTI_MAX
 
@@ -224,6 +226,9 @@ def test_state_dict_round_trip_keeps_packed_int8():
     assert s2["exp_avg_sq"].dtype == torch.int8
     assert float(s2["step"]) == 3.0 and s2["step"].dtype == torch.float32
     assert s2["exp_avg_qstate"]["overhead"]["max1"].dtype == torch.float64  # float state follows the parameter
+    # ... except the maps: the kernels read them as floats, and a rounded map would decode the codes differently
+    assert s2["exp_avg_qstate"]["qmap"].dtype == torch.float32 and s2["exp_avg_sq_qstate"]["qmap"].dtype == torch.float32
+    assert torch.equal(s2["exp_avg_qstate"]["qmap"], state["exp_avg_qstate"]["qmap"])
     oh = s2["exp_avg_sq_qstate"]["overhead"]
     assert oh["scaled_shape"] == torch.Size((64, 65)) and oh["dtype"] == torch.float32 and oh["dim"] == 2
     assert isinstance(oh["max_dims"], list) and oh["max_dims"][1].shape == (1, 65)
