@@ -261,3 +261,47 @@ def test_rank1_nd_statistics_at_size(oracle, qmaps, shape):
     np.testing.assert_array_equal(to_np(codes).view(np.uint8), want_codes)
     back = F.vectorwise_dequant(codes, qmap=dq, shape=dx.shape, **{**gen, **md})
     np.testing.assert_array_equal(to_np(back), oracle.dequant_rank1_nd_bits(want_codes, want_stats, qmaps[1], 4, shape))
+
+
+@pytest.mark.parametrize("v_scale", ["rank1", "group"])
+def test_half_step_kernels_at_4096x11008(oracle, qmaps, v_scale):
+    """float16 parameters with fused=False at a LLaMA-7B MLP shape through the optimizer (the two-pass half
+    kernels under the default configuration, the one-pass kernel with a block-wise second moment) against
+    the oracle's float16 restatement of the reference's chain, two steps, bit for bit."""
+    import os
+
+    import lpmm
+
+    qm, qv = qmaps
+    shape = (4096, 11008)
+    rng = np.random.default_rng(77)
+    host = (rng.standard_normal(shape, dtype=np.float32) * 0.02).astype(np.float16)
+    p = torch.nn.Parameter(to_dev(host.copy()))
+    cfg = os.path.join(os.path.dirname(lpmm.config.__file__), "configs",
+                       "default.yml" if v_scale == "rank1" else "2nd_moment_group_128.yml")
+    hyper = dict(lr=1e-3, betas=(0.9, 0.999), eps=1e-3, weight_decay=0.01)
+    opt = lpmm.optim.AdamW([p], fused=False, qconfig=cfg, **hyper)
+    state = oracle.NonFusedState(shape, v_scale)
+
+    def same(got, want, what):
+        got, want = np.ascontiguousarray(got).reshape(-1), np.ascontiguousarray(want).reshape(-1)
+        assert got.dtype == want.dtype == np.float16, what
+        assert np.array_equal(got.view(np.uint16), want.view(np.uint16)), what
+
+    for step in (1, 2):
+        g = (rng.standard_normal(shape, dtype=np.float32) * 0.05).astype(np.float16)
+        p.grad = to_dev(g)
+        opt.step()
+        torch.cuda.synchronize()
+        oracle.nonfused_step_f16(host, g, state, qm, qv, hyper["lr"], 0.9, 0.999, hyper["eps"], 0.01)
+        st = opt.state[p]
+        same(to_np(p.detach()), host, f"step {step}: p")
+        same(to_np(st["exp_avg_qstate"]["overhead"]["max1"]), state.m[1], f"step {step}: m max1")
+        np.testing.assert_array_equal(to_np(st["exp_avg"]).view(np.uint8), state.m[0])
+        np.testing.assert_array_equal(to_np(st["exp_avg_sq"]).view(np.uint8), state.v[0])
+        oh_v = st["exp_avg_sq_qstate"]["overhead"]
+        if v_scale == "rank1":
+            same(to_np(oh_v["max_dims"][0]), state.v[1], f"step {step}: row statistics")
+            same(to_np(oh_v["max_dims"][1]), state.v[2], f"step {step}: column statistics")
+        else:
+            same(to_np(oh_v["max1"]), state.v[1], f"step {step}: v max1")
