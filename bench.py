@@ -19,7 +19,8 @@ Two further workloads measure the other kernels of the path with the same JSON s
 `--workload nonfused_group|nonfused_rank1` (fused=False on the LLaMA-7B-shaped set; with the suffix
 `_m32` under the configurations that quantise the second moment only: fp32 first moment;
 `nonfused_rank1_mgroup`: first-moment groups of 1024 values; `nonfused_rank1 --bits 5..8`: the
-configurations with wider codes) and
+configurations with wider codes; `--shapes gpt2xl|conv`: the GPT-2-XL-shaped set or the convolution
+weights of a wide ResNet-152 instead; `--half`: float16 parameters and gradients) and
 `--workload sgd` (4-bit SGD momentum on the same set).
 """
 import argparse
