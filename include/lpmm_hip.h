@@ -367,7 +367,8 @@ int lpmm_nonfused_adamw4bit_rank1_pass_multi(const lpmm_nonfused_rank1_tensor *t
  * statistics the v codes are scaled by, v_rowmax_next / v_colmax_next receive those of the new
  * second moment (must not alias the current ones: the caller swaps the pairs); `work` is scratch
  * of ((R + 3) / 4 * 4 + C) floats, 16-byte aligned, whose contents do not matter before and
- * after the call.  p and g 16-byte aligned. */
+ * after the call.  p, g and v_colmax 16-byte aligned, the code arrays, m_max1 and v_rowmax 4-byte,
+ * the next statistics 2-byte. */
 typedef struct lpmm_adamw4bit_f16_tensor {
     void *p;
     const void *g;
