@@ -1,5 +1,6 @@
-// Non-fused AdamW step on float16 parameters with 4-bit states: the one-pass kernel for a block-wise
-// second moment and the two passes for the rank-1 second moment.
+// AdamW steps on float16 parameters with 4-bit states: the non-fused step as one pass (block-wise second
+// moment) and as two passes (rank-1 second moment), and the fused operator's half instantiation (the
+// one-pass kernel with that operator's arithmetic and layout, adamw4bit_half_kernel<true>).
 //
 // With fused=False the reference runs its chain of PyTorch ops in the parameters' type
 // (lpmm/optim/adamw.py:367-369, :394-434): every op converts its half operands to float, computes as
