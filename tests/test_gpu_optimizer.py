@@ -848,6 +848,42 @@ def test_half_parameters_take_the_hip_step_kernels(oracle, qmaps, v_scale):
     same(to_np(m), oracle.dequant_group_f16(states[0].m[0], states[0].m[1], qm, host[0].size), "dequantised m")
 
 
+def test_half_and_float_parameters_in_one_group(oracle, qmaps):
+    """A parameter group that holds float16 and float32 tensors (fused=False, default configuration): each
+    goes to the kernels of its type, and both match their oracles bit for bit over three steps."""
+    import lpmm
+
+    qm, qv = qmaps
+    rng = np.random.default_rng(33)
+    shape = (64, 256)
+    hyper = dict(lr=1e-2, betas=(0.9, 0.999), eps=1e-3, weight_decay=0.01)
+    host_h = (rng.standard_normal(shape) * 0.5).astype(np.float16)
+    host_f = (rng.standard_normal(shape) * 0.5).astype(np.float32)
+    ph, pf = torch.nn.Parameter(to_dev(host_h.copy())), torch.nn.Parameter(to_dev(host_f.copy()))
+    opt = lpmm.optim.AdamW([pf, ph], fused=False, **hyper,
+                           qconfig=os.path.join(os.path.dirname(lpmm.config.__file__), "configs", "default.yml"))
+    st_h, st_f = oracle.NonFusedState(shape, "rank1"), oracle.NonFusedState(shape, "rank1")
+    for step in range(1, 4):
+        gh = (rng.standard_normal(shape) * 0.1).astype(np.float16)
+        gf = (rng.standard_normal(shape) * 0.1).astype(np.float32)
+        ph.grad, pf.grad = to_dev(gh), to_dev(gf)
+        opt.step()
+        torch.cuda.synchronize()
+        oracle.nonfused_step_f16(host_h, gh, st_h, qm, qv, hyper["lr"], 0.9, 0.999, hyper["eps"], 0.01)
+        oracle.nonfused_step(host_f, gf, st_f, qm, qv, hyper["lr"], 0.9, 0.999, hyper["eps"], 0.01)
+        assert np.array_equal(to_np(ph.detach()).view(np.uint16), host_h.view(np.uint16)), step
+        assert_params(to_np(pf.detach()), host_f, host_f, f"float parameter, step {step}")
+        for p, st in ((ph, st_h), (pf, st_f)):
+            s = opt.state[p]
+            np.testing.assert_array_equal(to_np(s["exp_avg"]).view(np.uint8), st.m[0])
+            np.testing.assert_array_equal(to_np(s["exp_avg_sq"]).view(np.uint8), st.v[0])
+            dims = s["exp_avg_sq_qstate"]["overhead"]["max_dims"]
+            assert dims[0].dtype is p.dtype and s["exp_avg_qstate"]["overhead"]["max1"].dtype is p.dtype
+            np.testing.assert_array_equal(to_np(dims[0]).reshape(-1), st.v[1])
+            np.testing.assert_array_equal(to_np(dims[1]).reshape(-1), st.v[2])
+        pf.data.copy_(torch.from_numpy(host_f))  # the float update is near-exact: continue from the oracle's values
+
+
 @pytest.mark.parametrize("v_scale", ["rank1", "group"])
 def test_double_parameters_on_the_nonfused_path(v_scale):
     """float64 parameters with fused=False: the reference's chain of PyTorch ops in double
