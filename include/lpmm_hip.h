@@ -201,8 +201,9 @@ int lpmm_rank1_row_scale_nd(const float *const *stats, int ndim, const int64_t *
  * vector's dimensions, in one launch for up to 32 vectors -- what lies between the two passes of
  * lpmm_nonfused_adamw4bit_rank1_pass_multi for tensors of more than two dimensions, whose trailing
  * dimensions are the vector's.  ndim 1..7, at most 8192 statistics entries per vector (the sum of
- * its dimensions), fewer than 2^31 elements; records live in host memory and are consumed during
- * the call. */
+ * its dimensions), fewer than 2^31 elements; one workgroup works through a vector, so the call
+ * is for vectors of thousands of values (a long one is better served by the two calls it stands
+ * for); records live in host memory and are consumed during the call. */
 typedef struct lpmm_rank1_small_vector {
     const float *x;
     float *scale;

@@ -11,6 +11,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "liblpmm_hip.so")
 MULTI_MAX = 48  # tensors per launch of the fused step (LPMM_MULTI_MAX in include/lpmm_hip.h)
 RANK1_SMALL_SLOTS = 8192  # statistics entries of a vector lpmm_rank1_small_fold_scale_multi takes (kNdSmallSlots)
+RANK1_SMALL_VALUES = 1 << 16  # longest vector worth the single workgroup that call gives it
 RANK1_MULTI_MAX = 32  # tensors per launch of the two-pass rank-1 step (kR1Max in csrc/nonfused_rank1.hip)
 SGD_MULTI_MAX = 64  # tensors per launch of the one-pass SGD step (kSgdMax in csrc/sgd.hip)
 V4BIT_MULTI_MAX = 48  # tensors per launch of the one-pass step with an fp32 first moment (kV4Max in csrc/nonfused_m32.hip)

@@ -842,7 +842,9 @@ class AdamW(LowBitOptimizer):
                     small = []
                     for p, nxt, raw, scale, trailing in between:
                         dims = tuple(p.shape[1:])
-                        if sum(dims) <= _native.RANK1_SMALL_SLOTS:
+                        # one workgroup per vector: for the few thousand values of a convolution weight's
+                        # trailing dimensions, not for the millions of a stack of matrices
+                        if sum(dims) <= _native.RANK1_SMALL_SLOTS and raw.numel() <= _native.RANK1_SMALL_VALUES:
                             pad = 7 - len(dims)
                             small.append((raw.data_ptr(), scale.data_ptr(), tuple(t.data_ptr() for t in nxt[1:]) + (0,) * pad,
                                           dims + (1,) * pad, len(dims), 0))
