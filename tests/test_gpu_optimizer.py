@@ -188,6 +188,7 @@ def test_nonfused_rank1_on_tensors_of_more_than_two_dimensions(oracle, qmaps):
     # 128 with an even shape[0]: double rows), the last two the staged path
     shapes = [(6, 40, 64), (64, 64, 3, 3), (16, 4, 8, 32), (12, 3, 128), (6, 2, 4, 4, 32), (32, 16, 3, 3), (4, 24, 130)]
     shapes += [(48, 16, 3, 3), (16, 8, 8, 8)] * 15  # 35 tensors on the two passes: more than one launch holds
+    shapes += [(4, 300, 256)]  # trailing dimensions of 76800 values: folded by the general statistics kernels
     host, params = _params(shapes, rng)
     cfg = os.path.join(os.path.dirname(lpmm.config.__file__), "configs", "default.yml")
     opt = lpmm.optim.AdamW(params, fused=False, qconfig=cfg, **H)
