@@ -35,6 +35,20 @@ def _two_pass_columns(rows, cols):
     return cols % 128 == 0 or (cols % 128 == 64 and rows % 2 == 0)
 
 
+def _two_pass_nd(shape):
+    """Tensors of more than two dimensions that take the two passes on their shape[0] x rest view.  The
+    kernels' tiles are 64 rows tall: a large tensor with a handful of rows (a stack of a few matrices)
+    fills an eighth of every tile and pays one column atomic per few elements -- measured 1.20 against
+    0.47 ms for 3 x 4096 x 4096 and 0.66 against 0.58 ms for 8 x 2048 x 4096, level at 16 rows -- so it
+    stays with the staged path; small tensors gain from the batched launches whatever their shape."""
+    rows, numel = shape[0], 1
+    for d in shape:
+        numel *= d
+    if rows == 0 or not _two_pass_columns(rows, numel // rows):
+        return False
+    return rows >= 16 or numel <= (1 << 20)
+
+
 def _is_placeholder(t):
     # a state that has not been materialised yet is a 0-dim tensor (adamw.py:121, :128);
     # the reference tests numel() <= 1 (adamw.py:394, :402, :509, :544)
@@ -491,7 +505,7 @@ class AdamW(LowBitOptimizer):
                         launch_group(key, pending)
                         pending.clear()
                     continue
-                if v_rank1 and 2 < p.dim() <= RANK1_ND_MAX and _two_pass_columns(p.shape[0], p.numel() // p.shape[0]):
+                if v_rank1 and 2 < p.dim() <= RANK1_ND_MAX and _two_pass_nd(p.shape):
                     # a convolution weight and its like, viewed as shape[0] x the rest
                     nd_work.setdefault(key, []).append((p, dense, grad, state, step))
                     continue
