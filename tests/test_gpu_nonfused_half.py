@@ -89,6 +89,8 @@ def test_one_pass_half_step(oracle, qmaps, eps):
                _Flat(oracle, 11008, rng, offset=1), _Flat(oracle, 2048 * 2 + 128, rng, offset=3)]
     for step in range(1, 5):
         grads = [(rng.standard_normal(t.n) * 0.3 * 10.0 ** -step).astype(f16) for t in tensors]
+        grads[0][128:384] = 0  # two groups that never see a gradient: scale 0, 0 / 0 -> the NaN code throughout
+        grads[1][4992:] = 0    # ... and the partial last group of a ragged tensor
         records = [t.record(g, step) for t, g in zip(tensors, grads)]
         table = np.array(records, dtype=nat.ADAMW4BIT_TENSOR)
         st = lib.lpmm_nonfused_adamw4bit_f16_step_multi(table.ctypes.data, len(records), dqm.data_ptr(), dqv.data_ptr(),
@@ -104,6 +106,8 @@ def test_one_pass_half_step(oracle, qmaps, eps):
         assert all(np.isfinite(t.host_p).all() for t in tensors)
     else:
         assert any(not np.isfinite(t.host_p).all() for t in tensors)
+    st = tensors[0].state
+    assert st.m[1][1] == 0 and st.v[1][2] == 0 and np.all(st.m[0][64:192] == 0xFF) and np.all(st.v[0][64:192] == 0xFF)
 
 
 class _Matrix:
