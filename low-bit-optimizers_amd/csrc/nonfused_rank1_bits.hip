@@ -92,21 +92,52 @@ __global__ __launch_bounds__(kThreads) void rank1_update_bits_kernel(const Multi
         uint32_t *red = colred + slot * kRedSlotWords + lane16;
         float co[kEltsPerLane];
         unpack8(*reinterpret_cast<const float4 *>(cop), *reinterpret_cast<const float4 *>(cop + 64), co);
+        // the operands of a pass are requested one pass ahead, so that a wave has two passes' loads in
+        // flight (LLaMA-7B-shaped set, 8 bits: 24.9-25.1 -> 24.5-24.6 ms per step)
+        struct Fetch {
+            float4 a0, a1, b0, b1;
+            uint32_t wm0, wm1, wv0, wv1;
+            float sm, ro;
+        };
+        auto fetch = [&](int it) {
+            Fetch x;
+            const int64_t r = q.row0 + it * q.step;
+            const int64_t grp = r * t.col_blocks + q.cg;
+            const int64_t gbase = grp * kGroup;
+            const float *pp = t.p + gbase + lane16 * 4;
+            const float *gp = t.g + gbase + lane16 * 4;
+            const uint32_t *mcp = reinterpret_cast<const uint32_t *>(t.mc + gbase) + lane16;
+            const uint32_t *vcp = reinterpret_cast<const uint32_t *>(t.vc + gbase) + lane16;
+            x.a0 = load4(pp);
+            x.a1 = load4(pp + 64);
+            x.b0 = load4(gp);
+            x.b1 = load4(gp + 64);
+            x.wm0 = load_u32(mcp);
+            x.wm1 = load_u32(mcp + 16);
+            x.wv0 = load_u32(vcp);
+            x.wv1 = load_u32(vcp + 16);
+            x.sm = t.ms[grp];
+            x.ro = t.row_old[r];
+            return x;
+        };
+        Fetch nxt;
+        if (q.row0 < t.rows)
+            nxt = fetch(0);
 #pragma unroll 1
         for (int it = 0; it < q.passes; ++it) {
             const int64_t r = q.row0 + it * q.step;
             if (r >= t.rows)
                 break;
+            const Fetch cur = nxt;
+            if (it + 1 < q.passes && r + q.step < t.rows)
+                nxt = fetch(it + 1);
             const int64_t grp = r * t.col_blocks + q.cg;
             const int64_t gbase = grp * kGroup;
             float *pp = t.p + gbase + lane16 * 4;
-            const float *gp = t.g + gbase + lane16 * 4;
             uint32_t *mcp = reinterpret_cast<uint32_t *>(t.mc + gbase) + lane16;
-            const uint32_t *vcp = reinterpret_cast<const uint32_t *>(t.vc + gbase) + lane16;
-            const float4 a0 = load4(pp), a1 = load4(pp + 64), b0 = load4(gp), b1 = load4(gp + 64);
-            const uint32_t wm0 = load_u32(mcp), wm1 = load_u32(mcp + 16);
-            const uint32_t wv0 = load_u32(vcp), wv1 = load_u32(vcp + 16);
-            const float sm = t.ms[grp], ro = t.row_old[r];
+            const float4 a0 = cur.a0, a1 = cur.a1, b0 = cur.b0, b1 = cur.b1;
+            const uint32_t wm0 = cur.wm0, wm1 = cur.wm1, wv0 = cur.wv0, wv1 = cur.wv1;
+            const float sm = cur.sm, ro = cur.ro;
             float pv[kEltsPerLane], gv[kEltsPerLane], m[kEltsPerLane], v[kEltsPerLane];
             unpack8(a0, a1, pv);
             unpack8(b0, b1, gv);
