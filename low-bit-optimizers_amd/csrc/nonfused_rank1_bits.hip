@@ -13,7 +13,7 @@ namespace lpmm {
 // caller passes one, or by the closed form of the evenly spaced map (the second moment's in every
 // shipped configuration; lpmm_search.hpp).  Same tiles and statistics as above; a lane's eight
 // codes are two dwords.  21.06 bytes per parameter cross HBM (p 8, g 4 + 4, m codes 2, v codes
-// 1 + 2, scales).  LLaMA-7B-shaped set: 25.0 ms per step with 5 bits, 25.3 ms with 8 (the staged
+// 1 + 2, scales).  LLaMA-7B-shaped set: 24.2 ms per step with 5 bits, 24.4 ms with 8 (the staged
 // path 67.6 ms).  Both passes run within 5 % of the rate of their 4-bit counterparts per byte:
 // with the arithmetic taken out, with the table instead of the search and with 8-byte instead of
 // 4-byte code accesses they take the same time -- the tile structure sets it, not the codes.
