@@ -261,3 +261,63 @@ def test_fused_operator_on_half_tensors(oracle, qmaps, n):
         fused_adamw.adamw4bit_single_tensor(p, g, mc, vc, ms.float(), vs, dqm, dqv, *hyper, 4.0)
     with pytest.raises(RuntimeError, match="float32 is required"):
         fused_adamw.adamw4bit_single_tensor(p, g, mc, vc, ms, vs, dqm.half(), dqv, *hyper, 4.0)
+
+
+@pytest.mark.parametrize("eps", [1e-3, 1e-8])
+def test_one_pass_half_step_on_every_gradient_value(oracle, qmaps, eps):
+    """Every float16 gradient of magnitude up to 256 (subnormals and both zeros included; beyond that the
+    second moment overflows in half), in shuffled order, on states that three ordinary steps have filled:
+    parameters, codes and scales bit for bit.  The sweep takes the square root, the two divisions and the
+    encoders of the kernel through 46 octaves of second moments, down to the ones that underflow to zero."""
+    nat = _native()
+    lib = nat.lib()
+    qm, qv = qmaps
+    dqm, dqv = to_dev(qm), to_dev(qv)
+    rng = np.random.default_rng(61)
+    mags = np.arange(0, 0x5C01, dtype=np.uint16)  # 0 ... 256.0
+    sweep = np.concatenate([mags, mags | 0x8000]).view(f16)
+    reps = 3
+    t = _Flat(oracle, sweep.size * reps, rng)
+    hyper = dict(lr=1e-2, beta1=0.9, beta2=0.999, wd=0.01)
+    for step in range(1, 6):
+        if step <= 3:
+            g = (rng.standard_normal(t.n) * 0.3).astype(f16)
+        else:
+            g = np.concatenate([rng.permutation(sweep) for _ in range(reps)])
+        table = np.array([t.record(g, step)], dtype=nat.ADAMW4BIT_TENSOR)
+        st = lib.lpmm_nonfused_adamw4bit_f16_step_multi(table.ctypes.data, 1, dqm.data_ptr(), dqv.data_ptr(),
+                                                        hyper["beta1"], hyper["beta2"], hyper["lr"], hyper["wd"], eps,
+                                                        nat.current_stream(torch.device("cuda:0")))
+        assert st == 0
+        torch.cuda.synchronize()
+        oracle.nonfused_step_f16(t.host_p, g, t.state, qm, qv, hyper["lr"], hyper["beta1"], hyper["beta2"], eps,
+                                 hyper["wd"])
+        t.check(f"step {step}")
+    assert np.isfinite(t.state.v[1].astype(np.float32)).all() and float(t.state.v[1].max()) > 50.0
+
+
+def test_fused_operator_on_every_half_gradient_value(oracle, qmaps):
+    """The same sweep through the fused operator's half instantiation (float eps: no division by zero)."""
+    from lpmm.cpp_extension import fused_adamw
+
+    qm, qv = qmaps
+    dqm, dqv = to_dev(qm), to_dev(qv)
+    rng = np.random.default_rng(62)
+    mags = np.arange(0, 0x5C01, dtype=np.uint16)
+    sweep = np.concatenate([mags, mags | 0x8000]).view(f16)
+    n = sweep.size * 2
+    nb, ng = n // 2, (n + 127) // 128
+    hp = (rng.standard_normal(n) * 0.1).astype(f16)
+    hmc, hvc, hms, hvs = np.zeros(nb, np.uint8), np.zeros(nb, np.uint8), np.zeros(ng, f16), np.zeros(ng, f16)
+    p, mc, vc, ms, vs = (to_dev(a.copy()) for a in (hp, hmc, hvc, hms, hvs))
+    hyper = (0.9, 0.999, 1e-3, 0.01, 1e-8)
+    for step in range(1, 5):
+        hg = (rng.standard_normal(n) * 0.05).astype(f16) if step <= 2 else np.concatenate([rng.permutation(sweep) for _ in range(2)])
+        fused_adamw.adamw4bit_single_tensor(p, to_dev(hg), mc, vc, ms, vs, dqm, dqv, *hyper, float(step))
+        torch.cuda.synchronize()
+        oracle.adamw4bit_step_f16(hp, hg, hmc, hvc, hms, hvs, qm, qv, *hyper, float(step))
+        np.testing.assert_array_equal(to_np(mc), hmc, err_msg=f"step {step}: m codes")
+        np.testing.assert_array_equal(to_np(vc), hvc, err_msg=f"step {step}: v codes")
+        _same_halfs(to_np(ms), hms, f"step {step}: m scales")
+        _same_halfs(to_np(vs), hvs, f"step {step}: v scales")
+        _same_halfs(to_np(p), hp, f"step {step}: p")
